@@ -1,0 +1,77 @@
+// Shared host-side helpers of the device layer: error capture, handle types, dtype helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include "../../include/gpreempt_hip.h"
+#include "tile_loop.hpp"
+
+struct gp_stream_s { hipStream_t s; int priority; };
+struct gp_event_s { hipEvent_t e; };
+struct gp_graph_s { hipGraph_t g; hipGraphExec_t x; };
+
+namespace gp {
+
+void set_error(const char *fmt, ...);
+int device_cus();
+
+#define GP_HIP(call)                                                                           \
+    do {                                                                                       \
+        hipError_t e_ = (call);                                                                \
+        if (e_ != hipSuccess) {                                                                \
+            gp::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__, __LINE__); \
+            return GP_FAIL;                                                                    \
+        }                                                                                      \
+    } while (0)
+
+#define GP_REQUIRE(cond, ...)                                                                  \
+    do {                                                                                       \
+        if (!(cond)) {                                                                         \
+            gp::set_error(__VA_ARGS__);                                                        \
+            return GP_OUTOFRANGE;                                                              \
+        }                                                                                      \
+    } while (0)
+
+inline hipStream_t native(gp_stream s) { return s ? s->s : nullptr; }
+
+inline size_t dtype_size(int dt) {
+    switch (dt) {
+        case GP_F32: return 4; case GP_F16: return 2; case GP_BF16: return 2;
+        case GP_I32: return 4; case GP_I64: return 8; default: return 0;
+    }
+}
+
+// Resolves the launch geometry of one preemptible kernel, as Model::add_block_preemption_param
+// does in the reference (src/model.cpp:366-396): total_block = sx*sy*sz; persistent grid =
+// min(total_block, resident workgroups the device can hold); a NULL context keeps one
+// workgroup per tile.
+template <class Kernel>
+int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int sz,
+                const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info) {
+    long total = (long)sx * sy * sz;
+    GP_REQUIRE(total > 0 && total < (1L << 31), "tile count %ld out of range", total);
+    blp->total = (int)total; blp->sx = sx; blp->sy = sy;
+    if (ctx) {
+        GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
+        blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;
+        blp->kernel_id = ctx->kernel_id; blp->inject_at = ctx->inject_at;
+        int per_cu = 0;
+        GP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, lds_bytes));
+        if (per_cu < 1) per_cu = 1;
+        long resident = (long)per_cu * device_cus();
+        if (ctx->max_workgroups > 0 && resident > ctx->max_workgroups) resident = ctx->max_workgroups;
+        *grid = (int)(total < resident ? total : resident);
+    } else {
+        blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
+        blp->kernel_id = 0; blp->inject_at = -1;
+        *grid = (int)total;
+    }
+    if (info) {
+        info->total_tiles = (int)total; info->shape[0] = sx; info->shape[1] = sy; info->shape[2] = sz;
+        info->grid = *grid; info->block = block;
+    }
+    return GP_SUCC;
+}
+
+}  // namespace gp

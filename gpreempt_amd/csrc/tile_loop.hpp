@@ -1,0 +1,81 @@
+// Block-level-preemption dispatcher for gfx950 kernels.
+//
+// Restates the persistent-block wrapper that the reference generates around every kernel
+// (scripts/compile/convert_to_blp.py:40-69): a workgroup repeatedly (1) reads the preempt
+// flag, (2) claims the next tile index from the kernel's atomic counter, (3) decodes the
+// index into the original grid coordinates, (4) runs the kernel body on that tile.  When the
+// flag is up it records the kernel id in *stop_index (first writer wins) and leaves; the
+// counter then holds exactly the number of tiles already owed to completed claims, so a
+// relaunch continues with the next unclaimed tile: no tile is redone or skipped.
+//
+// Differences from the generated wrapper, all deliberate:
+//  * the flag lives in fine-grained pinned host memory and is read with a system-scope load
+//    (the reference polls a GDRCopy-mapped device int, src/cuda-clients/blpclient.cpp:45-76);
+//  * the claimed index is handed to the other waves through a two-slot LDS mailbox indexed by
+//    iteration parity, which removes the reference's reuse race on its single __shared__ slot
+//    with one barrier per tile;
+//  * *stop_index is claimed with a compare-and-swap instead of a test followed by a store;
+//  * with executed == nullptr the same kernel runs non-preemptibly, one workgroup per tile
+//    (the reference builds a second, untransformed module for that: mod.cubin vs mod.tr.cubin).
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace gp {
+
+struct BlpArgs {
+    int *flag;        // nullptr: never preempted
+    int *stop_index;
+    int *executed;    // nullptr: static mapping, tile = blockIdx.x
+    int total;        // total_block
+    int sx, sy;       // shape.x, shape.y (shape.z = total / (sx*sy))
+    int kernel_id;
+    int inject_at;    // -1 = off
+};
+
+struct TileIdx { int x, y, z; };
+
+__device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy) {
+    // x = idx % sx; y = (idx / sx) % sy; z = idx / (sx*sy)   (convert_to_blp.py:52-54)
+    TileIdx t;
+    int q = idx / sx;
+    t.x = idx - q * sx;
+    t.z = q / sy;
+    t.y = q - t.z * sy;
+    return t;
+}
+
+// Runs body(TileIdx) for every tile this workgroup obtains.  All threads of the workgroup must
+// call it; the body may use barriers freely.
+template <class Body>
+__device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
+    if (b.executed == nullptr) {
+        int idx = blockIdx.x;
+        if (idx < b.total) body(decode_tile(idx, b.sx, b.sy));
+        return;
+    }
+    __shared__ int mailbox[2];
+    const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    for (int it = 0;; ++it) {
+        if (leader) {
+            int idx = -1;
+            int stop = b.flag ? __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : 0;
+            if (!stop) {
+                idx = atomicAdd(b.executed, 1);
+                if (idx >= b.total) {
+                    idx = -1;
+                } else if (idx == b.inject_at && b.flag) {
+                    __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+            } else {
+                atomicCAS(b.stop_index, -1, b.kernel_id);
+            }
+            mailbox[it & 1] = idx;
+        }
+        __syncthreads();
+        int idx = mailbox[it & 1];
+        if (idx < 0) return;
+        body(decode_tile(idx, b.sx, b.sy));
+    }
+}
+
+}  // namespace gp

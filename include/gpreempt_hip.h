@@ -1,0 +1,234 @@
+/*
+ * gpreempt_hip.h — C ABI of libgpreempt_hip.so, the MI355X (gfx950) device layer of the
+ * preemptible inference executor.
+ *
+ * This is the drop-in boundary: the C++ host classes (foo::Executor / foo::BLPExecutor /
+ * foo::Model, gpreempt.h) reach the GPU only through these entry points.  Each entry point
+ * names the interface of the reference (thustorage/GPreempt) that it replaces.
+ *
+ * Conventions: every function returns 0 on success and a non-zero gp_status otherwise; it never
+ * throws and never aborts; gp_last_error() gives the message of the calling thread's last
+ * failure.  All pointers are plain device or host addresses; sizes are bytes unless named
+ * otherwise.  Callable from any host thread.
+ */
+#ifndef GPREEMPT_HIP_H
+#define GPREEMPT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Mirrors `enum Status` of the reference (include/util/common.h:16-23). */
+enum gp_status { GP_SUCC = 0, GP_FAIL = 1, GP_TIMEOUT = 2, GP_NOTFOUND = 3, GP_OUTOFRANGE = 4, GP_FULL = 5 };
+
+enum gp_dtype { GP_F32 = 0, GP_F16 = 1, GP_BF16 = 2, GP_I32 = 3, GP_I64 = 4 };
+enum gp_act { GP_ACT_NONE = 0, GP_ACT_RELU = 1, GP_ACT_GELU = 2 };
+
+typedef struct gp_stream_s *gp_stream; /* opaque; wraps one HIP stream */
+typedef struct gp_event_s *gp_event;
+typedef struct gp_graph_s *gp_graph;
+
+/* ---- device / errors ---------------------------------------------------------------------
+ * Replaces foo::util::init_cuda (src/util/gpu_util.cpp:14-25): selects the device for the
+ * calling thread.  Safe to call once per thread, as the reference's clients do. */
+int gp_init(int device);
+const char *gp_last_error(void);
+/* Number of compute units, wavefront clock in kHz and the device name (name_len bytes). */
+int gp_device_info(int *compute_units, int *clock_khz, char *name, size_t name_len);
+
+/* ---- streams, events ---------------------------------------------------------------------
+ * Replaces GPUStreamCreate / GPUStreamSynchronize (include/util/gpu_util.h:74-139).  `priority`
+ * is the tenant priority of the reference (0 = high, 1 = low, larger = lower); it is recorded
+ * on the handle and selects which preempt flag level the tenant obeys.  The HIP stream itself
+ * is always created at the default hardware priority. */
+int gp_stream_create(int priority, gp_stream *out);
+int gp_stream_destroy(gp_stream s);
+int gp_stream_sync(gp_stream s);
+int gp_stream_query(gp_stream s, int *idle); /* *idle = 1 when all work has completed */
+int gp_stream_priority(gp_stream s, int *priority);
+void *gp_stream_native(gp_stream s); /* the hipStream_t, for callers that own HIP code */
+
+int gp_event_create(gp_event *out);
+int gp_event_destroy(gp_event e);
+int gp_event_record(gp_event e, gp_stream s);
+int gp_event_sync(gp_event e);
+int gp_event_elapsed_ms(gp_event start, gp_event stop, float *ms);
+
+/* ---- memory ------------------------------------------------------------------------------
+ * Replaces GPUMemAlloc / GPUMemFree / GPUMemcpy* / GPUMemsetAsync / GPUMemHostAlloc
+ * (include/util/gpu_util.h:74-139; uses in src/model.cpp:101-113,268-279,296-327). */
+int gp_malloc(void **dev, size_t bytes);
+int gp_free(void *dev);
+int gp_host_alloc(void **host, size_t bytes); /* pinned */
+int gp_host_free(void *host);
+int gp_memcpy_h2d(void *dev, const void *host, size_t bytes);
+int gp_memcpy_d2h(void *host, const void *dev, size_t bytes);
+int gp_memcpy_h2d_async(void *dev, const void *host, size_t bytes, gp_stream s);
+int gp_memcpy_d2h_async(void *host, const void *dev, size_t bytes, gp_stream s);
+int gp_memcpy_d2d_async(void *dst, const void *src, size_t bytes, gp_stream s);
+/* Fills `count` 32-bit words with `value` using a fill kernel (safe inside a captured graph). */
+int gp_fill32_async(void *dev, uint32_t value, size_t count, gp_stream s);
+
+/* ---- preempt flag ------------------------------------------------------------------------
+ * Replaces the GDRCopy-mapped device int of src/cuda-clients/blpclient.cpp:45-76 and the
+ * managed int of src/hip-clients/blpclient.cpp:106: one int in fine-grained, coherent pinned
+ * host memory.  The host sets it with a plain store through *host_ptr; kernels poll *dev_ptr
+ * with system-scope loads. */
+int gp_flag_create(volatile int **host_ptr, void **dev_ptr);
+int gp_flag_destroy(volatile int *host_ptr);
+
+/* ---- block-level preemption context ------------------------------------------------------
+ * The six trailing arguments that scripts/compile/convert_to_blp.py:35 appends to every kernel
+ * (`int* preempted, int* pStopIndex, int total_block, int* executed, dim3 shape, int
+ * kernel_id`), as one struct.  total_block and shape are derived by the launcher from the
+ * operator's own tiling, as src/model.cpp:366-396 derives them from the launch grid.
+ * A NULL context launches the same kernel non-preemptibly: one workgroup per tile. */
+typedef struct gp_preempt_ctx {
+    int *flag;       /* device address of the preempt flag (gp_flag_create's dev_ptr)          */
+    int *stop_index; /* device int, -1 when no kernel has been stopped                          */
+    int *executed;   /* device int: this kernel's tile claim counter                            */
+    int kernel_id;   /* index written to *stop_index by the first workgroup that sees the flag */
+    int inject_at;   /* test hook: the workgroup whose claim returns this value raises *flag    */
+                     /* itself right after the claim; -1 = off                                  */
+    int max_workgroups; /* 0 = occupancy-sized persistent grid; >0 caps it                      */
+} gp_preempt_ctx;
+
+/* What a launch did: filled when the `info` argument of a launcher is non-NULL. */
+typedef struct gp_launch_info {
+    int total_tiles;    /* = total_block of the reference                     */
+    int shape[3];       /* = dim3 shape of the reference (tile grid)          */
+    int grid;           /* workgroups launched                                */
+    int block;          /* threads per workgroup                              */
+} gp_launch_info;
+
+/* ---- operators ---------------------------------------------------------------------------
+ * These replace the TVM-generated device kernels that src/executor.cpp:157-162 launches by
+ * name (fused_nn_conv2d_add_nn_relu*, fused_nn_dense*, fused_nn_softmax*, pooling, add,
+ * layer_norm, erf GELU, take, batch_matmul; names implied by patch/tvm.patch:296-311).
+ * Accumulation is fp32 for every dtype. */
+
+/* C[b] = act(alpha * A[b] * op(B[b]) + bias[n] + residual[b]); A is M x K row-major.
+ * b_is_nk = 0: B is K x N row-major; 1: B is N x K row-major (dense weights).
+ * Batch strides are in elements; batch = 1 ignores them.  bias / residual may be NULL;
+ * bias has the dtype of C; residual shares ldc / stride_c. */
+typedef struct gp_gemm_params {
+    int dtype;
+    int M, N, K;
+    const void *A; long lda; long stride_a;
+    const void *B; long ldb; long stride_b; int b_is_nk;
+    void *C; long ldc; long stride_c;
+    const void *bias;
+    const void *residual;
+    float alpha;
+    int act;
+    int batch;
+    /* second-level batch (attention heads): offset = (b / batch_inner) * stride_*_outer +
+     * (b % batch_inner) * stride_*; batch_inner = 0 disables it. */
+    int batch_inner; long stride_a_outer, stride_b_outer, stride_c_outer;
+    int tile_m, tile_n; /* 0 = chosen by the launcher */
+} gp_gemm_params;
+int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* Implicit-GEMM convolution.  Activations are NHWC with a pixel stride (in elements) that may
+ * exceed the channel count, so a layer can read or write a channel slice of a wider buffer
+ * (DenseNet concatenation without a copy).  Weights are [Cout][R][S][Cin] ("OHWI").
+ * Requires Cin % 4 == 0 (fp32) or Cin % 8 == 0 (fp16 / bf16).
+ * out[n,ho,wo,co] = act(sum in[n,ho*sh-ph+r,wo*sw-pw+s,ci] * w[co,r,s,ci] + bias[co] + residual). */
+typedef struct gp_conv_params {
+    int dtype;
+    int N, H, W, Cin, Cout, R, S, stride_h, stride_w, pad_h, pad_w;
+    const void *in; long in_pix_stride;
+    const void *weight;
+    const void *bias;
+    const void *residual; long res_pix_stride;
+    void *out; long out_pix_stride;
+    int act;
+    int tile_m, tile_n;
+} gp_conv_params;
+int gp_launch_conv2d(const gp_conv_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* NCHW -> NHWC with zero padding of the channel count up to c_pad (input adapter: the
+ * reference's "data" tensor is NCHW, src/tests/test-dnn.cpp:25-30). */
+typedef struct gp_layout_params {
+    int dtype_in, dtype_out;
+    int N, C, H, W, c_pad;
+    const void *in; void *out;
+} gp_layout_params;
+int gp_launch_nchw_to_nhwc(const gp_layout_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* Pooling on NHWC.  mode 0 = max, 1 = average (padding excluded from the count),
+ * 2 = global average (R,S,stride,pad ignored; output N x 1 x 1 x C). */
+typedef struct gp_pool_params {
+    int dtype;
+    int N, H, W, C, R, S, stride, pad, mode;
+    const void *in; long in_pix_stride;
+    void *out; long out_pix_stride;
+} gp_pool_params;
+int gp_launch_pool2d(const gp_pool_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* Elementwise over `rows` pixels of `cols` channels:
+ *   out = act((a [+ b]) * scale[c] + shift[c]); b, scale, shift may be NULL. */
+typedef struct gp_eltwise_params {
+    int dtype;
+    long rows; int cols;
+    const void *a; long a_stride;
+    const void *b; long b_stride;
+    const void *scale; const void *shift; /* per channel, dtype of a */
+    void *out; long out_stride;
+    int act;
+} gp_eltwise_params;
+int gp_launch_eltwise(const gp_eltwise_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* Row softmax over the last axis: out = softmax(scale * x). */
+typedef struct gp_softmax_params {
+    int dtype;
+    long rows; int cols;
+    const void *x; void *out;
+    float scale;
+} gp_softmax_params;
+int gp_launch_softmax(const gp_softmax_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* out = layer_norm(x [+ residual]) * gamma + beta over the last axis (biased variance). */
+typedef struct gp_layernorm_params {
+    int dtype;
+    long rows; int cols;
+    const void *x; const void *residual;
+    const void *gamma; const void *beta;
+    void *out;
+    float eps;
+} gp_layernorm_params;
+int gp_launch_layernorm(const gp_layernorm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* out[t,:] = tok[ids[t],:] + pos[t % seq,:] (+ seg[0,:]); ids are int64 (the reference feeds
+ * BERT int64 token ids, src/tests/test-dnn.cpp:21-23). */
+typedef struct gp_embed_params {
+    int dtype;
+    long tokens; int seq; int hidden; long vocab;
+    const int64_t *ids;
+    const void *tok; const void *pos; const void *seg;
+    void *out;
+} gp_embed_params;
+int gp_launch_embed(const gp_embed_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+/* ---- gate kernels --------------------------------------------------------------------------
+ * Replace gpu_block / gpu_noop (src/block.cu:1-7): one wave spins until *stop != 0.  Unlike the
+ * reference the wait is bounded: after spin_limit polls the kernel leaves and stores 1 to
+ * *timed_out (may be NULL), so a lost release can never hang the device. */
+int gp_launch_gate(const int *stop, unsigned long long spin_limit, int *timed_out, gp_stream s);
+int gp_launch_noop(gp_stream s);
+
+/* ---- graphs --------------------------------------------------------------------------------
+ * Replace GPUStreamBeginCapture / EndCapture / GraphInstantiate / GraphLaunch
+ * (src/executor.cpp:119-122,176-196). */
+int gp_graph_begin(gp_stream s);
+int gp_graph_end(gp_stream s, gp_graph *out);
+int gp_graph_launch(gp_graph g, gp_stream s);
+int gp_graph_destroy(gp_graph g);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPREEMPT_HIP_H */

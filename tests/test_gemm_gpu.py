@@ -1,0 +1,158 @@
+"""Parity of the preemptible GEMM (C ABI gp_launch_gemm) with the CPU oracle, and bit-exact
+preempt/resume (BASELINE config 1; protocol of reference src/tests/test-dnn-blp.cpp:36-42)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+# Tolerances stated by the north star: 1e-4 relative for fp32, 1e-2 for fp16 / bf16.  "Relative"
+# is taken against the magnitude of the output tensor (max |ref|), because single elements of a
+# GEMM can cancel to ~0 where an element-wise ratio is meaningless.
+TOL = {"f32": 1e-4, "f16": 1e-2, "bf16": 1e-2}
+
+
+def rel_err(got, ref):
+    return float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None, tile=0, batch=1, alpha=1.0):
+    rng = np.random.default_rng(seed)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    A = O.round_to(rng.uniform(-1, 1, (batch, M, K)).astype(np.float32), dt)
+    Bshape = (batch, N, K) if b_is_nk else (batch, K, N)
+    B = O.round_to(rng.uniform(-1, 1, Bshape).astype(np.float32), dt)
+    bias = O.round_to(rng.uniform(-0.1, 0.1, N).astype(np.float32), dt) if use_bias else None
+    res = O.round_to(rng.uniform(-1, 1, (batch, M, N)).astype(np.float32), dt) if use_res else None
+    dA, dB = gp.DevBuf.from_array(A, dtype), gp.DevBuf.from_array(B, dtype)
+    dbias = gp.DevBuf.from_array(bias, dtype) if use_bias else None
+    dres = gp.DevBuf.from_array(res, dtype) if use_res else None
+    dC = gp.DevBuf(batch * M * N * gp.DTYPE_SIZE[dtype])
+    dC.fill32(0xFFFFFFFF if dt == "f32" else 0x7E007E00)  # NaN pattern: unwritten elements show up
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, stride_a=M * K, B=dB.ptr,
+                      ldb=K if b_is_nk else N, stride_b=N * K, b_is_nk=int(b_is_nk), C=dC.ptr, ldc=N,
+                      stride_c=M * N, bias=gp._ptr(dbias), residual=gp._ptr(dres), alpha=alpha, act=act,
+                      batch=batch, tile_m=tile, tile_n=tile)
+    info = ctx_fn(p, dC) if ctx_fn else gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    got = dC.download(dtype, (batch, M, N)).copy()
+    ref = np.stack([O.gemm_bias_act(A[b] * np.float32(alpha), B[b], bias, None if res is None else res[b], act, b_is_nk)
+                    for b in range(batch)])
+    return got, ref, info
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("b_is_nk", [False, True])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (200, 136, 72), (64, 1000, 512), (1, 8, 8), (130, 264, 40)])
+def test_gemm_matches_oracle(gp, dt, b_is_nk, shape):
+    M, N, K = shape
+    for tile in (64, 128):
+        got, ref, info = run_gemm(gp, dt, M, N, K, b_is_nk, gp.ACT_RELU, True, True, seed=M + N + K, tile=tile)
+        assert info.total_tiles == -(-M // tile) * -(-N // tile)
+        assert np.isfinite(got).all()
+        assert rel_err(got, ref) < TOL[dt], (dt, shape, tile)
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+def test_gemm_batched_alpha_gelu(gp, dt):
+    got, ref, info = run_gemm(gp, dt, 128, 64, 64, True, gp.ACT_GELU, True, False, seed=3, batch=6, alpha=0.125)
+    assert info.shape[2] == 6
+    assert rel_err(got, ref) < TOL[dt]
+
+
+def test_gemm_known_answers(gp):
+    """Identity, permutation and all-ones operands: results fixed by the mathematics."""
+    n = 128
+    eye = np.eye(n, dtype=np.float32)
+    rng = np.random.default_rng(1)
+    X = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    perm = rng.permutation(n)
+    for A, B, want in ((eye, X, X), (X, eye, X), (eye[perm], X, X[perm]), (np.ones((n, n), np.float32), np.ones((n, n), np.float32), np.full((n, n), n, np.float32))):
+        dA, dB, dC = gp.DevBuf.from_array(A, gp.F32), gp.DevBuf.from_array(B, gp.F32), gp.DevBuf(4 * n * n)
+        p = gp.GemmParams(dtype=gp.F32, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=0, C=dC.ptr, ldc=n, alpha=1.0, batch=1)
+        gp.launch("gp_launch_gemm", p)
+        gp.check(gp.lib().gp_stream_sync(None))
+        assert np.array_equal(dC.download(gp.F32, (n, n)), want)
+
+
+def test_gemm_rejects_bad_arguments(gp):
+    d = gp.DevBuf(4096)
+    bad = gp.GemmParams(dtype=gp.F32, M=8, N=8, K=6, A=d.ptr, lda=6, B=d.ptr, ldb=8, C=d.ptr, ldc=8, batch=1)
+    with pytest.raises(gp.GpError) as e:
+        gp.launch("gp_launch_gemm", bad)
+    assert e.value.status == gp.OUTOFRANGE and "multiples" in str(e.value)
+    bad = gp.GemmParams(dtype=7, M=8, N=8, K=8, A=d.ptr, lda=8, B=d.ptr, ldb=8, C=d.ptr, ldc=8, batch=1)
+    with pytest.raises(gp.GpError):
+        gp.launch("gp_launch_gemm", bad)
+
+
+# ---- config 1: 1024^3 fp32 GEMM + bias + ReLU, preempt at 25/50/75 %, resume, bit-exact ----
+
+def _config1(gp, tile):
+    rng = np.random.default_rng(0xC0FFEE)
+    A = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    bias = rng.uniform(-0.1, 0.1, 1024).astype(np.float32)
+    dA, dB, db = (gp.DevBuf.from_array(x, gp.F32) for x in (A, B, bias))
+    dC = gp.DevBuf(4 * 1024 * 1024)
+    p = gp.GemmParams(dtype=gp.F32, M=1024, N=1024, K=1024, A=dA.ptr, lda=1024, B=dB.ptr, ldb=1024, b_is_nk=0,
+                      C=dC.ptr, ldc=1024, bias=db.ptr, alpha=1.0, act=gp.ACT_RELU, batch=1, tile_m=tile, tile_n=tile)
+    return A, B, bias, p, dC, (dA, dB, db)
+
+
+@pytest.mark.parametrize("tile", [64, 128])
+def test_config1_preempt_resume_bit_exact(gp, tile):
+    A, B, bias, p, dC, keep = _config1(gp, tile)
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    # uninterrupted, non-preemptible launch (BaseExecutor path)
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    base = dC.download(gp.F32, (1024, 1024)).copy()
+    ref = O.gemm_bias_act(A, B, bias, act=O.ACT_RELU)
+    assert rel_err(base, ref) < 1e-4
+    # uninterrupted, preemptible launch: same bits
+    dC.fill32(0xFFFFFFFF)
+    info = gp.launch("gp_launch_gemm", p, st.ctx())
+    gp.check(gp.lib().gp_stream_sync(None))
+    total = info.total_tiles
+    assert total == (1024 // tile) ** 2 and info.grid <= total
+    assert np.array_equal(dC.download(gp.F32, (1024, 1024)), base)
+    assert st.stop_index() == -1
+    assert st.counters()[0] == total + info.grid  # every workgroup overshoots once (convert_to_blp.py:48-51)
+    for frac in (0.25, 0.5, 0.75):
+        k = int(np.ceil(frac * total))
+        st.reset()
+        flag.set(0)
+        dC.fill32(0xFFFFFFFF)
+        gp.launch("gp_launch_gemm", p, st.ctx(inject_at=k - 1))  # claim number k raises the flag
+        gp.check(gp.lib().gp_stream_sync(None))
+        assert flag.get() == 1
+        assert st.stop_index() == 0
+        done = st.counters()[0]
+        assert k <= done <= min(total, k + info.grid), (k, done, info.grid)
+        part = dC.download(gp.F32, (1024, 1024))
+        assert np.isnan(part).any() or done == total  # really interrupted
+        # host: *flag = 0; resume (executor.cpp:280-298): counters are NOT reset
+        flag.set(0)
+        st.clear_stop()
+        gp.launch("gp_launch_gemm", p, st.ctx())
+        gp.check(gp.lib().gp_stream_sync(None))
+        assert np.array_equal(dC.download(gp.F32, (1024, 1024)), base), f"resume after {frac:.0%} differs"
+        assert st.stop_index() == -1
+
+
+def test_flag_set_before_launch_does_no_tiles(gp):
+    A, B, bias, p, dC, keep = _config1(gp, 128)
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    flag.set(1)
+    dC.fill32(0xFFFFFFFF)
+    gp.launch("gp_launch_gemm", p, st.ctx())
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert st.counters()[0] == 0 and st.stop_index() == 0
+    assert np.isnan(dC.download(gp.F32, (1024, 1024))).all()
+    flag.set(0)
