@@ -1,0 +1,216 @@
+"""Parity of every operator kernel behind the C ABI with the CPU oracle, on seeded inputs."""
+import numpy as np
+import pytest
+
+from oracle import oracle as O
+from helpers import TOL, gpu_conv2d, nchw_to_nhwc, nhwc_to_nchw, rel_err, sync
+
+pytestmark = pytest.mark.gpu
+DTS = ["f32", "f16", "bf16"]
+
+
+def rnd(rng, shape, dt, lo=-1.0, hi=1.0):
+    return O.round_to(rng.uniform(lo, hi, shape).astype(np.float32), dt)
+
+
+CONV_CASES = [
+    # N, Cin, H, W, Cout, k, stride, pad
+    (1, 3, 32, 32, 64, 7, 2, 3),     # stem: Cin padded to the vector width
+    (2, 64, 14, 14, 64, 1, 1, 0),    # 1x1 == GEMM
+    (1, 64, 15, 13, 96, 3, 1, 1),    # odd sizes, ragged tiles
+    (1, 128, 16, 16, 256, 3, 2, 1),  # strided 3x3
+    (2, 256, 8, 8, 512, 1, 2, 0),    # strided 1x1 (projection shortcut)
+    (1, 8, 5, 5, 8, 5, 1, 2),        # window as large as the image
+]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_matches_oracle(gp, dt, case):
+    N, Cin, H, W, Cout, k, stride, pad = case
+    rng = np.random.default_rng(hash(case) % 2**31)
+    x = rnd(rng, (N, Cin, H, W), dt)
+    w = rnd(rng, (Cout, Cin, k, k), dt, -0.2, 0.2)
+    b = rnd(rng, (Cout,), dt, -0.1, 0.1)
+    Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
+    res = rnd(rng, (N, Cout, Ho, Wo), dt)
+    ref = O.conv2d(x, w, b, stride, pad, res, O.ACT_RELU)
+    for tile in (64, 128):
+        got, info, _ = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=tile)
+        assert np.isfinite(got).all()
+        assert rel_err(got, ref) < TOL[dt], (dt, case, tile)
+
+
+def test_conv2d_channel_slices(gp):
+    """Reading and writing channel slices of wider NHWC buffers (concatenation without a copy)."""
+    rng = np.random.default_rng(5)
+    N, H, W, Cin, Cout, Cbuf = 1, 6, 6, 32, 32, 96
+    x = rnd(rng, (N, Cin, H, W), "f32")
+    w = rnd(rng, (Cout, Cin, 3, 3), "f32", -0.2, 0.2)
+    buf = np.zeros((N, H, W, Cbuf), np.float32)
+    buf[..., :Cin] = nchw_to_nhwc(x)
+    dbuf = gp.DevBuf.from_array(buf, gp.F32)
+    dw = gp.DevBuf.from_array(np.ascontiguousarray(np.transpose(w, (0, 2, 3, 1))), gp.F32)
+    p = gp.ConvParams(dtype=gp.F32, N=N, H=H, W=W, Cin=Cin, Cout=Cout, R=3, S=3, stride_h=1, stride_w=1, pad_h=1, pad_w=1,
+                      in_=dbuf.ptr, in_pix_stride=Cbuf, weight=dw.ptr, out=dbuf.ptr + 4 * 64, out_pix_stride=Cbuf)
+    gp.launch("gp_launch_conv2d", p)
+    sync(gp)
+    out = dbuf.download(gp.F32, (N, H, W, Cbuf))
+    assert np.array_equal(out[..., :Cin], buf[..., :Cin]) and np.all(out[..., Cin:64] == 0)
+    assert rel_err(nhwc_to_nchw(out[..., 64:]), O.conv2d(x, w, None, 1, 1)) < 1e-4
+
+
+@pytest.mark.parametrize("dt_in,dt_out", [("f32", "f32"), ("f32", "f16"), ("f16", "f16"), ("f32", "bf16")])
+def test_nchw_to_nhwc(gp, dt_in, dt_out):
+    rng = np.random.default_rng(2)
+    N, Cc, H, W = 2, 3, 19, 23
+    cp = 4 if dt_out == "f32" else 8
+    x = rnd(rng, (N, Cc, H, W), dt_in)
+    di = gp.DevBuf.from_array(x, gp.DTYPE_BY_NAME[dt_in])
+    do = gp.DevBuf(N * H * W * cp * gp.DTYPE_SIZE[gp.DTYPE_BY_NAME[dt_out]])
+    p = gp.LayoutParams(gp.DTYPE_BY_NAME[dt_in], gp.DTYPE_BY_NAME[dt_out], N, Cc, H, W, cp, di.ptr, do.ptr)
+    info = gp.launch("gp_launch_nchw_to_nhwc", p)
+    sync(gp)
+    got = do.download(gp.DTYPE_BY_NAME[dt_out], (N, H, W, cp))
+    assert np.array_equal(got, O.round_to(nchw_to_nhwc(x, cp), dt_out))  # a pure copy/convert: exact
+    assert info.total_tiles == N * -(-H * W // 256)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("cfg", [(3, 2, 1, "max"), (2, 2, 0, "max"), (2, 2, 0, "avg"), (3, 1, 1, "avg"), (7, 1, 0, "gap")])
+def test_pool2d(gp, dt, cfg):
+    k, stride, pad, mode = cfg
+    rng = np.random.default_rng(k * 10 + stride)
+    N, Cc, H, W = 2, 24, 14, 14 if mode != "gap" else 7
+    if mode == "gap":
+        H = 7
+    x = rnd(rng, (N, Cc, H, W), dt)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    di = gp.DevBuf.from_array(nchw_to_nhwc(x), dtype)
+    if mode == "gap":
+        ref = O.global_avgpool(x).reshape(N, Cc, 1, 1)
+        Ho = Wo = 1
+    else:
+        ref = O.pool2d(x, k, stride, pad, mode)
+        Ho, Wo = ref.shape[2:]
+    do = gp.DevBuf(N * Ho * Wo * Cc * gp.DTYPE_SIZE[dtype])
+    p = gp.PoolParams(dtype, N, H, W, Cc, k, k, stride, pad, {"max": 0, "avg": 1, "gap": 2}[mode], di.ptr, Cc, do.ptr, Cc)
+    gp.launch("gp_launch_pool2d", p)
+    sync(gp)
+    got = nhwc_to_nchw(do.download(dtype, (N, Ho, Wo, Cc)))
+    if mode == "max":
+        assert np.array_equal(got, ref)  # selection only: exact in every dtype
+    else:
+        assert rel_err(got, ref) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_eltwise_add_scale_shift_relu(gp, dt):
+    rng = np.random.default_rng(4)
+    rows, cols = 777, 40
+    a, b = rnd(rng, (rows, cols), dt), rnd(rng, (rows, cols), dt)
+    sc, sh = rnd(rng, (cols,), dt, 0.5, 1.5), rnd(rng, (cols,), dt)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    da, db, dsc, dsh = (gp.DevBuf.from_array(v, dtype) for v in (a, b, sc, sh))
+    do = gp.DevBuf(rows * cols * gp.DTYPE_SIZE[dtype])
+    # add + relu (residual join)
+    p = gp.EltwiseParams(dtype, rows, cols, da.ptr, cols, db.ptr, cols, None, None, do.ptr, cols, gp.ACT_RELU)
+    gp.launch("gp_launch_eltwise", p)
+    sync(gp)
+    assert rel_err(do.download(dtype, (rows, cols)), O.add_act(a, b, O.ACT_RELU)) < TOL[dt]
+    # per-channel affine + relu (unfolded batch-norm), checked through the NCHW oracle
+    p = gp.EltwiseParams(dtype, rows, cols, da.ptr, cols, None, 0, dsc.ptr, dsh.ptr, do.ptr, cols, gp.ACT_RELU)
+    gp.launch("gp_launch_eltwise", p)
+    sync(gp)
+    ref = O.scale_shift_act(a.T.reshape(1, cols, rows, 1), sc, sh, O.ACT_RELU).reshape(cols, rows).T
+    assert rel_err(do.download(dtype, (rows, cols)), ref) < TOL[dt]
+    # gelu
+    p = gp.EltwiseParams(dtype, rows, cols, da.ptr, cols, None, 0, None, None, do.ptr, cols, gp.ACT_GELU)
+    gp.launch("gp_launch_eltwise", p)
+    sync(gp)
+    assert rel_err(do.download(dtype, (rows, cols)), O.add_act(a, None, O.ACT_GELU)) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape", [(12 * 128, 128), (5, 1000), (3, 7), (33, 384)])
+def test_softmax(gp, dt, shape):
+    rng = np.random.default_rng(shape[1])
+    x = rnd(rng, shape, dt, -8, 8)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    dx = gp.DevBuf.from_array(x, dtype)
+    do = gp.DevBuf(x.size * gp.DTYPE_SIZE[dtype])
+    gp.launch("gp_launch_softmax", gp.SoftmaxParams(dtype, shape[0], shape[1], dx.ptr, do.ptr, 0.125))
+    sync(gp)
+    got = do.download(dtype, shape)
+    assert rel_err(got, O.softmax(x * np.float32(0.125))) < TOL[dt]
+    assert np.abs(got.sum(axis=1) - 1).max() < (1e-5 if dt == "f32" else 2e-2)
+
+
+@pytest.mark.parametrize("dt", DTS)
+@pytest.mark.parametrize("shape", [(128, 768), (7, 3072), (5, 8)])
+def test_layernorm(gp, dt, shape):
+    rng = np.random.default_rng(shape[1])
+    x, r = rnd(rng, shape, dt, -2, 2), rnd(rng, shape, dt, -2, 2)
+    g, b = rnd(rng, (shape[1],), dt, 0.5, 1.5), rnd(rng, (shape[1],), dt)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    dx, dr, dg, db = (gp.DevBuf.from_array(v, dtype) for v in (x, r, g, b))
+    do = gp.DevBuf(x.size * gp.DTYPE_SIZE[dtype])
+    for res in (None, dr):
+        p = gp.LayernormParams(dtype, shape[0], shape[1], dx.ptr, gp._ptr(res), dg.ptr, db.ptr, do.ptr, 1e-12)
+        gp.launch("gp_launch_layernorm", p)
+        sync(gp)
+        ref = O.layernorm(x, g, b, 1e-12, None if res is None else r)
+        assert rel_err(do.download(dtype, shape), ref) < TOL[dt]
+
+
+@pytest.mark.parametrize("dt", DTS)
+def test_embed(gp, dt):
+    rng = np.random.default_rng(9)
+    vocab, seq, hidden, batch = 500, 16, 64, 3
+    ids = rng.integers(0, vocab, batch * seq)
+    tok, pos, seg = rnd(rng, (vocab, hidden), dt), rnd(rng, (seq, hidden), dt), rnd(rng, (1, hidden), dt)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    dids = gp.DevBuf.from_array(ids.astype(np.int64))
+    dt_, dp, ds = (gp.DevBuf.from_array(v, dtype) for v in (tok, pos, seg))
+    do = gp.DevBuf(batch * seq * hidden * gp.DTYPE_SIZE[dtype])
+    p = gp.EmbedParams(dtype, batch * seq, seq, hidden, vocab, dids.ptr, dt_.ptr, dp.ptr, ds.ptr, do.ptr)
+    gp.launch("gp_launch_embed", p)
+    sync(gp)
+    assert rel_err(do.download(dtype, (batch * seq, hidden)), O.embed(ids, tok, pos, seg[0], seq)) < TOL[dt]
+
+
+def test_every_op_resumes_bit_exact(gp):
+    """Each memory-bound kernel, preempted at a tile boundary and resumed, equals its
+    uninterrupted run bit for bit."""
+    rng = np.random.default_rng(11)
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    rows, cols = 4096, 256
+    a = rnd(rng, (rows, cols), "f16")
+    g = rnd(rng, (cols,), "f16")
+    da, dg = gp.DevBuf.from_array(a, gp.F16), gp.DevBuf.from_array(g, gp.F16)
+    do = gp.DevBuf(rows * cols * 2)
+    cases = {
+        "gp_launch_eltwise": gp.EltwiseParams(gp.F16, rows, cols, da.ptr, cols, da.ptr, cols, dg.ptr, dg.ptr, do.ptr, cols, gp.ACT_GELU),
+        "gp_launch_softmax": gp.SoftmaxParams(gp.F16, rows, cols, da.ptr, do.ptr, 1.0),
+        "gp_launch_layernorm": gp.LayernormParams(gp.F16, rows, cols, da.ptr, da.ptr, dg.ptr, dg.ptr, do.ptr, 1e-5),
+        "gp_launch_pool2d": gp.PoolParams(gp.F16, 1, 64, 64, cols, 3, 3, 2, 1, 0, da.ptr, cols, do.ptr, cols),
+    }
+    for fn, p in cases.items():
+        do.fill32(0)
+        info = gp.launch(fn, p)
+        sync(gp)
+        base = do.download().copy()
+        st.reset()
+        do.fill32(0)
+        gp.launch(fn, p, st.ctx(inject_at=info.total_tiles // 3, max_workgroups=8))
+        sync(gp)
+        assert flag.get() == 1 and st.stop_index() == 0, fn
+        assert st.counters()[0] < info.total_tiles, fn
+        assert not np.array_equal(do.download(), base), fn
+        flag.set(0)
+        st.clear_stop()
+        gp.launch(fn, p, st.ctx())
+        sync(gp)
+        assert np.array_equal(do.download(), base), fn
+        assert st.stop_index() == -1
