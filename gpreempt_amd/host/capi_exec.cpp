@@ -1,0 +1,100 @@
+// extern "C" forwarding layer over foo::Executor / foo::BLPExecutor (include/gpreempt_exec_c.h).
+#include <cstring>
+#include "executor.h"
+#include "gpreempt_exec_c.h"
+
+using namespace foo;
+
+namespace {
+struct Handle {
+    std::unique_ptr<Executor> ex;
+    BLPExecutor *blp = nullptr;
+};
+Handle *H(gpx_executor e) { return static_cast<Handle *>(e); }
+void copy_str(char *dst, size_t n, const std::string &s) {
+    if (!dst || !n) return;
+    std::strncpy(dst, s.c_str(), n - 1);
+    dst[n - 1] = 0;
+}
+}  // namespace
+
+extern "C" {
+
+gpx_executor gpx_create(int blp) {
+    Handle *h = new Handle();
+    if (blp) { h->blp = new BLPExecutor(); h->ex.reset(h->blp); }
+    else h->ex.reset(new BaseExecutor());
+    return h;
+}
+void gpx_destroy(gpx_executor e) { delete H(e); }
+int gpx_init(gpx_executor e, const char *workload) { return H(e)->ex->init(workload); }
+int gpx_set_input(gpx_executor e, const char *key, void *value, size_t len, gp_stream s) { return H(e)->ex->set_input(key, value, len, s); }
+int gpx_get_output(gpx_executor e, const char *key, void *value, size_t len, gp_stream s) { return H(e)->ex->get_output(key, value, len, s); }
+size_t gpx_get_data_size(gpx_executor e, const char *key) { return H(e)->ex->get_data_size(key); }
+int gpx_execute(gpx_executor e, gp_stream s) { return H(e)->ex->execute(s); }
+int gpx_launch_kernel(gpx_executor e, size_t idx, gp_stream s) { return H(e)->ex->launch_kernel(idx, s); }
+size_t gpx_get_kernel_num(gpx_executor e) { return H(e)->ex->get_kernel_num(); }
+int gpx_capture_graph(gpx_executor e, gp_stream s) {
+    H(e)->ex->capture_graph(s);
+    return H(e)->ex->uses_graph() ? Status::Succ : Status::Fail;  // capture_graph itself returns void
+}
+void gpx_clear(gpx_executor e) { H(e)->ex->clear(); }
+
+int gpx_set_flag(gpx_executor e, void *dp) { if (!H(e)->blp) return Status::Fail; H(e)->blp->dpStop = dp; return Status::Succ; }
+int gpx_set_running(gpx_executor e, int r) { if (!H(e)->blp) return Status::Fail; H(e)->blp->running = r != 0; return Status::Succ; }
+int gpx_resume(gpx_executor e, gp_stream s) { return H(e)->blp ? H(e)->blp->resume(s) : Status::Fail; }
+int gpx_get_stop_point(gpx_executor e, gp_stream s, int *stop) {
+    if (!H(e)->blp) return Status::Fail;
+    Status st = H(e)->blp->getStopPoint(s);
+    if (stop) *stop = H(e)->blp->last_stop_index();
+    return st;
+}
+int gpx_last_stop_index(gpx_executor e) { return H(e)->blp ? H(e)->blp->last_stop_index() : -1; }
+int gpx_inject_preempt(gpx_executor e, int kernel, int claim) { if (!H(e)->blp) return Status::Fail; H(e)->blp->inject_preempt(kernel, claim); return Status::Succ; }
+int gpx_read_counters(gpx_executor e, int *out, size_t n) {
+    if (!H(e)->blp) return Status::Fail;
+    std::vector<int> v;
+    Status st = H(e)->blp->read_counters(v);
+    if (st != Status::Succ) return st;
+    std::memcpy(out, v.data(), sizeof(int) * std::min(n, v.size()));
+    return Status::Succ;
+}
+
+size_t gpx_storage_num(gpx_executor e) { auto m = H(e)->ex->get_model(); return m ? m->get_storage_num() : 0; }
+
+int gpx_kernel_info(gpx_executor e, size_t idx, char *name, size_t name_len, double *flops, double *bytes, int *total_blocks, int *grid) {
+    auto m = H(e)->ex->get_model();
+    if (!m || idx >= m->get_kernel_num()) return Status::OutOfRange;
+    KernelInfo &k = m->get_kernel_info(idx);
+    copy_str(name, name_len, k.name);
+    if (flops) *flops = k.flops;
+    if (bytes) *bytes = k.bytes;
+    if (total_blocks) *total_blocks = k.total_blocks;
+    if (grid) *grid = (int)k.launch_params[0];
+    return Status::Succ;
+}
+
+int gpx_read_storage(gpx_executor e, const char *key, void *out, size_t len) {
+    auto m = H(e)->ex->get_model();
+    if (!m) return Status::Fail;
+    Status st = m->get(key, out, len, nullptr);
+    if (st != Status::Succ) return st;
+    return gp_stream_sync(nullptr) == 0 ? Status::Succ : Status::Fail;
+}
+
+}  // extern "C"
+
+extern "C" int gpx_storage_info(gpx_executor e, size_t idx, char *name, size_t name_len, char *stype, size_t stype_len,
+                                size_t *bytes, int *is_param, size_t *disk_elems, int dims[8]) {
+    auto m = H(e)->ex->get_model();
+    if (!m || idx >= m->get_storage_num()) return Status::OutOfRange;
+    StorageInfo &s = m->get_storage_info(idx);
+    const ParamLayout &L = m->get_param_layout(idx);
+    copy_str(name, name_len, s.name);
+    copy_str(stype, stype_len, s.stype);
+    if (bytes) *bytes = s.size;
+    if (is_param) *is_param = L.is_param;
+    if (disk_elems) *disk_elems = L.disk_elems;
+    if (dims) { int d[8] = {(int)L.kind, L.o, L.i, L.r, L.s, L.c, L.h, L.w}; std::memcpy(dims, d, sizeof(d)); }
+    return Status::Succ;
+}

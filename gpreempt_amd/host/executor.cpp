@@ -1,0 +1,191 @@
+// Executor launch loop and the block-level-preemption protocol on the host side.
+// Behaviour follows the reference's src/executor.cpp (cited per function).
+#include "executor.h"
+
+#include <cstdlib>
+#include <set>
+
+namespace foo {
+
+static const std::set<std::string> kNotBuilt = {"cc", "bfs", "pagerank", "sssp", "miniweather"};
+
+static std::string model_root() {
+    const char *e = std::getenv("GPREEMPT_MODEL_PATH");
+    return e && *e ? std::string(e) : std::string("./model");
+}
+
+Status Executor::set_graph_path(const std::string &path) {
+    graph_path = path;
+    return Status::Succ;
+}
+
+Executor::~Executor() {
+    if (graph_exec) gp_graph_destroy(graph_exec);
+}
+
+// reference executor.cpp:23-45 (dnn branch)
+Status Executor::init(std::string workload) {
+    if (kNotBuilt.count(workload)) {
+        std::fprintf(stderr, "workload '%s' is not part of this build\n", workload.c_str());
+        return Status::NotFound;
+    }
+    type = "dnn";
+    RETURN_STATUS(this->load_model(model_root() + "/" + workload));
+    RETURN_STATUS(this->load_param(model_root() + "/" + workload));
+    return Status::Succ;
+}
+
+// reference executor.cpp:47-95
+Status Executor::set_input(const std::string &key, void *value, size_t len, GPUstream stream) {
+    size_t idx;
+    if (!model || model->find_storage_idx(key, idx) != Status::Succ) return Status::NotFound;
+    return model->set(idx, value, len, stream);
+}
+Status Executor::set_input(const std::string &key, std::vector<float> &value, GPUstream stream) {
+    return set_input(key, value.data(), value.size() * sizeof(float), stream);
+}
+Status Executor::get_output(const std::string &key, void *value, size_t len, GPUstream stream) {
+    size_t idx;
+    if (!model || model->find_storage_idx(key, idx) != Status::Succ) return Status::NotFound;
+    return model->get(idx, value, len, stream);
+}
+Status Executor::get_output(const std::string &key, std::vector<float> &value, GPUstream stream) {
+    return get_output(key, value.data(), value.size() * sizeof(float), stream);
+}
+size_t Executor::get_data_size(const std::string &key) {
+    size_t idx;
+    if (!model || model->find_storage_idx(key, idx) != Status::Succ) return 0;
+    return model->get_storage_size(idx);
+}
+
+void Executor::clear() {
+    if (model) model->clear();
+}
+
+// reference executor.cpp:110-117
+Status Executor::load_model(std::string model_path) {
+    model = std::make_shared<Model>();
+    return model->load_model(model_path + "/mod.json", model_path + "/host.json", model_path + "/mod.co");
+}
+Status Executor::load_param(std::string model_path) { return model->load_param((model_path + "/mod.params").c_str()); }
+
+// reference executor.cpp:119-134
+Status Executor::execute(GPUstream stream) {
+    if (use_cuda_graph) {
+        CUDA_RETURN_STATUS(gp_graph_launch(graph_exec, stream));
+        return Status::Succ;
+    }
+    for (size_t i = 0; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
+    return Status::Succ;
+}
+
+// reference executor.cpp:136-164
+Status Executor::launch_kernel(size_t kernel_offset, GPUstream stream) { return model->launch(kernel_offset, stream); }
+
+size_t Executor::get_kernel_num() const { return model ? model->get_kernel_num() : 0; }
+
+// reference executor.cpp:176-196.  On failure the executor stays in launch-by-launch mode.
+void Executor::capture_graph(GPUstream stream) {
+    if (graph_exec) { gp_graph_destroy(graph_exec); graph_exec = nullptr; }
+    use_cuda_graph = false;
+    if (gp_graph_begin(stream) != 0) return;
+    bool ok = true;
+    for (size_t i = 0; i < get_kernel_num() && ok; i++) ok = launch_kernel(i, stream) == Status::Succ;
+    gp_graph g = nullptr;
+    if (gp_graph_end(stream, &g) != 0 || !ok) {
+        if (g) gp_graph_destroy(g);
+        std::fprintf(stderr, "capture_graph failed: %s\n", gp_last_error());
+        return;
+    }
+    graph_exec = g;
+    use_cuda_graph = true;
+}
+
+BaseExecutor::BaseExecutor() {}
+BaseExecutor::~BaseExecutor() {}
+
+BLPExecutor::BLPExecutor() {}
+
+BLPExecutor::~BLPExecutor() {
+    if (dpStopIndex) gp_free(dpStopIndex);
+    if (executed) gp_free(executed);
+    if (stop_host) gp_host_free(stop_host);
+}
+
+// reference executor.cpp:300-342 (dnn branch): build the model, allocate the stop index (-1) and
+// one counter per kernel, append (flag, stop index) by reference to every kernel and the
+// per-kernel preemption arguments, then load parameters.
+Status BLPExecutor::init(std::string workload) {
+    if (kNotBuilt.count(workload)) {
+        std::fprintf(stderr, "workload '%s' is not part of this build\n", workload.c_str());
+        return Status::NotFound;
+    }
+    type = "dnn";
+    model = std::make_shared<Model>();
+    std::string model_path = model_root() + "/" + workload;
+    RETURN_STATUS(model->load_model(model_path + "/mod.json", model_path + "/host.json", model_path + "/mod.tr.co"));
+    CUDA_RETURN_STATUS(gp_malloc(&dpStopIndex, sizeof(int)));
+    CUDA_RETURN_STATUS(gp_host_alloc((void **)&stop_host, sizeof(int)));
+    stopIndex = -1;
+    CUDA_RETURN_STATUS(gp_memcpy_h2d(dpStopIndex, &stopIndex, sizeof(int)));
+    model->batchAddParam(&this->dpStop);
+    model->batchAddParam(&this->dpStopIndex);
+    CUDA_RETURN_STATUS(gp_malloc(&executed, sizeof(int) * model->get_kernel_num()));
+    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num(), nullptr));
+    CUDA_RETURN_STATUS(gp_stream_sync(nullptr));
+    RETURN_STATUS(model->add_block_preemption_param(executed));
+    RETURN_STATUS(this->load_param(model_path));
+    return Status::Succ;
+}
+
+Status BLPExecutor::launch_kernel(size_t kernel_offset, GPUstream stream) {
+    int inject = ((int)kernel_offset == inject_kernel) ? inject_claim : -1;
+    return model->launch(kernel_offset, stream, inject);
+}
+
+// reference executor.cpp:211-232: zero every tile counter, then launch (or replay the graph).
+// The counters are cleared by a fill kernel outside the captured graph.
+Status BLPExecutor::execute(GPUstream stream) {
+    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num(), stream));
+    if (use_cuda_graph) {
+        CUDA_RETURN_STATUS(gp_graph_launch(graph_exec, stream));
+        return Status::Succ;
+    }
+    for (size_t i = 0; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
+    return Status::Succ;
+}
+
+void BLPExecutor::capture_graph(GPUstream stream) { Executor::capture_graph(stream); }
+
+void BLPExecutor::clear() {
+    if (model) model->clear();
+}
+
+// reference executor.cpp:269-278
+Status BLPExecutor::getStopPoint(GPUstream stream) {
+    CUDA_RETURN_STATUS(gp_memcpy_d2h_async(stop_host, dpStopIndex, sizeof(int), stream));
+    CUDA_RETURN_STATUS(gp_stream_sync(stream));
+    stopIndex = *stop_host;
+    if (stopIndex == -1) return Status::Succ;
+    CUDA_RETURN_STATUS(gp_fill32_async(dpStopIndex, 0xFFFFFFFFu, 1, stream));
+    return Status::Succ;
+}
+
+// reference executor.cpp:280-298: no-op unless running; kernels before the stop index completed,
+// the one at the stop index continues from its counter, later ones start from zero claims.
+// Always launch-by-launch, never through the captured graph.
+Status BLPExecutor::resume(GPUstream stream) {
+    if (!running) return Status::Succ;
+    RETURN_STATUS(getStopPoint(stream));
+    if (stopIndex == -1) return Status::Succ;
+    for (size_t i = (size_t)stopIndex; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
+    return Status::Succ;
+}
+
+Status BLPExecutor::read_counters(std::vector<int> &out) {
+    out.resize(model->get_kernel_num());
+    CUDA_RETURN_STATUS(gp_memcpy_d2h(out.data(), executed, sizeof(int) * out.size()));
+    return Status::Succ;
+}
+
+}  // namespace foo

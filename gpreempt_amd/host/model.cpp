@@ -1,0 +1,345 @@
+// foo::Model: storage planning, parameter loading and kernel launch over the C ABI.
+// Follows the behaviour of the reference's src/model.cpp (cited per function); the graph itself
+// comes from the native builders in zoo.cpp instead of TVM's mod.json / host.json.
+#include "model.h"
+
+#include <cmath>
+#include <cstring>
+#include <fstream>
+
+#include "numeric.h"
+#include "zoo.h"
+
+namespace foo {
+
+static const char kParamMagic[] = "TVM_MODEL_PARAMS";  // 16 chars + NUL = 17 bytes on disk
+
+// File layout (reference src/model.cpp:15-55): magic[17] | u64 count | count x { key\0 | u64 n | f32[n] }.
+ModelParam *ModelParamParser::parse_from_file(const char *param_file) {
+    FILE *fp = std::fopen(param_file, "rb");
+    if (!fp) return nullptr;
+    std::unique_ptr<ModelParam> params(new ModelParam());
+    char magic[sizeof(kParamMagic)];
+    uint64_t count = 0;
+    bool ok = std::fread(magic, 1, sizeof(magic), fp) == sizeof(magic) && std::memcmp(magic, kParamMagic, sizeof(magic)) == 0 &&
+              std::fread(&count, sizeof(count), 1, fp) == 1 && count != 0;
+    for (uint64_t i = 0; ok && i < count; ++i) {
+        std::string key;
+        int c;
+        while ((c = std::fgetc(fp)) != EOF && c != 0 && key.size() < 255) key.push_back((char)c);
+        uint64_t n = 0;
+        ok = c == 0 && std::fread(&n, sizeof(n), 1, fp) == 1 && n != 0 && n < (1ull << 34);
+        if (!ok) break;
+        std::vector<float> values(n);
+        ok = std::fread(values.data(), sizeof(float), n, fp) == n;
+        if (ok) (*params)[key] = std::move(values);
+    }
+    std::fclose(fp);
+    if (!ok) {
+        std::fprintf(stderr, "malformed parameter file %s\n", param_file);
+        return nullptr;
+    }
+    return params.release();
+}
+
+Model::Model() {}
+
+Model::Model(const std::string &device_json, const std::string &host_json, const std::string &cuda_module) {
+    load_model(device_json, host_json, cuda_module);
+}
+
+Model::~Model() { clear(); }
+
+// reference src/model.cpp:69-77, extended with the 16-bit float types the configurations need
+size_t Model::get_stype_size(std::string &stype) {
+    if (stype == "float32") return 4;
+    if (stype == "float16" || stype == "bfloat16") return 2;
+    if (stype == "int64") return 8;
+    if (stype == "int32") return 4;
+    if (stype == "byte" || stype == "uint1") return 1;
+    std::fprintf(stderr, "Unknown stype: %s\n", stype.c_str());
+    return 0;
+}
+
+static std::string parent_dir_name(const std::string &path) {
+    size_t end = path.find_last_of('/');
+    if (end == std::string::npos) return "";
+    std::string dir = path.substr(0, end);
+    while (!dir.empty() && dir.back() == '/') dir.pop_back();
+    size_t b = dir.find_last_of('/');
+    return b == std::string::npos ? dir : dir.substr(b + 1);
+}
+
+Status Model::load_model(const std::string &device_json, const std::string & /*host_json*/, const std::string & /*module*/) {
+    if (is_loaded()) {
+        std::fprintf(stderr, "The model is already loaded\n");  // reference model.cpp:81-84
+        return Status::Fail;
+    }
+    std::string name = parent_dir_name(device_json);
+    if (name.empty()) return Status::NotFound;
+    return build(name);
+}
+
+Status Model::build(const std::string &workload) {
+    if (is_loaded()) return Status::Fail;
+    workload_ = workload;
+    Status s = zoo_build(*this, workload);
+    if (s != Status::Succ) {
+        storage_infos.clear(); layouts.clear(); kernel_infos.clear();
+        return s;
+    }
+    return allocate_and_bind();
+}
+
+// One zero-filled device buffer per storage, then resolve every kernel's pointer slots
+// (reference src/model.cpp:100-124).
+Status Model::allocate_and_bind() {
+    storages.assign(storage_infos.size(), nullptr);
+    for (size_t i = 0; i < storage_infos.size(); ++i) {
+        size_t bytes = storage_infos[i].size;
+        CUDA_RETURN_STATUS(gp_malloc(&storages[i], bytes));
+        CUDA_RETURN_STATUS(gp_fill32_async(storages[i], 0, bytes / 4, nullptr));
+        if (bytes % 4) {
+            std::vector<char> z(bytes % 4, 0);
+            CUDA_RETURN_STATUS(gp_memcpy_h2d((char *)storages[i] + bytes - bytes % 4, z.data(), z.size()));
+        }
+        storages_idx.emplace(storage_infos[i].name, i);
+    }
+    CUDA_RETURN_STATUS(gp_stream_sync(nullptr));
+    for (KernelInfo &k : kernel_infos) {
+        k.args.clear();
+        k.args_index.clear();
+        k.args.reserve(k.refs.size() + 10);
+        for (const ArgRef &r : k.refs) {
+            k.args_index.push_back(r.storage);
+            k.args.push_back(r.storage == SIZE_MAX ? nullptr : (GPUdeviceptr)((char *)storages[r.storage] + r.byte_offset));
+        }
+        bind_pointers(k);
+    }
+    loaded_ = true;
+    // seeded random initialisation of every parameter (overwritten by load_param when a file exists)
+    uint64_t seed = 0x5EEDull;
+    for (size_t i = 0; i < storage_infos.size(); ++i) {
+        const ParamLayout &L = layouts[i];
+        if (!L.is_param) continue;
+        std::vector<float> host(L.disk_elems, 0.f);
+        numeric::Rng rng(seed + 7919 * (uint64_t)i);
+        switch (L.init) {
+            case ParamLayout::InitZero: break;
+            case ParamLayout::InitConst: for (float &v : host) v = L.init_a; break;
+            case ParamLayout::InitUniform: for (float &v : host) v = rng.uniform(L.init_a, L.init_b); break;
+            case ParamLayout::InitNormal: for (float &v : host) v = rng.normal() * L.init_a; break;
+        }
+        RETURN_STATUS(upload_param(i, host.data(), host.size()));
+    }
+    return Status::Succ;
+}
+
+// Slot order per operator is fixed by the builders in zoo.cpp.
+void Model::bind_pointers(KernelInfo &k) {
+    auto P = [&](size_t j) -> void * { return j < k.args.size() ? k.args[j] : nullptr; };
+    switch (k.op) {
+        case OpKind::Nop: break;
+        case OpKind::Gemm: k.p.gemm.A = P(0); k.p.gemm.B = P(1); k.p.gemm.bias = P(2); k.p.gemm.residual = P(3); k.p.gemm.C = P(4); break;
+        case OpKind::Conv: k.p.conv.in = P(0); k.p.conv.weight = P(1); k.p.conv.bias = P(2); k.p.conv.residual = P(3); k.p.conv.out = P(4); break;
+        case OpKind::Layout: k.p.layout.in = P(0); k.p.layout.out = P(1); break;
+        case OpKind::Pool: k.p.pool.in = P(0); k.p.pool.out = P(1); break;
+        case OpKind::Eltwise: k.p.eltwise.a = P(0); k.p.eltwise.b = P(1); k.p.eltwise.scale = P(2); k.p.eltwise.shift = P(3); k.p.eltwise.out = P(4); break;
+        case OpKind::Softmax: k.p.softmax.x = P(0); k.p.softmax.out = P(1); break;
+        case OpKind::Layernorm: k.p.layernorm.x = P(0); k.p.layernorm.residual = P(1); k.p.layernorm.gamma = P(2); k.p.layernorm.beta = P(3); k.p.layernorm.out = P(4); break;
+        case OpKind::Embed: k.p.embed.ids = (const int64_t *)P(0); k.p.embed.tok = P(1); k.p.embed.pos = P(2); k.p.embed.seg = P(3); k.p.embed.out = P(4); break;
+    }
+}
+
+// disk convention (fp32, OIHW / dense over CHW) -> device layout and dtype
+Status Model::upload_param(size_t idx, const float *disk, size_t n) {
+    const ParamLayout &L = layouts[idx];
+    StorageInfo &info = storage_infos[idx];
+    size_t es = get_stype_size(info.stype);
+    size_t dev_elems = info.size / es;
+    if (n < L.disk_elems) return Status::OutOfRange;
+    std::vector<float> dev(dev_elems, 0.f);
+    switch (L.kind) {
+        case ParamLayout::Plain:
+            std::memcpy(dev.data(), disk, sizeof(float) * std::min(dev_elems, n));
+            break;
+        case ParamLayout::ConvOIHW:
+            for (int o = 0; o < L.o; ++o)
+                for (int i = 0; i < L.i; ++i)
+                    for (int r = 0; r < L.r; ++r)
+                        for (int s = 0; s < L.s; ++s)
+                            dev[(((size_t)o * L.r + r) * L.s + s) * L.i_pad + i] = disk[(((size_t)o * L.i + i) * L.r + r) * L.s + s];
+            break;
+        case ParamLayout::DenseOverCHW: {
+            size_t feat = (size_t)L.c * L.h * L.w;
+            for (int o = 0; o < L.o; ++o)
+                for (int c = 0; c < L.c; ++c)
+                    for (int h = 0; h < L.h; ++h)
+                        for (int w = 0; w < L.w; ++w)
+                            dev[o * feat + ((size_t)h * L.w + w) * L.c + c] = disk[o * feat + ((size_t)c * L.h + h) * L.w + w];
+            break;
+        }
+    }
+    if (info.stype == "float32") {
+        CUDA_RETURN_STATUS(gp_memcpy_h2d(storages[idx], dev.data(), info.size));
+    } else {
+        std::vector<uint16_t> half(dev_elems);
+        const bool bf = info.stype == "bfloat16";
+        for (size_t i = 0; i < dev_elems; ++i) half[i] = bf ? numeric::f32_to_bf16(dev[i]) : numeric::f32_to_f16(dev[i]);
+        CUDA_RETURN_STATUS(gp_memcpy_h2d(storages[idx], half.data(), info.size));
+    }
+    return Status::Succ;
+}
+
+// reference src/model.cpp:263-282: copy a tensor only if a storage of the same name exists
+Status Model::load_param(const char *param_file_path) {
+    if (!is_loaded()) return Status::Fail;
+    std::ifstream probe(param_file_path, std::ios::binary);
+    if (!probe.is_open()) return Status::Succ;  // random-init model
+    probe.close();
+    std::unique_ptr<ModelParam> params(ModelParamParser::parse_from_file(param_file_path));
+    if (!params) return Status::Fail;
+    for (size_t i = 0; i < storages.size(); ++i) {
+        auto it = params->find(storage_infos[i].name);
+        if (it == params->end()) continue;
+        if (!layouts[i].is_param) continue;
+        RETURN_STATUS(upload_param(i, it->second.data(), it->second.size()));
+    }
+    return Status::Succ;
+}
+
+bool Model::is_loaded() { return loaded_; }
+
+Status Model::find_storage_idx(const std::string &name, size_t &idx) {
+    auto it = storages_idx.find(name);
+    if (it == storages_idx.end()) return Status::NotFound;
+    idx = it->second;
+    return Status::Succ;
+}
+
+// reference src/model.cpp:296-313: `len` is the caller's buffer size; exactly storage.size bytes move
+Status Model::get(size_t idx, void *out, size_t len, GPUstream stream) {
+    if (idx >= storages.size()) return Status::OutOfRange;
+    size_t size = storage_infos[idx].size;
+    if (len < size) return Status::Fail;
+    CUDA_RETURN_STATUS(gp_memcpy_d2h_async(out, storages[idx], size, stream));
+    return Status::Succ;
+}
+Status Model::get(const std::string &key, void *out, size_t len, GPUstream stream) {
+    size_t idx;
+    if (find_storage_idx(key, idx) != Status::Succ) return Status::NotFound;
+    return get(idx, out, len, stream);
+}
+// reference src/model.cpp:315-330
+Status Model::set(size_t idx, void *value, size_t len, GPUstream stream) {
+    if (idx >= storages.size()) return Status::OutOfRange;
+    size_t size = storage_infos[idx].size;
+    if (len < size) return Status::OutOfRange;
+    CUDA_RETURN_STATUS(gp_memcpy_h2d_async(storages[idx], value, size, stream));
+    return Status::Succ;
+}
+Status Model::set(const std::string &key, void *value, size_t len, GPUstream stream) {
+    size_t idx;
+    if (find_storage_idx(key, idx) != Status::Succ) return Status::NotFound;
+    return set(idx, value, len, stream);
+}
+
+size_t Model::get_kernel_num() const { return kernel_infos.size(); }
+size_t Model::get_storage_num() const { return storage_infos.size(); }
+StorageInfo &Model::get_storage_info(size_t idx) { return storage_infos[idx]; }
+GPUdeviceptr Model::get_storage_ptr(size_t idx) { return storages[idx]; }
+size_t Model::get_storage_size(size_t idx) { return storage_infos[idx].size; }
+KernelInfo &Model::get_kernel_info(size_t idx) { return kernel_infos[idx]; }
+
+// The reference resolves a symbol of the loaded GPU module (model.cpp:353-356); the native
+// kernels have no module-level globals, so a name can only denote a storage.
+Status Model::get_global_ptr(const std::string &name, GPUdeviceptr *ptr) {
+    size_t idx;
+    if (find_storage_idx(name, idx) != Status::Succ) return Status::NotFound;
+    *ptr = storages[idx];
+    return Status::Succ;
+}
+
+Status Model::clear() {
+    if (!loaded_) return Status::Succ;
+    for (GPUdeviceptr p : storages) CUDA_RETURN_STATUS(gp_free(p));
+    storage_infos.clear(); layouts.clear(); kernel_infos.clear(); storages.clear(); storages_idx.clear();
+    loaded_ = false;
+    return Status::Succ;
+}
+
+// Appends one by-reference argument to every kernel, "nop" included (reference model.cpp:358-364).
+// BLPExecutor::init calls it twice: first &dpStop (the flag), then &dpStopIndex.
+Status Model::batchAddParam(GPUdeviceptr *ptr) {
+    for (KernelInfo &k : kernel_infos) k.args_ptr.push_back(ptr);
+    return Status::Succ;
+}
+
+// Per kernel: total_blocks, &executed[i], kernel id i; "nop" kernels are skipped but keep their
+// index (reference model.cpp:366-396).  The persistent grid (min(total_blocks, resident
+// workgroups)) is resolved by the device layer at launch.
+Status Model::add_block_preemption_param(GPUdeviceptr ptr) {
+    for (size_t i = 0; i < kernel_infos.size(); ++i) {
+        KernelInfo &k = kernel_infos[i];
+        if (k.name == "nop") continue;
+        if (k.args_ptr.size() < 2) return Status::Fail;
+        k.preemptible = true;
+        k.executed = (GPUdeviceptr)((char *)ptr + i * sizeof(int));
+        k.kernel_id = (int)i;
+    }
+    return Status::Succ;
+}
+
+Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
+    if (idx >= kernel_infos.size()) return Status::OutOfRange;
+    KernelInfo &k = kernel_infos[idx];
+    if (k.op == OpKind::Nop) {
+        // reference src/executor.cpp:139-146: copy size(args_index[0]) bytes, args[1] <- args[0]
+        size_t size = get_storage_size(k.args_index[0]);
+        CUDA_RETURN_STATUS(gp_memcpy_d2d_async(k.args[1], k.args[0], size, stream));
+        return Status::Succ;
+    }
+    gp_preempt_ctx ctx{};
+    const gp_preempt_ctx *pc = nullptr;
+    if (k.preemptible) {
+        size_t n = k.args_ptr.size();
+        ctx.flag = (int *)*k.args_ptr[n - 2];
+        ctx.stop_index = (int *)*k.args_ptr[n - 1];
+        ctx.executed = (int *)k.executed;
+        ctx.kernel_id = k.kernel_id;
+        ctx.inject_at = inject_at;
+        ctx.max_workgroups = 0;
+        pc = &ctx;
+    }
+    gp_launch_info info{};
+    int rc = GP_FAIL;
+    switch (k.op) {
+        case OpKind::Gemm: rc = gp_launch_gemm(&k.p.gemm, pc, stream, &info); break;
+        case OpKind::Conv: rc = gp_launch_conv2d(&k.p.conv, pc, stream, &info); break;
+        case OpKind::Layout: rc = gp_launch_nchw_to_nhwc(&k.p.layout, pc, stream, &info); break;
+        case OpKind::Pool: rc = gp_launch_pool2d(&k.p.pool, pc, stream, &info); break;
+        case OpKind::Eltwise: rc = gp_launch_eltwise(&k.p.eltwise, pc, stream, &info); break;
+        case OpKind::Softmax: rc = gp_launch_softmax(&k.p.softmax, pc, stream, &info); break;
+        case OpKind::Layernorm: rc = gp_launch_layernorm(&k.p.layernorm, pc, stream, &info); break;
+        case OpKind::Embed: rc = gp_launch_embed(&k.p.embed, pc, stream, &info); break;
+        case OpKind::Nop: break;
+    }
+    CUDA_RETURN_STATUS(rc);
+    k.total_blocks = info.total_tiles;
+    k.launch_params[0] = (uint32_t)info.grid; k.launch_params[1] = 1; k.launch_params[2] = 1;
+    k.launch_params[3] = (uint32_t)info.block; k.launch_params[4] = 1; k.launch_params[5] = 1;
+    return Status::Succ;
+}
+
+double Model::total_flops() const {
+    double f = 0;
+    for (const KernelInfo &k : kernel_infos) f += k.flops;
+    return f;
+}
+double Model::total_bytes() const {
+    double b = 0;
+    for (const KernelInfo &k : kernel_infos) b += k.bytes;
+    return b;
+}
+
+}  // namespace foo

@@ -1,0 +1,476 @@
+// Native graph builders: the model set the reference exports through TVM
+// (scripts/compile/compile.py:28-44: resnet, vgg, densenet, inception; compile-bert.py) rebuilt
+// as kernel lists over the operators of libgpreempt_hip.so, at the shapes the benchmark
+// configurations name.  Activations are NHWC with 16-byte aligned channel counts; parameters are
+// declared in the reference's on-disk convention (fp32, OIHW) and re-laid-out at load time.
+#include "zoo.h"
+
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <sstream>
+
+namespace foo {
+
+namespace {
+
+struct Tensor {            // NHWC view into a storage
+    size_t st = SIZE_MAX;
+    size_t off = 0;        // element offset of channel 0 of pixel 0
+    int N = 0, H = 0, W = 0, C = 0;
+    long ps = 0;           // pixel stride in elements
+};
+
+}  // namespace
+
+class GraphBuilder {
+public:
+    GraphBuilder(Model &m, const std::string &dt) : m_(m), dt_(dt) {
+        if (dt == "f32") { stype_ = "float32"; gp_dt_ = GP_F32; es_ = 4; vec_ = 4; }
+        else if (dt == "f16") { stype_ = "float16"; gp_dt_ = GP_F16; es_ = 2; vec_ = 8; }
+        else { stype_ = "bfloat16"; gp_dt_ = GP_BF16; es_ = 2; vec_ = 8; }
+        m_.dtype_ = dt;
+    }
+    int vec() const { return vec_; }
+    int gp_dtype() const { return gp_dt_; }
+    size_t es() const { return es_; }
+    int pad_c(int c) const { return (c + vec_ - 1) / vec_ * vec_; }
+
+    size_t add_storage(const std::string &name, size_t elems, const std::string &stype, const ParamLayout &L = ParamLayout()) {
+        StorageInfo info;
+        info.name = name; info.stype = stype;
+        std::string st = stype;
+        info.size = elems * Model::get_stype_size(st);
+        m_.storage_infos.push_back(info);
+        m_.layouts.push_back(L);
+        return m_.storage_infos.size() - 1;
+    }
+    size_t add_param(const std::string &name, size_t dev_elems, ParamLayout L) {
+        L.is_param = true;
+        return add_storage(name, dev_elems, stype_, L);
+    }
+    Tensor activation(const std::string &name, int N, int H, int W, int C) {
+        Tensor t;
+        t.st = add_storage(name, (size_t)N * H * W * C, stype_);
+        t.N = N; t.H = H; t.W = W; t.C = C; t.ps = C;
+        return t;
+    }
+    static Tensor slice(const Tensor &t, int c0, int c) {
+        Tensor s = t;
+        s.off += c0; s.C = c;
+        return s;
+    }
+    ArgRef ref(const Tensor &t) const { ArgRef r; r.storage = t.st; r.byte_offset = t.off * es_; return r; }
+    static ArgRef ref(size_t st, size_t byte_off = 0) { ArgRef r; r.storage = st; r.byte_offset = byte_off; return r; }
+    static ArgRef none() { return ArgRef(); }
+
+    KernelInfo &add_kernel(const std::string &name, OpKind op, std::vector<ArgRef> refs, double flops, double bytes) {
+        KernelInfo k;
+        k.name = name; k.op = op; k.refs = std::move(refs); k.flops = flops; k.bytes = bytes;
+        std::memset(&k.p, 0, sizeof(k.p));
+        std::memset(k.launch_params, 0, sizeof(k.launch_params));
+        m_.kernel_infos.push_back(std::move(k));
+        return m_.kernel_infos.back();
+    }
+
+    // conv + folded-BN bias + optional residual + activation; writes into `into` when given
+    Tensor conv(const std::string &name, const Tensor &in, int cout, int k, int stride, int pad, int act,
+                const Tensor *residual = nullptr, const Tensor *into = nullptr, int cin_logical = -1, float init_gain = 1.f) {
+        int Ho = (in.H + 2 * pad - k) / stride + 1, Wo = (in.W + 2 * pad - k) / stride + 1;
+        int cin = cin_logical > 0 ? cin_logical : in.C;
+        ParamLayout L;
+        L.kind = ParamLayout::ConvOIHW; L.o = cout; L.i = cin; L.r = k; L.s = k; L.i_pad = in.C;
+        L.disk_elems = (size_t)cout * cin * k * k;
+        L.init = ParamLayout::InitNormal; L.init_a = init_gain * std::sqrt(2.f / (float)(cin * k * k));  // He-normal
+        size_t w = add_param(name + ".weight", (size_t)cout * k * k * in.C, L);
+        ParamLayout LB; LB.disk_elems = cout; LB.init = ParamLayout::InitZero;
+        size_t b = add_param(name + ".bias", cout, LB);
+        Tensor out = into ? *into : activation(name + ".out", in.N, Ho, Wo, cout);
+        double flops = 2.0 * in.N * Ho * Wo * cout * (double)cin * k * k;
+        double bytes = es_ * ((double)in.N * in.H * in.W * cin + (double)cout * cin * k * k + cout + (double)in.N * Ho * Wo * cout * (residual ? 2 : 1));
+        KernelInfo &ki = add_kernel("conv2d", OpKind::Conv, {ref(in), ref(w), ref(b), residual ? ref(*residual) : none(), ref(out)}, flops, bytes);
+        gp_conv_params &p = ki.p.conv;
+        p.dtype = gp_dt_; p.N = in.N; p.H = in.H; p.W = in.W; p.Cin = in.C; p.Cout = cout; p.R = k; p.S = k;
+        p.stride_h = p.stride_w = stride; p.pad_h = p.pad_w = pad;
+        p.in_pix_stride = in.ps; p.res_pix_stride = residual ? residual->ps : 0; p.out_pix_stride = out.ps; p.act = act;
+        Tensor o = out; o.N = in.N; o.H = Ho; o.W = Wo; o.C = cout;
+        return o;
+    }
+
+    Tensor pool(const std::string &name, const Tensor &in, int k, int stride, int pad, int mode, const Tensor *into = nullptr) {
+        int Ho = mode == 2 ? 1 : (in.H + 2 * pad - k) / stride + 1, Wo = mode == 2 ? 1 : (in.W + 2 * pad - k) / stride + 1;
+        Tensor out = into ? *into : activation(name + ".out", in.N, Ho, Wo, in.C);
+        double bytes = es_ * ((double)in.N * in.H * in.W * in.C + (double)in.N * Ho * Wo * in.C);
+        KernelInfo &ki = add_kernel("pool2d", OpKind::Pool, {ref(in), ref(out)}, 0, bytes);
+        gp_pool_params &p = ki.p.pool;
+        p.dtype = gp_dt_; p.N = in.N; p.H = in.H; p.W = in.W; p.C = in.C; p.R = k; p.S = k; p.stride = stride; p.pad = pad; p.mode = mode;
+        p.in_pix_stride = in.ps; p.out_pix_stride = out.ps;
+        Tensor o = out; o.N = in.N; o.H = Ho; o.W = Wo; o.C = in.C;
+        return o;
+    }
+
+    // out = act((a [+ b]) * scale + shift); scale/shift are parameters when affine_name is set
+    Tensor eltwise(const std::string &name, const Tensor &a, const Tensor *b, const std::string &affine_name, int act, const Tensor *into = nullptr) {
+        Tensor out = into ? *into : activation(name + ".out", a.N, a.H, a.W, a.C);
+        size_t sc = SIZE_MAX, sh = SIZE_MAX;
+        if (!affine_name.empty()) {
+            ParamLayout L1; L1.disk_elems = a.C; L1.init = ParamLayout::InitConst; L1.init_a = 1.f;
+            sc = add_param(affine_name + ".scale", a.C, L1);
+            ParamLayout L0; L0.disk_elems = a.C; L0.init = ParamLayout::InitZero;
+            sh = add_param(affine_name + ".shift", a.C, L0);
+        }
+        double elems = (double)a.N * a.H * a.W * a.C;
+        KernelInfo &ki = add_kernel("eltwise", OpKind::Eltwise, {ref(a), b ? ref(*b) : none(), sc == SIZE_MAX ? none() : ref(sc), sh == SIZE_MAX ? none() : ref(sh), ref(out)},
+                                    elems, es_ * elems * (b ? 3 : 2));
+        gp_eltwise_params &p = ki.p.eltwise;
+        p.dtype = gp_dt_; p.rows = (long)a.N * a.H * a.W; p.cols = a.C; p.a_stride = a.ps; p.b_stride = b ? b->ps : 0; p.out_stride = out.ps; p.act = act;
+        Tensor o = out; o.N = a.N; o.H = a.H; o.W = a.W; o.C = a.C;
+        return o;
+    }
+
+    // dense layer: rows x in_features -> rows x units; weight on disk [units][in_features]
+    size_t dense(const std::string &name, size_t in_st, size_t in_off_bytes, long rows, int in_f, long lda, int units, int act,
+                 size_t residual_st, size_t out_st, size_t out_off_bytes, long ldc, float init_std, const ParamLayout *wl = nullptr) {
+        ParamLayout L;
+        if (wl) L = *wl;
+        L.o = units; L.disk_elems = (size_t)units * in_f; L.init = ParamLayout::InitNormal; L.init_a = init_std;
+        size_t w = add_param(name + ".weight", (size_t)units * in_f, L);
+        ParamLayout LB; LB.disk_elems = units; LB.init = ParamLayout::InitZero;
+        size_t b = add_param(name + ".bias", units, LB);
+        double flops = 2.0 * rows * units * (double)in_f;
+        double bytes = es_ * ((double)rows * in_f + (double)units * in_f + units + (double)rows * units * (residual_st == SIZE_MAX ? 1 : 2));
+        KernelInfo &ki = add_kernel("dense", OpKind::Gemm, {ref(in_st, in_off_bytes), ref(w), ref(b), residual_st == SIZE_MAX ? none() : ref(residual_st), ref(out_st, out_off_bytes)}, flops, bytes);
+        gp_gemm_params &p = ki.p.gemm;
+        p.dtype = gp_dt_; p.M = (int)rows; p.N = units; p.K = in_f; p.lda = lda; p.ldb = in_f; p.b_is_nk = 1; p.ldc = ldc; p.alpha = 1.f; p.act = act; p.batch = 1;
+        return w;
+    }
+
+    void softmax(size_t x_st, size_t out_st, long rows, int cols, float scale) {
+        double e = (double)rows * cols;
+        KernelInfo &ki = add_kernel("softmax", OpKind::Softmax, {ref(x_st), ref(out_st)}, 5 * e, 2 * es_ * e);
+        gp_softmax_params &p = ki.p.softmax;
+        p.dtype = gp_dt_; p.rows = rows; p.cols = cols; p.scale = scale;
+    }
+
+    Tensor input_nchw(int N, int C, int H, int W) {
+        // "data" is NCHW in the model dtype, as the reference feeds it (src/tests/test-dnn.cpp:25-30)
+        size_t data = add_storage("data", (size_t)N * C * H * W, stype_);
+        Tensor t = activation("data.nhwc", N, H, W, pad_c(C));
+        double e = (double)N * H * W;
+        KernelInfo &ki = add_kernel("nchw_to_nhwc", OpKind::Layout, {ref(data), ref(t)}, 0, es_ * e * (C + t.C));
+        gp_layout_params &p = ki.p.layout;
+        p.dtype_in = p.dtype_out = gp_dt_; p.N = N; p.C = C; p.H = H; p.W = W; p.c_pad = t.C;
+        return t;
+    }
+
+    Model &m_;
+    std::string dt_, stype_;
+    int gp_dt_ = 0, vec_ = 4;
+    size_t es_ = 4;
+};
+
+namespace {
+
+// ---- option parsing: "name@key=value,key=value" ------------------------------------------------
+struct Options {
+    std::string name;
+    std::map<std::string, std::string> kv;
+    int geti(const std::string &k, int d) const { auto it = kv.find(k); return it == kv.end() ? d : std::atoi(it->second.c_str()); }
+    std::string gets(const std::string &k, const std::string &d) const { auto it = kv.find(k); return it == kv.end() ? d : it->second; }
+};
+
+Options parse(const std::string &workload) {
+    Options o;
+    size_t at = workload.find('@');
+    o.name = workload.substr(0, at);
+    if (at != std::string::npos) {
+        std::stringstream ss(workload.substr(at + 1));
+        std::string item;
+        while (std::getline(ss, item, ',')) {
+            size_t eq = item.find('=');
+            if (eq != std::string::npos) o.kv[item.substr(0, eq)] = item.substr(eq + 1);
+        }
+    }
+    return o;
+}
+
+bool valid_dtype(const std::string &d) { return d == "f32" || d == "f16" || d == "bf16"; }
+
+// ---- config 1 / config 5: C = act(A * B + bias) as a one-kernel model --------------------------
+// storages: "data" = A (M x K), "B" (K x N, or N x K with layout=nk), "bias" (N), "heads" = C.
+Status build_gemm(Model &m, const Options &o, int M, int N, int K, const std::string &dt_default, int act_default) {
+    std::string dt = o.gets("dtype", dt_default);
+    if (!valid_dtype(dt)) return Status::OutOfRange;
+    GraphBuilder g(m, dt);
+    M = o.geti("m", M); N = o.geti("n", N); K = o.geti("k", K);
+    bool nk = o.gets("layout", "kn") == "nk";
+    int act = o.geti("act", act_default);
+    int tile = o.geti("tile", 0);
+    size_t a = g.add_storage("data", (size_t)M * K, g.stype_);
+    ParamLayout LB; LB.disk_elems = (size_t)K * N; LB.init = ParamLayout::InitUniform; LB.init_a = -1.f; LB.init_b = 1.f;
+    size_t b = g.add_param("B", (size_t)K * N, LB);
+    ParamLayout Lb; Lb.disk_elems = N; Lb.init = ParamLayout::InitUniform; Lb.init_a = -0.1f; Lb.init_b = 0.1f;
+    size_t bias = g.add_param("bias", N, Lb);
+    size_t c = g.add_storage("heads", (size_t)M * N, g.stype_);
+    bool use_bias = o.geti("bias", 1) != 0;
+    double flops = 2.0 * M * N * (double)K + (use_bias ? 2.0 * M * N : 0);
+    double bytes = g.es() * ((double)M * K + (double)K * N + (use_bias ? N : 0) + (double)M * N);
+    KernelInfo &k = g.add_kernel("gemm", OpKind::Gemm, {GraphBuilder::ref(a), GraphBuilder::ref(b), use_bias ? GraphBuilder::ref(bias) : GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(c)}, flops, bytes);
+    gp_gemm_params &p = k.p.gemm;
+    p.dtype = g.gp_dtype(); p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = nk ? K : N; p.b_is_nk = nk; p.ldc = N; p.alpha = 1.f; p.act = act; p.batch = 1;
+    p.tile_m = p.tile_n = tile;
+    return Status::Succ;
+}
+
+// ---- ResNet v1 with bottleneck blocks ----------------------------------------------------------
+// conv7x7/2-64 -> maxpool3x3/2 -> stages of [1x1, 3x3, 1x1(+shortcut)] -> global average pool ->
+// FC 1000 -> softmax.  Batch-norm is folded into each convolution's weight and bias.  The stride
+// of a down-sampling block sits on its first 1x1 convolution (the original "v1" placement) and
+// on the 1x1 projection shortcut.
+Status build_resnet(Model &m, const Options &o, const int (&blocks)[4], int batch_default, const std::string &dt_default) {
+    std::string dt = o.gets("dtype", dt_default);
+    if (!valid_dtype(dt)) return Status::OutOfRange;
+    GraphBuilder g(m, dt);
+    int N = o.geti("b", batch_default), HW = o.geti("hw", 224), classes = o.geti("classes", 1000);
+    int base = o.geti("width", 64);
+    Tensor x = g.input_nchw(N, 3, HW, HW);
+    x = g.conv("conv1", x, base, 7, 2, 3, GP_ACT_RELU, nullptr, nullptr, 3);
+    x = g.pool("pool1", x, 3, 2, 1, 0);
+    for (int s = 0; s < 4; ++s) {
+        int width = base << s;
+        for (int b = 0; b < blocks[s]; ++b) {
+            std::string n = "layer" + std::to_string(s + 1) + "." + std::to_string(b);
+            int stride = (b == 0 && s > 0) ? 2 : 1;
+            Tensor shortcut = x;
+            if (b == 0) shortcut = g.conv(n + ".downsample", x, width * 4, 1, stride, 0, GP_ACT_NONE);
+            Tensor y = g.conv(n + ".conv1", x, width, 1, stride, 0, GP_ACT_RELU);
+            y = g.conv(n + ".conv2", y, width, 3, 1, 1, GP_ACT_RELU);
+            // The block's last convolution starts small (a folded batch-norm with a small gamma):
+            // without it 50 un-normalised residual additions overflow fp16.
+            x = g.conv(n + ".conv3", y, width * 4, 1, 1, 0, GP_ACT_RELU, &shortcut, nullptr, -1, 0.2f);
+        }
+    }
+    Tensor gap = g.pool("avgpool", x, 0, 1, 0, 2);
+    size_t logits = g.add_storage("fc.out", (size_t)N * classes, g.stype_);
+    g.dense("fc", gap.st, 0, N, gap.C, gap.C, classes, GP_ACT_NONE, SIZE_MAX, logits, 0, classes, 0.01f);
+    size_t heads = g.add_storage("heads", (size_t)N * classes, g.stype_);
+    g.softmax(logits, heads, N, classes, 1.f);
+    return Status::Succ;
+}
+
+// ---- VGG-16 -----------------------------------------------------------------------------------
+Status build_vgg16(Model &m, const Options &o) {
+    std::string dt = o.gets("dtype", "f16");
+    if (!valid_dtype(dt)) return Status::OutOfRange;
+    GraphBuilder g(m, dt);
+    int N = o.geti("b", 16), HW = o.geti("hw", 224), classes = o.geti("classes", 1000), fc = o.geti("fc", 4096);
+    int div = o.geti("wdiv", 1);
+    const int cfg[] = {64, 64, -1, 128, 128, -1, 256, 256, 256, -1, 512, 512, 512, -1, 512, 512, 512, -1};
+    Tensor x = g.input_nchw(N, 3, HW, HW);
+    int ci = 0, pi = 0;
+    bool first = true;
+    for (int c : cfg) {
+        if (c < 0) x = g.pool("pool" + std::to_string(++pi), x, 2, 2, 0, 0);
+        else {
+            x = g.conv("conv" + std::to_string(++ci), x, c / div, 3, 1, 1, GP_ACT_RELU, nullptr, nullptr, first ? 3 : -1);
+            first = false;
+        }
+    }
+    // flatten is a view (the reference copies through a "__nop" kernel, src/model.cpp:201-207);
+    // fc1's weight is declared over the NCHW flatten and permuted to NHWC order at load time.
+    int feat = x.H * x.W * x.C;
+    ParamLayout L; L.kind = ParamLayout::DenseOverCHW; L.c = x.C; L.h = x.H; L.w = x.W;
+    size_t h1 = g.add_storage("fc1.out", (size_t)N * fc, g.stype_);
+    g.dense("fc1", x.st, 0, N, feat, feat, fc, GP_ACT_RELU, SIZE_MAX, h1, 0, fc, std::sqrt(2.f / feat), &L);
+    size_t h2 = g.add_storage("fc2.out", (size_t)N * fc, g.stype_);
+    g.dense("fc2", h1, 0, N, fc, fc, fc, GP_ACT_RELU, SIZE_MAX, h2, 0, fc, std::sqrt(2.f / fc));
+    size_t logits = g.add_storage("fc3.out", (size_t)N * classes, g.stype_);
+    g.dense("fc3", h2, 0, N, fc, fc, classes, GP_ACT_NONE, SIZE_MAX, logits, 0, classes, 0.01f);
+    size_t heads = g.add_storage("heads", (size_t)N * classes, g.stype_);
+    g.softmax(logits, heads, N, classes, 1.f);
+    return Status::Succ;
+}
+
+// ---- DenseNet-201 -----------------------------------------------------------------------------
+// conv7x7/2 -> maxpool -> dense blocks [6,12,48,32] with growth 32 and 1x1 bottlenecks of 128,
+// transitions halve channels and average-pool 2x2.  Batch-norm precedes each convolution here,
+// so only the norm that FOLLOWS a convolution (stem, bottleneck 1x1) folds into it; the others
+// run as per-channel scale-shift-ReLU kernels.  A dense block is one NHWC buffer as wide as its
+// final channel count: every layer writes its 32 new channels into its slice of that buffer,
+// which is concatenation without a copy.
+Status build_densenet201(Model &m, const Options &o) {
+    std::string dt = o.gets("dtype", "f16");
+    if (!valid_dtype(dt)) return Status::OutOfRange;
+    GraphBuilder g(m, dt);
+    int N = o.geti("b", 4), HW = o.geti("hw", 224), classes = o.geti("classes", 1000);
+    int growth = o.geti("growth", 32), init_c = o.geti("init", 64), bn_size = 4;
+    int blocks[4] = {o.geti("l1", 6), o.geti("l2", 12), o.geti("l3", 48), o.geti("l4", 32)};
+    Tensor x = g.input_nchw(N, 3, HW, HW);
+    x = g.conv("conv0", x, init_c, 7, 2, 3, GP_ACT_RELU, nullptr, nullptr, 3);  // + norm0 folded + relu
+    int C = init_c;
+    int H = (x.H + 2 - 3) / 2 + 1;
+    Tensor buf = g.activation("block1.buf", N, H, H, C + blocks[0] * growth);
+    Tensor first = GraphBuilder::slice(buf, 0, C);
+    g.pool("pool0", x, 3, 2, 1, 0, &first);
+    for (int b = 0; b < 4; ++b) {
+        std::string bn = "block" + std::to_string(b + 1);
+        for (int l = 0; l < blocks[b]; ++l) {
+            std::string n = bn + ".layer" + std::to_string(l + 1);
+            Tensor in = GraphBuilder::slice(buf, 0, C);
+            Tensor t = g.eltwise(n + ".norm1", in, nullptr, n + ".norm1", GP_ACT_RELU);
+            t = g.conv(n + ".conv1", t, bn_size * growth, 1, 1, 0, GP_ACT_RELU);          // + norm2 folded + relu
+            Tensor dst = GraphBuilder::slice(buf, C, growth);
+            g.conv(n + ".conv2", t, growth, 3, 1, 1, GP_ACT_NONE, nullptr, &dst);
+            C += growth;
+        }
+        if (b < 3) {
+            std::string n = "transition" + std::to_string(b + 1);
+            if ((C / 2) % g.vec() != 0) return Status::OutOfRange;  // halved channel count must stay 16-byte aligned
+            Tensor t = g.eltwise(n + ".norm", buf, nullptr, n + ".norm", GP_ACT_RELU);
+            t = g.conv(n + ".conv", t, C / 2, 1, 1, 0, GP_ACT_NONE);
+            C /= 2;
+            Tensor next = g.activation("block" + std::to_string(b + 2) + ".buf", N, t.H / 2, t.W / 2, C + blocks[b + 1] * growth);
+            Tensor dst = GraphBuilder::slice(next, 0, C);
+            g.pool(n + ".pool", t, 2, 2, 0, 1, &dst);
+            buf = next;
+        }
+    }
+    Tensor t = g.eltwise("norm5", buf, nullptr, "norm5", GP_ACT_RELU);
+    Tensor gap = g.pool("avgpool", t, 0, 1, 0, 2);
+    size_t logits = g.add_storage("classifier.out", (size_t)N * classes, g.stype_);
+    g.dense("classifier", gap.st, 0, N, gap.C, gap.C, classes, GP_ACT_NONE, SIZE_MAX, logits, 0, classes, 0.01f);
+    size_t heads = g.add_storage("heads", (size_t)N * classes, g.stype_);
+    g.softmax(logits, heads, N, classes, 1.f);
+    return Status::Succ;
+}
+
+// ---- BERT encoder -----------------------------------------------------------------------------
+// token + position + segment-0 embedding -> LayerNorm -> L x { fused QKV dense, per-head
+// softmax(Q K^T / sqrt(d)) V as two batched GEMMs over head slices of the QKV buffer, output
+// dense + residual, LayerNorm, FFN dense + erf-GELU, dense + residual, LayerNorm }; eps 1e-12.
+// "data" holds int64 token ids (reference src/tests/test-dnn.cpp:21-23); "heads" is the last
+// hidden state [batch*seq, hidden].
+Status build_bert(Model &m, const Options &o) {
+    std::string dt = o.gets("dtype", "f16");
+    if (!valid_dtype(dt)) return Status::OutOfRange;
+    GraphBuilder g(m, dt);
+    int B = o.geti("b", 1), S = o.geti("s", 128), L = o.geti("layers", 12), Hd = o.geti("hidden", 768);
+    int heads = o.geti("heads", 12), F = o.geti("ffn", 3072), vocab = o.geti("vocab", 30522), maxpos = o.geti("maxpos", 512);
+    if (Hd % heads || S > maxpos) return Status::OutOfRange;
+    int d = Hd / heads;
+    long T = (long)B * S;
+    const float std_ = 0.02f;
+    size_t es = g.es();
+    auto table = [&](const std::string &name, size_t rows) {
+        ParamLayout P; P.o = (int)rows; P.disk_elems = rows * Hd; P.init = ParamLayout::InitNormal; P.init_a = std_;
+        return g.add_param(name, rows * Hd, P);
+    };
+    auto ln_params = [&](const std::string &name, size_t &gamma, size_t &beta) {
+        ParamLayout G; G.disk_elems = Hd; G.init = ParamLayout::InitConst; G.init_a = 1.f;
+        gamma = g.add_param(name + ".gamma", Hd, G);
+        ParamLayout Bt; Bt.disk_elems = Hd; Bt.init = ParamLayout::InitZero;
+        beta = g.add_param(name + ".beta", Hd, Bt);
+    };
+    auto layernorm = [&](const std::string &name, size_t x, size_t res, size_t out) {
+        size_t ga, be;
+        ln_params(name, ga, be);
+        double e = (double)T * Hd;
+        KernelInfo &k = g.add_kernel("layernorm", OpKind::Layernorm, {GraphBuilder::ref(x), res == SIZE_MAX ? GraphBuilder::none() : GraphBuilder::ref(res), GraphBuilder::ref(ga), GraphBuilder::ref(be), GraphBuilder::ref(out)},
+                                     8 * e, es * e * (res == SIZE_MAX ? 2 : 3));
+        gp_layernorm_params &p = k.p.layernorm;
+        p.dtype = g.gp_dtype(); p.rows = T; p.cols = Hd; p.eps = 1e-12f;
+    };
+
+    size_t ids = g.add_storage("data", (size_t)T, "int64");
+    size_t tok = table("embeddings.word", vocab), pos = table("embeddings.position", maxpos), seg = table("embeddings.token_type", 1);
+    size_t emb = g.add_storage("embeddings.sum", (size_t)T * Hd, g.stype_);
+    {
+        KernelInfo &k = g.add_kernel("embed", OpKind::Embed, {GraphBuilder::ref(ids), GraphBuilder::ref(tok), GraphBuilder::ref(pos), GraphBuilder::ref(seg), GraphBuilder::ref(emb)},
+                                     2.0 * T * Hd, 8.0 * T + es * 4.0 * T * Hd);
+        gp_embed_params &p = k.p.embed;
+        p.dtype = g.gp_dtype(); p.tokens = T; p.seq = S; p.hidden = Hd; p.vocab = vocab;
+    }
+    size_t x = g.add_storage("embeddings.out", (size_t)T * Hd, g.stype_);
+    layernorm("embeddings.ln", emb, SIZE_MAX, x);
+
+    for (int l = 0; l < L; ++l) {
+        std::string n = "layer" + std::to_string(l);
+        size_t qkv = g.add_storage(n + ".qkv", (size_t)T * 3 * Hd, g.stype_);
+        g.dense(n + ".attn.qkv", x, 0, T, Hd, Hd, 3 * Hd, GP_ACT_NONE, SIZE_MAX, qkv, 0, 3 * Hd, std_);
+        size_t sc = g.add_storage(n + ".scores", (size_t)B * heads * S * S, g.stype_);
+        {   // scores[b,h] = Q[b,h] K[b,h]^T / sqrt(d)
+            double flops = 2.0 * B * heads * (double)S * S * d;
+            KernelInfo &k = g.add_kernel("batch_matmul_qk", OpKind::Gemm, {GraphBuilder::ref(qkv, 0), GraphBuilder::ref(qkv, (size_t)Hd * es), GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(sc)},
+                                         flops, es * (2.0 * T * Hd + (double)B * heads * S * S));
+            gp_gemm_params &p = k.p.gemm;
+            p.dtype = g.gp_dtype(); p.M = S; p.N = S; p.K = d; p.lda = 3 * Hd; p.ldb = 3 * Hd; p.b_is_nk = 1; p.ldc = S;
+            p.alpha = 1.f / std::sqrt((float)d); p.act = GP_ACT_NONE; p.batch = B * heads; p.batch_inner = heads;
+            p.stride_a = d; p.stride_b = d; p.stride_c = (long)S * S;
+            p.stride_a_outer = (long)S * 3 * Hd; p.stride_b_outer = (long)S * 3 * Hd; p.stride_c_outer = (long)heads * S * S;
+        }
+        size_t pr = g.add_storage(n + ".probs", (size_t)B * heads * S * S, g.stype_);
+        g.softmax(sc, pr, (long)B * heads * S, S, 1.f);
+        size_t ctx = g.add_storage(n + ".context", (size_t)T * Hd, g.stype_);
+        {   // context[b,:,h] = probs[b,h] V[b,h]
+            double flops = 2.0 * B * heads * (double)S * S * d;
+            KernelInfo &k = g.add_kernel("batch_matmul_pv", OpKind::Gemm, {GraphBuilder::ref(pr), GraphBuilder::ref(qkv, (size_t)2 * Hd * es), GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(ctx)},
+                                         flops, es * ((double)B * heads * S * S + 2.0 * T * Hd));
+            gp_gemm_params &p = k.p.gemm;
+            p.dtype = g.gp_dtype(); p.M = S; p.N = d; p.K = S; p.lda = S; p.ldb = 3 * Hd; p.b_is_nk = 0; p.ldc = Hd;
+            p.alpha = 1.f; p.act = GP_ACT_NONE; p.batch = B * heads; p.batch_inner = heads;
+            p.stride_a = (long)S * S; p.stride_b = d; p.stride_c = d;
+            p.stride_a_outer = (long)heads * S * S; p.stride_b_outer = (long)S * 3 * Hd; p.stride_c_outer = (long)S * Hd;
+        }
+        size_t ao = g.add_storage(n + ".attn.out", (size_t)T * Hd, g.stype_);
+        g.dense(n + ".attn.proj", ctx, 0, T, Hd, Hd, Hd, GP_ACT_NONE, x, ao, 0, Hd, std_);   // + residual x
+        size_t x1 = g.add_storage(n + ".ln1.out", (size_t)T * Hd, g.stype_);
+        layernorm(n + ".ln1", ao, SIZE_MAX, x1);
+        size_t f1 = g.add_storage(n + ".ffn1.out", (size_t)T * F, g.stype_);
+        g.dense(n + ".ffn1", x1, 0, T, Hd, Hd, F, GP_ACT_GELU, SIZE_MAX, f1, 0, F, std_);
+        size_t f2 = g.add_storage(n + ".ffn2.out", (size_t)T * Hd, g.stype_);
+        g.dense(n + ".ffn2", f1, 0, T, F, F, Hd, GP_ACT_NONE, x1, f2, 0, Hd, std_);          // + residual x1
+        size_t x2 = g.add_storage(l == L - 1 ? std::string("heads") : n + ".ln2.out", (size_t)T * Hd, g.stype_);
+        layernorm(n + ".ln2", f2, SIZE_MAX, x2);
+        x = x2;
+    }
+    return Status::Succ;
+}
+
+// ---- a tiny chain with a "nop" copy, used to test the executor plumbing ------------------------
+Status build_toy(Model &m, const Options &o) {
+    std::string dt = o.gets("dtype", "f32");
+    if (!valid_dtype(dt)) return Status::OutOfRange;
+    GraphBuilder g(m, dt);
+    int rows = o.geti("rows", 64), cols = o.geti("cols", 64), n = o.geti("n", 3);
+    size_t cur = g.add_storage("data", (size_t)rows * cols, g.stype_);
+    for (int i = 0; i < n; ++i) {
+        Tensor a; a.st = cur; a.N = 1; a.H = 1; a.W = rows; a.C = cols; a.ps = cols;
+        Tensor t = g.eltwise("scale" + std::to_string(i), a, &a, "", GP_ACT_NONE);  // x -> 2x
+        size_t copy = g.add_storage(i == n - 1 ? std::string("heads") : "copy" + std::to_string(i), (size_t)rows * cols, g.stype_);
+        KernelInfo &k = g.add_kernel("nop", OpKind::Nop, {GraphBuilder::ref(t.st), GraphBuilder::ref(copy)}, 0, 2.0 * g.es() * rows * cols);
+        (void)k;
+        cur = copy;
+    }
+    return Status::Succ;
+}
+
+}  // namespace
+
+Status zoo_build(Model &m, const std::string &workload) {
+    Options o = parse(workload);
+    const std::string &n = o.name;
+    static const int r50[4] = {3, 4, 6, 3}, r101[4] = {3, 4, 23, 3}, r152[4] = {3, 8, 36, 3};
+    if (n == "gemm" || n == "gemm1024") return build_gemm(m, o, 1024, 1024, 1024, "f32", GP_ACT_RELU);
+    if (n == "gemm8192") { Options q = o; if (!q.kv.count("layout")) q.kv["layout"] = "nk"; if (!q.kv.count("bias")) q.kv["bias"] = "0"; return build_gemm(m, q, 8192, 8192, 8192, "bf16", GP_ACT_NONE); }
+    if (n == "resnet50") return build_resnet(m, o, r50, 1, "f32");
+    if (n == "resnet101") return build_resnet(m, o, r101, 1, "f16");
+    if (n == "resnet152" || n == "resnet") return build_resnet(m, o, r152, 8, "f16");
+    if (n == "vgg" || n == "vgg16") return build_vgg16(m, o);
+    if (n == "densenet" || n == "densenet201") return build_densenet201(m, o);
+    if (n == "bert") return build_bert(m, o);
+    if (n == "toy") return build_toy(m, o);
+    std::fprintf(stderr, "unknown workload '%s' (known: gemm1024 gemm8192 resnet50 resnet101 resnet152 vgg16 densenet201 bert toy)\n", n.c_str());
+    return Status::NotFound;
+}
+
+}  // namespace foo

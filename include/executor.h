@@ -1,0 +1,101 @@
+// foo::Executor / BaseExecutor / BLPExecutor — the model-level API of the preemptible executor:
+// load, set input, submit, preempt (by the shared flag), resume, read output.
+//
+// Interface of the reference's include/executor.h:14-84: same class names, method names,
+// argument meaning, public data members (BLPExecutor::dpStop, BLPExecutor::running) and Status
+// results.  Workload names select natively built graphs; the reference's graph-analytics and
+// miniWeather workloads ("cc", "bfs", "pagerank", "sssp", "miniweather") are not part of this
+// build and init() answers Status::NotFound for them.
+#pragma once
+#include <atomic>
+#include <memory>
+#include <string>
+#include <vector>
+#include "model.h"
+
+namespace foo {
+
+class Executor {
+public:
+    Status set_graph_path(const std::string &path);
+
+    // model_path = <MODEL_PATH>/<workload>; the workload's graph is built natively.
+    virtual Status load_model(std::string model_path);
+    // Loads <model_path>/mod.params when it exists; otherwise the seeded random init stays.
+    virtual Status load_param(std::string model_path);
+
+    // Submits the whole model asynchronously on `stream`.
+    virtual Status execute(GPUstream stream);
+    virtual Status launch_kernel(size_t kernel_offset, GPUstream stream = 0);
+
+    // Root directory of model files: $GPREEMPT_MODEL_PATH, else "./model".
+    virtual Status init(std::string workload);
+    virtual Status set_input(const std::string &key, void *value, size_t len, GPUstream stream);
+    virtual Status set_input(const std::string &key, std::vector<float> &value, GPUstream stream);
+    virtual Status get_output(const std::string &key, void *value, size_t len, GPUstream stream);
+    virtual Status get_output(const std::string &key, std::vector<float> &value, GPUstream stream);
+    virtual size_t get_data_size(const std::string &key);
+
+    virtual void clear();
+    size_t get_kernel_num() const;
+    virtual void capture_graph(GPUstream stream);
+    virtual ~Executor();
+
+    // additions over the reference
+    std::shared_ptr<Model> get_model() const { return model; }
+    bool uses_graph() const { return use_cuda_graph; }
+
+protected:
+    std::shared_ptr<Model> model;
+    std::string type;
+    bool use_cuda_graph = false;
+    GPUgraphExec graph_exec = nullptr;
+    std::string graph_path;
+};
+
+class BaseExecutor : public Executor {
+public:
+    BaseExecutor();
+    virtual ~BaseExecutor();
+};
+
+class BLPExecutor : public Executor {
+public:
+    BLPExecutor();
+    virtual ~BLPExecutor();
+    // Reads the stop index back (blocks on `stream`); re-arms it to -1 when a kernel was stopped.
+    Status getStopPoint(GPUstream stream);
+    // Relaunches kernels [stop index, N) without resetting their tile counters.
+    Status resume(GPUstream stream);
+    virtual Status init(std::string workload) override;
+    virtual Status execute(GPUstream stream) override;
+    virtual Status launch_kernel(size_t kernel_offset, GPUstream stream = 0) override;
+    virtual void capture_graph(GPUstream stream) override;
+    virtual void clear() override;
+    void set_lc_be_tasks(std::atomic<int> &lc_tasks, std::atomic<int> &be_tasks) {
+        this->lc_tasks = &lc_tasks;
+        this->be_tasks = &be_tasks;
+    }
+
+    // additions over the reference (test and measurement hooks)
+    int last_stop_index() const { return stopIndex; }
+    // Arms deterministic preemption: the workgroup whose claim on kernel `kernel` returns
+    // `claim` raises the flag itself.  Applies to the next execute()/resume(); -1 disarms.
+    void inject_preempt(int kernel, int claim) { inject_kernel = kernel; inject_claim = claim; }
+    Status read_counters(std::vector<int> &out);
+
+public:
+    GPUdeviceptr dpStop = nullptr;  // the preempt flag: allocated by the caller, shared by all best-effort tenants
+    std::atomic<bool> running{false};
+
+private:
+    GPUdeviceptr dpStopIndex = nullptr;  // owned
+    GPUdeviceptr executed = nullptr;     // owned: one tile counter per kernel
+    int stopIndex = -1;
+    int *stop_host = nullptr;            // pinned landing slot for the stop index
+    int inject_kernel = -1, inject_claim = -1;
+    std::atomic<int> *lc_tasks = nullptr;
+    std::atomic<int> *be_tasks = nullptr;
+};
+
+}  // namespace foo

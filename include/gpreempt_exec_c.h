@@ -1,0 +1,52 @@
+/*
+ * gpreempt_exec_c.h — C view of the C++ executor classes (include/executor.h, include/model.h)
+ * for callers that bind through an FFI (ctypes, cgo, JNI) instead of linking C++.
+ * Every function forwards to the method of foo::Executor / foo::BLPExecutor named in its
+ * comment, which in turn replaces the method of the same name in the reference
+ * (include/executor.h:14-84).  Results are the `Status` values of include/util/common.h
+ * (0 = Succ) unless stated otherwise.
+ */
+#ifndef GPREEMPT_EXEC_C_H
+#define GPREEMPT_EXEC_C_H
+#include <stddef.h>
+#include "gpreempt_hip.h"
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *gpx_executor;
+
+gpx_executor gpx_create(int block_level_preemptible); /* 0: foo::BaseExecutor, 1: foo::BLPExecutor */
+void gpx_destroy(gpx_executor e);
+int gpx_init(gpx_executor e, const char *workload);                 /* Executor::init */
+int gpx_set_input(gpx_executor e, const char *key, void *value, size_t len, gp_stream s);  /* Executor::set_input */
+int gpx_get_output(gpx_executor e, const char *key, void *value, size_t len, gp_stream s); /* Executor::get_output */
+size_t gpx_get_data_size(gpx_executor e, const char *key);          /* Executor::get_data_size */
+int gpx_execute(gpx_executor e, gp_stream s);                        /* Executor::execute */
+int gpx_launch_kernel(gpx_executor e, size_t idx, gp_stream s);      /* Executor::launch_kernel */
+size_t gpx_get_kernel_num(gpx_executor e);                           /* Executor::get_kernel_num */
+int gpx_capture_graph(gpx_executor e, gp_stream s);                  /* Executor::capture_graph; 0 when a graph is in use afterwards */
+void gpx_clear(gpx_executor e);                                      /* Executor::clear */
+
+/* BLPExecutor only (Status::Fail on a BaseExecutor) */
+int gpx_set_flag(gpx_executor e, void *dp_stop);                     /* BLPExecutor::dpStop = dp_stop */
+int gpx_set_running(gpx_executor e, int running);                    /* BLPExecutor::running = running */
+int gpx_resume(gpx_executor e, gp_stream s);                         /* BLPExecutor::resume */
+int gpx_get_stop_point(gpx_executor e, gp_stream s, int *stop_index);/* BLPExecutor::getStopPoint */
+int gpx_last_stop_index(gpx_executor e);                             /* value read by the last getStopPoint / resume */
+int gpx_inject_preempt(gpx_executor e, int kernel, int claim);       /* BLPExecutor::inject_preempt (test hook) */
+int gpx_read_counters(gpx_executor e, int *out, size_t n);           /* BLPExecutor::read_counters */
+
+/* Model introspection (foo::Model::get_storage_info / get_kernel_info) */
+size_t gpx_storage_num(gpx_executor e);
+/* dims = {kind, o, i, r, s, c, h, w}: kind 0 plain, 1 conv weight stored OIHW on disk, 2 dense over a CHW flatten */
+int gpx_storage_info(gpx_executor e, size_t idx, char *name, size_t name_len, char *stype, size_t stype_len,
+                     size_t *bytes, int *is_param, size_t *disk_elems, int dims[8]);
+int gpx_kernel_info(gpx_executor e, size_t idx, char *name, size_t name_len, double *flops, double *bytes,
+                    int *total_blocks, int *grid);
+int gpx_read_storage(gpx_executor e, const char *key, void *out, size_t len); /* blocking Model::get */
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,148 @@
+// foo::Model — storages + kernel list of one DNN, and its on-disk parameter format.
+//
+// Public interface of the reference's include/model.h:12-100 (same class and method names,
+// argument meaning and Status results).  What differs underneath: the reference loads a
+// TVM-compiled GPU module and two JSON files; here the kernel list is built natively from the
+// workload name and every kernel is an operator of libgpreempt_hip.so.
+#pragma once
+#include <cstdint>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+#include "util/common.h"
+#include "util/gpu_util.h"
+
+namespace foo {
+
+using namespace foo::util;
+
+class StorageInfo {
+public:
+    std::string name;
+    size_t size;        // bytes
+    std::string stype;  // "float32" "float16" "bfloat16" "int64" "int32" "byte" "uint1"
+};
+
+// How a parameter that is stored on disk in the reference's convention (fp32; OIHW convolution
+// weights; dense weights [out][in] over an NCHW flatten) maps onto the device layout
+// (model dtype; [O][H][W][I padded]; dense over an NHWC flatten).
+struct ParamLayout {
+    enum Kind { Plain, ConvOIHW, DenseOverCHW } kind = Plain;
+    int o = 0, i = 0, r = 0, s = 0, i_pad = 0;  // ConvOIHW
+    int c = 0, h = 0, w = 0;                    // DenseOverCHW: input features were flattened from C x H x W
+    size_t disk_elems = 0;                      // fp32 values expected on disk
+    bool is_param = false;
+    // seeded initial value when no parameter file is given
+    enum Init { InitZero, InitNormal /* N(0, a) */, InitUniform /* U[a, b] */, InitConst /* a */ } init = InitZero;
+    float init_a = 0.f, init_b = 0.f;
+};
+
+enum class OpKind { Nop, Gemm, Conv, Layout, Pool, Eltwise, Softmax, Layernorm, Embed };
+
+struct ArgRef {
+    size_t storage = SIZE_MAX;  // SIZE_MAX = absent
+    size_t byte_offset = 0;
+};
+
+class KernelInfo {
+public:
+    std::string name;            // operator name; "nop" is a device-to-device copy (reference model.cpp:201-207)
+    uint32_t launch_params[6];   // grid x,y,z and block x,y,z as last planned by the device layer
+    OpKind op = OpKind::Nop;
+    union {
+        gp_gemm_params gemm;
+        gp_conv_params conv;
+        gp_layout_params layout;
+        gp_pool_params pool;
+        gp_eltwise_params eltwise;
+        gp_softmax_params softmax;
+        gp_layernorm_params layernorm;
+        gp_embed_params embed;
+    } p;
+    std::vector<size_t> args_index;       // storage index per pointer slot (SIZE_MAX = absent)
+    std::vector<ArgRef> refs;             // same slots with byte offsets into the storage
+    std::vector<GPUdeviceptr> args;       // resolved device pointers
+    std::vector<GPUdeviceptr *> args_ptr; // extra by-reference arguments appended by batchAddParam
+    // block-level preemption arguments (reference model.cpp:366-396)
+    bool preemptible = false;
+    int total_blocks = 0;
+    GPUdeviceptr executed = nullptr;
+    int kernel_id = 0;
+    double flops = 0, bytes = 0;          // algorithmic work of one launch
+};
+
+class Model {
+public:
+    Model();
+    Model(const std::string &device_json, const std::string &host_json, const std::string &cuda_module);
+    ~Model();
+
+    // The three paths name files inside MODEL_PATH/<workload>/ as in the reference
+    // (src/executor.cpp:110-113); the workload is the name of that directory and the graph is
+    // built natively from it.  `workload` may carry options: "resnet152@b=8,dtype=f16".
+    Status load_model(const std::string &device_json, const std::string &host_json, const std::string &cuda_module);
+    Status build(const std::string &workload);
+
+    // Reads a "TVM_MODEL_PARAMS" file (format of reference src/model.cpp:15-55) and uploads every
+    // tensor whose key names a storage.  Parameters missing from the file keep their seeded
+    // random initialisation.  A missing file is not an error: the model stays random-init.
+    Status load_param(const char *param_file_path);
+
+    bool is_loaded();
+    size_t get_kernel_num() const;
+    size_t get_storage_num() const;
+    size_t get_storage_size(size_t idx);
+    StorageInfo &get_storage_info(size_t idx);
+    KernelInfo &get_kernel_info(size_t idx);
+    GPUdeviceptr get_storage_ptr(size_t idx);
+    const ParamLayout &get_param_layout(size_t idx) const { return layouts[idx]; }
+
+    Status get(size_t idx, void *out, size_t len, GPUstream stream);
+    Status get(const std::string &key, void *out, size_t len, GPUstream stream);
+    Status set(size_t idx, void *value, size_t len, GPUstream stream);
+    Status set(const std::string &key, void *value, size_t len, GPUstream stream);
+
+    static size_t get_stype_size(std::string &stype);
+    Status find_storage_idx(const std::string &name, size_t &idx);
+    Status get_global_ptr(const std::string &name, GPUdeviceptr *ptr);
+    Status clear();
+
+    Status batchAddParam(GPUdeviceptr *ptr);
+    Status add_block_preemption_param(GPUdeviceptr ptr);
+
+    // Launches kernel `idx` on `stream` (what src/executor.cpp:136-164 does with
+    // GPULaunchKernel); preemptible kernels take their flag and stop index from the by-reference
+    // arguments added with batchAddParam.  inject_at is a test hook (-1 = off).
+    Status launch(size_t idx, GPUstream stream, int inject_at = -1);
+
+    const std::string &workload() const { return workload_; }
+    const std::string &dtype() const { return dtype_; }
+    double total_flops() const;
+    double total_bytes() const;
+
+    friend class GraphBuilder;
+
+private:
+    bool loaded_ = false;
+    std::string workload_, dtype_;
+    std::vector<StorageInfo> storage_infos;
+    std::vector<ParamLayout> layouts;
+    std::vector<KernelInfo> kernel_infos;
+    std::vector<GPUdeviceptr> storages;
+    std::unordered_map<std::string, size_t> storages_idx;
+
+    Status allocate_and_bind();
+    Status upload_param(size_t idx, const float *disk, size_t n);
+    void bind_pointers(KernelInfo &k);
+};
+
+typedef std::unordered_map<std::string, std::vector<float>> ModelParam;
+
+class ModelParamParser {
+public:
+    // nullptr when the file is missing or malformed (the reference aborts instead).
+    static ModelParam *parse_from_file(const char *param_file);
+};
+
+}  // namespace foo

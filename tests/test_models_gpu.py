@@ -1,0 +1,212 @@
+"""Whole-model parity: the C++ Executor (through its C view) against the layer-by-layer oracle
+on the same seeded weights, which travel through a TVM_MODEL_PARAMS file as in the reference
+(src/model.cpp:263-282), plus the preempt-then-resume protocol of src/tests/test-dnn-blp.cpp."""
+import os
+
+import numpy as np
+import pytest
+
+from oracle import models as OM
+from oracle import oracle as O
+from helpers import TOL, rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ex_mod(gp):
+    from gpreempt_amd import executor
+    return executor
+
+
+def make_model(ex_mod, tmp_path, workload, family, seed, blp=False):
+    """Builds the executor once to learn the parameter shapes, writes seeded parameters to
+    <root>/<workload>/mod.params, and builds it again so that they load from the file."""
+    root = str(tmp_path)
+    probe = ex_mod.Executor(workload, model_root=root)
+    shapes = probe.param_shapes()
+    probe.destroy()
+    params = OM.random_params(shapes, seed, family)
+    os.makedirs(os.path.join(root, workload), exist_ok=True)
+    ex_mod.write_params(os.path.join(root, workload, "mod.params"), params)
+    return ex_mod.Executor(workload, blp=blp, model_root=root), params
+
+
+def run(gp, ex, x_raw, dtype, out_shape):
+    ex.set_input("data", x_raw)
+    ex.execute()
+    return gp.from_storage(ex.get_output("heads"), dtype).reshape(out_shape).copy()
+
+
+def test_gemm1024_workload_matches_oracle(gp, ex_mod, tmp_path):
+    ex, params = make_model(ex_mod, tmp_path, "gemm1024", "gemm", 1)
+    A = np.random.default_rng(0xC0FFEE).uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    got = run(gp, ex, A, gp.F32, (1024, 1024))
+    ref = O.gemm_bias_act(A, params["B"].reshape(1024, 1024), params["bias"], act=O.ACT_RELU)
+    assert rel_err(got, ref) < TOL["f32"]
+
+
+@pytest.mark.parametrize("workload,dt,blocks", [
+    ("resnet50", "f32", OM.RESNET_BLOCKS["resnet50"]),                 # BASELINE config 2 at full size
+    ("resnet152@b=2,hw=64", "f16", OM.RESNET_BLOCKS["resnet152"]),     # config 3's tenant, reduced image
+])
+def test_resnet_matches_oracle(gp, ex_mod, tmp_path, workload, dt, blocks):
+    ex, params = make_model(ex_mod, tmp_path, workload, "cnn", 2)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    n = 2 if "b=2" in workload else 1
+    hw = 64 if "hw=64" in workload else 224
+    x = O.round_to(np.random.default_rng(3).normal(0, 1, (n, 3, hw, hw)).astype(np.float32), dt)
+    got = run(gp, ex, gp.to_storage(x, dtype), dtype, (n, 1000))
+    ref = OM.resnet(params, x, blocks, dt)
+    assert np.isfinite(got).all()
+    assert rel_err(got, ref) < TOL[dt]
+    assert abs(got.sum(axis=1) - 1).max() < 2e-2
+
+
+def test_vgg16_matches_oracle(gp, ex_mod, tmp_path):
+    wl = "vgg16@b=2,hw=64,fc=512"
+    ex, params = make_model(ex_mod, tmp_path, wl, "cnn", 4)
+    x = O.round_to(np.random.default_rng(5).normal(0, 1, (2, 3, 64, 64)).astype(np.float32), "f16")
+    got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (2, 1000))
+    assert rel_err(got, OM.vgg16(params, x, "f16")) < TOL["f16"]
+
+
+def test_densenet_matches_oracle(gp, ex_mod, tmp_path):
+    wl = "densenet201@b=1,hw=64,l1=2,l2=4,l3=5,l4=3"
+    ex, params = make_model(ex_mod, tmp_path, wl, "cnn", 6)
+    x = O.round_to(np.random.default_rng(7).normal(0, 1, (1, 3, 64, 64)).astype(np.float32), "f16")
+    got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (1, 1000))
+    assert rel_err(got, OM.densenet(params, x, "f16", (2, 4, 5, 3))) < TOL["f16"]
+
+
+@pytest.mark.parametrize("workload,kw", [
+    ("bert", dict(batch=1, seq=128, layers=12)),                       # config 3's high-priority tenant, full size
+    ("bert@b=2,s=48,layers=2,dtype=f32", dict(batch=2, seq=48, layers=2)),
+])
+def test_bert_matches_oracle(gp, ex_mod, tmp_path, workload, kw):
+    dt = "f32" if "f32" in workload else "f16"
+    ex, params = make_model(ex_mod, tmp_path, workload, "bert", 8)
+    ids = np.random.default_rng(9).integers(0, 30522, kw["batch"] * kw["seq"]).astype(np.int64)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    got = run(gp, ex, ids, dtype, (kw["batch"] * kw["seq"], 768))
+    ref = OM.bert(params, ids, dt, **kw)
+    assert rel_err(got, ref) < TOL[dt]
+
+
+def test_toy_chain_with_nop_copies(gp, ex_mod, tmp_path):
+    ex = ex_mod.Executor("toy@n=3", model_root=str(tmp_path))
+    assert [k["name"] for k in ex.kernels()] == ["eltwise", "nop"] * 3
+    x = np.arange(64 * 64, dtype=np.float32)
+    got = run(gp, ex, x, gp.F32, (64 * 64,))
+    assert np.array_equal(got, 8 * x)
+
+
+def test_executor_error_paths(gp, ex_mod, tmp_path):
+    with pytest.raises(ex_mod.StatusError) as e:
+        ex_mod.Executor("no_such_model", model_root=str(tmp_path))
+    assert e.value.status == 3  # NotFound
+    with pytest.raises(ex_mod.StatusError) as e:
+        ex_mod.Executor("miniweather", model_root=str(tmp_path))  # reference workload outside this build
+    assert e.value.status == 3
+    ex = ex_mod.Executor("toy", model_root=str(tmp_path))
+    with pytest.raises(ex_mod.StatusError) as e:
+        ex.set_input("data", np.zeros(8, np.float32))  # shorter than the storage: OutOfRange (model.cpp:319)
+    assert e.value.status == 4
+    with pytest.raises(ex_mod.StatusError) as e:
+        ex.set_input("nope", np.zeros(8, np.float32))
+    assert e.value.status == 3
+    assert ex.data_size("nope") == 0
+    with pytest.raises(ex_mod.StatusError):
+        ex.resume()  # BaseExecutor has no resume
+
+
+# ---- preempt-then-resume on whole models ----------------------------------------------------
+
+def _blp_roundtrip(gp, ex_mod, tmp_path, workload, x_raw, injections, graph=False):
+    root = str(tmp_path)
+    base = ex_mod.Executor(workload, blp=False, model_root=root)
+    base.set_input("data", x_raw)
+    base.execute()
+    want = base.get_output("heads").copy()
+    ex = ex_mod.Executor(workload, blp=True, model_root=root)
+    flag = gp.Flag()
+    ex.set_flag(flag)
+    stream = gp.Stream(1)
+    if graph:
+        ex.capture_graph(stream)
+    ex.set_input("data", x_raw, stream)
+    # uninterrupted preemptible run: same bits as the non-preemptible executor
+    ex.execute(stream)
+    ex.set_running(True)
+    assert np.array_equal(ex.get_output("heads", stream), want)
+    assert ex.stop_point(stream) == -1
+    n = ex.kernel_num()
+    for kernel, claim in injections:
+        kernel = kernel if kernel >= 0 else n + kernel
+        flag.set(0)
+        ex.inject_preempt(kernel, claim)
+        if graph:
+            ex.capture_graph(stream)  # the injection point is a kernel argument: re-capture
+        ex.execute(stream)
+        ex.set_running(True)
+        stream.sync()
+        assert flag.get() == 1, (kernel, claim)
+        cnt = ex.counters()
+        assert (cnt[kernel + 1:] == 0).all()  # every later kernel left at its first flag check
+        ex.inject_preempt(-1, -1)
+        flag.set(0)  # host clears the flag, then resumes (test-dnn-blp.cpp:41-42)
+        ex.resume(stream)
+        assert ex.last_stop_index() in (kernel, kernel + 1), (ex.last_stop_index(), kernel)
+        stream.sync()
+        assert np.array_equal(ex.get_output("heads", stream), want), (kernel, claim)
+        assert ex.stop_point(stream) == -1
+        ex.resume(stream)  # nothing stopped: must be a no-op
+        assert np.array_equal(ex.get_output("heads", stream), want)
+    ex.set_running(False)
+    return ex
+
+
+def test_resnet50_preempt_resume_bit_exact(gp, ex_mod, tmp_path):
+    x = np.random.default_rng(1).normal(0, 1, (1, 3, 224, 224)).astype(np.float32)
+    _blp_roundtrip(gp, ex_mod, tmp_path, "resnet50", x, [(1, 10), (20, 3), (-3, 0), (5, 0)])
+
+
+def test_resnet50_preempt_resume_bit_exact_with_graph(gp, ex_mod, tmp_path):
+    x = np.random.default_rng(2).normal(0, 1, (1, 3, 224, 224)).astype(np.float32)
+    _blp_roundtrip(gp, ex_mod, tmp_path, "resnet50", x, [(7, 5), (40, 1)], graph=True)
+
+
+def test_bert_preempt_resume_bit_exact(gp, ex_mod, tmp_path):
+    ids = np.random.default_rng(3).integers(0, 30522, 128).astype(np.int64)
+    _blp_roundtrip(gp, ex_mod, tmp_path, "bert", ids, [(0, 3), (2, 17), (57, 0), (-1, 10)])
+
+
+def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path):
+    """src/tests/test-dnn-blp.cpp:36-42 verbatim: execute; set the flag from the host right
+    away; sync; clear; resume; sync.  Where the flag lands is up to timing; the result is not."""
+    root = str(tmp_path)
+    x = gp.to_storage(np.full((8, 3, 224, 224), 10.0, np.float32), gp.F16)  # the reference's all-10.0 image
+    base = ex_mod.Executor("resnet152", model_root=root)
+    base.set_input("data", x)
+    base.execute()
+    want = base.get_output("heads").copy()
+    ex = ex_mod.Executor("resnet152", blp=True, model_root=root)
+    flag = gp.Flag()
+    ex.set_flag(flag)
+    stream = gp.Stream(1)
+    ex.set_input("data", x, stream)
+    stream.sync()
+    stops = []
+    for _ in range(5):
+        ex.execute(stream)
+        ex.set_running(True)
+        flag.set(1)
+        stream.sync()
+        flag.set(0)
+        ex.resume(stream)
+        stops.append(ex.last_stop_index())
+        stream.sync()
+        assert np.array_equal(ex.get_output("heads", stream), want)
+    assert any(s != -1 for s in stops), stops  # at least one run was really interrupted
+    ex.set_running(False)
+    ex.resume(stream)  # running == false: no-op (executor.cpp:281)
