@@ -1,0 +1,159 @@
+#!/usr/bin/env python3
+"""Headline benchmark: BASELINE.json config 3 on one MI355X.
+
+High-priority tenant: BERT-base fp16, batch 1, seq 128, Poisson arrivals at 200 req/s.
+Best-effort tenant: ResNet-152 fp16, batch 8, 224x224, back to back, block-level preemptible.
+A "step" is one high-priority request served while the best-effort tenant co-runs; inputs are
+synthetic and resident before the timed region; weights are seeded random-init.
+
+Prints ONE JSON line.  `value` = co-run p99 latency of the high-priority tenant / its isolated
+p99 (the first figure of BASELINE.json's metric); the other two (preemption latency, best-effort
+throughput kept) and the absolute latencies ride along in the same line, together with
+  roofline      the dominant kernel (MFMA implicit-GEMM convolution of the best-effort model),
+                timed live with HIP events on the stream it is launched on
+  cpu_baseline  the same high-priority graph on the host cores (CPU oracle), bounded sample
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
+HBM_PEAK_GBS = 8000.0
+
+
+def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
+    from gpreempt_amd import executor as gx
+    cfg = {
+        "time": max(5.0, 4.0 * steps / hp_rate), "policy": policy, "hp_requests": steps,
+        "warmups": warmup, "standalone_runs": 100,
+        "tasks": [
+            {"id": "hp", "load": {"type": "poisson", "frequency": hp_rate, "seed": 2025},
+             "client": {"name": "hp", "model_name": hp_model, "priority": 0, "use_cuda_graph": True, "preprocess_time": 0}},
+            {"id": "be", "load": {"type": "continuous"},
+             "client": {"name": "be", "model_name": be_model, "priority": 1, "use_cuda_graph": True, "preprocess_time": 0}},
+        ],
+    }
+    buf = C.create_string_buffer(1 << 20)
+    rc = gx.lib().gpx_run_scenario(json.dumps(cfg).encode(), buf, C.c_size_t(len(buf)))
+    if rc != 0:
+        raise RuntimeError(f"scenario failed with Status {rc}: {buf.value[:400]!r}")
+    return json.loads(buf.value.decode())
+
+
+def roofline(workload, iters, dt):
+    """Times every launch of the model's MFMA convolution kernel with HIP events on the stream
+    the kernel runs on; achieved = algorithmic flop of those launches / their summed duration."""
+    from gpreempt_amd import capi as gp
+    from gpreempt_amd import executor as gx
+    ex = gx.Executor(workload, blp=True)
+    flag = gp.Flag()
+    ex.set_flag(flag)
+    stream = gp.Stream(1)
+    kernels = ex.kernels()
+    conv = [i for i, k in enumerate(kernels) if k["name"] == "conv2d"]
+    ex.execute(stream)  # warm-up, also resolves launch geometry
+    stream.sync()
+    ev = [(gp.Event(), gp.Event()) for _ in conv]
+    total_ms, total_flop, total_bytes, launches = 0.0, 0.0, 0.0, 0
+    for _ in range(iters):
+        # one pass through the reference's launch_kernel API, events around each convolution
+        ex.reset_counters(stream)
+        j = 0
+        for i in range(len(kernels)):
+            if j < len(conv) and conv[j] == i:
+                ev[j][0].record(stream)
+                ex.launch_kernel(i, stream)
+                ev[j][1].record(stream)
+                j += 1
+            else:
+                ex.launch_kernel(i, stream)
+        stream.sync()
+        for (a, b), i in zip(ev, conv):
+            total_ms += a.elapsed_ms(b)
+            total_flop += kernels[i]["flops"]
+            total_bytes += kernels[i]["bytes"]
+            launches += 1
+    ex.destroy()
+    achieved = total_flop / (total_ms * 1e-3) / 1e12
+    return {"bound": "mfma", "kernel": "mat_kernel<TileKernel<f16,conv>> (implicit-GEMM conv2d of " + workload + ")",
+            "achieved": achieved, "peak": PEAK[dt], "unit": "TFLOP/s", "frac": achieved / PEAK[dt], "traffic": None,
+            "launches": launches, "avg_launch_us": total_ms * 1e3 / launches,
+            "algorithmic_flop_per_launch": total_flop / launches, "algorithmic_bytes_per_launch": total_bytes / launches}
+
+
+def cpu_baseline(requests):
+    """The high-priority graph (BERT-base, seq 128, fp16 storage) on the host cores through the
+    CPU oracle.  Bounded sample: `requests` whole requests."""
+    import numpy as np
+    from oracle import models as OM
+    H, F, L = 768, 3072, 12
+    shapes = {"embeddings.word": (30522, H), "embeddings.position": (512, H), "embeddings.token_type": (1, H),
+              "embeddings.ln.gamma": (H,), "embeddings.ln.beta": (H,)}
+    for l in range(L):
+        n = f"layer{l}"
+        shapes.update({n + ".attn.qkv.weight": (3 * H, H), n + ".attn.qkv.bias": (3 * H,), n + ".attn.proj.weight": (H, H),
+                       n + ".attn.proj.bias": (H,), n + ".ln1.gamma": (H,), n + ".ln1.beta": (H,), n + ".ffn1.weight": (F, H),
+                       n + ".ffn1.bias": (F,), n + ".ffn2.weight": (H, F), n + ".ffn2.bias": (H,), n + ".ln2.gamma": (H,), n + ".ln2.beta": (H,)})
+    params = OM.random_params(shapes, 0, "bert")
+    ids = np.random.default_rng(0).integers(0, 30522, 128)
+    OM.bert(params, ids, "f16", 1, 128, 1)  # touch the library
+    t0 = time.perf_counter()
+    for _ in range(requests):
+        OM.bert(params, ids, "f16", 1, 128, L)
+    dt = (time.perf_counter() - t0) / requests
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": dt * 1e3, "unit": "ms per high-priority request (isolated)", "cores": cores, "kind": "port",
+            "sample": f"{requests} BERT-base b1 s128 requests through oracle/models.py (double accumulation, fp16 storage rounding, OpenMP)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=600)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--policy", default="wb")
+    ap.add_argument("--hp-rate", type=float, default=200.0)
+    ap.add_argument("--hp-model", default="bert")
+    ap.add_argument("--be-model", default="resnet152")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | cpu")
+    ap.add_argument("--cpu-requests", type=int, default=4)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the executor is a single-device path); run with --gpus 1")
+
+    from gpreempt_amd import capi as gp
+    gp.init(0)
+    out = {"metric": "HP p99 latency vs isolated (co-run p99 / isolated p99); preemption latency (us); BE throughput kept",
+           "unit": "x (ratio)", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": False,
+           "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic (seeded random-init weights, N(0,1) images, uniform token ids)",
+           "config": {"workload": "BASELINE config 3: HP BERT-base fp16 b1 s128 Poisson %g req/s + BE ResNet-152 fp16 b8 224x224 back-to-back" % args.hp_rate,
+                      "policy": args.policy, "hp_model": args.hp_model, "be_model": args.be_model}}
+    if args.only in ("", "scenario"):
+        rep = scenario(args.steps, args.warmup, args.policy, args.hp_rate, args.be_model, args.hp_model)
+        hp, be = rep["tasks"]["hp"], rep["tasks"]["be"]
+        out.update({
+            "value": rep["hp_p99_vs_isolated"], "steps": hp["requests"],
+            "ms_per_step": hp["totalLatency(us)"]["mean"] / 1e3,
+            "hp_isolated_ms": {k: hp["standAlone(us)"][k] / 1e3 for k in ("mean", "p50", "p99")},
+            "hp_corun_ms": {k: hp["totalLatency(us)"][k] / 1e3 for k in ("mean", "p50", "p99", "max")},
+            "hp_throughput_req_s": hp["avgThroughput(req/s)"],
+            "preemption_latency_us": {k: rep["preemptLatency(us)"][k] for k in ("count", "mean", "p50", "p99", "max")},
+            "be_throughput_kept": rep["be_throughput_kept"],
+            "be_throughput_req_s": be["avgThroughput(req/s)"], "be_isolated_req_s": be["standAloneThroughput(req/s)"],
+            "be_preemptions": be["preemptions"], "hp_busy_fraction": rep["hp_busy_fraction"],
+            "hp_kernels": hp["kernels"], "be_kernels": be["kernels"]})
+    if args.only in ("", "roofline"):
+        out["roofline"] = roofline(args.be_model, 3, "f16")
+    if args.only in ("", "cpu"):
+        out["cpu_baseline"] = cpu_baseline(args.cpu_requests)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

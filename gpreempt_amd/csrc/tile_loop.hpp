@@ -14,7 +14,8 @@
 //  * the claimed index is handed to the other waves through a two-slot LDS mailbox indexed by
 //    iteration parity, which removes the reference's reuse race on its single __shared__ slot
 //    with one barrier per tile;
-//  * *stop_index is claimed with a compare-and-swap instead of a test followed by a store;
+//  * *stop_index is claimed with a compare-and-swap instead of a test followed by a store, and a
+//    workgroup also leaves when *stop_index is already set (see "Sticky" below);
 //  * with executed == nullptr the same kernel runs non-preemptibly, one workgroup per tile
 //    (the reference builds a second, untransformed module for that: mod.cubin vs mod.tr.cubin).
 #pragma once
@@ -59,6 +60,11 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
         if (leader) {
             int idx = -1;
             int stop = b.flag ? __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : 0;
+            // Sticky: once a kernel of this executor has been stopped, every later kernel of the
+            // same submission leaves too until the host re-arms the stop index, even if the flag
+            // has been lowered in between.  Otherwise a kernel queued behind a stopped one could
+            // run to completion on incomplete inputs.
+            stop |= __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
             if (!stop) {
                 idx = atomicAdd(b.executed, 1);
                 if (idx >= b.total) {

@@ -14,8 +14,8 @@ vp = C.c_void_p
 
 SYMBOLS = """gpx_create gpx_destroy gpx_init gpx_set_input gpx_get_output gpx_get_data_size gpx_execute
 gpx_launch_kernel gpx_get_kernel_num gpx_capture_graph gpx_clear gpx_set_flag gpx_set_running gpx_resume
-gpx_get_stop_point gpx_last_stop_index gpx_inject_preempt gpx_read_counters gpx_storage_num gpx_storage_info
-gpx_kernel_info gpx_read_storage""".split()
+gpx_get_stop_point gpx_last_stop_index gpx_inject_preempt gpx_read_counters gpx_reset_counters gpx_storage_num gpx_storage_info
+gpx_kernel_info gpx_read_storage gpx_run_scenario gpx_preempt_probe gpx_parse_params""".split()
 
 STATUS = ["Succ", "Fail", "Timeout", "NotFound", "OutOfRange", "Full"]
 _lib = None
@@ -167,6 +167,9 @@ class Executor:
         out = np.zeros(self.kernel_num(), np.int32)
         _chk(lib().gpx_read_counters(self.h, out.ctypes.data_as(vp), C.c_size_t(out.size)), "read_counters")
         return out
+
+    def reset_counters(self, stream=None):
+        _chk(lib().gpx_reset_counters(self.h, stream.h if stream else None), "reset_counters")
 
     def destroy(self):
         if self.h:

@@ -2,6 +2,7 @@
 #include <cstring>
 #include "executor.h"
 #include "gpreempt_exec_c.h"
+#include "harness.h"
 
 using namespace foo;
 
@@ -51,6 +52,7 @@ int gpx_get_stop_point(gpx_executor e, gp_stream s, int *stop) {
 }
 int gpx_last_stop_index(gpx_executor e) { return H(e)->blp ? H(e)->blp->last_stop_index() : -1; }
 int gpx_inject_preempt(gpx_executor e, int kernel, int claim) { if (!H(e)->blp) return Status::Fail; H(e)->blp->inject_preempt(kernel, claim); return Status::Succ; }
+int gpx_reset_counters(gpx_executor e, gp_stream s) { return H(e)->blp ? H(e)->blp->reset_counters(s) : Status::Fail; }
 int gpx_read_counters(gpx_executor e, int *out, size_t n) {
     if (!H(e)->blp) return Status::Fail;
     std::vector<int> v;
@@ -97,4 +99,36 @@ extern "C" int gpx_storage_info(gpx_executor e, size_t idx, char *name, size_t n
     if (disk_elems) *disk_elems = L.disk_elems;
     if (dims) { int d[8] = {(int)L.kind, L.o, L.i, L.r, L.s, L.c, L.h, L.w}; std::memcpy(dims, d, sizeof(d)); }
     return Status::Succ;
+}
+
+static int copy_report(Status st, const std::string &rep, char *report, size_t report_len) {
+    if (report && report_len) {
+        std::strncpy(report, rep.c_str(), report_len - 1);
+        report[report_len - 1] = 0;
+    }
+    if (st == Status::Succ && rep.size() + 1 > report_len) return Status::Full;
+    return st;
+}
+
+extern "C" int gpx_run_scenario(const char *config_json, char *report, size_t report_len) {
+    std::string rep;
+    Status st = foo::run_scenario(config_json ? config_json : "", rep);
+    return copy_report(st, rep, report, report_len);
+}
+
+extern "C" int gpx_preempt_probe(const char *workload, int trials, int use_graph, unsigned long long seed, char *report, size_t report_len) {
+    std::string rep;
+    Status st = foo::preempt_probe(workload ? workload : "", trials, use_graph != 0, seed, rep);
+    return copy_report(st, rep, report, report_len);
+}
+
+extern "C" long gpx_parse_params(const char *path, const char *key, float *out, size_t n, size_t *len) {
+    std::unique_ptr<ModelParam> params(ModelParamParser::parse_from_file(path));
+    if (!params) return -1;
+    if (key) {
+        auto it = params->find(key);
+        if (len) *len = it == params->end() ? 0 : it->second.size();
+        if (it != params->end() && out) std::memcpy(out, it->second.data(), sizeof(float) * std::min(n, it->second.size()));
+    }
+    return (long)params->size();
 }

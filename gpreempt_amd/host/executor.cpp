@@ -146,7 +146,7 @@ Status BLPExecutor::launch_kernel(size_t kernel_offset, GPUstream stream) {
 // reference executor.cpp:211-232: zero every tile counter, then launch (or replay the graph).
 // The counters are cleared by a fill kernel outside the captured graph.
 Status BLPExecutor::execute(GPUstream stream) {
-    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num(), stream));
+    RETURN_STATUS(reset_counters(stream));
     if (use_cuda_graph) {
         CUDA_RETURN_STATUS(gp_graph_launch(graph_exec, stream));
         return Status::Succ;
@@ -179,6 +179,11 @@ Status BLPExecutor::resume(GPUstream stream) {
     RETURN_STATUS(getStopPoint(stream));
     if (stopIndex == -1) return Status::Succ;
     for (size_t i = (size_t)stopIndex; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
+    return Status::Succ;
+}
+
+Status BLPExecutor::reset_counters(GPUstream stream) {
+    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num(), stream));
     return Status::Succ;
 }
 

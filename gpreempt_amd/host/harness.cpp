@@ -1,0 +1,545 @@
+// Multi-tenant benchmark harness: tenants with priorities share one GPU; the policy decides how
+// a higher-priority request takes the GPU from lower-priority work.
+//
+// It plays the role of the reference's DISB suite (third_party/disb/src/benchmark.cpp:182-338,
+// load.cpp:71-260, analyzer.cpp:90-170) together with the client programs that carry the
+// scheduling policies (src/cuda-clients/blpclient.cpp:163-198 "wb", src/common-clients/
+// baseclient.cpp "np", seqclient.cpp:82-102 "seq", rtonlyclient.cpp:120-141 "lco"), and reads
+// the same task-file schema (config/A.json).  Unlike DISB it keeps every request's latency, so
+// percentiles can be reported, and it seeds the Poisson generator from the task file instead of
+// the clock (load.cpp:190).
+#include "harness.h"
+
+#include <algorithm>
+#include <atomic>
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <mutex>
+#include <thread>
+
+#include "executor.h"
+#include "mini_json.h"
+#include "numeric.h"
+
+namespace foo {
+
+using clock_type = std::chrono::steady_clock;
+static inline int64_t now_ns() { return std::chrono::duration_cast<std::chrono::nanoseconds>(clock_type::now().time_since_epoch()).count(); }
+static inline void spin_pause() { __builtin_ia32_pause(); }
+
+namespace {
+
+constexpr int kMaxLevels = 8;
+constexpr int kWarmups = 10;          // third_party/disb/include/benchmark.h:39
+constexpr int kStandAloneRuns = 100;  // third_party/disb/include/benchmark.h:40
+
+// ---- arrival processes (third_party/disb/src/load.cpp) -----------------------------------------
+struct Load {
+    std::string type = "continuous";
+    double frequency = 0;
+    uint64_t seed = 1;
+    int64_t next = 0, end = 0;
+    numeric::Rng rng{1};
+
+    int64_t gap_ns() {
+        if (type == "poisson") {  // exponential gaps: -ln(u) / frequency (load.cpp:230-237)
+            double u = rng.uniform01();
+            if (u < 1e-12) u = 1e-12;
+            return (int64_t)(-std::log(u) / frequency * 1e9);
+        }
+        return (int64_t)(1e9 / frequency);
+    }
+    void start(int64_t begin, int64_t end_) {
+        next = begin; end = end_;
+        rng = numeric::Rng(seed);
+    }
+    // Returns false when the run is over.  A launch whose successor is already due is given up,
+    // as in DISB ("always choose the newest frame", load.cpp:196-222).  *scheduled receives the
+    // arrival time of the request that is served.
+    bool wait_next(int64_t *scheduled) {
+        int64_t now = now_ns();
+        if (type == "continuous") {
+            *scheduled = now;
+            return now < end;
+        }
+        if (frequency <= 0) return false;
+        int64_t nn = next + gap_ns();
+        while (nn < now) { next = nn; nn = next + gap_ns(); }
+        if (next >= end) return false;
+        while (now_ns() < next) {
+            int64_t left = next - now_ns();
+            if (left > 200000) std::this_thread::sleep_for(std::chrono::nanoseconds(left - 100000));
+            else spin_pause();
+        }
+        *scheduled = next;
+        next = nn;
+        return true;
+    }
+};
+
+struct Stats {
+    std::vector<double> v;  // microseconds
+    void add(double us) { v.push_back(us); }
+    double pct(double p) const {
+        if (v.empty()) return 0;
+        std::vector<double> s(v);
+        std::sort(s.begin(), s.end());
+        double idx = p * (s.size() - 1);
+        size_t lo = (size_t)idx;
+        size_t hi = std::min(lo + 1, s.size() - 1);
+        return s[lo] + (s[hi] - s[lo]) * (idx - lo);
+    }
+    double mean() const {
+        if (v.empty()) return 0;
+        double t = 0;
+        for (double x : v) t += x;
+        return t / v.size();
+    }
+    double max() const { return v.empty() ? 0 : *std::max_element(v.begin(), v.end()); }
+    json::Value to_json() const {
+        json::Value o = json::Value::object();
+        o.set("count") = v.size();
+        o.set("mean") = mean(); o.set("p50") = pct(0.5); o.set("p90") = pct(0.9); o.set("p99") = pct(0.99); o.set("max") = max();
+        return o;
+    }
+};
+
+// ---- shared scheduling state -------------------------------------------------------------------
+// Level p tenants obey flag word p-1, which is up while any tenant of a level < p is active
+// (the reference has two levels and one word, blpclient.cpp:185-195; the three-tenant
+// configuration needs one word per level).
+struct Shared {
+    std::string policy;
+    int levels = 2;
+    volatile int *flag_host[kMaxLevels] = {nullptr};
+    void *flag_dev[kMaxLevels] = {nullptr};
+    std::atomic<int> active[kMaxLevels];   // requests of this level that want or hold the GPU
+    std::atomic<int> on_gpu[kMaxLevels];   // preemptible tenants of this level with work in flight
+    std::atomic<int64_t> flag_raised_ns[kMaxLevels];
+    std::mutex flag_mu, seq_mu;
+    std::mutex stats_mu;
+    Stats preempt_latency;                 // flag store -> lower-priority stream drained
+    std::atomic<int64_t> hp_busy_ns{0};
+    std::atomic<int> cores{0};
+    long hp_requests = 0;                  // > 0: the run ends once every priority-0 tenant served this many
+    std::atomic<int> hp_unfinished{0};
+    std::atomic<bool> stop{false};
+
+    Shared() {
+        for (int i = 0; i < kMaxLevels; ++i) { active[i] = 0; on_gpu[i] = 0; flag_raised_ns[i] = 0; }
+    }
+    int active_above(int p) const {
+        int n = 0;
+        for (int i = 0; i < p; ++i) n += active[i].load(std::memory_order_acquire);
+        return n;
+    }
+    int on_gpu_below(int p) const {
+        int n = 0;
+        for (int i = p + 1; i < levels; ++i) n += on_gpu[i].load(std::memory_order_acquire);
+        return n;
+    }
+    void update_flags() {  // flag[j] = any active at level <= j
+        std::lock_guard<std::mutex> g(flag_mu);
+        int run = 0;
+        for (int j = 0; j + 1 < levels; ++j) {
+            run += active[j].load();
+            int want = run > 0;
+            if (*flag_host[j] != want) {
+                if (want) flag_raised_ns[j].store(now_ns());
+                *flag_host[j] = want;
+            }
+        }
+    }
+};
+
+struct Tenant {
+    std::string id, name, model_name;
+    int priority = 0;
+    bool use_graph = true;
+    int64_t preprocess_us = 0;
+    Load load;
+    std::unique_ptr<Executor> ex;
+    BLPExecutor *blp = nullptr;
+    GPUstream stream = nullptr;
+    void *input = nullptr, *output = nullptr;
+    size_t input_size = 0, output_size = 0;
+    Stats standalone, total, infer, queueing;
+    int64_t preemptions = 0, requests = 0;
+    int64_t first_ns = 0, last_ns = 0;
+    Status error = Status::Succ;
+};
+
+void fill_input(Tenant &t) {
+    // synthetic input: N(0,1) values for images, uniform token ids for BERT (int64 storage)
+    numeric::Rng rng(0xDA7A + std::hash<std::string>()(t.id) % 1000);
+    auto m = t.ex->get_model();
+    size_t idx = 0;
+    m->find_storage_idx("data", idx);
+    const std::string &st = m->get_storage_info(idx).stype;
+    if (st == "int64") { int64_t *p = (int64_t *)t.input; for (size_t i = 0; i < t.input_size / 8; ++i) p[i] = (int64_t)(rng.next() % 30522); }
+    else if (st == "float32") { float *p = (float *)t.input; for (size_t i = 0; i < t.input_size / 4; ++i) p[i] = rng.normal(); }
+    else if (st == "float16") { uint16_t *p = (uint16_t *)t.input; for (size_t i = 0; i < t.input_size / 2; ++i) p[i] = numeric::f32_to_f16(rng.normal()); }
+    else { uint16_t *p = (uint16_t *)t.input; for (size_t i = 0; i < t.input_size / 2; ++i) p[i] = numeric::f32_to_bf16(rng.normal()); }
+}
+
+Status init_tenant(Tenant &t, Shared &sh) {
+    const bool preemptible = t.priority > 0 && (sh.policy == "wb" || sh.policy == "wb-async");
+    if (preemptible) { t.blp = new BLPExecutor(); t.ex.reset(t.blp); }
+    else t.ex.reset(new BaseExecutor());
+    RETURN_STATUS(t.ex->init(t.model_name));
+    t.input_size = t.ex->get_data_size("data");
+    t.output_size = t.ex->get_data_size("heads");
+    CUDA_RETURN_STATUS(gp_host_alloc(&t.input, t.input_size));
+    CUDA_RETURN_STATUS(gp_host_alloc(&t.output, t.output_size));
+    fill_input(t);
+    CUDA_RETURN_STATUS(gp_stream_create(t.priority, &t.stream));
+    if (t.blp) {
+        int level = std::min(t.priority, sh.levels - 1);
+        t.blp->dpStop = sh.flag_dev[level - 1];
+    }
+    if (t.use_graph) t.ex->capture_graph(t.stream);
+    return Status::Succ;
+}
+
+// Waits until the stream is idle by polling, which reacts faster than a blocking wait.
+Status drain(GPUstream s) {
+    for (;;) {
+        int idle = 0;
+        CUDA_RETURN_STATUS(gp_stream_query(s, &idle));
+        if (idle) return Status::Succ;
+        spin_pause();
+    }
+}
+
+// One inference under the policy.  Mirrors FooClient::infer of the reference's clients.
+Status infer(Tenant &t, Shared &sh) {
+    const int p = std::min(t.priority, sh.levels - 1);
+    const std::string &pol = sh.policy;
+    if (pol == "seq") {
+        // seqclient.cpp:82-102: one model at a time; a best-effort tenant yields while a
+        // latency-critical request is waiting.
+        if (p > 0) while (sh.active_above(p) > 0) spin_pause();
+        else sh.active[0].fetch_add(1);
+        std::lock_guard<std::mutex> g(sh.seq_mu);
+        RETURN_STATUS(t.ex->execute(t.stream));
+        RETURN_STATUS(drain(t.stream));
+        if (p == 0) sh.active[0].fetch_sub(1);
+        return Status::Succ;
+    }
+    if (pol == "np" || pol == "lco" || !(pol == "wb" || pol == "wb-async")) {
+        // baseclient.cpp: every tenant submits on its own stream, nothing is preempted
+        int64_t t0 = now_ns();
+        RETURN_STATUS(t.ex->execute(t.stream));
+        RETURN_STATUS(drain(t.stream));
+        if (p == 0) sh.hp_busy_ns.fetch_add(now_ns() - t0);
+        return Status::Succ;
+    }
+    // ---- "wb": cooperative block-level preemption ------------------------------------------
+    // 1. announce: raises the flag words of every lower level (blpclient.cpp:185-188)
+    sh.active[p].fetch_add(1, std::memory_order_acq_rel);
+    if (p + 1 < sh.levels) sh.update_flags();
+    int64_t t0 = now_ns();
+    // 2. "wb": wait until lower-priority work has left the GPU (blpclient.cpp:189); "wb-async"
+    //    submits at once and lets the hardware start workgroups as the others retire.
+    if (pol == "wb") while (sh.on_gpu_below(p) > 0) spin_pause();
+    Status st = Status::Succ;
+    if (!t.blp) {
+        st = t.ex->execute(t.stream);
+        if (st == Status::Succ) st = drain(t.stream);
+    } else {
+        // 3. preemptible tenant (blpclient.cpp:163-183): run, and after every drain ask whether a
+        //    kernel was stopped; if so wait for the higher levels to finish and resume.
+        while (sh.active_above(p) > 0) spin_pause();
+        sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
+        t.blp->running = true;
+        st = t.blp->execute(t.stream);
+        while (st == Status::Succ) {
+            st = drain(t.stream);
+            if (st != Status::Succ) break;
+            int64_t drained = now_ns();
+            const bool contended = sh.active_above(p) > 0;
+            sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
+            if (contended) {
+                int64_t raised = sh.flag_raised_ns[p - 1].load();
+                if (raised > 0 && drained >= raised) {
+                    std::lock_guard<std::mutex> g(sh.stats_mu);
+                    sh.preempt_latency.add((drained - raised) / 1e3);
+                }
+                while (sh.active_above(p) > 0) spin_pause();
+            }
+            sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
+            st = t.blp->resume(t.stream);  // reads the stop index; -1 means the model had finished
+            if (st != Status::Succ) break;
+            if (t.blp->last_stop_index() == -1) break;
+            ++t.preemptions;
+        }
+        t.blp->running = false;
+        sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
+    }
+    // 4. retire: lowers the flag words when this was the last active request of its level
+    sh.active[p].fetch_sub(1, std::memory_order_acq_rel);
+    if (p + 1 < sh.levels) sh.update_flags();
+    if (p == 0) sh.hp_busy_ns.fetch_add(now_ns() - t0);
+    return st;
+}
+
+// One request: the six DISB phases (benchmark.cpp:66-135); prepareInput and postprocess are empty
+// in the reference's clients, preprocess sleeps preprocess_time (blpclient.cpp:153-155).
+Status infer_once(Tenant &t, Shared &sh, double *total_us, double *infer_us) {
+    int64_t t0 = now_ns();
+    if (t.preprocess_us > 0) std::this_thread::sleep_for(std::chrono::microseconds(t.preprocess_us));
+    RETURN_STATUS(t.ex->set_input("data", t.input, t.input_size, t.stream));
+    CUDA_RETURN_STATUS(gp_stream_sync(t.stream));
+    int64_t t1 = now_ns();
+    RETURN_STATUS(infer(t, sh));
+    int64_t t2 = now_ns();
+    RETURN_STATUS(t.ex->get_output("heads", t.output, t.output_size, t.stream));
+    CUDA_RETURN_STATUS(gp_stream_sync(t.stream));
+    int64_t t3 = now_ns();
+    *total_us = (t3 - t0) / 1e3;
+    *infer_us = (t2 - t1) / 1e3;
+    return Status::Succ;
+}
+
+void tenant_thread(Tenant *t, Shared *sh, std::atomic<int> *ready, int n_tasks, int64_t begin, int64_t end) {
+    bind_core(sh->cores.fetch_add(1));  // blpclient.cpp:147
+    util::init_cuda();
+    ready->fetch_add(1);
+    while (ready->load() < n_tasks) spin_pause();
+    t->load.start(begin, end);
+    int64_t scheduled = 0;
+    bool counted = false;
+    while (!sh->stop.load(std::memory_order_acquire) && t->load.wait_next(&scheduled)) {
+        if (sh->stop.load(std::memory_order_acquire)) break;
+        double total = 0, inf = 0;
+        int64_t start = now_ns();
+        Status s = infer_once(*t, *sh, &total, &inf);
+        if (s != Status::Succ) { t->error = s; break; }
+        if (t->requests == 0) t->first_ns = start;
+        t->last_ns = now_ns();
+        ++t->requests;
+        t->total.add(total);
+        t->infer.add(inf);
+        t->queueing.add((start - scheduled) / 1e3);
+        if (sh->hp_requests > 0 && t->priority == 0 && !counted && t->requests >= sh->hp_requests) {
+            counted = true;
+            if (sh->hp_unfinished.fetch_sub(1) == 1) sh->stop.store(true, std::memory_order_release);
+            break;
+        }
+    }
+    if (sh->hp_requests > 0 && t->priority == 0 && !counted && sh->hp_unfinished.fetch_sub(1) == 1) sh->stop.store(true, std::memory_order_release);
+}
+
+}  // namespace
+
+Status run_scenario(const std::string &config_text, std::string &report_text) {
+    json::Value cfg;
+    if (!json::parse(config_text, cfg) || cfg.type != json::Value::Object) {
+        std::fprintf(stderr, "scenario: malformed JSON\n");
+        return Status::Fail;
+    }
+    util::init_cuda();
+    Shared sh;
+    sh.policy = cfg["policy"].string("wb");
+    double seconds = cfg["time"].number(5);
+    int standalone_runs = (int)cfg["standalone_runs"].number(kStandAloneRuns);
+    int warmups = (int)cfg["warmups"].number(kWarmups);
+    sh.hp_requests = (long)cfg["hp_requests"].number(0);
+    const json::Value &tasks = cfg["tasks"];
+    std::vector<std::unique_ptr<Tenant>> tenants;
+    int max_prio = 0;
+    for (const json::Value &tv : tasks.arr) {
+        std::unique_ptr<Tenant> t(new Tenant());
+        const json::Value &c = tv["client"], &l = tv["load"];
+        t->id = tv["id"].string(c["name"].string("task"));
+        t->name = c["name"].string(t->id);
+        t->model_name = c["model_name"].string();
+        t->priority = (int)c["priority"].number(0);
+        t->use_graph = c["use_cuda_graph"].boolean(true);
+        t->preprocess_us = (int64_t)c["preprocess_time"].number(0);
+        t->load.type = l["type"].string("continuous");
+        t->load.frequency = l["frequency"].number(0);
+        t->load.seed = (uint64_t)l["seed"].number(1 + (double)tenants.size());
+        if (sh.policy == "lco" && t->priority != 0) continue;  // rtonlyclient.cpp:120-141: keep the real-time tasks only
+        max_prio = std::max(max_prio, t->priority);
+        tenants.push_back(std::move(t));
+    }
+    if (tenants.empty()) return Status::NotFound;
+    sh.levels = std::min(max_prio + 1, kMaxLevels);
+    if (sh.levels < 2) sh.levels = 2;
+    for (int j = 0; j + 1 < sh.levels; ++j) CUDA_RETURN_STATUS(gp_flag_create(&sh.flag_host[j], &sh.flag_dev[j]));
+    for (auto &t : tenants) RETURN_STATUS(init_tenant(*t, sh));
+
+    // warm-up and stand-alone latency, one tenant at a time (benchmark.cpp:221-299)
+    for (auto &t : tenants) {
+        for (int i = 0; i < warmups + standalone_runs; ++i) {
+            double total = 0, inf = 0;
+            RETURN_STATUS(infer_once(*t, sh, &total, &inf));
+            if (i >= warmups) t->standalone.add(total);
+        }
+        t->preemptions = 0;
+    }
+    {
+        std::lock_guard<std::mutex> g(sh.stats_mu);
+        sh.preempt_latency = Stats();
+    }
+    sh.hp_busy_ns = 0;
+
+    // co-run
+    for (auto &t : tenants) if (t->priority == 0) sh.hp_unfinished.fetch_add(1);
+    std::atomic<int> ready{0};
+    int64_t begin = now_ns() + 50 * 1000 * 1000;
+    int64_t end = begin + (int64_t)(seconds * 1e9);
+    std::vector<std::thread> threads;
+    for (auto &t : tenants) threads.emplace_back(tenant_thread, t.get(), &sh, &ready, (int)tenants.size(), begin, end);
+    for (auto &th : threads) th.join();
+    double wall_s = (now_ns() - begin) / 1e9;
+
+    json::Value rep = json::Value::object();
+    rep.set("policy") = sh.policy;
+    rep.set("time(s)") = wall_s;
+    json::Value &jt = rep.set("tasks");
+    jt = json::Value::object();
+    double hp_ratio = 0, be_kept = 0;
+    int n_hp = 0, n_be = 0;
+    double busy_frac = std::min(1.0, sh.hp_busy_ns.load() / 1e9 / std::max(wall_s, 1e-9));
+    Status result = Status::Succ;
+    for (auto &t : tenants) {
+        json::Value &o = jt.set(t->id);
+        o = json::Value::object();
+        o.set("model") = t->model_name;
+        o.set("priority") = t->priority;
+        o.set("kernels") = t->ex->get_kernel_num();
+        o.set("requests") = (long)t->requests;
+        double span = t->requests > 0 ? (t->last_ns - t->first_ns) / 1e9 : 0;
+        double thr = span > 0 ? t->requests / span : 0;
+        o.set("avgThroughput(req/s)") = thr;
+        o.set("avgTotalLatency(us)") = t->total.mean();
+        o.set("standAloneTotalLatency(us)") = t->standalone.mean();
+        o.set("avgTotalLatencyIncrease(us)") = t->total.mean() - t->standalone.mean();
+        o.set("totalLatency(us)") = t->total.to_json();
+        o.set("inferLatency(us)") = t->infer.to_json();
+        o.set("queueing(us)") = t->queueing.to_json();
+        o.set("standAlone(us)") = t->standalone.to_json();
+        o.set("preemptions") = (long)t->preemptions;
+        double alone_thr = t->standalone.mean() > 0 ? 1e6 / t->standalone.mean() : 0;
+        o.set("standAloneThroughput(req/s)") = alone_thr;
+        if (t->priority == 0) {
+            double r = t->standalone.pct(0.99) > 0 ? t->total.pct(0.99) / t->standalone.pct(0.99) : 0;
+            o.set("p99_vs_isolated") = r;
+            hp_ratio = std::max(hp_ratio, r);
+            ++n_hp;
+        } else if (t->load.type == "continuous") {
+            // throughput the idle gaps allow = isolated throughput x fraction of time without a
+            // high-priority request on the GPU
+            double allowed = alone_thr * (1.0 - busy_frac);
+            double kept = allowed > 0 ? thr / allowed : 0;
+            o.set("throughput_kept") = kept;
+            be_kept += kept;
+            ++n_be;
+        }
+        if (t->error != Status::Succ) { o.set("error") = status_name(t->error); result = t->error; }
+    }
+    rep.set("hp_busy_fraction") = busy_frac;
+    rep.set("hp_p99_vs_isolated") = hp_ratio;
+    rep.set("be_throughput_kept") = n_be ? be_kept / n_be : 0.0;
+    rep.set("preemptLatency(us)") = sh.preempt_latency.to_json();
+    report_text = rep.dump();
+
+    for (auto &t : tenants) {
+        t->ex->clear();
+        gp_host_free(t->input);
+        gp_host_free(t->output);
+        gp_stream_destroy(t->stream);
+    }
+    tenants.clear();
+    for (int j = 0; j + 1 < sh.levels; ++j) gp_flag_destroy(sh.flag_host[j]);
+    return result;
+}
+
+// Per-kernel preemption and resume latency of one best-effort model: the model runs back to
+// back; an injector raises the flag at random instants, waits for the stream to drain, notes
+// which kernel was stopped (the stop index) and how long the drain took, then clears the flag
+// and the model resumes.
+Status preempt_probe(const std::string &workload, int trials, bool use_graph, uint64_t seed, std::string &report_text) {
+    util::init_cuda();
+    BLPExecutor ex;
+    RETURN_STATUS(ex.init(workload));
+    volatile int *flag_host = nullptr;
+    void *flag_dev = nullptr;
+    CUDA_RETURN_STATUS(gp_flag_create(&flag_host, &flag_dev));
+    ex.dpStop = flag_dev;
+    GPUstream stream;
+    CUDA_RETURN_STATUS(gp_stream_create(1, &stream));
+    if (use_graph) ex.capture_graph(stream);
+    size_t n = ex.get_kernel_num();
+    // isolated duration of one inference
+    Stats iso;
+    for (int i = 0; i < 12; ++i) {
+        int64_t t0 = now_ns();
+        RETURN_STATUS(ex.execute(stream));
+        RETURN_STATUS(drain(stream));
+        if (i >= 2) iso.add((now_ns() - t0) / 1e3);
+    }
+    double span_us = iso.mean();
+    std::vector<Stats> per_kernel(n), per_kernel_resume(n);
+    Stats all, all_resume;
+    numeric::Rng rng(seed);
+    int hits = 0;
+    for (int tr = 0; tr < trials; ++tr) {
+        ex.running = true;
+        RETURN_STATUS(ex.execute(stream));
+        int64_t wait = (int64_t)(rng.uniform01() * span_us * 0.95 * 1e3);
+        int64_t t0 = now_ns();
+        while (now_ns() - t0 < wait) spin_pause();
+        int64_t raised = now_ns();
+        *flag_host = 1;
+        RETURN_STATUS(drain(stream));
+        int64_t drained = now_ns();
+        *flag_host = 0;
+        int64_t r0 = now_ns();
+        RETURN_STATUS(ex.resume(stream));
+        int64_t r1 = now_ns();
+        int stop = ex.last_stop_index();
+        RETURN_STATUS(drain(stream));
+        if (stop >= 0 && (size_t)stop < n) {
+            ++hits;
+            per_kernel[stop].add((drained - raised) / 1e3);
+            per_kernel_resume[stop].add((r1 - r0) / 1e3);
+            all.add((drained - raised) / 1e3);
+            all_resume.add((r1 - r0) / 1e3);
+        }
+        ex.running = false;
+    }
+    json::Value rep = json::Value::object();
+    rep.set("workload") = workload;
+    rep.set("kernels") = n;
+    rep.set("trials") = trials;
+    rep.set("interrupted") = hits;
+    rep.set("isolated(us)") = iso.to_json();
+    rep.set("preemptLatency(us)") = all.to_json();
+    rep.set("resumeCall(us)") = all_resume.to_json();
+    json::Value &pk = rep.set("perKernel");
+    pk = json::Value::array();
+    auto model = ex.get_model();
+    for (size_t i = 0; i < n; ++i) {
+        if (per_kernel[i].v.empty()) continue;
+        json::Value o = json::Value::object();
+        o.set("kernel") = i;
+        o.set("name") = model->get_kernel_info(i).name;
+        o.set("tiles") = model->get_kernel_info(i).total_blocks;
+        o.set("samples") = per_kernel[i].v.size();
+        o.set("preempt_mean(us)") = per_kernel[i].mean();
+        o.set("preempt_max(us)") = per_kernel[i].max();
+        o.set("resume_mean(us)") = per_kernel_resume[i].mean();
+        pk.push(o);
+    }
+    report_text = rep.dump();
+    ex.clear();
+    gp_stream_destroy(stream);
+    gp_flag_destroy(flag_host);
+    return Status::Succ;
+}
+
+}  // namespace foo

@@ -83,6 +83,9 @@ public:
     // `claim` raises the flag itself.  Applies to the next execute()/resume(); -1 disarms.
     void inject_preempt(int kernel, int claim) { inject_kernel = kernel; inject_claim = claim; }
     Status read_counters(std::vector<int> &out);
+    // Zeroes every tile counter on `stream` (what execute() does first), for callers that
+    // launch kernel by kernel.
+    Status reset_counters(GPUstream stream);
 
 public:
     GPUdeviceptr dpStop = nullptr;  // the preempt flag: allocated by the caller, shared by all best-effort tenants

@@ -36,6 +36,7 @@ int gpx_get_stop_point(gpx_executor e, gp_stream s, int *stop_index);/* BLPExecu
 int gpx_last_stop_index(gpx_executor e);                             /* value read by the last getStopPoint / resume */
 int gpx_inject_preempt(gpx_executor e, int kernel, int claim);       /* BLPExecutor::inject_preempt (test hook) */
 int gpx_read_counters(gpx_executor e, int *out, size_t n);           /* BLPExecutor::read_counters */
+int gpx_reset_counters(gpx_executor e, gp_stream s);                 /* BLPExecutor::reset_counters */
 
 /* Model introspection (foo::Model::get_storage_info / get_kernel_info) */
 size_t gpx_storage_num(gpx_executor e);
@@ -45,6 +46,20 @@ int gpx_storage_info(gpx_executor e, size_t idx, char *name, size_t name_len, ch
 int gpx_kernel_info(gpx_executor e, size_t idx, char *name, size_t name_len, double *flops, double *bytes,
                     int *total_blocks, int *grid);
 int gpx_read_storage(gpx_executor e, const char *key, void *out, size_t len); /* blocking Model::get */
+
+/* Multi-tenant scenario runner: the role of the reference's client executables
+ * (src/cuda-clients/blpclient.cpp main() and the programs under src/common-clients) over a DISB task file
+ * (config/A.json schema) with an extra "policy" key: "wb" (block-level preemption, HP waits for
+ * the drain as blpclient.cpp:189 does), "wb-async" (HP submits at once), "np" (no preemption,
+ * baseclient.cpp), "seq" (seqclient.cpp), "lco" (high-priority tasks only, rtonlyclient.cpp).
+ * The JSON report is written to `report` (NUL-terminated, truncated to report_len). */
+int gpx_run_scenario(const char *config_json, char *report, size_t report_len);
+/* Per-kernel preemption / resume latency of one best-effort model (BASELINE config 2). */
+int gpx_preempt_probe(const char *workload, int trials, int use_graph, unsigned long long seed, char *report, size_t report_len);
+/* Parses a TVM_MODEL_PARAMS file (ModelParamParser::parse_from_file, reference src/model.cpp:15-55):
+ * returns the number of tensors (-1: missing or malformed); when `key` names a tensor, up to n of
+ * its values are copied to `out` and *len receives its length. */
+long gpx_parse_params(const char *path, const char *key, float *out, size_t n, size_t *len);
 
 #ifdef __cplusplus
 }
