@@ -12,6 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libgpreempt_hip.so")
 
 F32, F16, BF16, I32, I64 = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
+MAT_AUTO, MAT_STAGED, MAT_PIPE, MAT_PIPE_SPLITK = 0, 1, 2, 3
 SUCC, FAIL, TIMEOUT, NOTFOUND, OUTOFRANGE, FULL = range(6)
 DTYPE_SIZE = {F32: 4, F16: 2, BF16: 2, I32: 4, I64: 8}
 DTYPE_BY_NAME = {"f32": F32, "f16": F16, "bf16": BF16}
@@ -35,7 +36,7 @@ class GemmParams(C.Structure):
                 ("C", vp), ("ldc", C.c_long), ("stride_c", C.c_long),
                 ("bias", vp), ("residual", vp), ("alpha", C.c_float), ("act", C.c_int), ("batch", C.c_int),
                 ("batch_inner", C.c_int), ("stride_a_outer", C.c_long), ("stride_b_outer", C.c_long),
-                ("stride_c_outer", C.c_long), ("tile_m", C.c_int), ("tile_n", C.c_int)]
+                ("stride_c_outer", C.c_long), ("tile_m", C.c_int), ("tile_n", C.c_int), ("variant", C.c_int)]
 
 
 class ConvParams(C.Structure):
@@ -43,7 +44,7 @@ class ConvParams(C.Structure):
                 ("N", "H", "W", "Cin", "Cout", "R", "S", "stride_h", "stride_w", "pad_h", "pad_w")] + [
                 ("in_", vp), ("in_pix_stride", C.c_long), ("weight", vp), ("bias", vp),
                 ("residual", vp), ("res_pix_stride", C.c_long), ("out", vp), ("out_pix_stride", C.c_long),
-                ("act", C.c_int), ("tile_m", C.c_int), ("tile_n", C.c_int)]
+                ("act", C.c_int), ("tile_m", C.c_int), ("tile_n", C.c_int), ("variant", C.c_int)]
 
 
 class LayoutParams(C.Structure):

@@ -49,36 +49,39 @@ __device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy) {
 // call it; the body may use barriers freely.
 template <class Body>
 __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
-    if (b.executed == nullptr) {
-        int idx = blockIdx.x;
-        if (idx < b.total) body(decode_tile(idx, b.sx, b.sy));
-        return;
-    }
     __shared__ int mailbox[2];
+    const bool dynamic = b.executed != nullptr;
     const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    // One loop and one call site for both modes, so that the body is inlined into the kernel and
+    // the kernel arguments stay in scalar registers.
     for (int it = 0;; ++it) {
-        if (leader) {
-            int idx = -1;
-            int stop = b.flag ? __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : 0;
-            // Sticky: once a kernel of this executor has been stopped, every later kernel of the
-            // same submission leaves too until the host re-arms the stop index, even if the flag
-            // has been lowered in between.  Otherwise a kernel queued behind a stopped one could
-            // run to completion on incomplete inputs.
-            stop |= __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
-            if (!stop) {
-                idx = atomicAdd(b.executed, 1);
-                if (idx >= b.total) {
-                    idx = -1;
-                } else if (idx == b.inject_at && b.flag) {
-                    __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        int idx;
+        if (!dynamic) {
+            idx = (it == 0 && (int)blockIdx.x < b.total) ? (int)blockIdx.x : -1;
+        } else {
+            if (leader) {
+                int claim = -1;
+                int stop = b.flag ? __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : 0;
+                // Sticky: once a kernel of this executor has been stopped, every later kernel of the
+                // same submission leaves too until the host re-arms the stop index, even if the flag
+                // has been lowered in between.  Otherwise a kernel queued behind a stopped one could
+                // run to completion on incomplete inputs.
+                stop |= __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
+                if (!stop) {
+                    claim = atomicAdd(b.executed, 1);
+                    if (claim >= b.total) {
+                        claim = -1;
+                    } else if (claim == b.inject_at && b.flag) {
+                        __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    }
+                } else {
+                    atomicCAS(b.stop_index, -1, b.kernel_id);
                 }
-            } else {
-                atomicCAS(b.stop_index, -1, b.kernel_id);
+                mailbox[it & 1] = claim;
             }
-            mailbox[it & 1] = idx;
+            __syncthreads();
+            idx = mailbox[it & 1];
         }
-        __syncthreads();
-        int idx = mailbox[it & 1];
         if (idx < 0) return;
         body(decode_tile(idx, b.sx, b.sy));
     }

@@ -19,7 +19,7 @@ def rel_err(got, ref):
     return float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
 
 
-def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None, tile=0, batch=1, alpha=1.0):
+def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None, tile=0, batch=1, alpha=1.0, variant=0):
     rng = np.random.default_rng(seed)
     dtype = gp.DTYPE_BY_NAME[dt]
     A = O.round_to(rng.uniform(-1, 1, (batch, M, K)).astype(np.float32), dt)
@@ -35,7 +35,7 @@ def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None
     p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, stride_a=M * K, B=dB.ptr,
                       ldb=K if b_is_nk else N, stride_b=N * K, b_is_nk=int(b_is_nk), C=dC.ptr, ldc=N,
                       stride_c=M * N, bias=gp._ptr(dbias), residual=gp._ptr(dres), alpha=alpha, act=act,
-                      batch=batch, tile_m=tile, tile_n=tile)
+                      batch=batch, tile_m=tile, tile_n=tile, variant=variant)
     info = ctx_fn(p, dC) if ctx_fn else gp.launch("gp_launch_gemm", p)
     gp.check(gp.lib().gp_stream_sync(None))
     got = dC.download(dtype, (batch, M, N)).copy()
@@ -46,19 +46,26 @@ def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None
 
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("b_is_nk", [False, True])
-@pytest.mark.parametrize("shape", [(256, 256, 128), (200, 136, 72), (64, 1000, 512), (1, 8, 8), (130, 264, 40)])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (200, 136, 72), (64, 1000, 512), (1, 8, 8), (130, 264, 40), (128, 768, 3072), (1568, 256, 2304)])
 def test_gemm_matches_oracle(gp, dt, b_is_nk, shape):
     M, N, K = shape
-    for tile in (64, 128):
-        got, ref, info = run_gemm(gp, dt, M, N, K, b_is_nk, gp.ACT_RELU, True, True, seed=M + N + K, tile=tile)
-        assert info.total_tiles == -(-M // tile) * -(-N // tile)
-        assert np.isfinite(got).all()
-        assert rel_err(got, ref) < TOL[dt], (dt, shape, tile)
+    # every kernel variant and tile size that supports the layout (B stored K x N needs the
+    # register-staged kernel), plus the launcher's own choice
+    variants = [(64, gp.MAT_STAGED), (128, gp.MAT_STAGED), (0, gp.MAT_AUTO)]
+    if b_is_nk:
+        variants += [(64, gp.MAT_PIPE), (128, gp.MAT_PIPE), (64, gp.MAT_PIPE_SPLITK), (32, gp.MAT_PIPE_SPLITK)]
+    for tile, variant in variants:
+        got, ref, info = run_gemm(gp, dt, M, N, K, b_is_nk, gp.ACT_RELU, True, True, seed=M + N + K, tile=tile, variant=variant)
+        if tile:
+            assert info.total_tiles == -(-M // tile) * -(-N // tile)
+        assert np.isfinite(got).all(), (dt, shape, tile, variant)
+        assert rel_err(got, ref) < TOL[dt], (dt, shape, tile, variant)
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16"])
-def test_gemm_batched_alpha_gelu(gp, dt):
-    got, ref, info = run_gemm(gp, dt, 128, 64, 64, True, gp.ACT_GELU, True, False, seed=3, batch=6, alpha=0.125)
+@pytest.mark.parametrize("variant", [1, 2, 3])
+def test_gemm_batched_alpha_gelu(gp, dt, variant):
+    got, ref, info = run_gemm(gp, dt, 128, 64, 64, True, gp.ACT_GELU, True, False, seed=3, batch=6, alpha=0.125, variant=variant)
     assert info.shape[2] == 6
     assert rel_err(got, ref) < TOL[dt]
 
@@ -156,3 +163,39 @@ def test_flag_set_before_launch_does_no_tiles(gp):
     assert st.counters()[0] == 0 and st.stop_index() == 0
     assert np.isnan(dC.download(gp.F32, (1024, 1024))).all()
     flag.set(0)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("tile,variant", [(128, 2), (64, 2), (64, 3), (32, 3)])
+def test_pipelined_gemm_preempt_resume_bit_exact(gp, dt, tile, variant):
+    """The direct-to-LDS kernels (N x K weights) under the same protocol as config 1."""
+    M, N, K = 1024, 512, 1024
+    rng = np.random.default_rng(7)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), dt)
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32), dt)
+    bias = O.round_to(rng.uniform(-0.1, 0.1, N).astype(np.float32), dt)
+    dA, dB, db = (gp.DevBuf.from_array(x, dtype) for x in (A, B, bias))
+    dC = gp.DevBuf(M * N * gp.DTYPE_SIZE[dtype])
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, bias=db.ptr,
+                      alpha=1.0, act=gp.ACT_RELU, batch=1, tile_m=tile, tile_n=tile, variant=variant)
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    base = dC.download().copy()
+    ref = O.gemm_bias_act(A, B, bias, act=O.ACT_RELU, b_is_nk=True)
+    assert rel_err(dC.download(dtype, (M, N)), ref) < TOL[dt]
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    total = (M // tile) * (N // tile)
+    for frac in (0.25, 0.75):
+        st.reset()
+        flag.set(0)
+        dC.fill32(0)
+        info = gp.launch("gp_launch_gemm", p, st.ctx(inject_at=int(frac * total), max_workgroups=4))
+        gp.check(gp.lib().gp_stream_sync(None))
+        assert flag.get() == 1 and st.stop_index() == 0 and st.counters()[0] < total
+        flag.set(0)
+        st.clear_stop()
+        gp.launch("gp_launch_gemm", p, st.ctx())
+        gp.check(gp.lib().gp_stream_sync(None))
+        assert np.array_equal(dC.download(), base)

@@ -21,6 +21,8 @@ CONV_CASES = [
     (1, 128, 16, 16, 256, 3, 2, 1),  # strided 3x3
     (2, 256, 8, 8, 512, 1, 2, 0),    # strided 1x1 (projection shortcut)
     (1, 8, 5, 5, 8, 5, 1, 2),        # window as large as the image
+    (2, 96, 9, 9, 64, 3, 1, 1),      # Cin not a multiple of the K-step: taps straddle stages
+    (8, 256, 14, 14, 256, 3, 1, 1),  # the dominant layer of ResNet-152 at batch 8
 ]
 
 
@@ -35,10 +37,10 @@ def test_conv2d_matches_oracle(gp, dt, case):
     Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
     res = rnd(rng, (N, Cout, Ho, Wo), dt)
     ref = O.conv2d(x, w, b, stride, pad, res, O.ACT_RELU)
-    for tile in (64, 128):
-        got, info, _ = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=tile)
-        assert np.isfinite(got).all()
-        assert rel_err(got, ref) < TOL[dt], (dt, case, tile)
+    for tile, variant in ((64, 1), (128, 1), (0, 0), (64, 2), (128, 2), (64, 3), (32, 3)):
+        got, info, _ = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=tile, variant=variant)
+        assert np.isfinite(got).all(), (dt, case, tile, variant)
+        assert rel_err(got, ref) < TOL[dt], (dt, case, tile, variant)
 
 
 def test_conv2d_channel_slices(gp):
