@@ -56,6 +56,9 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
         blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;
         blp->kernel_id = ctx->kernel_id; blp->inject_at = ctx->inject_at;
+        int pe = ctx->poll_every > 0 ? ctx->poll_every : 8;
+        GP_REQUIRE((pe & (pe - 1)) == 0, "poll_every must be a power of two");
+        blp->poll_mask = pe - 1;
         int per_cu = 0;
         GP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, lds_bytes));
         if (per_cu < 1) per_cu = 1;
@@ -64,7 +67,7 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         *grid = (int)(total < resident ? total : resident);
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
-        blp->kernel_id = 0; blp->inject_at = -1;
+        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0;
         *grid = (int)total;
     }
     if (info) {

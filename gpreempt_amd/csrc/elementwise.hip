@@ -92,6 +92,13 @@ __global__ __launch_bounds__(NT) void nchw_to_nhwc_kernel(const TI *in, TO *out,
         if (pix >= HW) return;
         const TI *src = in + (long)t.y * C * HW + pix;
         TO *dst = out + ((long)t.y * HW + pix) * c_pad;
+        if (c_pad == VecIO<TO>::VEC) {  // the usual case (3 channels padded to one vector): one 16-byte store
+            float v[VecIO<TO>::VEC];
+#pragma unroll
+            for (int c = 0; c < VecIO<TO>::VEC; ++c) v[c] = c < C ? VecIO<TI>::ld1(src + (long)c * HW) : 0.f;
+            VecIO<TO>::store(dst, v);
+            return;
+        }
         for (int c = 0; c < c_pad; ++c) {
             float v = c < C ? VecIO<TI>::ld1(src + (long)c * HW) : 0.f;
             VecIO<TO>::st1(dst + c, v);

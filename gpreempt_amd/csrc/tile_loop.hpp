@@ -31,6 +31,7 @@ struct BlpArgs {
     int sx, sy;       // shape.x, shape.y (shape.z = total / (sx*sy))
     int kernel_id;
     int inject_at;    // -1 = off
+    int poll_mask;    // the claim numbered c reads the host flag when (c & poll_mask) == 0
 };
 
 struct TileIdx { int x, y, z; };
@@ -60,19 +61,28 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
             idx = (it == 0 && (int)blockIdx.x < b.total) ? (int)blockIdx.x : -1;
         } else {
             if (leader) {
+                // The stop index (device memory) doubles as the device-side mirror of the flag:
+                // every claim checks it, but only the workgroup about to make a claim whose number
+                // is a multiple of poll_every reads the flag itself from host memory.  Reads of
+                // fine-grained host memory are served one at a time (about 90 ns each on MI355X),
+                // so a poll per tile from every workgroup would dominate short kernels.
+                // The stop index is also sticky: once a kernel of this executor has been stopped,
+                // every later kernel of the same submission leaves too until the host re-arms it,
+                // even if the flag has been lowered in between; otherwise a kernel queued behind a
+                // stopped one could run to completion on incomplete inputs.
                 int claim = -1;
-                int stop = b.flag ? __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) : 0;
-                // Sticky: once a kernel of this executor has been stopped, every later kernel of the
-                // same submission leaves too until the host re-arms the stop index, even if the flag
-                // has been lowered in between.  Otherwise a kernel queued behind a stopped one could
-                // run to completion on incomplete inputs.
-                stop |= __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
+                int stop = __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
                 if (!stop) {
                     claim = atomicAdd(b.executed, 1);
                     if (claim >= b.total) {
                         claim = -1;
-                    } else if (claim == b.inject_at && b.flag) {
-                        __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    } else {
+                        if (claim == b.inject_at && b.flag)
+                            __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                        if ((claim & b.poll_mask) == 0 && b.flag &&
+                            __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
+                            atomicCAS(b.stop_index, -1, b.kernel_id);
+                        // the polling workgroup still owes the tile it has just claimed
                     }
                 } else {
                     atomicCAS(b.stop_index, -1, b.kernel_id);

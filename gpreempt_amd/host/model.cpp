@@ -309,6 +309,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.kernel_id = k.kernel_id;
         ctx.inject_at = inject_at;
         ctx.max_workgroups = 0;
+        ctx.poll_every = 0;
         pc = &ctx;
     }
     gp_launch_info info{};

@@ -97,6 +97,9 @@ typedef struct gp_preempt_ctx {
     int inject_at;   /* test hook: the workgroup whose claim returns this value raises *flag    */
                      /* itself right after the claim; -1 = off                                  */
     int max_workgroups; /* 0 = occupancy-sized persistent grid; >0 caps it                      */
+    int poll_every;  /* the claim numbered c reads the host flag when c % poll_every == 0; a power */
+                     /* of two; 0 = default (8).  All claims check *stop_index (device memory),   */
+                     /* which the polling workgroup sets, so 1 reproduces a poll per tile         */
 } gp_preempt_ctx;
 
 /* What a launch did: filled when the `info` argument of a launcher is non-NULL. */
