@@ -84,7 +84,9 @@ gp_event_sync gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free g
 gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy
 gp_launch_gemm gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
 gp_launch_layernorm gp_launch_embed gp_launch_gate gp_launch_noop gp_graph_begin gp_graph_end gp_graph_launch
-gp_graph_destroy""".split()
+gp_graph_destroy gp_program_create gp_program_destroy gp_program_add_gemm gp_program_add_conv2d
+gp_program_add_nchw_to_nhwc gp_program_add_pool2d gp_program_add_eltwise gp_program_add_softmax gp_program_add_layernorm
+gp_program_add_embed gp_program_add_copy gp_program_finalize gp_program_launch gp_program_layers gp_program_read_state""".split()
 
 _lib = None
 

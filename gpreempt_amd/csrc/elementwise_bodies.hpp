@@ -1,0 +1,371 @@
+// Tile bodies of the memory-bound operators: layout change, pooling, elementwise, softmax,
+// layer-norm, embedding, copy.  All are HBM-bound, so each thread moves 16 bytes per access,
+// consecutive lanes touch consecutive 16-byte chunks (coalesced wave64 accesses), arithmetic is
+// fp32, and row reductions stay inside one wavefront (cross-lane shuffles, no LDS round trip).
+// Each body processes one tile; the stand-alone kernels below and the whole-model program kernel
+// hand tiles to them, so every operator can be stopped at a tile boundary and resumed without
+// redoing or skipping a tile.
+#pragma once
+#include "common.hpp"
+
+namespace gp {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T> struct VecIO;
+template <> struct VecIO<float> {
+    static constexpr int VEC = 4;
+    static __device__ __forceinline__ void load(const float *p, float (&f)[4]) {
+        f32x4 v = *(const f32x4 *)p;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = v[i];
+    }
+    static __device__ __forceinline__ void store(float *p, const float (&f)[4]) {
+        f32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = f[i];
+        *(f32x4 *)p = v;
+    }
+    static __device__ __forceinline__ float ld1(const float *p) { return *p; }
+    static __device__ __forceinline__ void st1(float *p, float v) { *p = v; }
+};
+template <> struct VecIO<_Float16> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ void load(const _Float16 *p, float (&f)[8]) {
+        f16x8 v = *(const f16x8 *)p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+    }
+    static __device__ __forceinline__ void store(_Float16 *p, const float (&f)[8]) {
+        f16x8 v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (_Float16)f[i];
+        *(f16x8 *)p = v;
+    }
+    static __device__ __forceinline__ float ld1(const _Float16 *p) { return (float)*p; }
+    static __device__ __forceinline__ void st1(_Float16 *p, float v) { *p = (_Float16)v; }
+};
+template <> struct VecIO<__bf16> {
+    static constexpr int VEC = 8;
+    static __device__ __forceinline__ void load(const __bf16 *p, float (&f)[8]) {
+        bf16x8 v = *(const bf16x8 *)p;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+    }
+    static __device__ __forceinline__ void store(__bf16 *p, const float (&f)[8]) {
+        bf16x8 v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (__bf16)f[i];
+        *(bf16x8 *)p = v;
+    }
+    static __device__ __forceinline__ float ld1(const __bf16 *p) { return (float)*p; }
+    static __device__ __forceinline__ void st1(__bf16 *p, float v) { *p = (__bf16)v; }
+};
+
+__device__ __forceinline__ float act_f(float v, int act) {
+    if (act == GP_ACT_RELU) return v > 0.f ? v : 0.f;
+    if (act == GP_ACT_GELU) return 0.5f * v * (1.f + erff(v * 0.70710678118654752440f));
+    return v;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+constexpr int NT = 256;
+
+// ---- NCHW -> NHWC (channel padded) ---------------------------------------------------------
+// tile = 256 pixels of one image; a thread owns one pixel: C strided reads (coalesced across
+// the wave for each channel) and one contiguous c_pad-wide write.
+struct LayoutArgs { const void *in_; void *out_; int C, HW, c_pad; };
+template <typename TI, typename TO>
+__device__ __forceinline__ void layout_tile(const LayoutArgs &a, TileIdx t) {
+    const TI *in = (const TI *)a.in_;
+    TO *out = (TO *)a.out_;
+    const int C = a.C, HW = a.HW, c_pad = a.c_pad;
+    
+        int pix = t.x * NT + threadIdx.x;
+        if (pix >= HW) return;
+        const TI *src = in + (long)t.y * C * HW + pix;
+        TO *dst = out + ((long)t.y * HW + pix) * c_pad;
+        if (c_pad == VecIO<TO>::VEC) {  // the usual case (3 channels padded to one vector): one 16-byte store
+            float v[VecIO<TO>::VEC];
+#pragma unroll
+            for (int c = 0; c < VecIO<TO>::VEC; ++c) v[c] = c < C ? VecIO<TI>::ld1(src + (long)c * HW) : 0.f;
+            VecIO<TO>::store(dst, v);
+            return;
+        }
+        for (int c = 0; c < c_pad; ++c) {
+            float v = c < C ? VecIO<TI>::ld1(src + (long)c * HW) : 0.f;
+            VecIO<TO>::st1(dst + c, v);
+        }
+}
+template <typename TI, typename TO>
+__global__ __launch_bounds__(NT) void nchw_to_nhwc_kernel(LayoutArgs a, BlpArgs blp) {
+    tile_loop(blp, [&](TileIdx t) { layout_tile<TI, TO>(a, t); });
+}
+
+// ---- pooling, NHWC -------------------------------------------------------------------------
+// item = (output pixel, 16-byte channel chunk); tile = 256 items.
+struct PoolArgs { gp_pool_params p; int Ho, Wo; long items; };
+template <typename T>
+__device__ __forceinline__ void pool_tile(const PoolArgs &a, TileIdx t) {
+    const gp_pool_params &p = a.p;
+    const int Ho = a.Ho, Wo = a.Wo;
+    const long items = a.items;
+    constexpr int VEC = VecIO<T>::VEC;
+    const int chunks = p.C / VEC;
+    
+        long item = (long)t.x * NT + threadIdx.x;
+        if (item >= items) return;
+        int ch = (int)(item % chunks);
+        long pix = item / chunks;
+        const T *in = (const T *)p.in;
+        T *out = (T *)p.out;
+        float acc[VEC];
+        if (p.mode == 2) {  // global average: pix = n
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) acc[i] = 0.f;
+            const T *src = in + pix * p.H * p.W * p.in_pix_stride + ch * VEC;
+            for (int i = 0; i < p.H * p.W; ++i) {
+                float f[VEC];
+                VecIO<T>::load(src + (long)i * p.in_pix_stride, f);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] += f[j];
+            }
+            float inv = 1.f / (float)(p.H * p.W);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] *= inv;
+            VecIO<T>::store(out + pix * p.out_pix_stride + ch * VEC, acc);
+            return;
+        }
+        int wo = (int)(pix % Wo);
+        long q = pix / Wo;
+        int ho = (int)(q % Ho);
+        long n = q / Ho;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[i] = p.mode == 0 ? -INFINITY : 0.f;
+        int cnt = 0;
+        for (int r = 0; r < p.R; ++r) {
+            int hi = ho * p.stride - p.pad + r;
+            if ((unsigned)hi >= (unsigned)p.H) continue;
+            for (int s = 0; s < p.S; ++s) {
+                int wi = wo * p.stride - p.pad + s;
+                if ((unsigned)wi >= (unsigned)p.W) continue;
+                float f[VEC];
+                VecIO<T>::load(in + ((n * p.H + hi) * p.W + wi) * p.in_pix_stride + ch * VEC, f);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = p.mode == 0 ? fmaxf(acc[j], f[j]) : acc[j] + f[j];
+                ++cnt;
+            }
+        }
+        if (p.mode == 1) {
+            float inv = 1.f / (float)(cnt > 0 ? cnt : 1);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) acc[j] *= inv;
+        }
+        VecIO<T>::store(out + pix * p.out_pix_stride + ch * VEC, acc);
+}
+template <typename T>
+__global__ __launch_bounds__(NT) void pool_kernel(PoolArgs a, BlpArgs blp) {
+    tile_loop(blp, [&](TileIdx t) { pool_tile<T>(a, t); });
+}
+
+// ---- elementwise ---------------------------------------------------------------------------
+// item = (row, 16-byte chunk); tile = 1024 items (4 per thread, strided by 256 for coalescing).
+constexpr int ELT_PER = 4;
+struct EltwiseArgs { gp_eltwise_params p; long items; };
+template <typename T>
+__device__ __forceinline__ void eltwise_tile(const EltwiseArgs &a, TileIdx t) {
+    const gp_eltwise_params &p = a.p;
+    const long items = a.items;
+    constexpr int VEC = VecIO<T>::VEC;
+    const int chunks = p.cols / VEC;
+    
+#pragma unroll
+        for (int u = 0; u < ELT_PER; ++u) {
+            long item = ((long)t.x * ELT_PER + u) * NT + threadIdx.x;
+            if (item >= items) continue;
+            int ch = (int)(item % chunks);
+            long row = item / chunks;
+            float a[VEC];
+            VecIO<T>::load((const T *)p.a + row * p.a_stride + ch * VEC, a);
+            if (p.b) {
+                float b[VEC];
+                VecIO<T>::load((const T *)p.b + row * p.b_stride + ch * VEC, b);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) a[j] += b[j];
+            }
+            if (p.scale) {
+                float sc[VEC];
+                VecIO<T>::load((const T *)p.scale + ch * VEC, sc);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) a[j] *= sc[j];
+            }
+            if (p.shift) {
+                float sh[VEC];
+                VecIO<T>::load((const T *)p.shift + ch * VEC, sh);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) a[j] += sh[j];
+            }
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) a[j] = act_f(a[j], p.act);
+            VecIO<T>::store((T *)p.out + row * p.out_stride + ch * VEC, a);
+        }
+}
+template <typename T>
+__global__ __launch_bounds__(NT) void eltwise_kernel(EltwiseArgs a, BlpArgs blp) {
+    tile_loop(blp, [&](TileIdx t) { eltwise_tile<T>(a, t); });
+}
+
+// ---- softmax -------------------------------------------------------------------------------
+// one wavefront per row, 4 rows per tile; lane i reads elements i, i+64, ...
+template <typename T>
+__device__ __forceinline__ void softmax_tile(const gp_softmax_params &p, TileIdx t) {
+    
+        long row = (long)t.x * 4 + (threadIdx.x >> 6);
+        if (row >= p.rows) return;
+        const int lane = threadIdx.x & 63;
+        const T *x = (const T *)p.x + row * p.cols;
+        T *o = (T *)p.out + row * p.cols;
+        float mx = -INFINITY;
+        for (int c = lane; c < p.cols; c += 64) mx = fmaxf(mx, VecIO<T>::ld1(x + c) * p.scale);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int c = lane; c < p.cols; c += 64) sum += __expf(VecIO<T>::ld1(x + c) * p.scale - mx);
+        sum = wave_sum(sum);
+        float inv = 1.f / sum;
+        for (int c = lane; c < p.cols; c += 64) VecIO<T>::st1(o + c, __expf(VecIO<T>::ld1(x + c) * p.scale - mx) * inv);
+}
+template <typename T>
+__global__ __launch_bounds__(NT) void softmax_kernel(gp_softmax_params p, BlpArgs blp) {
+    tile_loop(blp, [&](TileIdx t) { softmax_tile<T>(p, t); });
+}
+
+// ---- layer norm ----------------------------------------------------------------------------
+// one wavefront per row, 4 rows per tile; the row (plus residual) is kept in registers
+// (up to MAXC 16-byte chunks per lane), so HBM sees one read and one write per element.
+template <typename T, int MAXC>
+__device__ __forceinline__ void layernorm_tile(const gp_layernorm_params &p, TileIdx t) {
+    constexpr int VEC = VecIO<T>::VEC;
+    const int chunks = p.cols / VEC;
+    
+        long row = (long)t.x * 4 + (threadIdx.x >> 6);
+        if (row >= p.rows) return;
+        const int lane = threadIdx.x & 63;
+        const T *x = (const T *)p.x + row * p.cols;
+        const T *r = p.residual ? (const T *)p.residual + row * p.cols : nullptr;
+        float v[MAXC][VEC];
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            int ch = lane + i * 64;
+            if (ch < chunks) {
+                VecIO<T>::load(x + ch * VEC, v[i]);
+                if (r) {
+                    float rr[VEC];
+                    VecIO<T>::load(r + ch * VEC, rr);
+#pragma unroll
+                    for (int j = 0; j < VEC; ++j) v[i][j] += rr[j];
+                }
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) sum += v[i][j];
+            }
+        }
+        float mean = wave_sum(sum) / (float)p.cols;
+        float sq = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            int ch = lane + i * 64;
+            if (ch < chunks) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) { float d = v[i][j] - mean; sq += d * d; }
+            }
+        }
+        float inv = rsqrtf(wave_sum(sq) / (float)p.cols + p.eps);
+        T *o = (T *)p.out + row * p.cols;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            int ch = lane + i * 64;
+            if (ch < chunks) {
+                float ga[VEC], be[VEC], y[VEC];
+                VecIO<T>::load((const T *)p.gamma + ch * VEC, ga);
+                VecIO<T>::load((const T *)p.beta + ch * VEC, be);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) y[j] = (v[i][j] - mean) * inv * ga[j] + be[j];
+                VecIO<T>::store(o + ch * VEC, y);
+            }
+        }
+}
+template <typename T, int MAXC>
+__global__ __launch_bounds__(NT) void layernorm_kernel(gp_layernorm_params p, BlpArgs blp) {
+    tile_loop(blp, [&](TileIdx t) { layernorm_tile<T, MAXC>(p, t); });
+}
+
+// ---- embedding -----------------------------------------------------------------------------
+// one wavefront per token, 4 tokens per tile.
+template <typename T>
+__device__ __forceinline__ void embed_tile(const gp_embed_params &p, TileIdx t) {
+    constexpr int VEC = VecIO<T>::VEC;
+    const int chunks = p.hidden / VEC;
+    
+        long tok = (long)t.x * 4 + (threadIdx.x >> 6);
+        if (tok >= p.tokens) return;
+        const int lane = threadIdx.x & 63;
+        long id = p.ids[tok];
+        if (id < 0) id = 0;
+        if (id >= p.vocab) id = p.vocab - 1;  // clamp like relay take(mode="clip")
+        const T *e = (const T *)p.tok + id * p.hidden;
+        const T *ps = (const T *)p.pos + (tok % p.seq) * p.hidden;
+        T *o = (T *)p.out + tok * p.hidden;
+        for (int ch = lane; ch < chunks; ch += 64) {
+            float a[VEC], b[VEC];
+            VecIO<T>::load(e + ch * VEC, a);
+            VecIO<T>::load(ps + ch * VEC, b);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) a[j] += b[j];
+            if (p.seg) {
+                VecIO<T>::load((const T *)p.seg + ch * VEC, b);
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) a[j] += b[j];
+            }
+            VecIO<T>::store(o + ch * VEC, a);
+        }
+}
+template <typename T>
+__global__ __launch_bounds__(NT) void embed_kernel(gp_embed_params p, BlpArgs blp) {
+    tile_loop(blp, [&](TileIdx t) { embed_tile<T>(p, t); });
+}
+
+
+// ---- copy ----------------------------------------------------------------------------------
+// The reference's "nop" kernel (a device-to-device copy, src/executor.cpp:139-146) as a tiled
+// operator: tile = 4096 bytes x 4 per thread.
+struct CopyArgs { const void *src; void *dst; long bytes; };
+constexpr int COPY_TILE_BYTES = NT * 16 * 4;
+__device__ __forceinline__ void copy_tile(const CopyArgs &a, TileIdx t) {
+    const char *s = (const char *)a.src;
+    char *d = (char *)a.dst;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        long off = ((long)t.x * 4 + u) * NT * 16 + (long)threadIdx.x * 16;
+        if (off + 16 <= a.bytes) *(u32x4 *)(d + off) = *(const u32x4 *)(s + off);
+        else for (long i = off; i < a.bytes; ++i) d[i] = s[i];
+    }
+}
+template <int UNUSED = 0>
+__global__ __launch_bounds__(NT) void copy_kernel(CopyArgs a, BlpArgs blp) {
+    tile_loop(blp, [&](TileIdx t) { copy_tile(a, t); });
+}
+
+}  // namespace gp

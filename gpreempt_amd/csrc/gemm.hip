@@ -14,6 +14,7 @@
 // (n, ho, wo) and column k is (r, s, ci) of an NHWC input, zero-filled outside the image.
 #include "gemm_tile.hpp"
 #include "gemm_pipe.hpp"
+#include "plans.hpp"
 
 namespace gp {
 
@@ -28,8 +29,7 @@ template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool CONV, bool 
 using TK = TileKernel<T, BM, BN, BK, WGM, WGN, CONV, B_KN>;
 
 template <class K>
-static int launch_mat(const MatArgs &g, int batch, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
-    int sx = (g.N + K::bn - 1) / K::bn, sy = (g.M + K::bm - 1) / K::bm;
+static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     BlpArgs blp;
     int grid = 0;
     auto kern = mat_kernel<K>;
@@ -40,78 +40,102 @@ static int launch_mat(const MatArgs &g, int batch, const gp_preempt_ctx *ctx, gp
             once = true;
         }
     }
-    int rc = plan_launch(kern, K::NT, K::LDS_BYTES, sx, sy, batch, ctx, &blp, &grid, info);
+    int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info);
     if (rc) return rc;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(K::NT), K::LDS_BYTES, native(s), g, blp);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(K::NT), K::LDS_BYTES, native(s), pl.g, blp);
     GP_HIP(hipGetLastError());
     return GP_SUCC;
 }
 
-enum { VAR_AUTO = 0, VAR_STAGED = 1, VAR_PIPE = 2, VAR_PIPE_SPLITK = 3 };
+template <typename T, int TILE, int STAGES, bool SPLITK>
+static int pipe_case(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    if (pl.conv) return launch_mat<PipeKernel<T, TILE, TILE, STAGES, true, SPLITK>>(pl, ctx, s, info);
+    return launch_mat<PipeKernel<T, TILE, TILE, STAGES, false, SPLITK>>(pl, ctx, s, info);
+}
 
-template <typename T, bool CONV, bool B_KN>
-static int dispatch_staged(const MatArgs &g, int batch, int tm, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
-    constexpr int BK = sizeof(T) == 4 ? 16 : 32;
-    if (tm == 128) return launch_mat<TK<T, 128, 128, BK, 2, 2, CONV, B_KN>>(g, batch, ctx, s, info);
-    if (tm == 64) return launch_mat<TK<T, 64, 64, BK, 2, 2, CONV, B_KN>>(g, batch, ctx, s, info);
-    set_error("unsupported tile %d for the register-staged kernel (128, 64)", tm);
+template <typename T>
+static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
+    switch (pl.body) {
+        case MB_PIPE128: return pipe_case<T, 128, 3, false>(pl, ctx, s, info);
+        case MB_PIPE64: return pipe_case<T, 64, 4, false>(pl, ctx, s, info);
+        case MB_PIPE64_SK: return pipe_case<T, 64, 4, true>(pl, ctx, s, info);
+        case MB_PIPE32_SK: return pipe_case<T, 32, 4, true>(pl, ctx, s, info);
+        case MB_STAGED128:
+            if (pl.conv) return launch_mat<TK<T, 128, 128, SBK, 2, 2, true, false>>(pl, ctx, s, info);
+            return pl.b_kn ? launch_mat<TK<T, 128, 128, SBK, 2, 2, false, true>>(pl, ctx, s, info)
+                           : launch_mat<TK<T, 128, 128, SBK, 2, 2, false, false>>(pl, ctx, s, info);
+        case MB_STAGED64:
+            if (pl.conv) return launch_mat<TK<T, 64, 64, SBK, 2, 2, true, false>>(pl, ctx, s, info);
+            return pl.b_kn ? launch_mat<TK<T, 64, 64, SBK, 2, 2, false, true>>(pl, ctx, s, info)
+                           : launch_mat<TK<T, 64, 64, SBK, 2, 2, false, false>>(pl, ctx, s, info);
+    }
+    set_error("unknown matrix kernel body %d", pl.body);
+    return GP_FAIL;
+}
+
+int launch_mat_plan(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    switch (pl.dtype) {
+        case GP_F32: return launch_typed<float>(pl, ctx, s, info);
+        case GP_F16: return launch_typed<_Float16>(pl, ctx, s, info);
+        case GP_BF16: return launch_typed<__bf16>(pl, ctx, s, info);
+    }
+    set_error("unsupported dtype %d for matrix kernels", pl.dtype);
     return GP_OUTOFRANGE;
 }
 
-template <typename T, bool CONV>
-static int dispatch_pipe(const MatArgs &g, int batch, int tm, bool splitk, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
-    if (!splitk) {
-        if (tm == 128) return launch_mat<PipeKernel<T, 128, 128, 3, CONV, false>>(g, batch, ctx, s, info);
-        if (tm == 64) return launch_mat<PipeKernel<T, 64, 64, 4, CONV, false>>(g, batch, ctx, s, info);
-    } else {
-        if (tm == 64) return launch_mat<PipeKernel<T, 64, 64, 4, CONV, true>>(g, batch, ctx, s, info);
-        if (tm == 32) return launch_mat<PipeKernel<T, 32, 32, 4, CONV, true>>(g, batch, ctx, s, info);
+static size_t body_lds_bytes(int body, int dtype) {
+    const size_t es = dtype == GP_F32 ? 4 : 2;
+    switch (body) {
+        case MB_PIPE128: return 3 * (128 + 128) * 128;
+        case MB_PIPE64: return 4 * (64 + 64) * 128;
+        case MB_PIPE64_SK: return 4 * (64 + 64) * 128;   // equals the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4)
+        case MB_PIPE32_SK: return 4 * (32 + 32) * 128;
+        case MB_STAGED128: return (128 + 128) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
+        case MB_STAGED64: return (64 + 64) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
     }
-    set_error("unsupported tile %d for the pipelined kernel%s", tm, splitk ? " with split K (64, 32)" : " (128, 64)");
-    return GP_OUTOFRANGE;
+    return 0;
 }
 
 // Kernel and tile choice.  B stored K x N needs the transposing, register-staged kernel.
 // Otherwise the pipelined kernel is used with the largest tile that still gives every compute
 // unit work; problems too small for that split K across the waves of a workgroup so that the
 // serial K loop shrinks instead.
-template <typename T, bool CONV>
-static int dispatch_any(bool b_kn, const MatArgs &g, int batch, int tile, int variant, const gp_preempt_ctx *ctx,
-                        gp_stream s, gp_launch_info *info) {
-    auto tiles = [&](int t) { return (long)((g.M + t - 1) / t) * ((g.N + t - 1) / t) * batch; };
+static int choose_body(MatPlan *pl, int tile, int variant) {
+    const MatArgs &g = pl->g;
+    auto tiles = [&](int t) { return (long)((g.M + t - 1) / t) * ((g.N + t - 1) / t) * pl->batch; };
     const long cus = device_cus();
-    if (b_kn || variant == VAR_STAGED) {
+    int body = -1;
+    if (pl->b_kn || variant == GP_MAT_STAGED) {
         int tm = tile ? tile : (tiles(128) >= cus ? 128 : 64);
-        if (CONV) return dispatch_staged<T, CONV, false>(g, batch, tm, ctx, s, info);
-        return b_kn ? dispatch_staged<T, false, true>(g, batch, tm, ctx, s, info) : dispatch_staged<T, false, false>(g, batch, tm, ctx, s, info);
+        body = tm == 128 ? MB_STAGED128 : tm == 64 ? MB_STAGED64 : -1;
+    } else if (variant == GP_MAT_PIPE) {
+        int tm = tile ? tile : (tiles(128) >= cus ? 128 : 64);
+        body = tm == 128 ? MB_PIPE128 : tm == 64 ? MB_PIPE64 : -1;
+    } else if (variant == GP_MAT_PIPE_SPLITK) {
+        int tm = tile ? tile : (tiles(64) >= cus / 2 ? 64 : 32);
+        body = tm == 64 ? MB_PIPE64_SK : tm == 32 ? MB_PIPE32_SK : -1;
+    } else if (variant == GP_MAT_AUTO) {
+        if (tile == 128 || (tile == 0 && tiles(128) >= cus)) body = MB_PIPE128;
+        else if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) body = MB_PIPE64;
+        else if (tile == 0 && tiles(64) >= cus / 2) body = MB_PIPE64_SK;
+        else if (tile == 0 || tile == 32) body = MB_PIPE32_SK;
     }
-    if (variant == VAR_PIPE) return dispatch_pipe<T, CONV>(g, batch, tile ? tile : (tiles(128) >= cus ? 128 : 64), false, ctx, s, info);
-    if (variant == VAR_PIPE_SPLITK) return dispatch_pipe<T, CONV>(g, batch, tile ? tile : (tiles(64) >= cus / 2 ? 64 : 32), true, ctx, s, info);
-    if (tile == 128 || (tile == 0 && tiles(128) >= cus)) return dispatch_pipe<T, CONV>(g, batch, 128, false, ctx, s, info);
-    if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) return dispatch_pipe<T, CONV>(g, batch, 64, false, ctx, s, info);
-    if (tile == 0 && tiles(64) >= cus / 2) return dispatch_pipe<T, CONV>(g, batch, 64, true, ctx, s, info);
-    return dispatch_pipe<T, CONV>(g, batch, 32, true, ctx, s, info);
-}
-
-template <bool CONV>
-static int dispatch_dtype(int dtype, bool b_kn, const MatArgs &g, int batch, int tile, int variant,
-                          const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
-    switch (dtype) {
-        case GP_F32: return dispatch_any<float, CONV>(b_kn, g, batch, tile, variant, ctx, s, info);
-        case GP_F16: return dispatch_any<_Float16, CONV>(b_kn, g, batch, tile, variant, ctx, s, info);
-        case GP_BF16: return dispatch_any<__bf16, CONV>(b_kn, g, batch, tile, variant, ctx, s, info);
+    if (body < 0) {
+        set_error("no matrix kernel for tile %d with variant %d (tiles: 128, 64; 64, 32 with split K)", tile, variant);
+        return GP_OUTOFRANGE;
     }
-    set_error("unsupported dtype %d for matrix kernels", dtype);
-    return GP_OUTOFRANGE;
+    const int t = (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
+    pl->body = body;
+    pl->sx = (g.N + t - 1) / t;
+    pl->sy = (g.M + t - 1) / t;
+    pl->lds_bytes = body_lds_bytes(body, pl->dtype);
+    return GP_SUCC;
 }
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
-}  // namespace gp
-
-using namespace gp;
-
-extern "C" int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+int plan_gemm(const gp_gemm_params *p, MatPlan *out) {
     GP_REQUIRE(p != nullptr, "null gemm params");
     GP_REQUIRE(p->dtype == GP_F32 || p->dtype == GP_F16 || p->dtype == GP_BF16, "gemm dtype %d", p->dtype);
     const int vec = p->dtype == GP_F32 ? 4 : 8;
@@ -127,7 +151,10 @@ extern "C" int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx
             GP_REQUIRE(p->stride_a_outer % vec == 0 && p->stride_b_outer % vec == 0, "gemm: outer batch strides must be multiples of %d elements", vec);
     }
     GP_REQUIRE(p->lda >= p->K && p->ldc >= p->N && p->ldb >= (p->b_is_nk ? p->K : p->N), "gemm: leading dimension smaller than the row");
-    MatArgs g{};
+    GP_REQUIRE(p->tile_m == p->tile_n, "gemm: square tiles only");
+    MatPlan &pl = *out;
+    pl = MatPlan{};
+    MatArgs &g = pl.g;
     g.M = p->M; g.N = p->N; g.K = p->K;
     g.A = p->A; g.lda = p->lda; g.stride_a = p->stride_a; g.stride_a_outer = p->stride_a_outer;
     g.B = p->B; g.ldb = p->ldb; g.stride_b = p->stride_b; g.stride_b_outer = p->stride_b_outer;
@@ -135,11 +162,11 @@ extern "C" int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx
     g.bias = p->bias; g.residual = p->residual; g.ldr = p->ldc;
     g.alpha = p->alpha == 0.f ? 1.f : p->alpha;
     g.act = p->act; g.batch_inner = batch > 1 ? p->batch_inner : 0;
-    GP_REQUIRE(p->tile_m == p->tile_n, "gemm: square tiles only");
-    return dispatch_dtype<false>(p->dtype, !p->b_is_nk, g, batch, p->tile_m, p->variant, ctx, s, info);
+    pl.dtype = p->dtype; pl.conv = 0; pl.b_kn = !p->b_is_nk; pl.batch = batch;
+    return choose_body(&pl, p->tile_m, p->variant);
 }
 
-extern "C" int gp_launch_conv2d(const gp_conv_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+int plan_conv2d(const gp_conv_params *p, MatPlan *out) {
     GP_REQUIRE(p != nullptr, "null conv params");
     GP_REQUIRE(p->dtype == GP_F32 || p->dtype == GP_F16 || p->dtype == GP_BF16, "conv dtype %d", p->dtype);
     const int vec = p->dtype == GP_F32 ? 4 : 8;
@@ -154,16 +181,35 @@ extern "C" int gp_launch_conv2d(const gp_conv_params *p, const gp_preempt_ctx *c
     GP_REQUIRE(Ho > 0 && Wo > 0, "conv: empty output");
     long M = (long)p->N * Ho * Wo;
     GP_REQUIRE(M < (1L << 31), "conv: too many output pixels");
-    MatArgs g{};
+    GP_REQUIRE(!p->residual || p->res_pix_stride >= p->Cout, "conv: residual pixel stride");
+    GP_REQUIRE(p->tile_m == p->tile_n, "conv: square tiles only");
+    MatPlan &pl = *out;
+    pl = MatPlan{};
+    MatArgs &g = pl.g;
     g.M = (int)M; g.N = p->Cout; g.K = p->R * p->S * p->Cin;
     g.A = p->in; g.lda = p->in_pix_stride;
     g.B = p->weight; g.ldb = g.K;
     g.C = p->out; g.ldc = p->out_pix_stride;
     g.bias = p->bias; g.residual = p->residual; g.ldr = p->residual ? p->res_pix_stride : 0;
-    GP_REQUIRE(!p->residual || p->res_pix_stride >= p->Cout, "conv: residual pixel stride");
     g.alpha = 1.f; g.act = p->act; g.batch_inner = 0;
     g.H = p->H; g.W = p->W; g.Cin = p->Cin; g.S = p->S; g.Ho = Ho; g.Wo = Wo;
     g.sh = p->stride_h; g.sw = p->stride_w; g.ph = p->pad_h; g.pw = p->pad_w;
-    GP_REQUIRE(p->tile_m == p->tile_n, "conv: square tiles only");
-    return dispatch_dtype<true>(p->dtype, false, g, 1, p->tile_m, p->variant, ctx, s, info);
+    pl.dtype = p->dtype; pl.conv = 1; pl.b_kn = 0; pl.batch = 1;
+    return choose_body(&pl, p->tile_m, p->variant);
+}
+
+}  // namespace gp
+
+using namespace gp;
+
+extern "C" int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    MatPlan pl;
+    int rc = plan_gemm(p, &pl);
+    return rc ? rc : launch_mat_plan(pl, ctx, s, info);
+}
+
+extern "C" int gp_launch_conv2d(const gp_conv_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    MatPlan pl;
+    int rc = plan_conv2d(p, &pl);
+    return rc ? rc : launch_mat_plan(pl, ctx, s, info);
 }

@@ -21,7 +21,8 @@
 
 namespace gp {
 
-__device__ __attribute__((aligned(64))) unsigned int g_zero_page[16] = {0};
+// one copy per translation unit; only ever read
+static __device__ __attribute__((aligned(64))) unsigned int g_zero_page[16] = {0};
 
 // Direct global -> LDS load of 16 bytes per lane: lane i's data lands at lds_byte + 16*i.
 // `lds_byte` must be wave-uniform (it travels in M0).  Written as inline assembly because the

@@ -1,0 +1,48 @@
+// Launch plans: the validated, resolved form of an operator call (argument block, tile grid,
+// kernel body).  The stand-alone launchers (gp_launch_*) launch a plan at once; the whole-model
+// program (program.hip) stores plans as layer descriptors of one persistent kernel.
+#pragma once
+#include "elementwise_bodies.hpp"
+#include "mma.hpp"
+
+namespace gp {
+
+enum MatBody { MB_PIPE128 = 0, MB_PIPE64 = 1, MB_PIPE64_SK = 2, MB_PIPE32_SK = 3, MB_STAGED128 = 4, MB_STAGED64 = 5 };
+
+struct MatPlan {
+    MatArgs g;
+    int dtype, body, conv, b_kn, batch;
+    int sx, sy;        // tile grid (x over N, y over M, z = batch)
+    size_t lds_bytes;
+};
+
+enum EltOp { OP_MAT = 0, OP_LAYOUT, OP_POOL, OP_ELTWISE, OP_SOFTMAX, OP_LAYERNORM, OP_EMBED, OP_COPY };
+
+struct EltPlan {
+    int op, dtype, sub;  // sub: layout -> (dtype_in * 4 + dtype_out); layernorm -> chunks kept per lane (2, 8, 16)
+    int sx, sy;
+    union {
+        LayoutArgs layout;
+        PoolArgs pool;
+        EltwiseArgs elt;
+        gp_softmax_params softmax;
+        gp_layernorm_params ln;
+        gp_embed_params embed;
+        CopyArgs copy;
+    } u;
+};
+
+int plan_gemm(const gp_gemm_params *p, MatPlan *out);
+int plan_conv2d(const gp_conv_params *p, MatPlan *out);
+int launch_mat_plan(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+int plan_layout(const gp_layout_params *p, EltPlan *out);
+int plan_pool2d(const gp_pool_params *p, EltPlan *out);
+int plan_eltwise(const gp_eltwise_params *p, EltPlan *out);
+int plan_softmax(const gp_softmax_params *p, EltPlan *out);
+int plan_layernorm(const gp_layernorm_params *p, EltPlan *out);
+int plan_embed(const gp_embed_params *p, EltPlan *out);
+int plan_copy(const void *src, void *dst, long bytes, EltPlan *out);
+int launch_elt_plan(const EltPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
+}  // namespace gp

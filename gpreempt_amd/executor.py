@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "libgpreempt_exec.so")
 vp = C.c_void_p
 
 SYMBOLS = """gpx_create gpx_destroy gpx_init gpx_set_input gpx_get_output gpx_get_data_size gpx_execute
-gpx_launch_kernel gpx_get_kernel_num gpx_capture_graph gpx_clear gpx_set_flag gpx_set_running gpx_resume
+gpx_launch_kernel gpx_get_kernel_num gpx_capture_graph gpx_uses_program gpx_clear gpx_set_flag gpx_set_running gpx_resume
 gpx_get_stop_point gpx_last_stop_index gpx_inject_preempt gpx_read_counters gpx_reset_counters gpx_storage_num gpx_storage_info
 gpx_kernel_info gpx_read_storage gpx_run_scenario gpx_preempt_probe gpx_parse_params""".split()
 
@@ -140,6 +140,9 @@ class Executor:
 
     def capture_graph(self, stream):
         _chk(lib().gpx_capture_graph(self.h, stream.h), "capture_graph")
+
+    def uses_program(self):
+        return bool(lib().gpx_uses_program(self.h))
 
     # -- block-level preemption
     def set_flag(self, flag):

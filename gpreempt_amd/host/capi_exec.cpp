@@ -39,6 +39,7 @@ int gpx_capture_graph(gpx_executor e, gp_stream s) {
     H(e)->ex->capture_graph(s);
     return H(e)->ex->uses_graph() ? Status::Succ : Status::Fail;  // capture_graph itself returns void
 }
+int gpx_uses_program(gpx_executor e) { return H(e)->ex->uses_program() ? 1 : 0; }
 void gpx_clear(gpx_executor e) { H(e)->ex->clear(); }
 
 int gpx_set_flag(gpx_executor e, void *dp) { if (!H(e)->blp) return Status::Fail; H(e)->blp->dpStop = dp; return Status::Succ; }

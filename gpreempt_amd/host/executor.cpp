@@ -71,6 +71,7 @@ Status Executor::load_param(std::string model_path) { return model->load_param((
 
 // reference executor.cpp:119-134
 Status Executor::execute(GPUstream stream) {
+    if (use_program) return model->launch_program(stream, true);
     if (use_cuda_graph) {
         CUDA_RETURN_STATUS(gp_graph_launch(graph_exec, stream));
         return Status::Succ;
@@ -85,9 +86,20 @@ Status Executor::launch_kernel(size_t kernel_offset, GPUstream stream) { return 
 size_t Executor::get_kernel_num() const { return model ? model->get_kernel_num() : 0; }
 
 // reference executor.cpp:176-196.  On failure the executor stays in launch-by-launch mode.
+static bool want_hipgraph() {
+    const char *e = std::getenv("GPREEMPT_USE_HIPGRAPH");
+    return e && *e && *e != '0';
+}
+
 void Executor::capture_graph(GPUstream stream) {
     if (graph_exec) { gp_graph_destroy(graph_exec); graph_exec = nullptr; }
     use_cuda_graph = false;
+    use_program = false;
+    if (!want_hipgraph()) {
+        if (model && model->build_program() == Status::Succ) { use_cuda_graph = true; use_program = true; }
+        else std::fprintf(stderr, "capture_graph: no program, staying with per-kernel launches\n");
+        return;
+    }
     if (gp_graph_begin(stream) != 0) return;
     bool ok = true;
     for (size_t i = 0; i < get_kernel_num() && ok; i++) ok = launch_kernel(i, stream) == Status::Succ;
@@ -146,6 +158,7 @@ Status BLPExecutor::launch_kernel(size_t kernel_offset, GPUstream stream) {
 // reference executor.cpp:211-232: zero every tile counter, then launch (or replay the graph).
 // The counters are cleared by a fill kernel outside the captured graph.
 Status BLPExecutor::execute(GPUstream stream) {
+    if (use_program) return model->launch_program(stream, true, inject_kernel, inject_claim);
     RETURN_STATUS(reset_counters(stream));
     if (use_cuda_graph) {
         CUDA_RETURN_STATUS(gp_graph_launch(graph_exec, stream));
@@ -178,6 +191,8 @@ Status BLPExecutor::resume(GPUstream stream) {
     if (!running) return Status::Succ;
     RETURN_STATUS(getStopPoint(stream));
     if (stopIndex == -1) return Status::Succ;
+    // the program continues from its own per-layer counters; per-kernel mode relaunches one by one
+    if (use_program) return model->launch_program(stream, false, inject_kernel, inject_claim);
     for (size_t i = (size_t)stopIndex; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
     return Status::Succ;
 }
@@ -188,6 +203,12 @@ Status BLPExecutor::reset_counters(GPUstream stream) {
 }
 
 Status BLPExecutor::read_counters(std::vector<int> &out) {
+    if (use_program) {
+        std::vector<int> done;
+        int error = 0;
+        RETURN_STATUS(model->read_program_counters(out, done, error));
+        return error ? Status::Timeout : Status::Succ;
+    }
     out.resize(model->get_kernel_num());
     CUDA_RETURN_STATUS(gp_memcpy_d2h(out.data(), executed, sizeof(int) * out.size()));
     return Status::Succ;

@@ -261,6 +261,7 @@ Status Model::get_global_ptr(const std::string &name, GPUdeviceptr *ptr) {
 }
 
 Status Model::clear() {
+    if (program_) { gp_program_destroy(program_); program_ = nullptr; }
     if (!loaded_) return Status::Succ;
     for (GPUdeviceptr p : storages) CUDA_RETURN_STATUS(gp_free(p));
     storage_infos.clear(); layouts.clear(); kernel_infos.clear(); storages.clear(); storages_idx.clear();
@@ -329,6 +330,68 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
     k.total_blocks = info.total_tiles;
     k.launch_params[0] = (uint32_t)info.grid; k.launch_params[1] = 1; k.launch_params[2] = 1;
     k.launch_params[3] = (uint32_t)info.block; k.launch_params[4] = 1; k.launch_params[5] = 1;
+    return Status::Succ;
+}
+
+Status Model::build_program() {
+    if (program_) return Status::Succ;
+    if (!loaded_) return Status::Fail;
+    int dt = dtype_ == "f32" ? GP_F32 : dtype_ == "f16" ? GP_F16 : GP_BF16;
+    gp_program pr = nullptr;
+    CUDA_RETURN_STATUS(gp_program_create(dt, &pr));
+    for (size_t i = 0; i < kernel_infos.size(); ++i) {
+        KernelInfo &k = kernel_infos[i];
+        int rc = GP_FAIL;
+        switch (k.op) {
+            case OpKind::Nop: rc = gp_program_add_copy(pr, k.args[0], k.args[1], get_storage_size(k.args_index[0])); break;
+            case OpKind::Gemm: rc = gp_program_add_gemm(pr, &k.p.gemm); break;
+            case OpKind::Conv: rc = gp_program_add_conv2d(pr, &k.p.conv); break;
+            case OpKind::Layout: rc = gp_program_add_nchw_to_nhwc(pr, &k.p.layout); break;
+            case OpKind::Pool: rc = gp_program_add_pool2d(pr, &k.p.pool); break;
+            case OpKind::Eltwise: rc = gp_program_add_eltwise(pr, &k.p.eltwise); break;
+            case OpKind::Softmax: rc = gp_program_add_softmax(pr, &k.p.softmax); break;
+            case OpKind::Layernorm: rc = gp_program_add_layernorm(pr, &k.p.layernorm); break;
+            case OpKind::Embed: rc = gp_program_add_embed(pr, &k.p.embed); break;
+        }
+        if (rc != 0) {
+            std::fprintf(stderr, "build_program: kernel %zu (%s): %s\n", i, k.name.c_str(), gp_last_error());
+            gp_program_destroy(pr);
+            return Status::Fail;
+        }
+    }
+    if (gp_program_finalize(pr) != 0) {
+        std::fprintf(stderr, "build_program: %s\n", gp_last_error());
+        gp_program_destroy(pr);
+        return Status::Fail;
+    }
+    program_ = pr;
+    return Status::Succ;
+}
+
+Status Model::launch_program(GPUstream stream, bool reset, int inject_layer, int inject_claim) {
+    if (!program_) return Status::Fail;
+    gp_preempt_ctx ctx{};
+    const gp_preempt_ctx *pc = nullptr;
+    // preemptible when the executor attached its flag and stop index (batchAddParam)
+    if (!kernel_infos.empty() && kernel_infos[0].args_ptr.size() >= 2) {
+        size_t n = kernel_infos[0].args_ptr.size();
+        ctx.flag = (int *)*kernel_infos[0].args_ptr[n - 2];
+        ctx.stop_index = (int *)*kernel_infos[0].args_ptr[n - 1];
+        ctx.kernel_id = inject_layer;
+        ctx.inject_at = inject_layer >= 0 ? inject_claim : -1;
+        pc = &ctx;
+    }
+    gp_launch_info info{};
+    CUDA_RETURN_STATUS(gp_program_launch(program_, pc, reset ? 1 : 0, stream, &info));
+    return Status::Succ;
+}
+
+Status Model::read_program_counters(std::vector<int> &executed, std::vector<int> &done, int &error) {
+    if (!program_) return Status::Fail;
+    executed.assign(kernel_infos.size(), 0);
+    done.assign(kernel_infos.size(), 0);
+    int cursor = 0;
+    CUDA_RETURN_STATUS(gp_program_read_state(program_, executed.data(), done.data(), &cursor, &error));
     return Status::Succ;
 }
 

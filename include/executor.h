@@ -38,17 +38,22 @@ public:
 
     virtual void clear();
     size_t get_kernel_num() const;
+    // Prepares the launch-free submission path: by default the whole model becomes one
+    // persistent device kernel (a "program"); with GPREEMPT_USE_HIPGRAPH=1 in the environment a
+    // HIP graph of the per-kernel launches is captured instead, as the reference does.
     virtual void capture_graph(GPUstream stream);
     virtual ~Executor();
 
     // additions over the reference
     std::shared_ptr<Model> get_model() const { return model; }
     bool uses_graph() const { return use_cuda_graph; }
+    bool uses_program() const { return use_program; }
 
 protected:
     std::shared_ptr<Model> model;
     std::string type;
-    bool use_cuda_graph = false;
+    bool use_cuda_graph = false;  // a launch-free path is active (program or HIP graph)
+    bool use_program = false;     // ... and it is the persistent program
     GPUgraphExec graph_exec = nullptr;
     std::string graph_path;
 };

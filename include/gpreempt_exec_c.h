@@ -26,6 +26,7 @@ int gpx_execute(gpx_executor e, gp_stream s);                        /* Executor
 int gpx_launch_kernel(gpx_executor e, size_t idx, gp_stream s);      /* Executor::launch_kernel */
 size_t gpx_get_kernel_num(gpx_executor e);                           /* Executor::get_kernel_num */
 int gpx_capture_graph(gpx_executor e, gp_stream s);                  /* Executor::capture_graph; 0 when a graph is in use afterwards */
+int gpx_uses_program(gpx_executor e);                                /* 1 when capture_graph built the persistent program */
 void gpx_clear(gpx_executor e);                                      /* Executor::clear */
 
 /* BLPExecutor only (Status::Fail on a BaseExecutor) */

@@ -221,6 +221,38 @@ typedef struct gp_embed_params {
 } gp_embed_params;
 int gp_launch_embed(const gp_embed_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
 
+/* ---- whole-model program -------------------------------------------------------------------
+ * The launch-bound inner loop of the reference (one GPULaunchKernel or graph node per kernel,
+ * src/executor.cpp:119-134,176-196) as ONE persistent kernel: layers are added in execution
+ * order with the same parameter blocks as the stand-alone launchers, each layer depends on the
+ * one before it, and the resident workgroups walk the list claiming tiles.  Preemption and
+ * resume work at tile granularity exactly as for single kernels; because nothing is queued
+ * behind the running kernel, a preempted model leaves the GPU within about one tile.
+ *   ctx->flag / ctx->stop_index  as for the launchers (stop_index receives the LAYER index)
+ *   ctx->executed                ignored: the program owns one counter per layer
+ *   ctx->kernel_id, inject_at    test hook: layer and claim number that raise the flag
+ * reset != 0 starts the model from its first tile (BLPExecutor::execute); reset == 0 continues
+ * from the counters left by a preempted run (BLPExecutor::resume).  A NULL ctx runs the model
+ * non-preemptibly (BaseExecutor). */
+typedef struct gp_program_s *gp_program;
+int gp_program_create(int dtype, gp_program *out);
+int gp_program_destroy(gp_program p);
+int gp_program_add_gemm(gp_program p, const gp_gemm_params *params);
+int gp_program_add_conv2d(gp_program p, const gp_conv_params *params);
+int gp_program_add_nchw_to_nhwc(gp_program p, const gp_layout_params *params);
+int gp_program_add_pool2d(gp_program p, const gp_pool_params *params);
+int gp_program_add_eltwise(gp_program p, const gp_eltwise_params *params);
+int gp_program_add_softmax(gp_program p, const gp_softmax_params *params);
+int gp_program_add_layernorm(gp_program p, const gp_layernorm_params *params);
+int gp_program_add_embed(gp_program p, const gp_embed_params *params);
+int gp_program_add_copy(gp_program p, const void *src, void *dst, size_t bytes); /* the reference's "nop" copy */
+int gp_program_finalize(gp_program p);
+int gp_program_launch(gp_program p, const gp_preempt_ctx *ctx, int reset, gp_stream s, gp_launch_info *info);
+int gp_program_layers(gp_program p, int *n_layers);
+/* Blocking read-back of per-layer claim / completion counters, the resume cursor and the error
+ * word (1 = a dependency wait gave up); any pointer may be NULL. */
+int gp_program_read_state(gp_program p, int *executed, int *done, int *cursor, int *error);
+
 /* ---- gate kernels --------------------------------------------------------------------------
  * Replace gpu_block / gpu_noop (src/block.cu:1-7): one wave spins until *stop != 0.  Unlike the
  * reference the wait is bounded: after spin_limit polls the kernel leaves and stores 1 to

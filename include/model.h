@@ -116,6 +116,15 @@ public:
     // arguments added with batchAddParam.  inject_at is a test hook (-1 = off).
     Status launch(size_t idx, GPUstream stream, int inject_at = -1);
 
+    // Whole-model program: all kernels as one persistent device kernel (the counterpart of the
+    // captured graph of src/executor.cpp:176-196).  build_program() is idempotent.
+    Status build_program();
+    bool has_program() const { return program_ != nullptr; }
+    // reset = true starts from the first tile, false continues from the counters of a stopped run.
+    Status launch_program(GPUstream stream, bool reset, int inject_layer = -1, int inject_claim = -1);
+    // per-layer claim counters of the program (blocking)
+    Status read_program_counters(std::vector<int> &executed, std::vector<int> &done, int &error);
+
     const std::string &workload() const { return workload_; }
     const std::string &dtype() const { return dtype_; }
     double total_flops() const;
@@ -125,6 +134,7 @@ public:
 
 private:
     bool loaded_ = false;
+    gp_program program_ = nullptr;
     std::string workload_, dtype_;
     std::vector<StorageInfo> storage_infos;
     std::vector<ParamLayout> layouts;

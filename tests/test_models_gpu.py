@@ -122,8 +122,9 @@ def test_executor_error_paths(gp, ex_mod, tmp_path):
 
 # ---- preempt-then-resume on whole models ----------------------------------------------------
 
-def _blp_roundtrip(gp, ex_mod, tmp_path, workload, x_raw, injections, graph=False):
+def _blp_roundtrip(gp, ex_mod, tmp_path, workload, x_raw, injections, graph=False, hipgraph=False):
     root = str(tmp_path)
+    os.environ["GPREEMPT_USE_HIPGRAPH"] = "1" if hipgraph else "0"
     base = ex_mod.Executor(workload, blp=False, model_root=root)
     base.set_input("data", x_raw)
     base.execute()
@@ -134,6 +135,8 @@ def _blp_roundtrip(gp, ex_mod, tmp_path, workload, x_raw, injections, graph=Fals
     stream = gp.Stream(1)
     if graph:
         ex.capture_graph(stream)
+        assert ex.uses_program() == (not hipgraph)
+    program = graph and not hipgraph
     ex.set_input("data", x_raw, stream)
     # uninterrupted preemptible run: same bits as the non-preemptible executor
     ex.execute(stream)
@@ -145,18 +148,22 @@ def _blp_roundtrip(gp, ex_mod, tmp_path, workload, x_raw, injections, graph=Fals
         kernel = kernel if kernel >= 0 else n + kernel
         flag.set(0)
         ex.inject_preempt(kernel, claim)
-        if graph:
+        if graph and hipgraph:
             ex.capture_graph(stream)  # the injection point is a kernel argument: re-capture
         ex.execute(stream)
         ex.set_running(True)
         stream.sync()
         assert flag.get() == 1, (kernel, claim)
         cnt = ex.counters()
-        assert (cnt[kernel + 1:] == 0).all()  # every later kernel left at its first flag check
+        # Per-kernel launches: every later kernel left at its first flag check.  Inside the
+        # program, workgroups that found a layer's counter exhausted may already hold claims on
+        # the next layers when the flag is seen, but nothing far ahead can have started.
+        slack = 4 if program else 1
+        assert (cnt[kernel + slack:] == 0).all(), (kernel, cnt)
         ex.inject_preempt(-1, -1)
         flag.set(0)  # host clears the flag, then resumes (test-dnn-blp.cpp:41-42)
         ex.resume(stream)
-        assert ex.last_stop_index() in (kernel, kernel + 1), (ex.last_stop_index(), kernel)
+        assert kernel <= ex.last_stop_index() <= kernel + slack, (ex.last_stop_index(), kernel)
         stream.sync()
         assert np.array_equal(ex.get_output("heads", stream), want), (kernel, claim)
         assert ex.stop_point(stream) == -1
@@ -171,9 +178,47 @@ def test_resnet50_preempt_resume_bit_exact(gp, ex_mod, tmp_path):
     _blp_roundtrip(gp, ex_mod, tmp_path, "resnet50", x, [(1, 10), (20, 3), (-3, 0), (5, 0)])
 
 
-def test_resnet50_preempt_resume_bit_exact_with_graph(gp, ex_mod, tmp_path):
+def test_resnet50_preempt_resume_bit_exact_with_hip_graph(gp, ex_mod, tmp_path):
     x = np.random.default_rng(2).normal(0, 1, (1, 3, 224, 224)).astype(np.float32)
-    _blp_roundtrip(gp, ex_mod, tmp_path, "resnet50", x, [(7, 5), (40, 1)], graph=True)
+    _blp_roundtrip(gp, ex_mod, tmp_path, "resnet50", x, [(7, 5), (40, 1)], graph=True, hipgraph=True)
+
+
+@pytest.mark.parametrize("workload,shape,injections", [
+    ("toy@n=3,rows=512,cols=512", (512 * 512,), [(0, 3), (3, 10), (5, 0)]),
+    ("resnet50", (1, 3, 224, 224), [(1, 10), (7, 5), (20, 3), (40, 1), (-3, 0), (-1, 0)]),
+    ("gemm@m=2048,n=2048,k=512,tile=64", (2048, 512), [(0, 64), (0, 300), (0, 700)]),  # 1024 tiles > resident workgroups
+])
+def test_program_preempt_resume_bit_exact(gp, ex_mod, tmp_path, workload, shape, injections):
+    """The whole model as one persistent kernel: stop inside a layer, leave, relaunch."""
+    x = np.random.default_rng(2).normal(0, 1, shape).astype(np.float32)
+    ex = _blp_roundtrip(gp, ex_mod, tmp_path, workload, x, injections, graph=True)
+    assert ex.uses_program()
+
+
+def test_program_bert_and_resnet152_match_per_kernel_path(gp, ex_mod, tmp_path):
+    """Program output == per-kernel output, bit for bit, with and without preemption."""
+    ids = np.random.default_rng(3).integers(0, 30522, 128).astype(np.int64)
+    _blp_roundtrip(gp, ex_mod, tmp_path, "bert", ids, [(0, 3), (2, 17), (57, 0), (-1, 10)], graph=True)
+    x = gp.to_storage(np.random.default_rng(4).normal(0, 1, (8, 3, 224, 224)).astype(np.float32), gp.F16)
+    _blp_roundtrip(gp, ex_mod, tmp_path, "resnet152", x, [(3, 100), (80, 7), (-2, 0)], graph=True)
+
+
+def test_program_non_preemptible_executor(gp, ex_mod, tmp_path):
+    """BaseExecutor (the high-priority tenant) through the program: same bits as launch by launch."""
+    os.environ["GPREEMPT_USE_HIPGRAPH"] = "0"
+    ids = np.random.default_rng(5).integers(0, 30522, 128).astype(np.int64)
+    a = ex_mod.Executor("bert", model_root=str(tmp_path))
+    a.set_input("data", ids)
+    a.execute()
+    want = a.get_output("heads").copy()
+    b = ex_mod.Executor("bert", model_root=str(tmp_path))
+    stream = gp.Stream(0)
+    b.capture_graph(stream)
+    assert b.uses_program()
+    b.set_input("data", ids, stream)
+    for _ in range(3):
+        b.execute(stream)
+        assert np.array_equal(b.get_output("heads", stream), want)
 
 
 def test_bert_preempt_resume_bit_exact(gp, ex_mod, tmp_path):
@@ -181,7 +226,8 @@ def test_bert_preempt_resume_bit_exact(gp, ex_mod, tmp_path):
     _blp_roundtrip(gp, ex_mod, tmp_path, "bert", ids, [(0, 3), (2, 17), (57, 0), (-1, 10)])
 
 
-def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path):
+@pytest.mark.parametrize("program", [False, True])
+def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path, program):
     """src/tests/test-dnn-blp.cpp:36-42 verbatim: execute; set the flag from the host right
     away; sync; clear; resume; sync.  Where the flag lands is up to timing; the result is not."""
     root = str(tmp_path)
@@ -194,6 +240,9 @@ def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path):
     flag = gp.Flag()
     ex.set_flag(flag)
     stream = gp.Stream(1)
+    os.environ["GPREEMPT_USE_HIPGRAPH"] = "0"
+    if program:
+        ex.capture_graph(stream)
     ex.set_input("data", x, stream)
     stream.sync()
     stops = []
