@@ -7,6 +7,7 @@
 // redoing or skipping a tile.
 #pragma once
 #include "common.hpp"
+#include "out_store.hpp"
 
 namespace gp {
 
@@ -27,10 +28,10 @@ template <> struct VecIO<float> {
         f32x4 v;
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = f[i];
-        *(f32x4 *)p = v;
+        st_out128(p, __builtin_bit_cast(out_u32x4, v));
     }
     static __device__ __forceinline__ float ld1(const float *p) { return *p; }
-    static __device__ __forceinline__ void st1(float *p, float v) { *p = v; }
+    static __device__ __forceinline__ void st1(float *p, float v) { st_elem<float>(p, v); }
 };
 template <> struct VecIO<_Float16> {
     static constexpr int VEC = 8;
@@ -43,10 +44,10 @@ template <> struct VecIO<_Float16> {
         f16x8 v;
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = (_Float16)f[i];
-        *(f16x8 *)p = v;
+        st_out128(p, __builtin_bit_cast(out_u32x4, v));
     }
     static __device__ __forceinline__ float ld1(const _Float16 *p) { return (float)*p; }
-    static __device__ __forceinline__ void st1(_Float16 *p, float v) { *p = (_Float16)v; }
+    static __device__ __forceinline__ void st1(_Float16 *p, float v) { st_elem<_Float16>(p, (_Float16)v); }
 };
 template <> struct VecIO<__bf16> {
     static constexpr int VEC = 8;
@@ -59,10 +60,10 @@ template <> struct VecIO<__bf16> {
         bf16x8 v;
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = (__bf16)f[i];
-        *(bf16x8 *)p = v;
+        st_out128(p, __builtin_bit_cast(out_u32x4, v));
     }
     static __device__ __forceinline__ float ld1(const __bf16 *p) { return (float)*p; }
-    static __device__ __forceinline__ void st1(__bf16 *p, float v) { *p = (__bf16)v; }
+    static __device__ __forceinline__ void st1(__bf16 *p, float v) { st_elem<__bf16>(p, (__bf16)v); }
 };
 
 __device__ __forceinline__ float act_f(float v, int act) {
@@ -359,8 +360,8 @@ __device__ __forceinline__ void copy_tile(const CopyArgs &a, TileIdx t) {
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         long off = ((long)t.x * 4 + u) * NT * 16 + (long)threadIdx.x * 16;
-        if (off + 16 <= a.bytes) *(u32x4 *)(d + off) = *(const u32x4 *)(s + off);
-        else for (long i = off; i < a.bytes; ++i) d[i] = s[i];
+        if (off + 16 <= a.bytes) st_out128(d + off, *(const u32x4 *)(s + off));
+        else for (long i = off; i < a.bytes; ++i) st_out8(d + i, (unsigned char)s[i]);
     }
 }
 template <int UNUSED = 0>

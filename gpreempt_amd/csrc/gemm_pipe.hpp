@@ -204,7 +204,7 @@ struct PipeKernel {
             if (n >= g.N || m >= g.M) return;
             float x = a * g.alpha + (bias ? Elem<T>::to_f(bias[n]) : 0.f);
             if (R) x += Elem<T>::to_f(R[(long)m * g.ldr + n]);
-            C[(long)m * g.ldc + n] = Elem<T>::from_f(apply_act(x, g.act));
+            st_elem<T>(&C[(long)m * g.ldc + n], Elem<T>::from_f(apply_act(x, g.act)));
         };
         if (!SPLITK) {
 #pragma unroll

@@ -172,7 +172,7 @@ struct TileKernel {
                     if (m >= g.M) continue;
                     float x = acc[i][j][v] * g.alpha + bv;
                     if (R) x += Elem<T>::to_f(R[(long)m * g.ldr + n]);
-                    C[(long)m * g.ldc + n] = Elem<T>::from_f(apply_act(x, g.act));
+                    st_elem<T>(&C[(long)m * g.ldc + n], Elem<T>::from_f(apply_act(x, g.act)));
                 }
             }
         }

@@ -1,6 +1,7 @@
 // Element types, MFMA wrappers and the argument block shared by the matrix kernels.
 #pragma once
 #include "common.hpp"
+#include "out_store.hpp"
 
 namespace gp {
 

@@ -121,6 +121,14 @@ extern "C" int gp_event_destroy(gp_event e) {
 }
 extern "C" int gp_event_record(gp_event e, gp_stream s) { GP_REQUIRE(e, "null event"); GP_HIP(hipEventRecord(e->e, native(s))); return GP_SUCC; }
 extern "C" int gp_event_sync(gp_event e) { GP_REQUIRE(e, "null event"); GP_HIP(hipEventSynchronize(e->e)); return GP_SUCC; }
+extern "C" int gp_event_query(gp_event e, int *done) {
+    GP_REQUIRE(e && done, "null event");
+    hipError_t r = hipEventQuery(e->e);
+    if (r == hipSuccess) { *done = 1; return GP_SUCC; }
+    if (r == hipErrorNotReady) { *done = 0; return GP_SUCC; }
+    set_error("hipEventQuery: %s", hipGetErrorString(r));
+    return GP_FAIL;
+}
 extern "C" int gp_event_elapsed_ms(gp_event a, gp_event b, float *ms) {
     GP_REQUIRE(a && b && ms, "null event");
     GP_HIP(hipEventElapsedTime(ms, a->e, b->e));

@@ -157,6 +157,7 @@ struct Tenant {
     std::string id, name, model_name;
     int priority = 0;
     bool use_graph = true;
+    std::string launch_mode;  // "program" | "graph" | "launch"; empty = "program" when use_cuda_graph, else "launch"
     int64_t preprocess_us = 0;
     Load load;
     std::unique_ptr<Executor> ex;
@@ -168,6 +169,7 @@ struct Tenant {
     int64_t preemptions = 0, requests = 0;
     int64_t first_ns = 0, last_ns = 0;
     Status error = Status::Succ;
+    gp_event chunk_events[3] = {nullptr, nullptr, nullptr};
 };
 
 void fill_input(Tenant &t) {
@@ -184,7 +186,7 @@ void fill_input(Tenant &t) {
 }
 
 Status init_tenant(Tenant &t, Shared &sh) {
-    const bool preemptible = t.priority > 0 && (sh.policy == "wb" || sh.policy == "wb-async");
+    const bool preemptible = t.priority > 0 && (sh.policy == "wb" || sh.policy == "wb-async" || sh.policy == "wb-chunk");
     if (preemptible) { t.blp = new BLPExecutor(); t.ex.reset(t.blp); }
     else t.ex.reset(new BaseExecutor());
     RETURN_STATUS(t.ex->init(t.model_name));
@@ -198,7 +200,14 @@ Status init_tenant(Tenant &t, Shared &sh) {
         int level = std::min(t.priority, sh.levels - 1);
         t.blp->dpStop = sh.flag_dev[level - 1];
     }
-    if (t.use_graph) t.ex->capture_graph(t.stream);
+    // "wb-chunk" feeds a preemptible tenant's kernels a few at a time, so it never uses a
+    // captured graph or program for that tenant.
+    const bool chunked = t.blp && sh.policy == "wb-chunk";
+    if (!chunked && t.launch_mode != "launch") {
+        setenv("GPREEMPT_USE_HIPGRAPH", t.launch_mode == "graph" ? "1" : "0", 1);
+        t.ex->capture_graph(t.stream);
+    }
+    if (chunked) for (int i = 0; i < 3; ++i) CUDA_RETURN_STATUS(gp_event_create(&t.chunk_events[i]));
     return Status::Succ;
 }
 
@@ -210,6 +219,66 @@ Status drain(GPUstream s) {
         if (idle) return Status::Succ;
         spin_pause();
     }
+}
+
+// "wb-chunk": the best-effort model is submitted launch by launch (Executor::launch_kernel, the
+// reference's own launch loop, src/executor.cpp:222-225) but never more than two chunks of
+// kChunk kernels ahead of the GPU.  A preempted model then has at most 2*kChunk queued kernels
+// to flush (each leaves at its first look at the stop index) instead of the rest of the network,
+// which bounds the drain at tens of microseconds while keeping per-kernel occupancy.
+constexpr int kChunk = 6;
+Status infer_chunked(Tenant &t, Shared &sh, int p) {
+    BLPExecutor *ex = t.blp;
+    const size_t n = ex->get_kernel_num();
+    Status st = ex->reset_counters(t.stream);
+    size_t next = 0;
+    int inflight = 0, head = 0, tail = 0;  // ring of 3 events, at most 2 in flight
+    ex->running = true;
+    sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
+    while (st == Status::Succ && (next < n || inflight > 0)) {
+        if (sh.active_above(p) > 0) {
+            // a higher level wants the GPU: stop feeding, let what is queued leave
+            st = drain(t.stream);
+            if (st != Status::Succ) break;
+            int64_t drained = now_ns();
+            inflight = 0; head = tail;
+            sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
+            int64_t raised = sh.flag_raised_ns[p - 1].load();
+            if (raised > 0 && drained >= raised) {
+                std::lock_guard<std::mutex> g(sh.stats_mu);
+                sh.preempt_latency.add((drained - raised) / 1e3);
+            }
+            while (sh.active_above(p) > 0) spin_pause();
+            sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
+            st = ex->getStopPoint(t.stream);  // re-arms the stop index
+            if (st != Status::Succ) break;
+            int stop = ex->last_stop_index();
+            if (stop >= 0) { next = (size_t)stop; ++t.preemptions; }  // kernels from the stopped one on are submitted again
+            continue;
+        }
+        if (next < n && inflight < 2) {
+            size_t end = std::min(n, next + kChunk);
+            for (size_t i = next; i < end && st == Status::Succ; ++i) st = ex->launch_kernel(i, t.stream);
+            if (st != Status::Succ) break;
+            if (gp_event_record(t.chunk_events[tail], t.stream) != 0) { st = Status::Fail; break; }
+            tail = (tail + 1) % 3;
+            ++inflight;
+            next = end;
+            continue;
+        }
+        int done = 0;
+        if (gp_event_query(t.chunk_events[head], &done) != 0) { st = Status::Fail; break; }
+        if (done) { head = (head + 1) % 3; --inflight; }
+        else spin_pause();
+        if (next >= n && inflight == 0) {
+            // everything was submitted and has left the GPU; a late stop may still have cut it short
+            st = ex->getStopPoint(t.stream);
+            if (st == Status::Succ && ex->last_stop_index() >= 0) { next = (size_t)ex->last_stop_index(); ++t.preemptions; }
+        }
+    }
+    ex->running = false;
+    sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
+    return st;
 }
 
 // One inference under the policy.  Mirrors FooClient::infer of the reference's clients.
@@ -227,7 +296,7 @@ Status infer(Tenant &t, Shared &sh) {
         if (p == 0) sh.active[0].fetch_sub(1);
         return Status::Succ;
     }
-    if (pol == "np" || pol == "lco" || !(pol == "wb" || pol == "wb-async")) {
+    if (pol == "np" || pol == "lco" || !(pol == "wb" || pol == "wb-async" || pol == "wb-chunk")) {
         // baseclient.cpp: every tenant submits on its own stream, nothing is preempted
         int64_t t0 = now_ns();
         RETURN_STATUS(t.ex->execute(t.stream));
@@ -236,20 +305,21 @@ Status infer(Tenant &t, Shared &sh) {
         return Status::Succ;
     }
     // ---- "wb": cooperative block-level preemption ------------------------------------------
-    // 1. announce: raises the flag words of every lower level (blpclient.cpp:185-188)
-    sh.active[p].fetch_add(1, std::memory_order_acq_rel);
-    if (p + 1 < sh.levels) sh.update_flags();
+    // (the request was announced by begin_request(): the flag words of every lower level are up)
     int64_t t0 = now_ns();
-    // 2. "wb": wait until lower-priority work has left the GPU (blpclient.cpp:189); "wb-async"
-    //    submits at once and lets the hardware start workgroups as the others retire.
-    if (pol == "wb") while (sh.on_gpu_below(p) > 0) spin_pause();
+    // "wb" / "wb-chunk": wait until lower-priority work has left the GPU (blpclient.cpp:189);
+    // "wb-async" submits at once and lets the hardware start workgroups as the others retire.
+    if (pol != "wb-async") while (sh.on_gpu_below(p) > 0) spin_pause();
     Status st = Status::Succ;
     if (!t.blp) {
         st = t.ex->execute(t.stream);
         if (st == Status::Succ) st = drain(t.stream);
+    } else if (pol == "wb-chunk") {
+        while (sh.active_above(p) > 0) spin_pause();
+        st = infer_chunked(t, sh, p);
     } else {
-        // 3. preemptible tenant (blpclient.cpp:163-183): run, and after every drain ask whether a
-        //    kernel was stopped; if so wait for the higher levels to finish and resume.
+        // preemptible tenant (blpclient.cpp:163-183): run, and after every drain ask whether a
+        // kernel was stopped; if so wait for the higher levels to finish and resume.
         while (sh.active_above(p) > 0) spin_pause();
         sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
         t.blp->running = true;
@@ -277,11 +347,30 @@ Status infer(Tenant &t, Shared &sh) {
         t.blp->running = false;
         sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
     }
-    // 4. retire: lowers the flag words when this was the last active request of its level
-    sh.active[p].fetch_sub(1, std::memory_order_acq_rel);
-    if (p + 1 < sh.levels) sh.update_flags();
     if (p == 0) sh.hp_busy_ns.fetch_add(now_ns() - t0);
     return st;
+}
+
+static bool preempting_policy(const Shared &sh) { return sh.policy == "wb" || sh.policy == "wb-async" || sh.policy == "wb-chunk"; }
+
+// A request of level p announces itself before it touches the GPU at all (its input copy
+// included): a persistent best-effort kernel leaves no gap for even a small copy kernel, so the
+// flag has to go up first.  This is where the reference posts its pre-preemption hint
+// (src/cuda-clients/gpreemptclient.cpp:203-219).  Raises the flag words of every lower level
+// (blpclient.cpp:185-188); end_request() lowers them when the level has no request left.
+void begin_request(Tenant &t, Shared &sh) {
+    if (!preempting_policy(sh)) return;
+    const int p = std::min(t.priority, sh.levels - 1);
+    if (p + 1 >= sh.levels) return;  // the lowest level preempts nobody
+    sh.active[p].fetch_add(1, std::memory_order_acq_rel);
+    sh.update_flags();
+}
+void end_request(Tenant &t, Shared &sh) {
+    if (!preempting_policy(sh)) return;
+    const int p = std::min(t.priority, sh.levels - 1);
+    if (p + 1 >= sh.levels) return;
+    sh.active[p].fetch_sub(1, std::memory_order_acq_rel);
+    sh.update_flags();
 }
 
 // One request: the six DISB phases (benchmark.cpp:66-135); prepareInput and postprocess are empty
@@ -289,6 +378,8 @@ Status infer(Tenant &t, Shared &sh) {
 Status infer_once(Tenant &t, Shared &sh, double *total_us, double *infer_us) {
     int64_t t0 = now_ns();
     if (t.preprocess_us > 0) std::this_thread::sleep_for(std::chrono::microseconds(t.preprocess_us));
+    begin_request(t, sh);
+    struct Retire { Tenant &t; Shared &sh; ~Retire() { end_request(t, sh); } } retire{t, sh};
     RETURN_STATUS(t.ex->set_input("data", t.input, t.input_size, t.stream));
     CUDA_RETURN_STATUS(gp_stream_sync(t.stream));
     int64_t t1 = now_ns();
@@ -357,6 +448,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         t->model_name = c["model_name"].string();
         t->priority = (int)c["priority"].number(0);
         t->use_graph = c["use_cuda_graph"].boolean(true);
+        t->launch_mode = c["launch_mode"].string(t->use_graph ? "program" : "launch");
         t->preprocess_us = (int64_t)c["preprocess_time"].number(0);
         t->load.type = l["type"].string("continuous");
         t->load.frequency = l["frequency"].number(0);
@@ -451,6 +543,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         t->ex->clear();
         gp_host_free(t->input);
         gp_host_free(t->output);
+        for (gp_event e : t->chunk_events) if (e) gp_event_destroy(e);
         gp_stream_destroy(t->stream);
     }
     tenants.clear();

@@ -58,6 +58,7 @@ int gp_event_create(gp_event *out);
 int gp_event_destroy(gp_event e);
 int gp_event_record(gp_event e, gp_stream s);
 int gp_event_sync(gp_event e);
+int gp_event_query(gp_event e, int *done); /* *done = 1 when the event has completed (hipEventQuery) */
 int gp_event_elapsed_ms(gp_event start, gp_event stop, float *ms);
 
 /* ---- memory ------------------------------------------------------------------------------
@@ -249,8 +250,9 @@ int gp_program_add_copy(gp_program p, const void *src, void *dst, size_t bytes);
 int gp_program_finalize(gp_program p);
 int gp_program_launch(gp_program p, const gp_preempt_ctx *ctx, int reset, gp_stream s, gp_launch_info *info);
 int gp_program_layers(gp_program p, int *n_layers);
-/* Blocking read-back of per-layer claim / completion counters, the resume cursor and the error
- * word (1 = a dependency wait gave up); any pointer may be NULL. */
+/* Blocking read-back of per-layer claim / completion counters, the number of tiles handed out
+ * so far over all layers (*cursor) and the error word (1 = a dependency wait gave up); any
+ * pointer may be NULL. */
 int gp_program_read_state(gp_program p, int *executed, int *done, int *cursor, int *error);
 
 /* ---- gate kernels --------------------------------------------------------------------------
