@@ -28,15 +28,19 @@ HBM_PEAK_GBS = 8000.0
 
 
 def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
+    """Two tenants through the C++ harness (gpx_run_scenario).  The high-priority tenant submits
+    launch by launch (it is never preempted and plain launches are its fastest path); the
+    best-effort tenant runs as one persistent, preemptible program kernel, except under
+    "wb-chunk", which feeds its kernels a few at a time."""
     from gpreempt_amd import executor as gx
     cfg = {
         "time": max(5.0, 4.0 * steps / hp_rate), "policy": policy, "hp_requests": steps,
         "warmups": warmup, "standalone_runs": 100,
         "tasks": [
             {"id": "hp", "load": {"type": "poisson", "frequency": hp_rate, "seed": 2025},
-             "client": {"name": "hp", "model_name": hp_model, "priority": 0, "use_cuda_graph": True, "preprocess_time": 0}},
+             "client": {"name": "hp", "model_name": hp_model, "priority": 0, "use_cuda_graph": False, "launch_mode": "launch", "preprocess_time": 0}},
             {"id": "be", "load": {"type": "continuous"},
-             "client": {"name": "be", "model_name": be_model, "priority": 1, "use_cuda_graph": True, "preprocess_time": 0}},
+             "client": {"name": "be", "model_name": be_model, "priority": 1, "use_cuda_graph": True, "launch_mode": "program", "preprocess_time": 0}},
         ],
     }
     buf = C.create_string_buffer(1 << 20)
@@ -44,6 +48,37 @@ def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
     if rc != 0:
         raise RuntimeError(f"scenario failed with Status {rc}: {buf.value[:400]!r}")
     return json.loads(buf.value.decode())
+
+
+def summarize(rep):
+    hp, be = rep["tasks"]["hp"], rep["tasks"]["be"]
+    return {
+        "hp_p99_vs_isolated": rep["hp_p99_vs_isolated"],
+        "hp_requests": hp["requests"],
+        "hp_isolated_ms": {k: hp["standAlone(us)"][k] / 1e3 for k in ("mean", "p50", "p99")},
+        "hp_corun_ms": {k: hp["totalLatency(us)"][k] / 1e3 for k in ("mean", "p50", "p99", "max")},
+        "hp_throughput_req_s": hp["avgThroughput(req/s)"],
+        "preemption_latency_us": {k: rep["preemptLatency(us)"][k] for k in ("count", "mean", "p50", "p99", "max")},
+        "be_throughput_kept": rep["be_throughput_kept"],
+        "be_throughput_req_s": be["avgThroughput(req/s)"], "be_isolated_req_s": be["standAloneThroughput(req/s)"],
+        "be_preemptions": be["preemptions"], "hp_busy_fraction": rep["hp_busy_fraction"],
+        "hp_kernels": hp["kernels"], "be_kernels": be["kernels"]}
+
+
+def probe(workload, trials):
+    """BASELINE config 2: per-kernel preemption / resume latency of one best-effort model."""
+    from gpreempt_amd import executor as gx
+    buf = C.create_string_buffer(1 << 20)
+    rc = gx.lib().gpx_preempt_probe(workload.encode(), trials, 1, C.c_ulonglong(7), buf, C.c_size_t(len(buf)))
+    if rc != 0:
+        raise RuntimeError(f"probe failed with Status {rc}")
+    r = json.loads(buf.value.decode())
+    worst = sorted(r["perKernel"], key=lambda k: -k["preempt_max(us)"])[:3]
+    return {"workload": workload, "kernels": r["kernels"], "trials": r["trials"], "interrupted": r["interrupted"],
+            "isolated_ms": r["isolated(us)"]["mean"] / 1e3,
+            "preemption_latency_us": {k: r["preemptLatency(us)"][k] for k in ("mean", "p50", "p99", "max")},
+            "resume_call_us": {k: r["resumeCall(us)"][k] for k in ("mean", "p99", "max")},
+            "slowest_kernels": [{"kernel": k["kernel"], "name": k["name"], "tiles": k["tiles"], "preempt_max_us": k["preempt_max(us)"]} for k in worst]}
 
 
 def roofline(workload, iters, dt):
@@ -87,6 +122,33 @@ def roofline(workload, iters, dt):
             "algorithmic_flop_per_launch": total_flop / launches, "algorithmic_bytes_per_launch": total_bytes / launches}
 
 
+def gemm_roofline(iters=10):
+    """BASELINE config 5's best-effort tenant alone: bf16 8192^3 GEMM (fp32 accumulate), preemptible."""
+    from gpreempt_amd import capi as gp
+    n = 8192
+    dA, dB, dC = gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2)
+    dA.fill32(0x3F803F80)
+    dB.fill32(0x3C003C00)
+    p = gp.GemmParams(dtype=gp.BF16, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=1, C=dC.ptr, ldc=n, alpha=1.0, batch=1)
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    stream = gp.Stream(1)
+    e0, e1 = gp.Event(), gp.Event()
+    ms = []
+    for i in range(iters + 2):
+        st.reset()
+        e0.record(stream)
+        info = gp.launch("gp_launch_gemm", p, st.ctx(), stream)
+        e1.record(stream)
+        e1.sync()
+        if i >= 2:
+            ms.append(e0.elapsed_ms(e1))
+    t = sorted(ms)[len(ms) // 2] * 1e-3
+    ach = 2.0 * n ** 3 / t / 1e12
+    return {"bound": "mfma", "achieved": ach, "peak": PEAK["bf16"], "unit": "TFLOP/s", "frac": ach / PEAK["bf16"], "ms": t * 1e3,
+            "tiles": info.total_tiles, "grid": info.grid}
+
+
 def cpu_baseline(requests):
     """The high-priority graph (BERT-base, seq 128, fp16 storage) on the host cores through the
     CPU oracle.  Bounded sample: `requests` whole requests."""
@@ -117,11 +179,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=600)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--policy", default="wb")
+    ap.add_argument("--policy", default="wb-async")
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
-    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | cpu")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | cpu")
     ap.add_argument("--cpu-requests", type=int, default=4)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -135,21 +197,20 @@ def main():
            "config": {"workload": "BASELINE config 3: HP BERT-base fp16 b1 s128 Poisson %g req/s + BE ResNet-152 fp16 b8 224x224 back-to-back" % args.hp_rate,
                       "policy": args.policy, "hp_model": args.hp_model, "be_model": args.be_model}}
     if args.only in ("", "scenario"):
-        rep = scenario(args.steps, args.warmup, args.policy, args.hp_rate, args.be_model, args.hp_model)
-        hp, be = rep["tasks"]["hp"], rep["tasks"]["be"]
-        out.update({
-            "value": rep["hp_p99_vs_isolated"], "steps": hp["requests"],
-            "ms_per_step": hp["totalLatency(us)"]["mean"] / 1e3,
-            "hp_isolated_ms": {k: hp["standAlone(us)"][k] / 1e3 for k in ("mean", "p50", "p99")},
-            "hp_corun_ms": {k: hp["totalLatency(us)"][k] / 1e3 for k in ("mean", "p50", "p99", "max")},
-            "hp_throughput_req_s": hp["avgThroughput(req/s)"],
-            "preemption_latency_us": {k: rep["preemptLatency(us)"][k] for k in ("count", "mean", "p50", "p99", "max")},
-            "be_throughput_kept": rep["be_throughput_kept"],
-            "be_throughput_req_s": be["avgThroughput(req/s)"], "be_isolated_req_s": be["standAloneThroughput(req/s)"],
-            "be_preemptions": be["preemptions"], "hp_busy_fraction": rep["hp_busy_fraction"],
-            "hp_kernels": hp["kernels"], "be_kernels": be["kernels"]})
+        rep = summarize(scenario(args.steps, args.warmup, args.policy, args.hp_rate, args.be_model, args.hp_model))
+        out.update({"value": rep["hp_p99_vs_isolated"], "steps": rep["hp_requests"], "ms_per_step": rep["hp_corun_ms"]["mean"]})
+        out.update({k: v for k, v in rep.items() if k not in ("hp_p99_vs_isolated", "hp_requests")})
+        if not args.only:
+            # the other policies and the single-tenant probe ride along as context
+            out["other_policies"] = {}
+            for pol in ("wb", "wb-async", "wb-chunk", "np"):
+                if pol != args.policy:
+                    out["other_policies"][pol] = summarize(scenario(max(200, args.steps // 2), args.warmup, pol, args.hp_rate, args.be_model, args.hp_model))
+            out["config2_resnet50_fp32_b1"] = probe("resnet50", 300)
     if args.only in ("", "roofline"):
         out["roofline"] = roofline(args.be_model, 3, "f16")
+    if args.only in ("", "gemm"):
+        out["config5_gemm8192_bf16"] = gemm_roofline()
     if args.only in ("", "cpu"):
         out["cpu_baseline"] = cpu_baseline(args.cpu_requests)
     print(json.dumps(out))
