@@ -149,6 +149,20 @@ def gemm_roofline(iters=10):
             "tiles": info.total_tiles, "grid": info.grid}
 
 
+def copy_calibration(mib=256, iters=10):
+    """A plain device-to-device copy of known size (the runtime's copy kernel), used to scale
+    the FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc runs."""
+    from gpreempt_amd import capi as gp
+    n = mib << 20
+    a, b = gp.DevBuf(n), gp.DevBuf(n)
+    a.fill32(1)
+    stream = gp.Stream(1)
+    for _ in range(iters):
+        gp.check(gp.lib().gp_memcpy_d2d_async(C.c_void_p(b.ptr), C.c_void_p(a.ptr), C.c_size_t(n), stream.h))
+    stream.sync()
+    return {"bytes_per_copy": n, "copies": iters}
+
+
 def cpu_baseline(requests):
     """The high-priority graph (BERT-base, seq 128, fp16 storage) on the host cores through the
     CPU oracle.  Bounded sample: `requests` whole requests."""
@@ -183,7 +197,7 @@ def main():
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
-    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | cpu")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | cpu | copycal")
     ap.add_argument("--cpu-requests", type=int, default=4)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -211,6 +225,8 @@ def main():
         out["roofline"] = roofline(args.be_model, 3, "f16")
     if args.only in ("", "gemm"):
         out["config5_gemm8192_bf16"] = gemm_roofline()
+    if args.only == "copycal":
+        out["copy_calibration"] = copy_calibration()
     if args.only in ("", "cpu"):
         out["cpu_baseline"] = cpu_baseline(args.cpu_requests)
     print(json.dumps(out))

@@ -1,0 +1,76 @@
+// Priority / preemption control over the cooperative flag (see include/gpreempt.h).
+#include "gpreempt.h"
+
+#include <algorithm>
+#include <chrono>
+
+int NvRmQuery(NvContext *ctx) { return ctx && ctx->stream ? 0 : -1; }
+
+int set_priority(NvContext &ctx, int priority) {
+    if (priority < 0 || priority >= foo::PreemptDomain::kMaxLevels) return -1;
+    ctx.priority = priority;
+    return 0;
+}
+
+namespace foo {
+
+static int64_t steady_ns() {
+    return std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+PreemptDomain::PreemptDomain(int levels) : levels_(std::min(std::max(levels, 2), kMaxLevels)) {
+    for (int i = 0; i < kMaxLevels; ++i) { active_[i] = 0; raised_[i] = 0; }
+    for (int j = 0; j + 1 < levels_; ++j)
+        if (gp_flag_create(&host_[j], &dev_[j]) != 0) ok_ = false;
+}
+
+PreemptDomain::~PreemptDomain() {
+    for (int j = 0; j + 1 < levels_; ++j)
+        if (host_[j]) gp_flag_destroy(host_[j]);
+}
+
+GPUdeviceptr PreemptDomain::flag_for(int priority) const {
+    int p = std::min(priority, levels_ - 1);
+    return p >= 1 ? dev_[p - 1] : nullptr;
+}
+
+// word j is up while any request of a level <= j is active
+void PreemptDomain::update() {
+    std::lock_guard<std::mutex> g(mu_);
+    int run = 0;
+    for (int j = 0; j + 1 < levels_; ++j) {
+        run += active_[j].load();
+        int want = run > 0;
+        if (*host_[j] != want) {
+            if (want) raised_[j].store(steady_ns());
+            *host_[j] = want;
+        }
+    }
+}
+
+void PreemptDomain::begin(int priority) {
+    int p = std::min(priority, levels_ - 1);
+    if (p + 1 >= levels_) return;  // the lowest level preempts nobody
+    active_[p].fetch_add(1, std::memory_order_acq_rel);
+    update();
+}
+
+void PreemptDomain::end(int priority) {
+    int p = std::min(priority, levels_ - 1);
+    if (p + 1 >= levels_) return;
+    active_[p].fetch_sub(1, std::memory_order_acq_rel);
+    update();
+}
+
+int PreemptDomain::active_above(int priority) const {
+    int p = std::min(priority, levels_ - 1), n = 0;
+    for (int i = 0; i < p; ++i) n += active_[i].load(std::memory_order_acquire);
+    return n;
+}
+
+int64_t PreemptDomain::raised_ns(int priority) const {
+    int p = std::min(priority, levels_ - 1);
+    return p >= 1 ? raised_[p - 1].load() : 0;
+}
+
+}  // namespace foo

@@ -19,6 +19,7 @@
 #include <thread>
 
 #include "executor.h"
+#include "gpreempt.h"
 #include "mini_json.h"
 #include "numeric.h"
 
@@ -112,44 +113,26 @@ struct Stats {
 struct Shared {
     std::string policy;
     int levels = 2;
-    volatile int *flag_host[kMaxLevels] = {nullptr};
-    void *flag_dev[kMaxLevels] = {nullptr};
-    std::atomic<int> active[kMaxLevels];   // requests of this level that want or hold the GPU
-    std::atomic<int> on_gpu[kMaxLevels];   // preemptible tenants of this level with work in flight
-    std::atomic<int64_t> flag_raised_ns[kMaxLevels];
-    std::mutex flag_mu, seq_mu;
+    std::unique_ptr<PreemptDomain> domain;  // flag words and per-level request counts (gpreempt.h)
+    std::atomic<int> on_gpu[kMaxLevels];    // preemptible tenants of this level with work in flight
+    std::atomic<int> seq_waiting{0};        // "seq": latency-critical requests waiting for the lock
+    std::mutex seq_mu;
     std::mutex stats_mu;
-    Stats preempt_latency;                 // flag store -> lower-priority stream drained
+    Stats preempt_latency;                  // flag store -> lower-priority stream drained
     std::atomic<int64_t> hp_busy_ns{0};
     std::atomic<int> cores{0};
-    long hp_requests = 0;                  // > 0: the run ends once every priority-0 tenant served this many
+    long hp_requests = 0;                   // > 0: the run ends once every priority-0 tenant served this many
     std::atomic<int> hp_unfinished{0};
     std::atomic<bool> stop{false};
 
     Shared() {
-        for (int i = 0; i < kMaxLevels; ++i) { active[i] = 0; on_gpu[i] = 0; flag_raised_ns[i] = 0; }
+        for (int i = 0; i < kMaxLevels; ++i) on_gpu[i] = 0;
     }
-    int active_above(int p) const {
-        int n = 0;
-        for (int i = 0; i < p; ++i) n += active[i].load(std::memory_order_acquire);
-        return n;
-    }
+    int active_above(int p) const { return domain->active_above(p); }
     int on_gpu_below(int p) const {
         int n = 0;
         for (int i = p + 1; i < levels; ++i) n += on_gpu[i].load(std::memory_order_acquire);
         return n;
-    }
-    void update_flags() {  // flag[j] = any active at level <= j
-        std::lock_guard<std::mutex> g(flag_mu);
-        int run = 0;
-        for (int j = 0; j + 1 < levels; ++j) {
-            run += active[j].load();
-            int want = run > 0;
-            if (*flag_host[j] != want) {
-                if (want) flag_raised_ns[j].store(now_ns());
-                *flag_host[j] = want;
-            }
-        }
     }
 };
 
@@ -197,8 +180,7 @@ Status init_tenant(Tenant &t, Shared &sh) {
     fill_input(t);
     CUDA_RETURN_STATUS(gp_stream_create(t.priority, &t.stream));
     if (t.blp) {
-        int level = std::min(t.priority, sh.levels - 1);
-        t.blp->dpStop = sh.flag_dev[level - 1];
+        t.blp->dpStop = sh.domain->flag_for(t.priority);
     }
     // "wb-chunk" feeds a preemptible tenant's kernels a few at a time, so it never uses a
     // captured graph or program for that tenant.
@@ -243,7 +225,7 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             int64_t drained = now_ns();
             inflight = 0; head = tail;
             sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
-            int64_t raised = sh.flag_raised_ns[p - 1].load();
+            int64_t raised = sh.domain->raised_ns(p);
             if (raised > 0 && drained >= raised) {
                 std::lock_guard<std::mutex> g(sh.stats_mu);
                 sh.preempt_latency.add((drained - raised) / 1e3);
@@ -288,12 +270,12 @@ Status infer(Tenant &t, Shared &sh) {
     if (pol == "seq") {
         // seqclient.cpp:82-102: one model at a time; a best-effort tenant yields while a
         // latency-critical request is waiting.
-        if (p > 0) while (sh.active_above(p) > 0) spin_pause();
-        else sh.active[0].fetch_add(1);
+        if (p > 0) while (sh.seq_waiting.load() > 0) spin_pause();
+        else sh.seq_waiting.fetch_add(1);
         std::lock_guard<std::mutex> g(sh.seq_mu);
         RETURN_STATUS(t.ex->execute(t.stream));
         RETURN_STATUS(drain(t.stream));
-        if (p == 0) sh.active[0].fetch_sub(1);
+        if (p == 0) sh.seq_waiting.fetch_sub(1);
         return Status::Succ;
     }
     if (pol == "np" || pol == "lco" || !(pol == "wb" || pol == "wb-async" || pol == "wb-chunk")) {
@@ -331,7 +313,7 @@ Status infer(Tenant &t, Shared &sh) {
             const bool contended = sh.active_above(p) > 0;
             sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
             if (contended) {
-                int64_t raised = sh.flag_raised_ns[p - 1].load();
+                int64_t raised = sh.domain->raised_ns(p);
                 if (raised > 0 && drained >= raised) {
                     std::lock_guard<std::mutex> g(sh.stats_mu);
                     sh.preempt_latency.add((drained - raised) / 1e3);
@@ -360,17 +342,11 @@ static bool preempting_policy(const Shared &sh) { return sh.policy == "wb" || sh
 // (blpclient.cpp:185-188); end_request() lowers them when the level has no request left.
 void begin_request(Tenant &t, Shared &sh) {
     if (!preempting_policy(sh)) return;
-    const int p = std::min(t.priority, sh.levels - 1);
-    if (p + 1 >= sh.levels) return;  // the lowest level preempts nobody
-    sh.active[p].fetch_add(1, std::memory_order_acq_rel);
-    sh.update_flags();
+    sh.domain->begin(t.priority);
 }
 void end_request(Tenant &t, Shared &sh) {
     if (!preempting_policy(sh)) return;
-    const int p = std::min(t.priority, sh.levels - 1);
-    if (p + 1 >= sh.levels) return;
-    sh.active[p].fetch_sub(1, std::memory_order_acq_rel);
-    sh.update_flags();
+    sh.domain->end(t.priority);
 }
 
 // One request: the six DISB phases (benchmark.cpp:66-135); prepareInput and postprocess are empty
@@ -460,7 +436,8 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     if (tenants.empty()) return Status::NotFound;
     sh.levels = std::min(max_prio + 1, kMaxLevels);
     if (sh.levels < 2) sh.levels = 2;
-    for (int j = 0; j + 1 < sh.levels; ++j) CUDA_RETURN_STATUS(gp_flag_create(&sh.flag_host[j], &sh.flag_dev[j]));
+    sh.domain.reset(new PreemptDomain(sh.levels));
+    if (!sh.domain->ok()) return Status::Fail;
     for (auto &t : tenants) RETURN_STATUS(init_tenant(*t, sh));
 
     // warm-up and stand-alone latency, one tenant at a time (benchmark.cpp:221-299)
@@ -547,7 +524,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         gp_stream_destroy(t->stream);
     }
     tenants.clear();
-    for (int j = 0; j + 1 < sh.levels; ++j) gp_flag_destroy(sh.flag_host[j]);
+    sh.domain.reset();
     return result;
 }
 

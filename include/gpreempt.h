@@ -1,0 +1,71 @@
+// gpreempt.h — priority and preemption control.
+//
+// In the reference this header wraps ioctls of a patched driver: `set_priority(NvContext, int)`
+// turns a context's timeslice into 1 s (priority 0) or 1 us (any other), and on HIP
+// `hipSuspendStreams` / `hipResumeStreams` stop and restart hardware queues through a patched
+// amdkfd (include/gpreempt.h:124-173,191-194; src/gpreempt.cpp:61-72,143-196).  Here nothing
+// below user space is modified: a tenant's priority selects the cooperative preempt flag it
+// obeys, "suspend" raises that flag (running best-effort kernels leave at their next tile
+// boundary) and "resume" lowers it (the tenant then calls BLPExecutor::resume).  The call shapes
+// are kept so that client code reads the same.
+#pragma once
+#include <atomic>
+#include <mutex>
+#include <vector>
+#include "util/gpu_util.h"
+
+// What the reference keeps per GPU context (NvContext: client / object handles and channel list
+// found by NvRmQuery for the calling thread): here the tenant's stream and its priority level.
+struct NvContext {
+    GPUstream stream = nullptr;
+    int priority = 1;  // 0 = high, larger = lower
+};
+
+// Fills ctx for the calling thread's tenant; with stock drivers there is nothing to look up, so
+// this only validates the stream.  Returns 0 on success (the reference's NV_OK).
+int NvRmQuery(NvContext *ctx);
+
+// priority 0 = high, 1 = low (reference include/gpreempt.h:165-173); further levels are allowed.
+// Records the level on the context and its stream; returns 0, or -1 for a bad argument.
+int set_priority(NvContext &ctx, int priority);
+
+namespace foo {
+
+// The preempt flags of one GPU: one word per priority boundary.  Level p tenants obey word p-1,
+// which is up while any request of a level < p is active.  The reference has two levels and one
+// word (src/cuda-clients/blpclient.cpp:36-41,185-195).
+class PreemptDomain {
+public:
+    static constexpr int kMaxLevels = 8;
+    explicit PreemptDomain(int levels = 2);
+    ~PreemptDomain();
+    PreemptDomain(const PreemptDomain &) = delete;
+    PreemptDomain &operator=(const PreemptDomain &) = delete;
+
+    int levels() const { return levels_; }
+    bool ok() const { return ok_; }
+    // device address of the flag a level-p (p >= 1) best-effort executor polls: BLPExecutor::dpStop
+    GPUdeviceptr flag_for(int priority) const;
+    // a request of `priority` starts / ends: raises / lowers the words of every lower level
+    void begin(int priority);
+    void end(int priority);
+    // requests currently active at levels above `priority`
+    int active_above(int priority) const;
+    // steady-clock nanoseconds at which the word obeyed by `priority` was last raised (0: never)
+    int64_t raised_ns(int priority) const;
+    // direct control, the counterparts of hipSuspendStreams / hipResumeStreams
+    void suspend_below(int priority) { begin(priority); }
+    void resume_below(int priority) { end(priority); }
+
+private:
+    void update();
+    int levels_;
+    bool ok_ = true;
+    volatile int *host_[kMaxLevels] = {nullptr};
+    void *dev_[kMaxLevels] = {nullptr};
+    std::atomic<int> active_[kMaxLevels];
+    std::atomic<int64_t> raised_[kMaxLevels];
+    std::mutex mu_;
+};
+
+}  // namespace foo
