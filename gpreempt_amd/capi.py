@@ -22,7 +22,7 @@ vp = C.c_void_p
 
 class PreemptCtx(C.Structure):
     _fields_ = [("flag", vp), ("stop_index", vp), ("executed", vp), ("kernel_id", C.c_int),
-                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int)]
+                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int)]
 
 
 class LaunchInfo(C.Structure):
@@ -276,7 +276,7 @@ class BlpState:
         self.executed.upload(np.zeros(self.n, np.int32))
 
     def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0):
-        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id, kernel_id, inject_at, max_workgroups, poll_every)
+        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id, kernel_id, inject_at, max_workgroups, poll_every, 0)
 
     def stop_index(self):
         return int(self.stop.download(np_dtype=np.int32)[0])

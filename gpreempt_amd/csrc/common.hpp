@@ -59,15 +59,19 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         int pe = ctx->poll_every > 0 ? ctx->poll_every : 8;
         GP_REQUIRE((pe & (pe - 1)) == 0, "poll_every must be a power of two");
         blp->poll_mask = pe - 1;
+        int ng = ctx->counter_groups > 1 ? ctx->counter_groups : 1;
+        GP_REQUIRE((ng & (ng - 1)) == 0 && ng <= 64, "counter_groups must be a power of two <= 64");
+        blp->groups = ng;
         int per_cu = 0;
         GP_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, lds_bytes));
         if (per_cu < 1) per_cu = 1;
         long resident = (long)per_cu * device_cus();
         if (ctx->max_workgroups > 0 && resident > ctx->max_workgroups) resident = ctx->max_workgroups;
         *grid = (int)(total < resident ? total : resident);
+        if (*grid < blp->groups) *grid = blp->groups;  // every counter needs a workgroup to serve its slice
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
-        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0;
+        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1;
         *grid = (int)total;
     }
     if (info) {

@@ -32,7 +32,23 @@ struct BlpArgs {
     int kernel_id;
     int inject_at;    // -1 = off
     int poll_mask;    // the claim numbered c reads the host flag when (c & poll_mask) == 0
+    int groups;       // claim counters per kernel (>= 1); counter g sits at executed + g * COUNTER_STRIDE
 };
+
+// Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
+// few hundred tiles claimed from a single counter spends 10-20 us on claims alone.  A caller may
+// therefore give a kernel `groups` counters, one per 64-byte line: workgroup w claims from counter
+// w % groups, which owns the contiguous slice [total*g/groups, total*(g+1)/groups) of the tiles.
+// groups == 1 is the reference's layout (one int per kernel).
+constexpr int COUNTER_STRIDE = 16;  // ints
+
+// First tile of group g's slice when `grid` workgroups are spread round-robin over `groups`
+// counters: groups [0, grid % groups) hold one workgroup more than the others.
+__host__ __device__ inline int group_slice_begin(int total, int g, int groups, int grid) {
+    const int q = grid / groups, r = grid % groups;
+    const long w = (long)g * q + (g < r ? g : r);  // workgroups in the groups before g
+    return (int)((long)total * w / grid);
+}
 
 struct TileIdx { int x, y, z; };
 
@@ -53,6 +69,12 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     __shared__ int mailbox[2];
     const bool dynamic = b.executed != nullptr;
     const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    // Slices are proportional to the number of workgroups that serve them (workgroup w serves
+    // group w % groups), so that a launch with one workgroup per tile gives every workgroup
+    // exactly one tile.
+    const int grp = b.groups > 1 ? (int)(blockIdx.x % (unsigned)b.groups) : 0;
+    const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
+    const int slice_n = (b.groups > 1 ? group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) : b.total) - slice_lo;
     // One loop and one call site for both modes, so that the body is inlined into the kernel and
     // the kernel arguments stay in scalar registers.
     for (int it = 0;; ++it) {
@@ -73,13 +95,15 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
                 int claim = -1;
                 int stop = __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
                 if (!stop) {
-                    claim = atomicAdd(b.executed, 1);
-                    if (claim >= b.total) {
+                    const int c = atomicAdd(b.executed + grp * COUNTER_STRIDE, 1);
+                    if (c >= slice_n) {
                         claim = -1;
                     } else {
+                        claim = slice_lo + c;
                         if (claim == b.inject_at && b.flag)
                             __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                        if ((claim & b.poll_mask) == 0 && b.flag &&
+                        // with several counters only the first four groups read the host flag
+                        if (grp < 4 && (c & b.poll_mask) == 0 && b.flag &&
                             __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
                             atomicCAS(b.stop_index, -1, b.kernel_id);
                         // the polling workgroup still owes the tile it has just claimed

@@ -2,6 +2,7 @@
 // Behaviour follows the reference's src/executor.cpp (cited per function).
 #include "executor.h"
 
+#include <algorithm>
 #include <cstdlib>
 #include <set>
 
@@ -142,10 +143,13 @@ Status BLPExecutor::init(std::string workload) {
     CUDA_RETURN_STATUS(gp_memcpy_h2d(dpStopIndex, &stopIndex, sizeof(int)));
     model->batchAddParam(&this->dpStop);
     model->batchAddParam(&this->dpStopIndex);
-    CUDA_RETURN_STATUS(gp_malloc(&executed, sizeof(int) * model->get_kernel_num()));
-    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num(), nullptr));
+    const size_t counter_ints = model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride;
+    CUDA_RETURN_STATUS(gp_malloc(&executed, sizeof(int) * counter_ints));
+    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, counter_ints, nullptr));
     CUDA_RETURN_STATUS(gp_stream_sync(nullptr));
-    RETURN_STATUS(model->add_block_preemption_param(executed));
+    // GPREEMPT_SINGLE_COUNTER=1 selects the reference's one-counter-per-kernel layout (for A/B timing)
+    const char *single = std::getenv("GPREEMPT_SINGLE_COUNTER");
+    RETURN_STATUS(model->add_block_preemption_param(executed, (single && *single == '1') ? 1 : kCounterGroups));
     RETURN_STATUS(this->load_param(model_path));
     return Status::Succ;
 }
@@ -198,7 +202,7 @@ Status BLPExecutor::resume(GPUstream stream) {
 }
 
 Status BLPExecutor::reset_counters(GPUstream stream) {
-    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num(), stream));
+    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride, stream));
     return Status::Succ;
 }
 
@@ -209,8 +213,26 @@ Status BLPExecutor::read_counters(std::vector<int> &out) {
         RETURN_STATUS(model->read_program_counters(out, done, error));
         return error ? Status::Timeout : Status::Succ;
     }
-    out.resize(model->get_kernel_num());
-    CUDA_RETURN_STATUS(gp_memcpy_d2h(out.data(), executed, sizeof(int) * out.size()));
+    // per-kernel claim count = sum over the counter groups, each clamped to its slice (a counter
+    // overshoots by one per workgroup that found its slice handed out)
+    const size_t n = model->get_kernel_num();
+    std::vector<int> raw(n * (size_t)kCounterGroups * kCounterStride);
+    CUDA_RETURN_STATUS(gp_memcpy_d2h(raw.data(), executed, sizeof(int) * raw.size()));
+    out.assign(n, 0);
+    for (size_t i = 0; i < n; ++i) {
+        const long total = model->get_kernel_info(i).total_blocks;
+        long sum = 0;
+        if (model->counter_groups() == 1) { out[i] = raw[i]; continue; }
+        // slices follow the workgroup distribution of the last launch (device layer, tile_loop.hpp)
+        const long grid = std::max<long>(1, model->get_kernel_info(i).launch_params[0]);
+        auto begin = [&](long g) { long q = grid / kCounterGroups, r = grid % kCounterGroups; return total * (g * q + std::min(g, r)) / grid; };
+        for (int g = 0; g < kCounterGroups; ++g) {
+            long size = begin(g + 1) - begin(g);
+            long c = raw[(i * kCounterGroups + g) * kCounterStride];
+            sum += total > 0 ? std::min(c, size) : c;
+        }
+        out[i] = (int)sum;
+    }
     return Status::Succ;
 }
 

@@ -279,13 +279,15 @@ Status Model::batchAddParam(GPUdeviceptr *ptr) {
 // Per kernel: total_blocks, &executed[i], kernel id i; "nop" kernels are skipped but keep their
 // index (reference model.cpp:366-396).  The persistent grid (min(total_blocks, resident
 // workgroups)) is resolved by the device layer at launch.
-Status Model::add_block_preemption_param(GPUdeviceptr ptr) {
+Status Model::add_block_preemption_param(GPUdeviceptr ptr, int counter_groups) {
+    counter_groups_ = counter_groups > 1 ? counter_groups : 1;
     for (size_t i = 0; i < kernel_infos.size(); ++i) {
         KernelInfo &k = kernel_infos[i];
         if (k.name == "nop") continue;
         if (k.args_ptr.size() < 2) return Status::Fail;
         k.preemptible = true;
-        k.executed = (GPUdeviceptr)((char *)ptr + i * sizeof(int));
+        const size_t per_kernel = counter_groups_ > 1 ? sizeof(int) * counter_groups_ * 16 : sizeof(int);
+        k.executed = (GPUdeviceptr)((char *)ptr + i * per_kernel);
         k.kernel_id = (int)i;
     }
     return Status::Succ;
@@ -311,6 +313,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.inject_at = inject_at;
         ctx.max_workgroups = 0;
         ctx.poll_every = 0;
+        ctx.counter_groups = counter_groups_;
         pc = &ctx;
     }
     gp_launch_info info{};

@@ -92,13 +92,19 @@ public:
     // launch kernel by kernel.
     Status reset_counters(GPUstream stream);
 
+    // Claim counters per kernel.  The reference keeps one int per kernel (src/executor.cpp:333);
+    // claims from several hundred workgroups serialise on a single address, so each kernel gets
+    // 32 counters here, each owning a slice of the kernel's tiles.
+    static constexpr int kCounterGroups = 32;
+    static constexpr int kCounterStride = 16;  // ints between counters
+
 public:
     GPUdeviceptr dpStop = nullptr;  // the preempt flag: allocated by the caller, shared by all best-effort tenants
     std::atomic<bool> running{false};
 
 private:
     GPUdeviceptr dpStopIndex = nullptr;  // owned
-    GPUdeviceptr executed = nullptr;     // owned: one tile counter per kernel
+    GPUdeviceptr executed = nullptr;     // owned: kCounterGroups tile counters per kernel, one per 64-byte line
     int stopIndex = -1;
     int *stop_host = nullptr;            // pinned landing slot for the stop index
     int inject_kernel = -1, inject_claim = -1;

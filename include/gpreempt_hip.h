@@ -101,6 +101,10 @@ typedef struct gp_preempt_ctx {
     int poll_every;  /* the claim numbered c reads the host flag when c % poll_every == 0; a power */
                      /* of two; 0 = default (8).  All claims check *stop_index (device memory),   */
                      /* which the polling workgroup sets, so 1 reproduces a poll per tile         */
+    int counter_groups; /* 0 or 1: *executed is one int (the reference's layout).  A power of two */
+                     /* n > 1: executed points at n counters spaced 16 ints (64 bytes) apart;     */
+                     /* workgroup w claims from counter w % n, which owns a contiguous slice of   */
+                     /* the tiles.  Spreads the claim atomics, which serialise on one address.   */
 } gp_preempt_ctx;
 
 /* What a launch did: filled when the `info` argument of a launcher is non-NULL. */

@@ -109,7 +109,9 @@ public:
     Status clear();
 
     Status batchAddParam(GPUdeviceptr *ptr);
-    Status add_block_preemption_param(GPUdeviceptr ptr);
+    // `ptr` holds the claim counters: counter_groups counters per kernel, 64 bytes apart
+    // (counter_groups = 1 is the reference's one int per kernel, src/model.cpp:366-396).
+    Status add_block_preemption_param(GPUdeviceptr ptr, int counter_groups = 1);
 
     // Launches kernel `idx` on `stream` (what src/executor.cpp:136-164 does with
     // GPULaunchKernel); preemptible kernels take their flag and stop index from the by-reference
@@ -125,6 +127,7 @@ public:
     // per-layer claim counters of the program (blocking)
     Status read_program_counters(std::vector<int> &executed, std::vector<int> &done, int &error);
 
+    int counter_groups() const { return counter_groups_; }
     const std::string &workload() const { return workload_; }
     const std::string &dtype() const { return dtype_; }
     double total_flops() const;
@@ -135,6 +138,7 @@ public:
 private:
     bool loaded_ = false;
     gp_program program_ = nullptr;
+    int counter_groups_ = 1;
     std::string workload_, dtype_;
     std::vector<StorageInfo> storage_infos;
     std::vector<ParamLayout> layouts;
