@@ -22,7 +22,7 @@ vp = C.c_void_p
 
 class PreemptCtx(C.Structure):
     _fields_ = [("flag", vp), ("stop_index", vp), ("executed", vp), ("kernel_id", C.c_int),
-                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int)]
+                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("left_host", vp)]
 
 
 class LaunchInfo(C.Structure):
@@ -81,7 +81,7 @@ class EmbedParams(C.Structure):
 SYMBOLS = """gp_init gp_last_error gp_device_info gp_stream_create gp_stream_destroy gp_stream_sync
 gp_stream_query gp_stream_priority gp_stream_native gp_event_create gp_event_destroy gp_event_record
 gp_event_sync gp_event_query gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free gp_memcpy_h2d gp_memcpy_d2h
-gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy
+gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_flag_relay_start
 gp_launch_gemm gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
 gp_launch_layernorm gp_launch_embed gp_launch_gate gp_launch_noop gp_graph_begin gp_graph_end gp_graph_launch
 gp_graph_destroy gp_program_create gp_program_destroy gp_program_add_gemm gp_program_add_conv2d
@@ -276,7 +276,7 @@ class BlpState:
         self.executed.upload(np.zeros(self.n, np.int32))
 
     def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0):
-        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id, kernel_id, inject_at, max_workgroups, poll_every, 0)
+        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id, kernel_id, inject_at, max_workgroups, poll_every, 0, None)
 
     def stop_index(self):
         return int(self.stop.download(np_dtype=np.int32)[0])

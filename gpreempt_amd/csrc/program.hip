@@ -68,6 +68,9 @@ struct ProgArgs {
     int inject_layer, inject_claim;
     int poll_mask;
     unsigned spin_limit;
+    int *exited;       // device counter of workgroups that have left this launch
+    int *left_host;    // optional host-visible word: set to `launch_tag` by the last workgroup to leave
+    int launch_tag;
     unsigned long long *prof;  // optional: 4 cycle counters per workgroup (claim, acquire, body, publish)
 };
 
@@ -198,6 +201,16 @@ __global__ __launch_bounds__(256, GP_EXP_WGS) void program_kernel(ProgArgs p) {
                             break;
                         }
                         stop_word = __hip_atomic_load(p.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        // a few workgroups use their idle time to watch the host flag, so a stop is
+                        // noticed within microseconds even between the claims that normally read it
+                        if (blockIdx.x < 4 && p.flag && stop_word == -1) {
+                            int f = 0;
+                            if (leader) f = __hip_atomic_load(p.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                            if (__builtin_amdgcn_readfirstlane(f) != 0) {
+                                if (leader) atomicCAS(p.stop_index, -1, L);
+                                stop_word = L;
+                            }
+                        }
                         continue;
                     }
                     ready_upto = L;  // completion is monotone: layers 0..L-1 stay complete
@@ -227,6 +240,12 @@ __global__ __launch_bounds__(256, GP_EXP_WGS) void program_kernel(ProgArgs p) {
         const int claim = __builtin_amdgcn_readfirstlane(mailbox[it & 1][1]);
         if (p.prof) { unsigned long long t1 = wall_clock64(); t_claim += t1 - t0; t0 = t1; }
         if (claim < 0) {
+            if (leader && p.left_host) {
+                // every workgroup of this launch has stopped touching the model's buffers once the
+                // count is complete: tell the host without waiting for the queue to report it
+                if (atomicAdd(p.exited, 1) == (int)gridDim.x - 1)
+                    __hip_atomic_store(p.left_host, p.launch_tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
             if (p.prof && leader) { p.prof[blockIdx.x * 4 + 0] = t_claim; p.prof[blockIdx.x * 4 + 1] = t_acq; p.prof[blockIdx.x * 4 + 2] = t_body; p.prof[blockIdx.x * 4 + 3] = t_pub; }
             return;
         }
@@ -264,7 +283,8 @@ struct gp_program_s {
     int dtype = GP_F32;
     std::vector<LayerDesc> layers;
     LayerDesc *d_layers = nullptr;
-    int *d_state = nullptr;  // error | internal stop word | pad.. (16 ints) | claimed[n][NG] | done[n][NG] | ldone[n], one counter per line
+    int launches = 0;
+    int *d_state = nullptr;  // error | internal stop word | exited | pad.. (16 ints) | claimed[n][NG] | done[n][NG] | ldone[n], one counter per line
     unsigned long long *d_prof = nullptr;
     int n_groups = 1;
     size_t lds_bytes = 0;
@@ -274,6 +294,7 @@ struct gp_program_s {
     int n() const { return (int)layers.size(); }
     int *error() const { return d_state; }
     int *own_stop() const { return d_state + 1; }
+    int *exited() const { return d_state + 2; }
     int *claimed() const { return d_state + 16; }
     int *done() const { return d_state + 16 + (size_t)n() * n_groups * 16; }
     int *ldone() const { return d_state + 16 + (size_t)2 * n() * n_groups * 16; }
@@ -404,8 +425,13 @@ extern "C" int gp_program_launch(gp_program p, const gp_preempt_ctx *ctx, int re
     ProgArgs a{};
     a.layers = p->d_layers; a.n_layers = n;
     a.n_groups = p->n_groups; a.poll_groups = p->n_groups < 4 ? p->n_groups : 4;
+    if (ctx && ctx->poll_every == 1) a.poll_groups = p->n_groups;  // the flag is cheap to read: every group looks
     a.claimed = p->claimed(); a.done = p->done(); a.ldone = p->ldone(); a.error = p->error();
     a.spin_limit = 1u << 22;  // seconds: only a broken dependency chain gets there
+    a.exited = p->exited();
+    a.left_host = ctx ? ctx->left_host : nullptr;
+    a.launch_tag = ++p->launches;
+    if (a.left_host) { int rc = gp_fill32_async(p->exited(), 0, 1, s); if (rc) return rc; }
     a.prof = p->d_prof;
     long grid = p->max_tiles < p->resident ? p->max_tiles : p->resident;
     if (ctx) {
@@ -421,7 +447,7 @@ extern "C" int gp_program_launch(gp_program p, const gp_preempt_ctx *ctx, int re
         a.flag = nullptr; a.stop_index = p->own_stop(); a.inject_layer = -1; a.inject_claim = -1; a.poll_mask = 0;
     }
     if (grid < p->n_groups) grid = p->n_groups;  // every group needs at least one workgroup to serve its slices
-    if (info) { info->total_tiles = 0; for (auto &l : p->layers) info->total_tiles += l.total; info->shape[0] = n; info->shape[1] = 1; info->shape[2] = 1; info->grid = (int)grid; info->block = 256; }
+    if (info) { info->total_tiles = 0; for (auto &l : p->layers) info->total_tiles += l.total; info->shape[0] = n; info->shape[1] = a.launch_tag; info->shape[2] = 1; info->grid = (int)grid; info->block = 256; }
     switch (p->dtype) {
         case GP_F32: hipLaunchKernelGGL(program_kernel<float>, dim3((unsigned)grid), dim3(256), p->lds_bytes, native(s), a); break;
         case GP_F16: hipLaunchKernelGGL(program_kernel<_Float16>, dim3((unsigned)grid), dim3(256), p->lds_bytes, native(s), a); break;

@@ -45,6 +45,29 @@ __global__ void gate_kernel(const int *stop, unsigned long long spin_limit, int 
 
 __global__ void noop_kernel() {}
 
+struct RelayArgs { const int *flags[8]; int *mirror; int n; const int *quit; unsigned long long spin_limit; };
+
+// Lane i mirrors flag word i into device memory; lane 0 also watches the quit word.
+__global__ void flag_relay_kernel(RelayArgs a) {
+    const int lane = threadIdx.x;
+    int last = 0;
+    for (unsigned long long it = 0; it < a.spin_limit; ++it) {
+        if (lane < a.n) {
+            int v = __hip_atomic_load(a.flags[lane], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            if (v != last) {
+                __hip_atomic_store(a.mirror + lane, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                last = v;
+            }
+        }
+        int q = 0;
+        if (lane == 0) q = __hip_atomic_load(a.quit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        if (__builtin_amdgcn_readfirstlane(q) != 0) break;
+        __builtin_amdgcn_s_sleep(4);
+    }
+    // leave the mirror lowered so that nothing stays stopped because the relay is gone
+    if (lane < a.n && last != 0) __hip_atomic_store(a.mirror + lane, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 }  // namespace gp
 
 using namespace gp;
@@ -174,6 +197,19 @@ extern "C" int gp_flag_create(volatile int **host_ptr, void **dev_ptr) {
     return GP_SUCC;
 }
 extern "C" int gp_flag_destroy(volatile int *host_ptr) { if (host_ptr) GP_HIP(hipHostFree((void *)host_ptr)); return GP_SUCC; }
+
+extern "C" int gp_flag_relay_start(void *const *flags_dev, int *mirror, int n, const int *quit_dev,
+                                   unsigned long long spin_limit, gp_stream s) {
+    GP_REQUIRE(flags_dev && mirror && quit_dev && s, "relay needs flags, mirror, quit flag and an explicit stream");
+    GP_REQUIRE(n >= 1 && n <= 8, "relay handles 1..8 flag words");
+    GP_REQUIRE(spin_limit > 0, "relay needs a finite spin limit");
+    RelayArgs a{};
+    for (int i = 0; i < n; ++i) { GP_REQUIRE(flags_dev[i] != nullptr, "null flag"); a.flags[i] = (const int *)flags_dev[i]; }
+    a.mirror = mirror; a.n = n; a.quit = quit_dev; a.spin_limit = spin_limit;
+    hipLaunchKernelGGL(flag_relay_kernel, dim3(1), dim3(64), 0, native(s), a);
+    GP_HIP(hipGetLastError());
+    return GP_SUCC;
+}
 
 extern "C" int gp_launch_gate(const int *stop, unsigned long long spin_limit, int *timed_out, gp_stream s) {
     GP_REQUIRE(stop != nullptr, "null gate flag");

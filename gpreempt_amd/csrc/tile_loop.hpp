@@ -102,8 +102,9 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
                         claim = slice_lo + c;
                         if (claim == b.inject_at && b.flag)
                             __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                        // with several counters only the first four groups read the host flag
-                        if (grp < 4 && (c & b.poll_mask) == 0 && b.flag &&
+                        // with several counters only the first four groups read the flag, unless it
+                        // is read on every claim (poll_mask == 0: the flag is cheap device memory)
+                        if ((grp < 4 || b.poll_mask == 0) && (c & b.poll_mask) == 0 && b.flag &&
                             __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
                             atomicCAS(b.stop_index, -1, b.kernel_id);
                         // the polling workgroup still owes the tile it has just claimed

@@ -123,6 +123,11 @@ BLPExecutor::~BLPExecutor() {
     if (dpStopIndex) gp_free(dpStopIndex);
     if (executed) gp_free(executed);
     if (stop_host) gp_host_free(stop_host);
+    if (left_host) gp_flag_destroy(left_host);
+}
+
+bool BLPExecutor::program_vacated() const {
+    return use_program && left_host && *left_host == model->last_launch_tag();
 }
 
 // reference executor.cpp:300-342 (dnn branch): build the model, allocate the stop index (-1) and
@@ -139,6 +144,8 @@ Status BLPExecutor::init(std::string workload) {
     RETURN_STATUS(model->load_model(model_path + "/mod.json", model_path + "/host.json", model_path + "/mod.tr.co"));
     CUDA_RETURN_STATUS(gp_malloc(&dpStopIndex, sizeof(int)));
     CUDA_RETURN_STATUS(gp_host_alloc((void **)&stop_host, sizeof(int)));
+    CUDA_RETURN_STATUS(gp_flag_create(&left_host, &left_dev));
+    model->set_left_word(left_dev);
     stopIndex = -1;
     CUDA_RETURN_STATUS(gp_memcpy_h2d(dpStopIndex, &stopIndex, sizeof(int)));
     model->batchAddParam(&this->dpStop);
@@ -155,6 +162,7 @@ Status BLPExecutor::init(std::string workload) {
 }
 
 Status BLPExecutor::launch_kernel(size_t kernel_offset, GPUstream stream) {
+    model->set_poll_every(poll_every);
     int inject = ((int)kernel_offset == inject_kernel) ? inject_claim : -1;
     return model->launch(kernel_offset, stream, inject);
 }
@@ -162,6 +170,7 @@ Status BLPExecutor::launch_kernel(size_t kernel_offset, GPUstream stream) {
 // reference executor.cpp:211-232: zero every tile counter, then launch (or replay the graph).
 // The counters are cleared by a fill kernel outside the captured graph.
 Status BLPExecutor::execute(GPUstream stream) {
+    model->set_poll_every(poll_every);
     if (use_program) return model->launch_program(stream, true, inject_kernel, inject_claim);
     RETURN_STATUS(reset_counters(stream));
     if (use_cuda_graph) {
@@ -196,6 +205,7 @@ Status BLPExecutor::resume(GPUstream stream) {
     RETURN_STATUS(getStopPoint(stream));
     if (stopIndex == -1) return Status::Succ;
     // the program continues from its own per-layer counters; per-kernel mode relaunches one by one
+    model->set_poll_every(poll_every);
     if (use_program) return model->launch_program(stream, false, inject_kernel, inject_claim);
     for (size_t i = (size_t)stopIndex; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
     return Status::Succ;

@@ -18,20 +18,42 @@ static int64_t steady_ns() {
     return std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
 
-PreemptDomain::PreemptDomain(int levels) : levels_(std::min(std::max(levels, 2), kMaxLevels)) {
+PreemptDomain::PreemptDomain(int levels, bool use_relay) : levels_(std::min(std::max(levels, 2), kMaxLevels)) {
     for (int i = 0; i < kMaxLevels; ++i) { active_[i] = 0; raised_[i] = 0; }
     for (int j = 0; j + 1 < levels_; ++j)
         if (gp_flag_create(&host_[j], &dev_[j]) != 0) ok_ = false;
+    if (ok_ && use_relay) {
+        const int n = levels_ - 1;
+        bool good = gp_malloc((void **)&mirror_, sizeof(int) * 16) == 0 && gp_fill32_async(mirror_, 0, 16, nullptr) == 0 &&
+                    gp_stream_sync(nullptr) == 0 && gp_flag_create(&quit_host_, &quit_dev_) == 0 &&
+                    gp_stream_create(0, &relay_stream_) == 0;
+        // ~10 minutes of polling at most; a scenario is far shorter
+        if (good) good = gp_flag_relay_start(dev_, mirror_, n, (const int *)quit_dev_, 400000000ull, relay_stream_) == 0;
+        relay_on_ = good;
+        if (!good) std::fprintf(stderr, "PreemptDomain: flag relay not started (%s); kernels poll host memory\n", gp_last_error());
+    }
+}
+
+void PreemptDomain::stop_relay() {
+    if (!relay_on_) return;
+    *quit_host_ = 1;
+    gp_stream_sync(relay_stream_);
+    relay_on_ = false;
 }
 
 PreemptDomain::~PreemptDomain() {
+    stop_relay();
+    if (relay_stream_) gp_stream_destroy(relay_stream_);
+    if (quit_host_) gp_flag_destroy(quit_host_);
+    if (mirror_) gp_free(mirror_);
     for (int j = 0; j + 1 < levels_; ++j)
         if (host_[j]) gp_flag_destroy(host_[j]);
 }
 
 GPUdeviceptr PreemptDomain::flag_for(int priority) const {
     int p = std::min(priority, levels_ - 1);
-    return p >= 1 ? dev_[p - 1] : nullptr;
+    if (p < 1) return nullptr;
+    return relay_on_ ? (GPUdeviceptr)(mirror_ + (p - 1)) : dev_[p - 1];
 }
 
 // word j is up while any request of a level <= j is active

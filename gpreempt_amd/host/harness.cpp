@@ -181,6 +181,7 @@ Status init_tenant(Tenant &t, Shared &sh) {
     CUDA_RETURN_STATUS(gp_stream_create(t.priority, &t.stream));
     if (t.blp) {
         t.blp->dpStop = sh.domain->flag_for(t.priority);
+        if (sh.domain->relayed()) t.blp->poll_every = 1;  // the flag is a device-memory mirror
     }
     // "wb-chunk" feeds a preemptible tenant's kernels a few at a time, so it never uses a
     // captured graph or program for that tenant.
@@ -190,6 +191,24 @@ Status init_tenant(Tenant &t, Shared &sh) {
         t.ex->capture_graph(t.stream);
     }
     if (chunked) for (int i = 0; i < 3; ++i) CUDA_RETURN_STATUS(gp_event_create(&t.chunk_events[i]));
+    return Status::Succ;
+}
+
+// Waits until a preemptible tenant's work has left the GPU.  In program mode the kernel itself
+// tells the host (BLPExecutor::program_vacated); *vacated_ns receives that moment.  What follows
+// on the stream (reading the stop index back, relaunching) is ordered behind the kernel anyway.
+Status drain(GPUstream s);
+Status drain_blp(BLPExecutor *ex, GPUstream s, int64_t *vacated_ns) {
+    for (int i = 0;; ++i) {
+        if (ex->program_vacated()) break;  // a plain load of host memory
+        if ((i & 15) == 15) {              // the queue is asked now and then as well (per-kernel mode, errors)
+            int idle = 0;
+            CUDA_RETURN_STATUS(gp_stream_query(s, &idle));
+            if (idle) break;
+        }
+        spin_pause();
+    }
+    *vacated_ns = now_ns();
     return Status::Succ;
 }
 
@@ -307,9 +326,9 @@ Status infer(Tenant &t, Shared &sh) {
         t.blp->running = true;
         st = t.blp->execute(t.stream);
         while (st == Status::Succ) {
-            st = drain(t.stream);
+            int64_t drained = 0;
+            st = drain_blp(t.blp, t.stream, &drained);
             if (st != Status::Succ) break;
-            int64_t drained = now_ns();
             const bool contended = sh.active_above(p) > 0;
             sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
             if (contended) {
@@ -415,6 +434,9 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     sh.hp_requests = (long)cfg["hp_requests"].number(0);
     const json::Value &tasks = cfg["tasks"];
     std::vector<std::unique_ptr<Tenant>> tenants;
+    // Declared after `tenants`, so it runs first on every exit path: executors free device memory
+    // when they are destroyed, and a free waits for the whole device, relay kernel included.
+    struct RelayGuard { Shared &sh; ~RelayGuard() { if (sh.domain) sh.domain->stop_relay(); } } relay_guard{sh};
     int max_prio = 0;
     for (const json::Value &tv : tasks.arr) {
         std::unique_ptr<Tenant> t(new Tenant());
@@ -436,7 +458,8 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     if (tenants.empty()) return Status::NotFound;
     sh.levels = std::min(max_prio + 1, kMaxLevels);
     if (sh.levels < 2) sh.levels = 2;
-    sh.domain.reset(new PreemptDomain(sh.levels));
+    const bool relay = cfg["flag_relay"].boolean(false);  // measured slower: a second resident kernel slows every launch
+    sh.domain.reset(new PreemptDomain(sh.levels, relay));
     if (!sh.domain->ok()) return Status::Fail;
     for (auto &t : tenants) RETURN_STATUS(init_tenant(*t, sh));
 
@@ -516,6 +539,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     rep.set("preemptLatency(us)") = sh.preempt_latency.to_json();
     report_text = rep.dump();
 
+    sh.domain->stop_relay();  // frees below synchronise the device
     for (auto &t : tenants) {
         t->ex->clear();
         gp_host_free(t->input);

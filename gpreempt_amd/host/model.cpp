@@ -312,7 +312,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.kernel_id = k.kernel_id;
         ctx.inject_at = inject_at;
         ctx.max_workgroups = 0;
-        ctx.poll_every = 0;
+        ctx.poll_every = poll_every_;
         ctx.counter_groups = counter_groups_;
         pc = &ctx;
     }
@@ -382,10 +382,13 @@ Status Model::launch_program(GPUstream stream, bool reset, int inject_layer, int
         ctx.stop_index = (int *)*kernel_infos[0].args_ptr[n - 1];
         ctx.kernel_id = inject_layer;
         ctx.inject_at = inject_layer >= 0 ? inject_claim : -1;
+        ctx.poll_every = poll_every_;
+        ctx.left_host = (int *)left_word_;
         pc = &ctx;
     }
     gp_launch_info info{};
     CUDA_RETURN_STATUS(gp_program_launch(program_, pc, reset ? 1 : 0, stream, &info));
+    last_launch_tag_ = info.shape[1];
     return Status::Succ;
 }
 

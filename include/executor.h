@@ -91,6 +91,10 @@ public:
     // Zeroes every tile counter on `stream` (what execute() does first), for callers that
     // launch kernel by kernel.
     Status reset_counters(GPUstream stream);
+    // True once every workgroup of the last program launch has left the GPU (read from a host
+    // word the kernel sets; cheaper and earlier than a stream query).  Always false when the
+    // executor is not in program mode.
+    bool program_vacated() const;
 
     // Claim counters per kernel.  The reference keeps one int per kernel (src/executor.cpp:333);
     // claims from several hundred workgroups serialise on a single address, so each kernel gets
@@ -101,12 +105,17 @@ public:
 public:
     GPUdeviceptr dpStop = nullptr;  // the preempt flag: allocated by the caller, shared by all best-effort tenants
     std::atomic<bool> running{false};
+    // How often kernels read *dpStop: the claim numbered c reads it when c % poll_every == 0
+    // (a power of two; 0 = the device layer's default, 8).  Use 1 when dpStop is device memory.
+    int poll_every = 0;
 
 private:
     GPUdeviceptr dpStopIndex = nullptr;  // owned
     GPUdeviceptr executed = nullptr;     // owned: kCounterGroups tile counters per kernel, one per 64-byte line
     int stopIndex = -1;
     int *stop_host = nullptr;            // pinned landing slot for the stop index
+    volatile int *left_host = nullptr;   // fine-grained host word written by a program's last leaving workgroup
+    void *left_dev = nullptr;
     int inject_kernel = -1, inject_claim = -1;
     std::atomic<int> *lc_tasks = nullptr;
     std::atomic<int> *be_tasks = nullptr;

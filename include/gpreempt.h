@@ -37,7 +37,13 @@ namespace foo {
 class PreemptDomain {
 public:
     static constexpr int kMaxLevels = 8;
-    explicit PreemptDomain(int levels = 2);
+    // use_relay: keep a device-memory mirror of the flag words up to date with a small resident
+    // kernel (gp_flag_relay_start) and hand the mirror to the executors, so that their kernels
+    // poll device memory on every claim.  Call stop_relay() (the destructor does) before freeing
+    // device memory elsewhere: frees synchronise the device and would wait for the relay.
+    explicit PreemptDomain(int levels = 2, bool use_relay = false);
+    void stop_relay();
+    bool relayed() const { return relay_on_; }
     ~PreemptDomain();
     PreemptDomain(const PreemptDomain &) = delete;
     PreemptDomain &operator=(const PreemptDomain &) = delete;
@@ -66,6 +72,11 @@ private:
     std::atomic<int> active_[kMaxLevels];
     std::atomic<int64_t> raised_[kMaxLevels];
     std::mutex mu_;
+    bool relay_on_ = false;
+    int *mirror_ = nullptr;             // device ints, one per word
+    volatile int *quit_host_ = nullptr; // host flag that ends the relay
+    void *quit_dev_ = nullptr;
+    GPUstream relay_stream_ = nullptr;
 };
 
 }  // namespace foo

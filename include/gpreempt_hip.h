@@ -83,6 +83,15 @@ int gp_fill32_async(void *dev, uint32_t value, size_t count, gp_stream s);
  * with system-scope loads. */
 int gp_flag_create(volatile int **host_ptr, void **dev_ptr);
 int gp_flag_destroy(volatile int *host_ptr);
+/* Flag relay: one small resident kernel copies n host flag words (device-visible addresses of
+ * gp_flag_create flags, flags_dev[i]) into device memory (mirror[i]) whenever they change, so
+ * that kernels can poll a device address on every claim instead of crossing PCIe; a host store
+ * reaches the mirror in a few microseconds.  The kernel leaves when *quit_dev (another
+ * gp_flag_create word) becomes non-zero or after spin_limit polls; it occupies one wavefront of
+ * stream `s` until then, so stop it (store 1 to the quit flag, then gp_stream_sync(s)) before
+ * any call that synchronises the whole device (gp_free, gp_host_free).  n <= 8. */
+int gp_flag_relay_start(void *const *flags_dev, int *mirror, int n, const int *quit_dev,
+                        unsigned long long spin_limit, gp_stream s);
 
 /* ---- block-level preemption context ------------------------------------------------------
  * The six trailing arguments that scripts/compile/convert_to_blp.py:35 appends to every kernel
@@ -105,6 +114,10 @@ typedef struct gp_preempt_ctx {
                      /* n > 1: executed points at n counters spaced 16 ints (64 bytes) apart;     */
                      /* workgroup w claims from counter w % n, which owns a contiguous slice of   */
                      /* the tiles.  Spreads the claim atomics, which serialise on one address.   */
+    int *left_host;  /* programs only, may be NULL: device-visible address of a gp_flag_create    */
+                     /* word; the last workgroup to leave a launch stores that launch's number    */
+                     /* (info->shape[1] of gp_program_launch) there, so the host learns that the  */
+                     /* GPU has been vacated without a queue query                                */
 } gp_preempt_ctx;
 
 /* What a launch did: filled when the `info` argument of a launcher is non-NULL. */
@@ -236,6 +249,7 @@ int gp_launch_embed(const gp_embed_params *p, const gp_preempt_ctx *ctx, gp_stre
  *   ctx->flag / ctx->stop_index  as for the launchers (stop_index receives the LAYER index)
  *   ctx->executed                ignored: the program owns one counter per layer
  *   ctx->kernel_id, inject_at    test hook: layer and claim number that raise the flag
+ * info->shape[1] receives the launch number that ctx->left_host will be set to.
  * reset != 0 starts the model from its first tile (BLPExecutor::execute); reset == 0 continues
  * from the counters left by a preempted run (BLPExecutor::resume).  A NULL ctx runs the model
  * non-preemptibly (BaseExecutor). */

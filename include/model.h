@@ -117,6 +117,11 @@ public:
     // GPULaunchKernel); preemptible kernels take their flag and stop index from the by-reference
     // arguments added with batchAddParam.  inject_at is a test hook (-1 = off).
     Status launch(size_t idx, GPUstream stream, int inject_at = -1);
+    void set_poll_every(int n) { poll_every_ = n; }
+    // device-visible address of a host word that a program's last leaving workgroup sets to the
+    // launch number returned by launch_program()
+    void set_left_word(GPUdeviceptr p) { left_word_ = p; }
+    int last_launch_tag() const { return last_launch_tag_; }
 
     // Whole-model program: all kernels as one persistent device kernel (the counterpart of the
     // captured graph of src/executor.cpp:176-196).  build_program() is idempotent.
@@ -139,6 +144,9 @@ private:
     bool loaded_ = false;
     gp_program program_ = nullptr;
     int counter_groups_ = 1;
+    int poll_every_ = 0;
+    GPUdeviceptr left_word_ = nullptr;
+    int last_launch_tag_ = 0;
     std::string workload_, dtype_;
     std::vector<StorageInfo> storage_infos;
     std::vector<ParamLayout> layouts;
