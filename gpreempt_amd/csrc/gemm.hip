@@ -47,6 +47,16 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     return GP_SUCC;
 }
 
+// ring depth per tile size (deeper rings were measured: no gain, lower occupancy)
+#ifndef GP_S128
+#define GP_S128 3
+#endif
+#ifndef GP_S64
+#define GP_S64 4
+#endif
+#ifndef GP_S32
+#define GP_S32 4
+#endif
 template <typename T, int TILE, int STAGES, bool SPLITK>
 static int pipe_case(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     if (pl.conv) return launch_mat<PipeKernel<T, TILE, TILE, STAGES, true, SPLITK>>(pl, ctx, s, info);
@@ -57,10 +67,11 @@ template <typename T>
 static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
     switch (pl.body) {
-        case MB_PIPE128: return pipe_case<T, 128, 3, false>(pl, ctx, s, info);
-        case MB_PIPE64: return pipe_case<T, 64, 4, false>(pl, ctx, s, info);
-        case MB_PIPE64_SK: return pipe_case<T, 64, 4, true>(pl, ctx, s, info);
-        case MB_PIPE32_SK: return pipe_case<T, 32, 4, true>(pl, ctx, s, info);
+        case MB_PIPE256: return pipe_case<T, 256, 2, false>(pl, ctx, s, info);
+        case MB_PIPE128: return pipe_case<T, 128, GP_S128, false>(pl, ctx, s, info);
+        case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
+        case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
+        case MB_PIPE32_SK: return pipe_case<T, 32, GP_S32, true>(pl, ctx, s, info);
         case MB_STAGED128:
             if (pl.conv) return launch_mat<TK<T, 128, 128, SBK, 2, 2, true, false>>(pl, ctx, s, info);
             return pl.b_kn ? launch_mat<TK<T, 128, 128, SBK, 2, 2, false, true>>(pl, ctx, s, info)
@@ -87,10 +98,11 @@ int launch_mat_plan(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
 static size_t body_lds_bytes(int body, int dtype) {
     const size_t es = dtype == GP_F32 ? 4 : 2;
     switch (body) {
-        case MB_PIPE128: return 3 * (128 + 128) * 128;
-        case MB_PIPE64: return 4 * (64 + 64) * 128;
-        case MB_PIPE64_SK: return 4 * (64 + 64) * 128;   // equals the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4)
-        case MB_PIPE32_SK: return 4 * (32 + 32) * 128;
+        case MB_PIPE256: return 2 * (256 + 256) * 128;
+        case MB_PIPE128: return GP_S128 * (128 + 128) * 128;
+        case MB_PIPE64: return GP_S64 * (64 + 64) * 128;
+        case MB_PIPE64_SK: return GP_S64 * (64 + 64) * 128;   // at least the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4 = 64 KB)
+        case MB_PIPE32_SK: return GP_S32 * (32 + 32) * 128;
         case MB_STAGED128: return (128 + 128) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
         case MB_STAGED64: return (64 + 64) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
     }
@@ -111,21 +123,22 @@ static int choose_body(MatPlan *pl, int tile, int variant) {
         body = tm == 128 ? MB_STAGED128 : tm == 64 ? MB_STAGED64 : -1;
     } else if (variant == GP_MAT_PIPE) {
         int tm = tile ? tile : (tiles(128) >= cus ? 128 : 64);
-        body = tm == 128 ? MB_PIPE128 : tm == 64 ? MB_PIPE64 : -1;
+        body = tm == 256 ? MB_PIPE256 : tm == 128 ? MB_PIPE128 : tm == 64 ? MB_PIPE64 : -1;
     } else if (variant == GP_MAT_PIPE_SPLITK) {
         int tm = tile ? tile : (tiles(64) >= cus / 2 ? 64 : 32);
         body = tm == 64 ? MB_PIPE64_SK : tm == 32 ? MB_PIPE32_SK : -1;
     } else if (variant == GP_MAT_AUTO) {
-        if (tile == 128 || (tile == 0 && tiles(128) >= cus)) body = MB_PIPE128;
+        if (tile == 256 || (tile == 0 && tiles(256) >= cus)) body = MB_PIPE256;
+        else if (tile == 128 || (tile == 0 && tiles(128) >= cus)) body = MB_PIPE128;
         else if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) body = MB_PIPE64;
         else if (tile == 0 && tiles(64) >= cus / 2) body = MB_PIPE64_SK;
         else if (tile == 0 || tile == 32) body = MB_PIPE32_SK;
     }
     if (body < 0) {
-        set_error("no matrix kernel for tile %d with variant %d (tiles: 128, 64; 64, 32 with split K)", tile, variant);
+        set_error("no matrix kernel for tile %d with variant %d (tiles: 256, 128, 64; 64, 32 with split K)", tile, variant);
         return GP_OUTOFRANGE;
     }
-    const int t = (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
+    const int t = body == MB_PIPE256 ? 256 : (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
     pl->body = body;
     pl->sx = (g.N + t - 1) / t;
     pl->sy = (g.M + t - 1) / t;

@@ -36,9 +36,20 @@ __device__ __forceinline__ void load_lds16(const void *gptr, unsigned lds_byte) 
                  : "memory", "m0");
 }
 
+#ifndef GP_LOAD_SPREAD
+#define GP_LOAD_SPREAD 0  // MFMAs between two loads of a stage; 0: chosen from the tile shape
+#endif
+
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// four consecutive output elements
+template <typename T> struct __attribute__((aligned(4 * sizeof(T)))) Vec4 { T v[4]; };
+template <typename T> __device__ __forceinline__ void st_vec4(T *p, Vec4<T> o) {
+    if constexpr (sizeof(T) == 4) st_out128(p, __builtin_bit_cast(out_u32x4, o));
+    else st_out64(p, __builtin_bit_cast(unsigned long long, o));
 }
 
 template <typename T, int BM, int BN, int STAGES, bool CONV, bool SPLITK>
@@ -55,7 +66,7 @@ struct PipeKernel {
     static constexpr int LPS = A_PW + B_PW;
     static constexpr int WGM = SPLITK ? 1 : 2, WGN = SPLITK ? 1 : 2;
     static constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 32, NI = WN / 32;
-    static constexpr size_t RED_BYTES = SPLITK ? (size_t)WAVES * MI * NI * 16 * 64 * 4 : 0;
+    static constexpr size_t RED_BYTES = (size_t)WAVES * (SPLITK ? MI : 1) * NI * 16 * 64 * 4;  // epilogue staging
     static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_BYTES > RED_BYTES ? (size_t)STAGES * STAGE_BYTES : RED_BYTES;
     static_assert(BM % 32 == 0 && BN % 32 == 0 && A_PW >= 1 && B_PW >= 1, "tile shape");
     static_assert(STAGES >= 2 && (STAGES - 2) * LPS < 64, "pipeline depth");
@@ -80,74 +91,77 @@ struct PipeKernel {
         const T *zero = (const T *)g_zero_page;
 
         // ---- loader slots -------------------------------------------------------------------
-        const int rig = lane >> 3, cpos = lane & 7;  // row within the 8-row group, chunk slot
-        const T *a_row[A_PW];       // GEMM: pointer to the row start; CONV: pointer to image n
-        int a_h0[A_PW], a_w0[A_PW]; // CONV: window origin of the output pixel
-        int a_c[A_PW];              // logical chunk this lane fetches for that slot
-        bool a_ok[A_PW];
+        // Slot j of a wave covers rows (wave*PW + j)*8 .. +7 of the operand block; lane -> (row in
+        // the group, chunk slot).  Only the wave's first row pointer is kept in registers: the
+        // other slots are a uniform number of rows further on, and the swizzled chunk depends on
+        // the slot's parity only ((row >> 1) & 7 = 4*(slot & 1) + (rig >> 1)).
+        const int rig = lane >> 3, cpos = lane & 7;
+        const int c_base = cpos ^ (rig >> 1);
+        auto chunk_of = [&](int slot) { return c_base ^ ((slot & 1) << 2); };
+        const int a_row0 = m0 + wave * A_PW * 8 + rig, b_row0 = n0 + wave * B_PW * 8 + rig;
+        const T *a_ptr = nullptr;   // GEMM: row a_row0 of A
+        const T *a_img[CONV ? A_PW : 1];  // CONV: image of the slot's output pixel
+        int a_h0[CONV ? A_PW : 1], a_w0[CONV ? A_PW : 1];
+        if (CONV) {
 #pragma unroll
-        for (int j = 0; j < A_PW; ++j) {
-            int row = (wave * A_PW + j) * 8 + rig;
-            a_c[j] = cpos ^ ((row >> 1) & 7);
-            int m = m0 + row;
-            a_ok[j] = m < g.M;
-            if (CONV) {
-                int mm = a_ok[j] ? m : 0;
+            for (int j = 0; j < A_PW; ++j) {
+                int m = a_row0 + j * 8;
+                int mm = m < g.M ? m : 0;
                 int n = mm / (g.Ho * g.Wo), rem = mm - n * (g.Ho * g.Wo);
                 int ho = rem / g.Wo, wo = rem - ho * g.Wo;
                 a_h0[j] = ho * g.sh - g.ph; a_w0[j] = wo * g.sw - g.pw;
-                a_row[j] = A + (long)n * g.H * g.W * g.lda;
-            } else {
-                a_row[j] = A + (long)(a_ok[j] ? m : 0) * g.lda;
-                a_h0[j] = a_w0[j] = 0;
+                a_img[j] = A + (long)n * g.H * g.W * g.lda;
             }
+        } else {
+            a_ptr = A + (long)a_row0 * g.lda;
         }
-        const T *b_row[B_PW];
-        int b_c[B_PW];
-        bool b_ok[B_PW];
-#pragma unroll
-        for (int j = 0; j < B_PW; ++j) {
-            int row = (wave * B_PW + j) * 8 + rig;
-            b_c[j] = cpos ^ ((row >> 1) & 7);
-            int n = n0 + row;
-            b_ok[j] = n < g.N;
-            b_row[j] = B + (long)(b_ok[j] ? n : 0) * g.ldb;
-        }
+        const T *b_ptr = B + (long)b_row0 * g.ldb;
         const bool conv_fast = CONV && (g.Cin % BK == 0);  // a K-step never straddles a filter tap
 
-        auto issue = [&](int kt) {
-            const unsigned sbase = lds0 + (unsigned)(kt % STAGES) * STAGE_BYTES;
-            const int k0 = kt * BK;
-            int r_u = 0, s_u = 0, ci_u = 0;
+        // Loads of one stage: slot l < A_PW is an A slot, the rest are B slots.  `StageAddr` holds
+        // the wave-uniform part, computed once per stage.
+        struct StageAddr { unsigned sbase; int k0, r_u, s_u, ci_u; };
+        auto stage_addr = [&](int kt) {
+            StageAddr sa;
+            sa.sbase = lds0 + (unsigned)(kt % STAGES) * STAGE_BYTES;
+            sa.k0 = kt * BK;
+            sa.r_u = sa.s_u = sa.ci_u = 0;
             if (conv_fast) {
-                int rs = k0 / g.Cin;
-                ci_u = k0 - rs * g.Cin;
-                r_u = rs / g.S; s_u = rs - r_u * g.S;
+                int rs = sa.k0 / g.Cin;
+                sa.ci_u = sa.k0 - rs * g.Cin;
+                sa.r_u = rs / g.S; sa.s_u = rs - sa.r_u * g.S;
             }
-#pragma unroll
-            for (int j = 0; j < A_PW; ++j) {
-                const int k = k0 + a_c[j] * VEC;
+            return sa;
+        };
+        auto issue_one = [&](const StageAddr &sa, int l) {  // l is a compile-time constant at every call
+            if (l < A_PW) {
+                const int j = l;
+                const int kc = chunk_of(wave * A_PW + j) * VEC, k = sa.k0 + kc;
                 const T *src = zero;
-                if (a_ok[j] && k < g.K) {
+                if (a_row0 + j * 8 < g.M && k < g.K) {
                     if (CONV) {
-                        int r, s, ci;
-                        if (conv_fast) { r = r_u; s = s_u; ci = ci_u + a_c[j] * VEC; }
-                        else { int rs = k / g.Cin; ci = k - rs * g.Cin; r = rs / g.S; s = rs - r * g.S; }
-                        int hi = a_h0[j] + r, wi = a_w0[j] + s;
+                        int r, s2, ci;
+                        if (conv_fast) { r = sa.r_u; s2 = sa.s_u; ci = sa.ci_u + kc; }
+                        else { int rs = k / g.Cin; ci = k - rs * g.Cin; r = rs / g.S; s2 = rs - r * g.S; }
+                        int hi = a_h0[CONV ? j : 0] + r, wi = a_w0[CONV ? j : 0] + s2;
                         if ((unsigned)hi < (unsigned)g.H && (unsigned)wi < (unsigned)g.W)
-                            src = a_row[j] + ((long)hi * g.W + wi) * g.lda + ci;
+                            src = a_img[CONV ? j : 0] + ((long)hi * g.W + wi) * g.lda + ci;
                     } else {
-                        src = a_row[j] + k;
+                        src = a_ptr + (long)(j * 8) * g.lda + k;
                     }
                 }
-                load_lds16(src, sbase + (unsigned)((wave * A_PW + j) * 8 * RB));
+                load_lds16(src, sa.sbase + (unsigned)((wave * A_PW + j) * 8 * RB));
+            } else {
+                const int j = l - A_PW;
+                const int k = sa.k0 + chunk_of(wave * B_PW + j) * VEC;
+                const T *src = (b_row0 + j * 8 < g.N && k < g.K) ? b_ptr + (long)(j * 8) * g.ldb + k : zero;
+                load_lds16(src, sa.sbase + (unsigned)(A_BYTES + (wave * B_PW + j) * 8 * RB));
             }
+        };
+        auto issue = [&](int kt) {
+            const StageAddr sa = stage_addr(kt);
 #pragma unroll
-            for (int j = 0; j < B_PW; ++j) {
-                const int k = k0 + b_c[j] * VEC;
-                const T *src = (b_ok[j] && k < g.K) ? b_row[j] + k : zero;
-                load_lds16(src, sbase + (unsigned)(A_BYTES + (wave * B_PW + j) * 8 * RB));
-            }
+            for (int l = 0; l < LPS; ++l) issue_one(sa, l);
         };
 
         f32x16 acc[MI][NI];
@@ -163,19 +177,78 @@ struct PipeKernel {
             int phys = chunk ^ ((row >> 1) & 7);
             return *(const u32x4 *)(lds_c + (size_t)stage * STAGE_BYTES + region_bytes + row * RB + phys * 16);
         };
-        auto compute = [&](int stage) {
+        // Operand fragments are double-buffered in registers: while the MFMAs of k-step ks run, the
+        // LDS reads of k-step ks+1 are in flight.  The last k-step of a stage is multiplied after
+        // the next stage's barrier, so that the first fragment read of that stage is hidden too.
+        u32x4 fa[2][MI], fb[2][NI];
+        auto read_frags = [&](int buf, int stage, int ks) {
 #pragma unroll
-            for (int kq = 0; kq < (SPLITK ? 1 : KSTEPS); ++kq) {
-                const int ks = SPLITK ? wave : kq;
-                u32x4 fa[MI], fb[NI];
+            for (int i = 0; i < MI; ++i) fa[buf][i] = frag(stage, 0, wm * WM + i * 32 + l32, ks * 2 + half);
 #pragma unroll
-                for (int i = 0; i < MI; ++i) fa[i] = frag(stage, 0, wm * WM + i * 32 + l32, ks * 2 + half);
+            for (int j = 0; j < NI; ++j) fb[buf][j] = frag(stage, A_BYTES, wn * WN + j * 32 + l32, ks * 2 + half);
+        };
+        auto mma_all = [&](int buf) {
 #pragma unroll
-                for (int j = 0; j < NI; ++j) fb[j] = frag(stage, A_BYTES, wn * WN + j * 32 + l32, ks * 2 + half);
+            for (int i = 0; i < MI; ++i)
 #pragma unroll
-                for (int i = 0; i < MI; ++i)
-#pragma unroll
-                    for (int j = 0; j < NI; ++j) Elem<T>::mma(fa[i], fb[j], acc[i][j]);
+                for (int j = 0; j < NI; ++j) Elem<T>::mma(fa[buf][i], fb[buf][j], acc[i][j]);
+        };
+
+        // One MFMA phase = the MI*NI products of one k-step; a k-tile has KSTEPS phases, i.e.
+        // KSTEPS*MI*NI MFMA slots.  When `ISSUE`, the loads of the stage being fetched follow every
+        // SPREAD-th MFMA, so that their address arithmetic issues while the matrix pipe is busy
+        // instead of in front of it, and the requests reach the memory system as a steady stream.
+        constexpr int NM = MI * NI;
+        constexpr int EVEN = KSTEPS * NM / LPS > 0 ? KSTEPS * NM / LPS : 1;
+        constexpr int SPREAD = GP_LOAD_SPREAD > 0 ? GP_LOAD_SPREAD : (EVEN >= 4 ? EVEN - 1 : EVEN);  // measured: slightly front-loaded beats even for the 256x256 tile
+        static_assert(SPLITK || LPS <= KSTEPS * NM, "every load of a stage needs an MFMA slot");
+        auto phase = [&](int buf, auto issue_c, const StageAddr &sa, auto p_c) {
+            constexpr bool ISSUE = decltype(issue_c)::value != 0;
+            constexpr int P = decltype(p_c)::value;
+            static_for<0, NM>([&](auto qc) {
+                constexpr int q = decltype(qc)::value, slot = P * NM + q;
+                Elem<T>::mma(fa[buf][q / NI], fb[buf][q % NI], acc[q / NI][q % NI]);
+                if constexpr (ISSUE && slot % SPREAD == 0 && slot / SPREAD < LPS) issue_one(sa, slot / SPREAD);
+                // the slots cannot hold every load at this spacing: the rest follow the last MFMA
+                if constexpr (ISSUE && slot == KSTEPS * NM - 1 && slot / SPREAD + 1 < LPS)
+                    static_for<slot / SPREAD + 1, LPS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
+                if constexpr (ISSUE) __builtin_amdgcn_sched_barrier(0);
+            });
+        };
+        // k-tile kt: wait for its stage, start fetching stage kt+STAGES-1 (ISSUE) and multiply.
+        auto ktile = [&](int kt, bool tail, auto issue_c) {
+            constexpr bool ISSUE = decltype(issue_c)::value != 0;
+            // stage kt has landed once at most the loads of the younger in-flight stages remain
+            if (!tail) wait_vmcnt<(STAGES - 2) * LPS>();
+            else wait_vmcnt<0>();
+            __syncthreads();  // everyone's part of stage kt is visible; stage kt-1's buffer is free
+            const int stage = kt % STAGES;
+            StageAddr sa = {};
+            if constexpr (ISSUE) sa = stage_addr(kt + STAGES - 1);
+            if constexpr (SPLITK) {
+                if constexpr (ISSUE) static_for<0, LPS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
+                read_frags(0, stage, wave);
+                mma_all(0);
+            } else {
+                constexpr int LAST = (KSTEPS - 1) & 1;
+                read_frags(0, stage, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (kt > 0) {
+                    phase(LAST, issue_c, sa, IntC<0>{});  // last k-step of stage kt-1 (in registers)
+                } else if constexpr (ISSUE) {
+                    static_for<0, NM>([&](auto qc) {  // first k-tile: phase 0 has loads but no MFMAs
+                        constexpr int slot = decltype(qc)::value;
+                        if constexpr (slot % SPREAD == 0 && slot / SPREAD < LPS) issue_one(sa, slot / SPREAD);
+                    });
+                }
+                static_for<0, KSTEPS - 1>([&](auto kc) {
+                    constexpr int ks = decltype(kc)::value;
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_frags((ks + 1) & 1, stage, ks + 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    phase(ks & 1, issue_c, sa, IntC<ks + 1>{});
+                });
+                __builtin_amdgcn_sched_barrier(0);
             }
         };
 
@@ -185,39 +258,79 @@ struct PipeKernel {
 #pragma unroll
         for (int s = 0; s < STAGES - 1; ++s)
             if (s < KT) issue(s);
-        for (int kt = 0; kt < KT; ++kt) {
-            // stage kt has landed once at most the loads of the younger in-flight stages remain
-            if (KT - kt - 1 >= STAGES - 2) wait_vmcnt<(STAGES - 2) * LPS>();
-            else wait_vmcnt<0>();
-            __syncthreads();  // everyone's part of stage kt is visible; stage kt-1's buffer is free
-            if (kt + STAGES - 1 < KT) issue(kt + STAGES - 1);
-            compute(kt % STAGES);
-        }
+        int kt = 0;
+        for (; kt + STAGES - 1 < KT; ++kt) ktile(kt, false, IntC<1>{});
+        for (; kt < KT; ++kt) ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
+        if (!SPLITK && KT > 0) mma_all((KSTEPS - 1) & 1);
 
         // ---- epilogue -------------------------------------------------------------------------
+        // Accumulators go through LDS once so that each lane finishes four consecutive columns of
+        // one row: bias and residual are read, and the result written, as 8- or 16-byte vectors in
+        // full rows instead of one element per lane.  Slice s = (block j, register v) of a wave's
+        // accumulators is stored as 64 consecutive floats (one per lane), which is exactly
+        // "row 8*(v/4) + 4*(lane/32) + v%4, columns 32*j + lane%32".
         T *C = (T *)g.C + offc;
         const T *R = g.residual ? (const T *)g.residual + offc : nullptr;
         const T *bias = (const T *)g.bias;
-        auto emit = [&](int i, int j, int v, float a) {
-            int n = n0 + wn * WN + j * 32 + l32;
-            int m = m0 + wm * WM + i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
-            if (n >= g.N || m >= g.M) return;
-            float x = a * g.alpha + (bias ? Elem<T>::to_f(bias[n]) : 0.f);
-            if (R) x += Elem<T>::to_f(R[(long)m * g.ldr + n]);
-            st_elem<T>(&C[(long)m * g.ldc + n], Elem<T>::from_f(apply_act(x, g.act)));
+        const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
+                            (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
+        auto finish4 = [&](int m, int n, f32x4 a) {  // row m, columns n..n+3 of the output
+            if (m >= g.M || n >= g.N) return;
+            float x[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) x[q] = a[q] * g.alpha;
+            if (vec_ok) {
+                if (bias) {
+                    Vec4<T> bv = *(const Vec4<T> *)(bias + n);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) x[q] += Elem<T>::to_f(bv.v[q]);
+                }
+                if (R) {
+                    Vec4<T> rv = *(const Vec4<T> *)(R + (long)m * g.ldr + n);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) x[q] += Elem<T>::to_f(rv.v[q]);
+                }
+                Vec4<T> o;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) o.v[q] = Elem<T>::from_f(apply_act(x[q], g.act));
+                st_vec4<T>(&C[(long)m * g.ldc + n], o);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (n + q >= g.N) break;
+                    float y = x[q] + (bias ? Elem<T>::to_f(bias[n + q]) : 0.f);
+                    if (R) y += Elem<T>::to_f(R[(long)m * g.ldr + n + q]);
+                    st_elem<T>(&C[(long)m * g.ldc + n + q], Elem<T>::from_f(apply_act(y, g.act)));
+                }
+            }
         };
+        float *red = (float *)lds_t;
+        __syncthreads();  // all waves are done reading the stage buffers
         if (!SPLITK) {
+            // each wave transposes its own 32-row strips through a private NI x 4 KB region
+            float *mine = red + (size_t)wave * NI * 16 * 64;
+            constexpr int L4 = 8 * NI;            // lanes per output row (4 columns each)
+            constexpr int PASSES = 32 * L4 / 64;  // row groups per strip
+            static_for<0, MI>([&](auto ic) {
+                constexpr int i = ic;
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
+                for (int j = 0; j < NI; ++j)
 #pragma unroll
-                for (int i = 0; i < MI; ++i)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) emit(i, j, v, acc[i][j][v]);
+                    for (int v = 0; v < 16; ++v) mine[(j * 16 + v) * 64 + lane] = acc[i][j][v];
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // same wave reads other lanes' values next
+#pragma unroll 1
+                for (int p = 0; p < PASSES; ++p) {
+                    int idx = p * 64 + lane, r = idx / L4, c4 = idx - r * L4;
+                    int j = c4 >> 3, col = (c4 & 7) * 4;
+                    int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
+                    f32x4 a = *(const f32x4 *)(mine + (j * 16 + v) * 64 + hf * 32 + col);
+                    finish4(m0 + wm * WM + i * 32 + r, n0 + wn * WN + j * 32 + col, a);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // strip i+1 overwrites the region
+            });
         } else {
             // partial sums -> LDS as [wave][slice][lane], slice = (i*NI + j)*16 + v
-            float *red = (float *)lds_t;
             constexpr int SLICES = MI * NI * 16;
-            __syncthreads();  // all waves are done reading the stage buffers
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -225,16 +338,21 @@ struct PipeKernel {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + j) * 16 + v) * 64 + lane] = acc[i][j][v];
             __syncthreads();
-            // wave w finishes slices w, w+4, ...: fixed summation order over the four partials
-#pragma unroll
-            for (int sidx = 0; sidx < SLICES / WAVES; ++sidx) {
-                int sl = sidx * WAVES + wave;
-                float a = red[((size_t)0 * SLICES + sl) * 64 + lane];
-                a += red[((size_t)1 * SLICES + sl) * 64 + lane];
-                a += red[((size_t)2 * SLICES + sl) * 64 + lane];
-                a += red[((size_t)3 * SLICES + sl) * 64 + lane];
-                int blk = sl / 16, v = sl % 16;
-                emit(blk / NI, blk % NI, v, a);
+            // the BM x BN block is finished by all 256 threads, 4 columns each, summing the four
+            // partials in the fixed order w0 + w1 + w2 + w3
+            constexpr int L4 = BN / 4;
+            constexpr int PASSES = BM * L4 / NT;
+#pragma unroll 1
+            for (int p = 0; p < PASSES; ++p) {
+                int idx = p * NT + tid, row = idx / L4, c4 = idx - row * L4;
+                int i = row >> 5, r = row & 31, j = c4 >> 3, col = (c4 & 7) * 4;
+                int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
+                size_t o = ((size_t)(i * NI + j) * 16 + v) * 64 + hf * 32 + col;
+                f32x4 a = *(const f32x4 *)(red + o);
+                a += *(const f32x4 *)(red + (size_t)1 * SLICES * 64 + o);
+                a += *(const f32x4 *)(red + (size_t)2 * SLICES * 64 + o);
+                a += *(const f32x4 *)(red + (size_t)3 * SLICES * 64 + o);
+                finish4(m0 + row, n0 + j * 32 + col, a);
             }
         }
     }

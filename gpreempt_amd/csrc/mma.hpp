@@ -11,6 +11,15 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// loop whose index is a compile-time constant in the body (register arrays stay registers)
+template <int I> struct IntC { static constexpr int value = I; constexpr operator int() const { return I; } };
+template <int B, int E, class F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (B < E) {
+        f(IntC<B>{});
+        static_for<B + 1, E>(f);
+    }
+}
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
     static constexpr int VEC = 4;

@@ -28,6 +28,10 @@ __device__ __forceinline__ void st_out32(void *p, unsigned int v) {
     if (kCoherentStores) __hip_atomic_store((unsigned int *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else *(unsigned int *)p = v;
 }
+__device__ __forceinline__ void st_out64(void *p, unsigned long long v) {
+    if (kCoherentStores) __hip_atomic_store((unsigned long long *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *(unsigned long long *)p = v;
+}
 __device__ __forceinline__ void st_out128(void *p, out_u32x4 v) {
     if (kCoherentStores) {
         unsigned long long lo = ((unsigned long long)v[1] << 32) | v[0], hi = ((unsigned long long)v[3] << 32) | v[2];

@@ -7,7 +7,7 @@
 
 namespace gp {
 
-enum MatBody { MB_PIPE128 = 0, MB_PIPE64 = 1, MB_PIPE64_SK = 2, MB_PIPE32_SK = 3, MB_STAGED128 = 4, MB_STAGED64 = 5 };
+enum MatBody { MB_PIPE128 = 0, MB_PIPE64 = 1, MB_PIPE64_SK = 2, MB_PIPE32_SK = 3, MB_STAGED128 = 4, MB_STAGED64 = 5, MB_PIPE256 = 6 };
 
 struct MatPlan {
     MatArgs g;

@@ -356,9 +356,23 @@ extern "C" int gp_program_destroy(gp_program p) {
 }
 
 #define GP_ADD_MAT(PLAN) MatPlan pl; int rc = PLAN; return rc ? rc : push_mat(pr, pl);
+// the 256x256 body needs 128 KB of LDS and is not part of the program kernel: fall back to 128x128
+template <class P, class PlanFn>
+static int add_mat_layer(gp_program pr, const P *p, PlanFn plan) {
+    MatPlan pl;
+    int rc = plan(p, &pl);
+    if (rc) return rc;
+    if (pl.body == MB_PIPE256) {
+        P q = *p;
+        q.tile_m = q.tile_n = 128;
+        rc = plan(&q, &pl);
+        if (rc) return rc;
+    }
+    return push_mat(pr, pl);
+}
 #define GP_ADD_ELT(PLAN) EltPlan pl; int rc = PLAN; return rc ? rc : push_elt(pr, pl);
-extern "C" int gp_program_add_gemm(gp_program pr, const gp_gemm_params *p) { GP_ADD_MAT(plan_gemm(p, &pl)) }
-extern "C" int gp_program_add_conv2d(gp_program pr, const gp_conv_params *p) { GP_ADD_MAT(plan_conv2d(p, &pl)) }
+extern "C" int gp_program_add_gemm(gp_program pr, const gp_gemm_params *p) { GP_REQUIRE(p, "null params"); return add_mat_layer(pr, p, plan_gemm); }
+extern "C" int gp_program_add_conv2d(gp_program pr, const gp_conv_params *p) { GP_REQUIRE(p, "null params"); return add_mat_layer(pr, p, plan_conv2d); }
 extern "C" int gp_program_add_nchw_to_nhwc(gp_program pr, const gp_layout_params *p) { GP_ADD_ELT(plan_layout(p, &pl)) }
 extern "C" int gp_program_add_pool2d(gp_program pr, const gp_pool_params *p) { GP_ADD_ELT(plan_pool2d(p, &pl)) }
 extern "C" int gp_program_add_eltwise(gp_program pr, const gp_eltwise_params *p) { GP_ADD_ELT(plan_eltwise(p, &pl)) }
