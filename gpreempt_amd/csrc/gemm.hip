@@ -128,8 +128,9 @@ static int choose_body(MatPlan *pl, int tile, int variant) {
         int tm = tile ? tile : (tiles(64) >= cus / 2 ? 64 : 32);
         body = tm == 64 ? MB_PIPE64_SK : tm == 32 ? MB_PIPE32_SK : -1;
     } else if (variant == GP_MAT_AUTO) {
-        if (tile == 256 || (tile == 0 && tiles(256) >= cus)) body = MB_PIPE256;
-        else if (tile == 128 || (tile == 0 && tiles(128) >= cus)) body = MB_PIPE128;
+        // a tile wider than the problem multiplies zero columns: N <= 64 never takes the larger tiles
+        if (tile == 256 || (tile == 0 && tiles(256) >= cus && g.N > 128 && g.M > 128)) body = MB_PIPE256;
+        else if (tile == 128 || (tile == 0 && tiles(128) >= cus && g.N > 64 && g.M > 64)) body = MB_PIPE128;
         else if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) body = MB_PIPE64;
         else if (tile == 0 && tiles(64) >= cus / 2) body = MB_PIPE64_SK;
         else if (tile == 0 || tile == 32) body = MB_PIPE32_SK;
@@ -226,3 +227,11 @@ extern "C" int gp_launch_conv2d(const gp_conv_params *p, const gp_preempt_ctx *c
     int rc = plan_conv2d(p, &pl);
     return rc ? rc : launch_mat_plan(pl, ctx, s, info);
 }
+
+#ifdef GP_TILE_PROF
+extern "C" int gp_debug_tile_prof(unsigned long long *out, int n) {
+    GP_HIP(hipDeviceSynchronize());
+    GP_HIP(hipMemcpyFromSymbol(out, HIP_SYMBOL(gp::g_tile_prof), sizeof(unsigned long long) * (size_t)n));
+    return GP_SUCC;
+}
+#endif

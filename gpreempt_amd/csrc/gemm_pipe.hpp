@@ -40,6 +40,18 @@ __device__ __forceinline__ void load_lds16(const void *gptr, unsigned lds_byte) 
 #define GP_LOAD_SPREAD 0  // MFMAs between two loads of a stage; 0: chosen from the tile shape
 #endif
 
+// Optional phase timestamps of the first workgroups (compile with -DGP_TILE_PROF; read back with
+// gp_debug_tile_prof).  Slot p of workgroup b is g_tile_prof[b * 8 + p], in shader-clock ticks.
+#ifdef GP_TILE_PROF
+static __device__ unsigned long long g_tile_prof[256 * 8];
+#define GP_PROBE(p)                                                                  \
+    do {                                                                             \
+        if (threadIdx.x == 0 && blockIdx.x < 256) g_tile_prof[blockIdx.x * 8 + (p)] = __builtin_amdgcn_s_memtime(); \
+    } while (0)
+#else
+#define GP_PROBE(p) do { } while (0)
+#endif
+
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -72,6 +84,7 @@ struct PipeKernel {
     static_assert(STAGES >= 2 && (STAGES - 2) * LPS < 64, "pipeline depth");
 
     static __device__ __forceinline__ void run(const MatArgs &g, TileIdx t, T *lds_t) {
+        GP_PROBE(0);
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
         const int tid = threadIdx.x, lane = tid & 63;
@@ -121,15 +134,20 @@ struct PipeKernel {
         // Loads of one stage: slot l < A_PW is an A slot, the rest are B slots.  `StageAddr` holds
         // the wave-uniform part, computed once per stage.
         struct StageAddr { unsigned sbase; int k0, r_u, s_u, ci_u; };
+        // Stages are fetched in increasing order, so the filter tap (r, s) and channel offset of
+        // the next stage advance incrementally instead of being divided out of k every time.
+        int nx_r = 0, nx_s = 0, nx_ci = 0;
         auto stage_addr = [&](int kt) {
             StageAddr sa;
             sa.sbase = lds0 + (unsigned)(kt % STAGES) * STAGE_BYTES;
             sa.k0 = kt * BK;
-            sa.r_u = sa.s_u = sa.ci_u = 0;
+            sa.r_u = nx_r; sa.s_u = nx_s; sa.ci_u = nx_ci;
             if (conv_fast) {
-                int rs = sa.k0 / g.Cin;
-                sa.ci_u = sa.k0 - rs * g.Cin;
-                sa.r_u = rs / g.S; sa.s_u = rs - sa.r_u * g.S;
+                nx_ci += BK;
+                if (nx_ci >= g.Cin) {
+                    nx_ci = 0;
+                    if (++nx_s == g.S) { nx_s = 0; ++nx_r; }
+                }
             }
             return sa;
         };
@@ -222,12 +240,13 @@ struct PipeKernel {
             if (!tail) wait_vmcnt<(STAGES - 2) * LPS>();
             else wait_vmcnt<0>();
             __syncthreads();  // everyone's part of stage kt is visible; stage kt-1's buffer is free
+            if (kt == 0) GP_PROBE(2);
             const int stage = kt % STAGES;
             StageAddr sa = {};
             if constexpr (ISSUE) sa = stage_addr(kt + STAGES - 1);
             if constexpr (SPLITK) {
+                read_frags(0, stage, wave);  // the address arithmetic of the loads overlaps the LDS latency
                 if constexpr (ISSUE) static_for<0, LPS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
-                read_frags(0, stage, wave);
                 mma_all(0);
             } else {
                 constexpr int LAST = (KSTEPS - 1) & 1;
@@ -254,6 +273,7 @@ struct PipeKernel {
 
         // ---- main loop ------------------------------------------------------------------------
         const int KT = (g.K + BK - 1) / BK;
+        GP_PROBE(1);
         __syncthreads();  // the previous tile of this workgroup may still be reading LDS
 #pragma unroll
         for (int s = 0; s < STAGES - 1; ++s)
@@ -262,6 +282,7 @@ struct PipeKernel {
         for (; kt + STAGES - 1 < KT; ++kt) ktile(kt, false, IntC<1>{});
         for (; kt < KT; ++kt) ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
         if (!SPLITK && KT > 0) mma_all((KSTEPS - 1) & 1);
+        GP_PROBE(3);
 
         // ---- epilogue -------------------------------------------------------------------------
         // Accumulators go through LDS once so that each lane finishes four consecutive columns of
@@ -274,87 +295,140 @@ struct PipeKernel {
         const T *bias = (const T *)g.bias;
         const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
                             (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
-        auto finish4 = [&](int m, int n, f32x4 a) {  // row m, columns n..n+3 of the output
-            if (m >= g.M || n >= g.N) return;
-            float x[4];
+        // A lane's four columns are the same in every pass, so its bias values are read once.
+        auto load_bias = [&](int n, float (&bq)[4]) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) x[q] = a[q] * g.alpha;
+            for (int q = 0; q < 4; ++q) bq[q] = 0.f;
+            if (!bias || n >= g.N) return;
             if (vec_ok) {
-                if (bias) {
-                    Vec4<T> bv = *(const Vec4<T> *)(bias + n);
+                Vec4<T> bv = *(const Vec4<T> *)(bias + n);
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) x[q] += Elem<T>::to_f(bv.v[q]);
-                }
-                if (R) {
-                    Vec4<T> rv = *(const Vec4<T> *)(R + (long)m * g.ldr + n);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) x[q] += Elem<T>::to_f(rv.v[q]);
-                }
-                Vec4<T> o;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) o.v[q] = Elem<T>::from_f(apply_act(x[q], g.act));
-                st_vec4<T>(&C[(long)m * g.ldc + n], o);
+                for (int q = 0; q < 4; ++q) bq[q] = Elem<T>::to_f(bv.v[q]);
             } else {
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if (n + q >= g.N) break;
-                    float y = x[q] + (bias ? Elem<T>::to_f(bias[n + q]) : 0.f);
-                    if (R) y += Elem<T>::to_f(R[(long)m * g.ldr + n + q]);
-                    st_elem<T>(&C[(long)m * g.ldc + n + q], Elem<T>::from_f(apply_act(y, g.act)));
+                for (int q = 0; q < 4; ++q)
+                    if (n + q < g.N) bq[q] = Elem<T>::to_f(bias[n + q]);
+            }
+        };
+        // Finishes G rows (m_first, m_first + m_step, ...) of columns n..n+3: the residual reads of
+        // the whole group are issued before the first result is needed.
+        auto finish_group = [&](auto g_c, int n, const float (&bq)[4], int m_first, int m_step, const f32x4 *a) {
+            constexpr int G = decltype(g_c)::value;
+            if (n >= g.N) return;
+            if (vec_ok) {
+                Vec4<T> rv[G];
+                if (R) {
+#pragma unroll
+                    for (int gi = 0; gi < G; ++gi) {
+                        int m = m_first + gi * m_step;
+                        if (m < g.M) rv[gi] = *(const Vec4<T> *)(R + (long)m * g.ldr + n);
+                    }
+                }
+#pragma unroll
+                for (int gi = 0; gi < G; ++gi) {
+                    int m = m_first + gi * m_step;
+                    if (m >= g.M) continue;
+                    Vec4<T> o;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float x = a[gi][q] * g.alpha + bq[q];
+                        if (R) x += Elem<T>::to_f(rv[gi].v[q]);
+                        o.v[q] = Elem<T>::from_f(apply_act(x, g.act));
+                    }
+                    st_vec4<T>(&C[(long)m * g.ldc + n], o);
+                }
+            } else {
+#pragma unroll
+                for (int gi = 0; gi < G; ++gi) {
+                    int m = m_first + gi * m_step;
+                    if (m >= g.M) continue;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (n + q >= g.N) break;
+                        float x = a[gi][q] * g.alpha + bq[q];
+                        if (R) x += Elem<T>::to_f(R[(long)m * g.ldr + n + q]);
+                        st_elem<T>(&C[(long)m * g.ldc + n + q], Elem<T>::from_f(apply_act(x, g.act)));
+                    }
                 }
             }
         };
         float *red = (float *)lds_t;
-        __syncthreads();  // all waves are done reading the stage buffers
+        float bq[4];
         if (!SPLITK) {
             // each wave transposes its own 32-row strips through a private NI x 4 KB region
             float *mine = red + (size_t)wave * NI * 16 * 64;
-            constexpr int L4 = 8 * NI;            // lanes per output row (4 columns each)
-            constexpr int PASSES = 32 * L4 / 64;  // row groups per strip
+            constexpr int L4 = 8 * NI;       // lanes per output row (4 columns each)
+            constexpr int RPP = 64 / L4;     // rows per pass of the wave
+            constexpr int PASSES = 32 / RPP;
+            constexpr int G = PASSES < 4 ? PASSES : 4;
+            const int c4 = lane % L4, r_in = lane / L4;
+            const int j = c4 >> 3, col = (c4 & 7) * 4;
+            const int n = n0 + wn * WN + j * 32 + col;
+            load_bias(n, bq);
+            __syncthreads();  // all waves are done reading the stage buffers
             static_for<0, MI>([&](auto ic) {
                 constexpr int i = ic;
 #pragma unroll
-                for (int j = 0; j < NI; ++j)
+                for (int jj = 0; jj < NI; ++jj)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) mine[(j * 16 + v) * 64 + lane] = acc[i][j][v];
+                    for (int v = 0; v < 16; ++v) mine[(jj * 16 + v) * 64 + lane] = acc[i][jj][v];
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // same wave reads other lanes' values next
 #pragma unroll 1
-                for (int p = 0; p < PASSES; ++p) {
-                    int idx = p * 64 + lane, r = idx / L4, c4 = idx - r * L4;
-                    int j = c4 >> 3, col = (c4 & 7) * 4;
-                    int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
-                    f32x4 a = *(const f32x4 *)(mine + (j * 16 + v) * 64 + hf * 32 + col);
-                    finish4(m0 + wm * WM + i * 32 + r, n0 + wn * WN + j * 32 + col, a);
+                for (int p = 0; p < PASSES; p += G) {
+                    f32x4 a[G];
+#pragma unroll
+                    for (int gi = 0; gi < G; ++gi) {
+                        int r = (p + gi) * RPP + r_in;
+                        int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
+                        a[gi] = *(const f32x4 *)(mine + (j * 16 + v) * 64 + hf * 32 + col);
+                    }
+                    finish_group(IntC<G>{}, n, bq, m0 + wm * WM + i * 32 + p * RPP + r_in, RPP, a);
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // strip i+1 overwrites the region
             });
         } else {
-            // partial sums -> LDS as [wave][slice][lane], slice = (i*NI + j)*16 + v
+            // partial sums -> LDS as [wave][slice][lane], slice = (i*NI + j)*16 + v; the BM x BN
+            // block is then finished by all 256 threads, 4 columns each, summing the four partials
+            // in the fixed order w0 + w1 + w2 + w3
             constexpr int SLICES = MI * NI * 16;
+            constexpr int L4 = BN / 4;
+            constexpr int RPP = NT / L4;     // rows per pass of the workgroup
+            constexpr int PASSES = BM / RPP;
+            constexpr int G = PASSES < 4 ? PASSES : 4;
+            const int c4 = tid % L4, r_in = tid / L4;
+            const int j = c4 >> 3, col = (c4 & 7) * 4;
+            const int n = n0 + j * 32 + col;
+            load_bias(n, bq);
+            __syncthreads();  // all waves are done reading the stage buffers
 #pragma unroll
             for (int i = 0; i < MI; ++i)
 #pragma unroll
-                for (int j = 0; j < NI; ++j)
+                for (int jj = 0; jj < NI; ++jj)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+                    for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + jj) * 16 + v) * 64 + lane] = acc[i][jj][v];
             __syncthreads();
-            // the BM x BN block is finished by all 256 threads, 4 columns each, summing the four
-            // partials in the fixed order w0 + w1 + w2 + w3
-            constexpr int L4 = BN / 4;
-            constexpr int PASSES = BM * L4 / NT;
 #pragma unroll 1
-            for (int p = 0; p < PASSES; ++p) {
-                int idx = p * NT + tid, row = idx / L4, c4 = idx - row * L4;
-                int i = row >> 5, r = row & 31, j = c4 >> 3, col = (c4 & 7) * 4;
-                int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
-                size_t o = ((size_t)(i * NI + j) * 16 + v) * 64 + hf * 32 + col;
-                f32x4 a = *(const f32x4 *)(red + o);
-                a += *(const f32x4 *)(red + (size_t)1 * SLICES * 64 + o);
-                a += *(const f32x4 *)(red + (size_t)2 * SLICES * 64 + o);
-                a += *(const f32x4 *)(red + (size_t)3 * SLICES * 64 + o);
-                finish4(m0 + row, n0 + j * 32 + col, a);
+            for (int p = 0; p < PASSES; p += G) {
+                f32x4 a[G];
+#pragma unroll
+                for (int gi = 0; gi < G; ++gi) {
+                    int row = (p + gi) * RPP + r_in;
+                    int i = row >> 5, r = row & 31;
+                    int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
+                    size_t o = ((size_t)(i * NI + j) * 16 + v) * 64 + hf * 32 + col;
+                    a[gi] = *(const f32x4 *)(red + o);
+                    a[gi] += *(const f32x4 *)(red + (size_t)1 * SLICES * 64 + o);
+                    a[gi] += *(const f32x4 *)(red + (size_t)2 * SLICES * 64 + o);
+                    a[gi] += *(const f32x4 *)(red + (size_t)3 * SLICES * 64 + o);
+                }
+                finish_group(IntC<G>{}, n, bq, m0 + p * RPP + r_in, RPP, a);
             }
         }
+#ifdef GP_TILE_PROF
+        GP_PROBE(4);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        GP_PROBE(5);
+#endif
     }
 };
 
