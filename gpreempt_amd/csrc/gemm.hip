@@ -67,7 +67,8 @@ template <typename T>
 static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
     switch (pl.body) {
-        case MB_PIPE256: return pipe_case<T, 256, 2, false>(pl, ctx, s, info);
+        case MB_PIPE256:  // GEMM only: the gathered A operand of a convolution does not fit its register budget
+            return launch_mat<PipeKernel<T, 256, 256, 2, false, false>>(pl, ctx, s, info);
         case MB_PIPE128: return pipe_case<T, 128, GP_S128, false>(pl, ctx, s, info);
         case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
         case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
@@ -123,13 +124,13 @@ static int choose_body(MatPlan *pl, int tile, int variant) {
         body = tm == 128 ? MB_STAGED128 : tm == 64 ? MB_STAGED64 : -1;
     } else if (variant == GP_MAT_PIPE) {
         int tm = tile ? tile : (tiles(128) >= cus ? 128 : 64);
-        body = tm == 256 ? MB_PIPE256 : tm == 128 ? MB_PIPE128 : tm == 64 ? MB_PIPE64 : -1;
+        body = (tm == 256 && !pl->conv) ? MB_PIPE256 : tm == 128 ? MB_PIPE128 : tm == 64 ? MB_PIPE64 : -1;
     } else if (variant == GP_MAT_PIPE_SPLITK) {
         int tm = tile ? tile : (tiles(64) >= cus / 2 ? 64 : 32);
         body = tm == 64 ? MB_PIPE64_SK : tm == 32 ? MB_PIPE32_SK : -1;
     } else if (variant == GP_MAT_AUTO) {
         // a tile wider than the problem multiplies zero columns: N <= 64 never takes the larger tiles
-        if (tile == 256 || (tile == 0 && tiles(256) >= cus && g.N > 128 && g.M > 128)) body = MB_PIPE256;
+        if (!pl->conv && (tile == 256 || (tile == 0 && tiles(256) >= cus && g.N > 128 && g.M > 128))) body = MB_PIPE256;
         else if (tile == 128 || (tile == 0 && tiles(128) >= cus && g.N > 64 && g.M > 64)) body = MB_PIPE128;
         else if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) body = MB_PIPE64;
         else if (tile == 0 && tiles(64) >= cus / 2) body = MB_PIPE64_SK;

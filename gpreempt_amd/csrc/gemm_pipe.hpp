@@ -112,8 +112,10 @@ struct PipeKernel {
         const int c_base = cpos ^ (rig >> 1);
         auto chunk_of = [&](int slot) { return c_base ^ ((slot & 1) << 2); };
         const int a_row0 = m0 + wave * A_PW * 8 + rig, b_row0 = n0 + wave * B_PW * 8 + rig;
-        const T *a_ptr = nullptr;   // GEMM: row a_row0 of A
-        const T *a_img[CONV ? A_PW : 1];  // CONV: image of the slot's output pixel
+        // Pointers with the lane's chunk already added, one per parity of the slot number j: a
+        // load's address is then this plus a wave-uniform offset.
+        const T *a_par[2] = {nullptr, nullptr};  // GEMM: row a_row0 of A
+        const T *a_org[CONV ? A_PW : 1];         // CONV: the slot's window origin (may lie outside the image)
         int a_h0[CONV ? A_PW : 1], a_w0[CONV ? A_PW : 1];
         if (CONV) {
 #pragma unroll
@@ -123,17 +125,20 @@ struct PipeKernel {
                 int n = mm / (g.Ho * g.Wo), rem = mm - n * (g.Ho * g.Wo);
                 int ho = rem / g.Wo, wo = rem - ho * g.Wo;
                 a_h0[j] = ho * g.sh - g.ph; a_w0[j] = wo * g.sw - g.pw;
-                a_img[j] = A + (long)n * g.H * g.W * g.lda;
+                a_org[j] = A + ((long)n * g.H * g.W + (long)a_h0[j] * g.W + a_w0[j]) * g.lda;
             }
         } else {
-            a_ptr = A + (long)a_row0 * g.lda;
+            a_par[0] = A + (long)a_row0 * g.lda + chunk_of(wave * A_PW) * VEC;
+            a_par[1] = A + (long)a_row0 * g.lda + chunk_of(wave * A_PW + 1) * VEC;
         }
-        const T *b_ptr = B + (long)b_row0 * g.ldb;
+        const T *b_par[2] = {B + (long)b_row0 * g.ldb + chunk_of(wave * B_PW) * VEC,
+                             B + (long)b_row0 * g.ldb + chunk_of(wave * B_PW + 1) * VEC};
         const bool conv_fast = CONV && (g.Cin % BK == 0);  // a K-step never straddles a filter tap
+        const bool k_full = g.K % BK == 0;                 // no K-chunk of any stage lies past K
 
         // Loads of one stage: slot l < A_PW is an A slot, the rest are B slots.  `StageAddr` holds
         // the wave-uniform part, computed once per stage.
-        struct StageAddr { unsigned sbase; int k0, r_u, s_u, ci_u; };
+        struct StageAddr { unsigned sbase; int k0, r_u, s_u, tap_off; };
         // Stages are fetched in increasing order, so the filter tap (r, s) and channel offset of
         // the next stage advance incrementally instead of being divided out of k every time.
         int nx_r = 0, nx_s = 0, nx_ci = 0;
@@ -141,7 +146,8 @@ struct PipeKernel {
             StageAddr sa;
             sa.sbase = lds0 + (unsigned)(kt % STAGES) * STAGE_BYTES;
             sa.k0 = kt * BK;
-            sa.r_u = nx_r; sa.s_u = nx_s; sa.ci_u = nx_ci;
+            sa.r_u = nx_r; sa.s_u = nx_s;
+            sa.tap_off = (nx_r * g.W + nx_s) * (int)g.lda + nx_ci;  // elements from the window origin
             if (conv_fast) {
                 nx_ci += BK;
                 if (nx_ci >= g.Cin) {
@@ -154,25 +160,33 @@ struct PipeKernel {
         auto issue_one = [&](const StageAddr &sa, int l) {  // l is a compile-time constant at every call
             if (l < A_PW) {
                 const int j = l;
-                const int kc = chunk_of(wave * A_PW + j) * VEC, k = sa.k0 + kc;
-                const T *src = zero;
-                if (a_row0 + j * 8 < g.M && k < g.K) {
-                    if (CONV) {
-                        int r, s2, ci;
-                        if (conv_fast) { r = sa.r_u; s2 = sa.s_u; ci = sa.ci_u + kc; }
-                        else { int rs = k / g.Cin; ci = k - rs * g.Cin; r = rs / g.S; s2 = rs - r * g.S; }
-                        int hi = a_h0[CONV ? j : 0] + r, wi = a_w0[CONV ? j : 0] + s2;
-                        if ((unsigned)hi < (unsigned)g.H && (unsigned)wi < (unsigned)g.W)
-                            src = a_img[CONV ? j : 0] + ((long)hi * g.W + wi) * g.lda + ci;
+                const int kc = chunk_of(wave * A_PW + j) * VEC;
+                const T *src;
+                if (CONV) {
+                    const int jj = CONV ? j : 0;
+                    int r, s2, off;
+                    bool ok = a_row0 + j * 8 < g.M;
+                    if (conv_fast) {
+                        r = sa.r_u; s2 = sa.s_u; off = sa.tap_off + kc;
                     } else {
-                        src = a_ptr + (long)(j * 8) * g.lda + k;
+                        int k = sa.k0 + kc, rs = k / g.Cin, ci = k - rs * g.Cin;
+                        r = rs / g.S; s2 = rs - r * g.S;
+                        off = (r * g.W + s2) * (int)g.lda + ci;
+                        ok = ok & (k < g.K);
                     }
+                    // selects, not branches: every lane computes an address and picks it or the zero page
+                    ok = ok & ((unsigned)(a_h0[jj] + r) < (unsigned)g.H) & ((unsigned)(a_w0[jj] + s2) < (unsigned)g.W);
+                    src = ok ? a_org[jj] + off : zero;
+                } else {
+                    const bool ok = (a_row0 + j * 8 < g.M) & (k_full | (sa.k0 + kc < g.K));
+                    src = ok ? a_par[j & 1] + ((long)(j * 8) * g.lda + sa.k0) : zero;
                 }
                 load_lds16(src, sa.sbase + (unsigned)((wave * A_PW + j) * 8 * RB));
             } else {
                 const int j = l - A_PW;
-                const int k = sa.k0 + chunk_of(wave * B_PW + j) * VEC;
-                const T *src = (b_row0 + j * 8 < g.N && k < g.K) ? b_ptr + (long)(j * 8) * g.ldb + k : zero;
+                const int kc = chunk_of(wave * B_PW + j) * VEC;
+                const bool ok = (b_row0 + j * 8 < g.N) & (k_full | (sa.k0 + kc < g.K));
+                const T *src = ok ? b_par[j & 1] + ((long)(j * 8) * g.ldb + sa.k0) : zero;
                 load_lds16(src, sa.sbase + (unsigned)(A_BYTES + (wave * B_PW + j) * 8 * RB));
             }
         };
@@ -271,6 +285,22 @@ struct PipeKernel {
             }
         };
 
+        // ---- output addressing; the lane's bias values are fetched before the main loop ---------
+        T *C = (T *)g.C + offc;
+        const T *R = g.residual ? (const T *)g.residual + offc : nullptr;
+        const T *bias = (const T *)g.bias;
+        const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
+                            (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
+        constexpr int EPI_L4 = SPLITK ? BN / 4 : 8 * NI;  // lanes per output row (4 columns each)
+        const int epi_c4 = (SPLITK ? tid : lane) % EPI_L4;
+        const int epi_n = n0 + wn * WN + (epi_c4 >> 3) * 32 + (epi_c4 & 7) * 4;
+        // A lane's four columns are the same in every pass, so its bias values are read once; they
+        // stay unconverted until the epilogue so that nothing waits for them before the main loop.
+        Vec4<T> bias_raw;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bias_raw.v[q] = Elem<T>::from_f(0.f);
+        if (bias && vec_ok && epi_n < g.N) bias_raw = *(const Vec4<T> *)(bias + epi_n);
+
         // ---- main loop ------------------------------------------------------------------------
         const int KT = (g.K + BK - 1) / BK;
         GP_PROBE(1);
@@ -290,26 +320,6 @@ struct PipeKernel {
         // full rows instead of one element per lane.  Slice s = (block j, register v) of a wave's
         // accumulators is stored as 64 consecutive floats (one per lane), which is exactly
         // "row 8*(v/4) + 4*(lane/32) + v%4, columns 32*j + lane%32".
-        T *C = (T *)g.C + offc;
-        const T *R = g.residual ? (const T *)g.residual + offc : nullptr;
-        const T *bias = (const T *)g.bias;
-        const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
-                            (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
-        // A lane's four columns are the same in every pass, so its bias values are read once.
-        auto load_bias = [&](int n, float (&bq)[4]) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) bq[q] = 0.f;
-            if (!bias || n >= g.N) return;
-            if (vec_ok) {
-                Vec4<T> bv = *(const Vec4<T> *)(bias + n);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) bq[q] = Elem<T>::to_f(bv.v[q]);
-            } else {
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    if (n + q < g.N) bq[q] = Elem<T>::to_f(bias[n + q]);
-            }
-        };
         // Finishes G rows (m_first, m_first + m_step, ...) of columns n..n+3: the residual reads of
         // the whole group are issued before the first result is needed.
         auto finish_group = [&](auto g_c, int n, const float (&bq)[4], int m_first, int m_step, const f32x4 *a) {
@@ -353,7 +363,26 @@ struct PipeKernel {
             }
         };
         float *red = (float *)lds_t;
+        // (the empty asm pins the conversion here: hoisted next to the load it would wait for it)
+        {
+            typedef unsigned int raw_t __attribute__((ext_vector_type(sizeof(Vec4<T>) / 4)));
+            raw_t raw = __builtin_bit_cast(raw_t, bias_raw);
+#pragma unroll
+            for (int w = 0; w < (int)(sizeof(Vec4<T>) / 4); ++w) {
+                unsigned int x = raw[w];
+                asm volatile("" : "+v"(x));
+                raw[w] = x;
+            }
+            bias_raw = __builtin_bit_cast(Vec4<T>, raw);
+        }
         float bq[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) bq[q] = Elem<T>::to_f(bias_raw.v[q]);
+        if (bias && !vec_ok) {  // unaligned or ragged output: element-wise
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                if (epi_n + q < g.N) bq[q] = Elem<T>::to_f(bias[epi_n + q]);
+        }
         if (!SPLITK) {
             // each wave transposes its own 32-row strips through a private NI x 4 KB region
             float *mine = red + (size_t)wave * NI * 16 * 64;
@@ -364,7 +393,6 @@ struct PipeKernel {
             const int c4 = lane % L4, r_in = lane / L4;
             const int j = c4 >> 3, col = (c4 & 7) * 4;
             const int n = n0 + wn * WN + j * 32 + col;
-            load_bias(n, bq);
             __syncthreads();  // all waves are done reading the stage buffers
             static_for<0, MI>([&](auto ic) {
                 constexpr int i = ic;
@@ -398,7 +426,6 @@ struct PipeKernel {
             const int c4 = tid % L4, r_in = tid / L4;
             const int j = c4 >> 3, col = (c4 & 7) * 4;
             const int n = n0 + j * 32 + col;
-            load_bias(n, bq);
             __syncthreads();  // all waves are done reading the stage buffers
 #pragma unroll
             for (int i = 0; i < MI; ++i)

@@ -166,8 +166,9 @@ def _blp_roundtrip(gp, ex_mod, tmp_path, workload, x_raw, injections, graph=Fals
         ex.inject_preempt(-1, -1)
         flag.set(0)  # host clears the flag, then resumes (test-dnn-blp.cpp:41-42)
         ex.resume(stream)
-        if program and ex.last_stop_index() == -1:
+        if ex.last_stop_index() == -1:
             # the flag went up so late that no later claim looked at it: the model had finished
+            # (only some claims read the flag, and the last kernels are short)
             assert kernel >= n - 3, (kernel, n)
         else:
             assert kernel <= ex.last_stop_index() <= kernel + slack, (ex.last_stop_index(), kernel)
