@@ -25,6 +25,11 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs of
+# `bench.py --only roofline` (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads
+# for the copy of `--only copycal`); the figures and commands are in the hbm_traffic summary
+# under profiles/.  Counters cannot be collected from inside this process.
+HBM_TRAFFIC_PER_LAUNCH = {("resnet152", "f16"): 10.55e6}
 
 
 def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
@@ -95,6 +100,16 @@ def roofline(workload, iters, dt):
     ex.execute(stream)  # warm-up, also resolves launch geometry
     stream.sync()
     ev = [(gp.Event(), gp.Event()) for _ in conv]
+    # what an event pair reads with nothing between its two records: subtracted from every bracket
+    # below, so that the figure is the kernel's own duration, as a kernel trace reports it
+    empty = []
+    for a, b in ev[:64]:
+        a.record(stream)
+        b.record(stream)
+    stream.sync()
+    for a, b in ev[:64]:
+        empty.append(a.elapsed_ms(b))
+    bracket_ms = sorted(empty)[len(empty) // 2]
     total_ms, total_flop, total_bytes, launches = 0.0, 0.0, 0.0, 0
     for _ in range(iters):
         # one pass through the reference's launch_kernel API, events around each convolution
@@ -110,15 +125,16 @@ def roofline(workload, iters, dt):
                 ex.launch_kernel(i, stream)
         stream.sync()
         for (a, b), i in zip(ev, conv):
-            total_ms += a.elapsed_ms(b)
+            total_ms += max(a.elapsed_ms(b) - bracket_ms, 1e-4)
             total_flop += kernels[i]["flops"]
             total_bytes += kernels[i]["bytes"]
             launches += 1
     ex.destroy()
     achieved = total_flop / (total_ms * 1e-3) / 1e12
-    return {"bound": "mfma", "kernel": "mat_kernel<TileKernel<f16,conv>> (implicit-GEMM conv2d of " + workload + ")",
-            "achieved": achieved, "peak": PEAK[dt], "unit": "TFLOP/s", "frac": achieved / PEAK[dt], "traffic": None,
-            "launches": launches, "avg_launch_us": total_ms * 1e3 / launches,
+    return {"bound": "mfma", "kernel": "mat_kernel<PipeKernel<f16,conv>> (implicit-GEMM conv2d of " + workload + ", preemptible launches)",
+            "achieved": achieved, "peak": PEAK[dt], "unit": "TFLOP/s", "frac": achieved / PEAK[dt],
+            "traffic": HBM_TRAFFIC_PER_LAUNCH.get((workload, dt)),
+            "launches": launches, "avg_launch_us": total_ms * 1e3 / launches, "event_bracket_us": bracket_ms * 1e3,
             "algorithmic_flop_per_launch": total_flop / launches, "algorithmic_bytes_per_launch": total_bytes / launches}
 
 

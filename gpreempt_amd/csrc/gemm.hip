@@ -42,6 +42,7 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     }
     int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info);
     if (rc) return rc;
+    blp.order = pl.order;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(K::NT), K::LDS_BYTES, native(s), pl.g, blp);
     GP_HIP(hipGetLastError());
     return GP_SUCC;
@@ -145,6 +146,12 @@ static int choose_body(MatPlan *pl, int tile, int variant) {
     pl->sx = (g.N + t - 1) / t;
     pl->sy = (g.M + t - 1) / t;
     pl->lds_bytes = body_lds_bytes(body, pl->dtype);
+    // Each XCD works on a contiguous eighth of the tile order (util/slice_map.h).  With x fastest
+    // that is a band of tile rows: every XCD fetches its share of A and all of B; with y fastest
+    // it is a band of tile columns: all of A and a share of B.  Take the cheaper one.
+    const double a_elems = pl->conv ? (double)(g.M / (g.Ho * g.Wo > 0 ? g.Ho * g.Wo : 1)) * g.H * g.W * g.Cin : (double)g.M * g.K;
+    const double b_elems = (double)g.N * g.K;
+    pl->order = b_elems > a_elems ? 1 : 0;
     return GP_SUCC;
 }
 

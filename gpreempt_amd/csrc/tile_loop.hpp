@@ -20,6 +20,7 @@
 //    (the reference builds a second, untransformed module for that: mod.cubin vs mod.tr.cubin).
 #pragma once
 #include <hip/hip_runtime.h>
+#include "../../include/util/slice_map.h"
 
 namespace gp {
 
@@ -33,32 +34,33 @@ struct BlpArgs {
     int inject_at;    // -1 = off
     int poll_mask;    // the claim numbered c reads the host flag when (c & poll_mask) == 0
     int groups;       // claim counters per kernel (>= 1); counter g sits at executed + g * COUNTER_STRIDE
+    int order;        // tile order: 0 = x fastest (the reference's), 1 = y fastest
 };
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
 // few hundred tiles claimed from a single counter spends 10-20 us on claims alone.  A caller may
-// therefore give a kernel `groups` counters, one per 64-byte line: workgroup w claims from counter
-// w % groups, which owns the contiguous slice [total*g/groups, total*(g+1)/groups) of the tiles.
+// therefore give a kernel `groups` counters, one per 64-byte line; util/slice_map.h says which
+// counter a workgroup claims from and which contiguous slice of the tile order that counter owns.
 // groups == 1 is the reference's layout (one int per kernel).
 constexpr int COUNTER_STRIDE = 16;  // ints
 
-// First tile of group g's slice when `grid` workgroups are spread round-robin over `groups`
-// counters: groups [0, grid % groups) hold one workgroup more than the others.
-__host__ __device__ inline int group_slice_begin(int total, int g, int groups, int grid) {
-    const int q = grid / groups, r = grid % groups;
-    const long w = (long)g * q + (g < r ? g : r);  // workgroups in the groups before g
-    return (int)((long)total * w / grid);
-}
-
 struct TileIdx { int x, y, z; };
 
-__device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy) {
-    // x = idx % sx; y = (idx / sx) % sy; z = idx / (sx*sy)   (convert_to_blp.py:52-54)
+__device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy, int order = 0) {
+    // x = idx % sx; y = (idx / sx) % sy; z = idx / (sx*sy)   (convert_to_blp.py:52-54);
+    // order 1 swaps the roles of x and y, so that consecutive indices share a tile column
     TileIdx t;
-    int q = idx / sx;
-    t.x = idx - q * sx;
-    t.z = q / sy;
-    t.y = q - t.z * sy;
+    if (order == 0) {
+        int q = idx / sx;
+        t.x = idx - q * sx;
+        t.z = q / sy;
+        t.y = q - t.z * sy;
+    } else {
+        int q = idx / sy;
+        t.y = idx - q * sy;
+        t.z = q / sx;
+        t.x = q - t.z * sx;
+    }
     return t;
 }
 
@@ -69,10 +71,8 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     __shared__ int mailbox[2];
     const bool dynamic = b.executed != nullptr;
     const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
-    // Slices are proportional to the number of workgroups that serve them (workgroup w serves
-    // group w % groups), so that a launch with one workgroup per tile gives every workgroup
-    // exactly one tile.
-    const int grp = b.groups > 1 ? (int)(blockIdx.x % (unsigned)b.groups) : 0;
+    // which counter this workgroup serves and the slice of the tile order that counter owns
+    const int grp = wg_group((int)blockIdx.x, b.groups);
     const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
     const int slice_n = (b.groups > 1 ? group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) : b.total) - slice_lo;
     // One loop and one call site for both modes, so that the body is inlined into the kernel and
@@ -80,7 +80,7 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     for (int it = 0;; ++it) {
         int idx;
         if (!dynamic) {
-            idx = (it == 0 && (int)blockIdx.x < b.total) ? (int)blockIdx.x : -1;
+            idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
         } else {
             if (leader) {
                 // The stop index (device memory) doubles as the device-side mirror of the flag:
@@ -118,7 +118,7 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
             idx = mailbox[it & 1];
         }
         if (idx < 0) return;
-        body(decode_tile(idx, b.sx, b.sy));
+        body(decode_tile(idx, b.sx, b.sy, b.order));
     }
 }
 

@@ -1,6 +1,7 @@
 // Executor launch loop and the block-level-preemption protocol on the host side.
 // Behaviour follows the reference's src/executor.cpp (cited per function).
 #include "executor.h"
+#include "util/slice_map.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -235,7 +236,7 @@ Status BLPExecutor::read_counters(std::vector<int> &out) {
         if (model->counter_groups() == 1) { out[i] = raw[i]; continue; }
         // slices follow the workgroup distribution of the last launch (device layer, tile_loop.hpp)
         const long grid = std::max<long>(1, model->get_kernel_info(i).launch_params[0]);
-        auto begin = [&](long g) { long q = grid / kCounterGroups, r = grid % kCounterGroups; return total * (g * q + std::min(g, r)) / grid; };
+        auto begin = [&](int g) { return (long)gp::group_slice_begin((int)total, g, kCounterGroups, (int)grid); };
         for (int g = 0; g < kCounterGroups; ++g) {
             long size = begin(g + 1) - begin(g);
             long c = raw[(i * kCounterGroups + g) * kCounterStride];
