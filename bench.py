@@ -36,11 +36,13 @@ def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
     """Two tenants through the C++ harness (gpx_run_scenario).  The high-priority tenant submits
     launch by launch (it is never preempted and plain launches are its fastest path); the
     best-effort tenant runs as one persistent, preemptible program kernel, except under
-    "wb-chunk", which feeds its kernels a few at a time."""
+    "wb-chunk" and "wb-chunk-async", which feed its preemptible kernels a few at a time.  Under the
+    "-async" policies the high-priority tenant submits as soon as it has raised the flag instead
+    of waiting for the best-effort tenant to have left the GPU."""
     from gpreempt_amd import executor as gx
     cfg = {
         "time": max(5.0, 4.0 * steps / hp_rate), "policy": policy, "hp_requests": steps,
-        "warmups": warmup, "standalone_runs": 100,
+        "warmups": warmup, "standalone_runs": 300,
         "tasks": [
             {"id": "hp", "load": {"type": "poisson", "frequency": hp_rate, "seed": 2025},
              "client": {"name": "hp", "model_name": hp_model, "priority": 0, "use_cuda_graph": False, "launch_mode": "launch", "preprocess_time": 0}},
@@ -209,7 +211,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=600)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--policy", default="wb-async")
+    ap.add_argument("--policy", default="wb-chunk-async")
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
@@ -233,7 +235,7 @@ def main():
         if not args.only:
             # the other policies and the single-tenant probe ride along as context
             out["other_policies"] = {}
-            for pol in ("wb", "wb-async", "wb-chunk", "np"):
+            for pol in ("wb", "wb-async", "wb-chunk", "wb-chunk-async", "np"):
                 if pol != args.policy:
                     out["other_policies"][pol] = summarize(scenario(max(200, args.steps // 2), args.warmup, pol, args.hp_rate, args.be_model, args.hp_model))
             out["config2_resnet50_fp32_b1"] = probe("resnet50", 300)

@@ -25,6 +25,12 @@
 
 namespace foo {
 
+// Policy names: "wb" (reference), "wb-async", "wb-chunk", "wb-chunk-async".
+static bool is_wb(const std::string &p) { return p == "wb" || p == "wb-async" || p == "wb-chunk" || p == "wb-chunk-async"; }
+static bool is_chunked(const std::string &p) { return p == "wb-chunk" || p == "wb-chunk-async"; }
+static bool is_async(const std::string &p) { return p == "wb-async" || p == "wb-chunk-async"; }
+
+
 using clock_type = std::chrono::steady_clock;
 static inline int64_t now_ns() { return std::chrono::duration_cast<std::chrono::nanoseconds>(clock_type::now().time_since_epoch()).count(); }
 static inline void spin_pause() { __builtin_ia32_pause(); }
@@ -169,7 +175,7 @@ void fill_input(Tenant &t) {
 }
 
 Status init_tenant(Tenant &t, Shared &sh) {
-    const bool preemptible = t.priority > 0 && (sh.policy == "wb" || sh.policy == "wb-async" || sh.policy == "wb-chunk");
+    const bool preemptible = t.priority > 0 && is_wb(sh.policy);
     if (preemptible) { t.blp = new BLPExecutor(); t.ex.reset(t.blp); }
     else t.ex.reset(new BaseExecutor());
     RETURN_STATUS(t.ex->init(t.model_name));
@@ -185,7 +191,7 @@ Status init_tenant(Tenant &t, Shared &sh) {
     }
     // "wb-chunk" feeds a preemptible tenant's kernels a few at a time, so it never uses a
     // captured graph or program for that tenant.
-    const bool chunked = t.blp && sh.policy == "wb-chunk";
+    const bool chunked = t.blp && is_chunked(sh.policy);
     if (!chunked && t.launch_mode != "launch") {
         setenv("GPREEMPT_USE_HIPGRAPH", t.launch_mode == "graph" ? "1" : "0", 1);
         t.ex->capture_graph(t.stream);
@@ -222,12 +228,18 @@ Status drain(GPUstream s) {
     }
 }
 
-// "wb-chunk": the best-effort model is submitted launch by launch (Executor::launch_kernel, the
-// reference's own launch loop, src/executor.cpp:222-225) but never more than two chunks of
-// kChunk kernels ahead of the GPU.  A preempted model then has at most 2*kChunk queued kernels
-// to flush (each leaves at its first look at the stop index) instead of the rest of the network,
-// which bounds the drain at tens of microseconds while keeping per-kernel occupancy.
-constexpr int kChunk = 6;
+// "wb-chunk" / "wb-chunk-async": the best-effort model is submitted launch by launch
+// (Executor::launch_kernel, the reference's own launch loop, src/executor.cpp:222-225) but never
+// more than two chunks of kernels ahead of the GPU.  A preempted model then has at most two chunks
+// of queued kernels to flush (each leaves at its first look at the stop index, about 6 us apiece
+// on MI355X) instead of the rest of the network, while every kernel keeps its own occupancy.
+// Measured with BERT over ResNet-152: chunks of 6 / 3 / 2 / 1 kernels drain in 88 / 55 / 44 / 32 us
+// (mean) and cost 0 / 3 / 6 / 14 % of the best-effort throughput; the default is 2
+// (environment variable GPREEMPT_CHUNK overrides it).
+static int chunk_size() {
+    static const int v = [] { const char *e = getenv("GPREEMPT_CHUNK"); int c = e ? atoi(e) : 2; return c < 1 ? 1 : c; }();
+    return v;
+}
 Status infer_chunked(Tenant &t, Shared &sh, int p) {
     BLPExecutor *ex = t.blp;
     const size_t n = ex->get_kernel_num();
@@ -258,7 +270,7 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             continue;
         }
         if (next < n && inflight < 2) {
-            size_t end = std::min(n, next + kChunk);
+            size_t end = std::min(n, next + (size_t)chunk_size());
             for (size_t i = next; i < end && st == Status::Succ; ++i) st = ex->launch_kernel(i, t.stream);
             if (st != Status::Succ) break;
             if (gp_event_record(t.chunk_events[tail], t.stream) != 0) { st = Status::Fail; break; }
@@ -297,7 +309,7 @@ Status infer(Tenant &t, Shared &sh) {
         if (p == 0) sh.seq_waiting.fetch_sub(1);
         return Status::Succ;
     }
-    if (pol == "np" || pol == "lco" || !(pol == "wb" || pol == "wb-async" || pol == "wb-chunk")) {
+    if (!is_wb(pol)) {  // "np", "lco" and anything unknown
         // baseclient.cpp: every tenant submits on its own stream, nothing is preempted
         int64_t t0 = now_ns();
         RETURN_STATUS(t.ex->execute(t.stream));
@@ -310,12 +322,12 @@ Status infer(Tenant &t, Shared &sh) {
     int64_t t0 = now_ns();
     // "wb" / "wb-chunk": wait until lower-priority work has left the GPU (blpclient.cpp:189);
     // "wb-async" submits at once and lets the hardware start workgroups as the others retire.
-    if (pol != "wb-async") while (sh.on_gpu_below(p) > 0) spin_pause();
+    if (!is_async(pol)) while (sh.on_gpu_below(p) > 0) spin_pause();
     Status st = Status::Succ;
     if (!t.blp) {
         st = t.ex->execute(t.stream);
         if (st == Status::Succ) st = drain(t.stream);
-    } else if (pol == "wb-chunk") {
+    } else if (is_chunked(pol)) {
         while (sh.active_above(p) > 0) spin_pause();
         st = infer_chunked(t, sh, p);
     } else {
@@ -352,7 +364,7 @@ Status infer(Tenant &t, Shared &sh) {
     return st;
 }
 
-static bool preempting_policy(const Shared &sh) { return sh.policy == "wb" || sh.policy == "wb-async" || sh.policy == "wb-chunk"; }
+static bool preempting_policy(const Shared &sh) { return is_wb(sh.policy); }
 
 // A request of level p announces itself before it touches the GPU at all (its input copy
 // included): a persistent best-effort kernel leaves no gap for even a small copy kernel, so the
