@@ -170,6 +170,10 @@ Status Model::upload_param(size_t idx, const float *disk, size_t n) {
                         for (int s = 0; s < L.s; ++s)
                             dev[(((size_t)o * L.r + r) * L.s + s) * L.i_pad + i] = disk[(((size_t)o * L.i + i) * L.r + r) * L.s + s];
             break;
+        case ParamLayout::MatKN:  // K x N -> N x K: the matrix kernels want both operands K-contiguous
+            for (int k = 0; k < L.i; ++k)
+                for (int nn = 0; nn < L.o; ++nn) dev[(size_t)nn * L.i + k] = disk[(size_t)k * L.o + nn];
+            break;
         case ParamLayout::DenseOverCHW: {
             size_t feat = (size_t)L.c * L.h * L.w;
             for (int o = 0; o < L.o; ++o)

@@ -198,6 +198,8 @@ bool valid_dtype(const std::string &d) { return d == "f32" || d == "f16" || d ==
 
 // ---- config 1 / config 5: C = act(A * B + bias) as a one-kernel model --------------------------
 // storages: "data" = A (M x K), "B" (K x N, or N x K with layout=nk), "bias" (N), "heads" = C.
+// B is a parameter: whatever its layout on disk, the device copy is N x K (K-contiguous rows feed
+// the direct-to-LDS loads), as convolution weights are re-laid out at load time.
 Status build_gemm(Model &m, const Options &o, int M, int N, int K, const std::string &dt_default, int act_default) {
     std::string dt = o.gets("dtype", dt_default);
     if (!valid_dtype(dt)) return Status::OutOfRange;
@@ -208,6 +210,7 @@ Status build_gemm(Model &m, const Options &o, int M, int N, int K, const std::st
     int tile = o.geti("tile", 0);
     size_t a = g.add_storage("data", (size_t)M * K, g.stype_);
     ParamLayout LB; LB.disk_elems = (size_t)K * N; LB.init = ParamLayout::InitUniform; LB.init_a = -1.f; LB.init_b = 1.f;
+    if (!nk) { LB.kind = ParamLayout::MatKN; LB.i = K; LB.o = N; }
     size_t b = g.add_param("B", (size_t)K * N, LB);
     ParamLayout Lb; Lb.disk_elems = N; Lb.init = ParamLayout::InitUniform; Lb.init_a = -0.1f; Lb.init_b = 0.1f;
     size_t bias = g.add_param("bias", N, Lb);
@@ -217,7 +220,7 @@ Status build_gemm(Model &m, const Options &o, int M, int N, int K, const std::st
     double bytes = g.es() * ((double)M * K + (double)K * N + (use_bias ? N : 0) + (double)M * N);
     KernelInfo &k = g.add_kernel("gemm", OpKind::Gemm, {GraphBuilder::ref(a), GraphBuilder::ref(b), use_bias ? GraphBuilder::ref(bias) : GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(c)}, flops, bytes);
     gp_gemm_params &p = k.p.gemm;
-    p.dtype = g.gp_dtype(); p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = nk ? K : N; p.b_is_nk = nk; p.ldc = N; p.alpha = 1.f; p.act = act; p.batch = 1;
+    p.dtype = g.gp_dtype(); p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = K; p.b_is_nk = 1; p.ldc = N; p.alpha = 1.f; p.act = act; p.batch = 1;
     p.tile_m = p.tile_n = tile;
     return Status::Succ;
 }

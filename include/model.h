@@ -28,8 +28,8 @@ public:
 // weights; dense weights [out][in] over an NCHW flatten) maps onto the device layout
 // (model dtype; [O][H][W][I padded]; dense over an NHWC flatten).
 struct ParamLayout {
-    enum Kind { Plain, ConvOIHW, DenseOverCHW } kind = Plain;
-    int o = 0, i = 0, r = 0, s = 0, i_pad = 0;  // ConvOIHW
+    enum Kind { Plain, ConvOIHW, DenseOverCHW, MatKN } kind = Plain;
+    int o = 0, i = 0, r = 0, s = 0, i_pad = 0;  // ConvOIHW; MatKN: a K x N matrix on disk (i = K, o = N), kept N x K on the device
     int c = 0, h = 0, w = 0;                    // DenseOverCHW: input features were flattened from C x H x W
     size_t disk_elems = 0;                      // fp32 values expected on disk
     bool is_param = false;
