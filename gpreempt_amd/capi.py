@@ -22,7 +22,8 @@ vp = C.c_void_p
 
 class PreemptCtx(C.Structure):
     _fields_ = [("flag", vp), ("stop_index", vp), ("executed", vp), ("kernel_id", C.c_int),
-                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("left_host", vp)]
+                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("left_host", vp),
+                ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong)]
 
 
 class LaunchInfo(C.Structure):
@@ -82,7 +83,7 @@ SYMBOLS = """gp_init gp_last_error gp_device_info gp_stream_create gp_stream_des
 gp_stream_query gp_stream_priority gp_stream_native gp_event_create gp_event_destroy gp_event_record
 gp_event_sync gp_event_query gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free gp_memcpy_h2d gp_memcpy_d2h
 gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_flag_relay_start
-gp_launch_gemm gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
+gp_launch_gemm gp_gemm_ckpt_bytes gp_ckpt_reset_async gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
 gp_launch_layernorm gp_launch_embed gp_launch_gate gp_launch_noop gp_graph_begin gp_graph_end gp_graph_launch
 gp_graph_destroy gp_program_create gp_program_destroy gp_program_add_gemm gp_program_add_conv2d
 gp_program_add_nchw_to_nhwc gp_program_add_pool2d gp_program_add_eltwise gp_program_add_softmax gp_program_add_layernorm
@@ -276,7 +277,25 @@ class BlpState:
         self.executed.upload(np.zeros(self.n, np.int32))
 
     def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0):
-        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id, kernel_id, inject_at, max_workgroups, poll_every, 0, None)
+        ck = getattr(self, "ckpt", None)
+        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id, kernel_id, inject_at, max_workgroups, poll_every, 0, None,
+                          ck.ptr if ck else None, ck.nbytes if ck else 0)
+
+    def enable_checkpoints(self, params):
+        """Allocates the workspace that lets the GEMM `params` leave its tiles half-way (if it can)."""
+        n = C.c_size_t(0)
+        check(lib().gp_gemm_ckpt_bytes(C.byref(params), C.byref(n)))
+        self.ckpt = DevBuf(n.value) if n.value else None
+        if self.ckpt:
+            check(lib().gp_ckpt_reset_async(vp(self.ckpt.ptr), None))
+            check(lib().gp_stream_sync(None))
+        return n.value
+
+    def checkpoint_headers(self, n):
+        """valid / kernel id / tile / next K-step of the first n workgroup slots."""
+        raw = np.empty(n * 16, np.int32)
+        check(lib().gp_memcpy_d2h(raw.ctypes.data_as(vp), vp(self.ckpt.ptr), C.c_size_t(raw.nbytes)))
+        return raw.reshape(n, 16)[:, :4].copy()
 
     def stop_index(self):
         return int(self.stop.download(np_dtype=np.int32)[0])

@@ -51,7 +51,7 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
                 const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info) {
     long total = (long)sx * sy * sz;
     GP_REQUIRE(total > 0 && total < (1L << 31), "tile count %ld out of range", total);
-    blp->total = (int)total; blp->sx = sx; blp->sy = sy; blp->order = 0;
+    blp->total = (int)total; blp->sx = sx; blp->sy = sy; blp->order = 0; blp->ckpt = nullptr;
     if (ctx) {
         GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
         blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;

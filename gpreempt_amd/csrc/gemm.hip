@@ -25,14 +25,33 @@ __global__ __launch_bounds__(TK::NT) void mat_kernel(MatArgs g, BlpArgs blp) {
     tile_loop(blp, [&](TileIdx t) { TK::run(g, t, lds); });
 }
 
+// bodies that can leave a tile between two K-steps (tile_loop_ckpt)
+template <class TK>
+__global__ __launch_bounds__(TK::NT) void mat_kernel_ckpt(MatArgs g, BlpArgs blp) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+    auto *lds = reinterpret_cast<typename TK::elem *>(lds_raw);
+    const CkptCtx cc = {blp.executed && blp.ckpt ? blp.stop_index : nullptr, blp.flag, blp.ckpt, blp.kernel_id};
+    tile_loop_ckpt(blp, [&](TileIdx t, int tile_index, int kt0) { return TK::run(g, t, lds, cc, tile_index, kt0); });
+}
+
 template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool CONV, bool B_KN>
 using TK = TileKernel<T, BM, BN, BK, WGM, WGN, CONV, B_KN>;
+
+template <class K> struct K_is_ckpt { static constexpr bool value = false; };
+template <typename T> struct K_is_ckpt<PipeKernel<T, 256, 256, 2, false, false, true>> { static constexpr bool value = true; };
+template <class K> struct KernelOf { static constexpr auto fn = mat_kernel<K>; };
+template <typename T> struct KernelOf<PipeKernel<T, 256, 256, 2, false, false, true>> {
+    static constexpr auto fn = mat_kernel_ckpt<PipeKernel<T, 256, 256, 2, false, false, true>>;
+};
+
+// bytes of checkpoint workspace a launch of body K needs (0: the body always finishes its tiles)
+static size_t ckpt_workspace_bytes(size_t slot_bytes) { return (size_t)CKPT_MAX_WGS * (CKPT_HEADER_INTS * 4 + slot_bytes); }
 
 template <class K>
 static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     BlpArgs blp;
     int grid = 0;
-    auto kern = mat_kernel<K>;
+    auto kern = KernelOf<K>::fn;
     if (K::LDS_BYTES > 48 * 1024) {
         static bool once = false;  // benign race: idempotent attribute
         if (!once) {
@@ -43,6 +62,10 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info);
     if (rc) return rc;
     blp.order = pl.order;
+    if constexpr (K_is_ckpt<K>::value) {
+        // mid-tile checkpoints need the caller's workspace and a slot per workgroup
+        if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
+    }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(K::NT), K::LDS_BYTES, native(s), pl.g, blp);
     GP_HIP(hipGetLastError());
     return GP_SUCC;
@@ -69,7 +92,9 @@ static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream 
     constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
     switch (pl.body) {
         case MB_PIPE256:  // GEMM only: the gathered A operand of a convolution does not fit its register budget
-            return launch_mat<PipeKernel<T, 256, 256, 2, false, false>>(pl, ctx, s, info);
+            // the checkpointing instantiation only when the caller brought a workspace
+            if (ctx && ctx->ckpt) return launch_mat<PipeKernel<T, 256, 256, 2, false, false, true>>(pl, ctx, s, info);
+            return launch_mat<PipeKernel<T, 256, 256, 2, false, false, false>>(pl, ctx, s, info);
         case MB_PIPE128: return pipe_case<T, 128, GP_S128, false>(pl, ctx, s, info);
         case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
         case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
@@ -100,7 +125,7 @@ int launch_mat_plan(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
 static size_t body_lds_bytes(int body, int dtype) {
     const size_t es = dtype == GP_F32 ? 4 : 2;
     switch (body) {
-        case MB_PIPE256: return 2 * (256 + 256) * 128;
+        case MB_PIPE256: return 2 * (256 + 256) * 128 + 16;
         case MB_PIPE128: return GP_S128 * (128 + 128) * 128;
         case MB_PIPE64: return GP_S64 * (64 + 64) * 128;
         case MB_PIPE64_SK: return GP_S64 * (64 + 64) * 128;   // at least the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4 = 64 KB)
@@ -243,3 +268,18 @@ extern "C" int gp_debug_tile_prof(unsigned long long *out, int n) {
     return GP_SUCC;
 }
 #endif
+
+// Checkpoint workspace of the bodies that can leave a tile half-way (only the 256 x 256 GEMM body).
+extern "C" int gp_gemm_ckpt_bytes(const gp_gemm_params *p, size_t *bytes) {
+    GP_REQUIRE(bytes != nullptr, "null bytes");
+    MatPlan pl;
+    int rc = plan_gemm(p, &pl);
+    if (rc) return rc;
+    *bytes = pl.body == MB_PIPE256 ? ckpt_workspace_bytes(PipeKernel<float, 256, 256, 2, false, false, true>::CKPT_SLOT_BYTES) : 0;
+    return GP_SUCC;
+}
+
+extern "C" int gp_ckpt_reset_async(void *ckpt, gp_stream s) {
+    GP_REQUIRE(ckpt != nullptr, "null checkpoint workspace");
+    return gp_fill32_async(ckpt, 0, (size_t)CKPT_MAX_WGS * CKPT_HEADER_INTS, s);
+}

@@ -64,7 +64,18 @@ template <typename T> __device__ __forceinline__ void st_vec4(T *p, Vec4<T> o) {
     else st_out64(p, __builtin_bit_cast(unsigned long long, o));
 }
 
-template <typename T, int BM, int BN, int STAGES, bool CONV, bool SPLITK>
+// CKPT = true (two-stage GEMM bodies only): the tile can be left between two K-steps; see
+// tile_loop_ckpt in tile_loop.hpp.  One lane of the workgroup reads the stop index once per
+// K-step (and, in the first eight workgroups, now and then the host flag); the answer reaches the
+// other waves through an LDS word one K-step later, so nothing waits for the stop-index read.
+struct CkptCtx {       // what a checkpointing body needs from the dispatcher, passed by value
+    int *stop_index;   // nullptr: never leave a tile
+    int *flag;
+    void *ckpt;
+    int kernel_id;
+};
+
+template <typename T, int BM, int BN, int STAGES, bool CONV, bool SPLITK, bool CKPT = false>
 struct PipeKernel {
     using elem = T;
     static constexpr int bm = BM, bn = BN;
@@ -79,11 +90,17 @@ struct PipeKernel {
     static constexpr int WGM = SPLITK ? 1 : 2, WGN = SPLITK ? 1 : 2;
     static constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 32, NI = WN / 32;
     static constexpr size_t RED_BYTES = (size_t)WAVES * (SPLITK ? MI : 1) * NI * 16 * 64 * 4;  // epilogue staging
-    static constexpr size_t LDS_BYTES = (size_t)STAGES * STAGE_BYTES > RED_BYTES ? (size_t)STAGES * STAGE_BYTES : RED_BYTES;
+    static constexpr size_t RING_BYTES = (size_t)STAGES * STAGE_BYTES > RED_BYTES ? (size_t)STAGES * STAGE_BYTES : RED_BYTES;
+    static constexpr size_t LDS_BYTES = RING_BYTES + (CKPT ? 16 : 0);  // + the stop words of a checkpointing body
+    static constexpr size_t CKPT_SLOT_BYTES = (size_t)WAVES * MI * NI * 16 * 64 * 4;  // one workgroup's accumulators
+    static constexpr bool ckpt = CKPT;
+    static_assert(!CKPT || (STAGES == 2 && !CONV && !SPLITK), "checkpointing is built for the two-stage GEMM body");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && A_PW >= 1 && B_PW >= 1, "tile shape");
     static_assert(STAGES >= 2 && (STAGES - 2) * LPS < 64, "pipeline depth");
 
-    static __device__ __forceinline__ void run(const MatArgs &g, TileIdx t, T *lds_t) {
+    // Returns true when the tile was left half-way (CKPT only); kt0 > 0 continues such a tile.
+    static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0},
+                                               int tile_index = 0, int kt0 = 0) {
         GP_PROBE(0);
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
@@ -203,6 +220,29 @@ struct PipeKernel {
             for (int j = 0; j < NI; ++j)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+        // checkpointing state
+        const bool can_ckpt = CKPT && cc.stop_index != nullptr && cc.ckpt != nullptr;
+        f32x4 *slot = nullptr;       // this wave's part of the workgroup's checkpoint slot
+        // two LDS words behind the ring, indexed by K-step parity
+        typedef __attribute__((address_space(3))) volatile int lds_vint;
+        lds_vint *stopw = (lds_vint *)(__attribute__((address_space(3))) void *)lds_t + RING_BYTES / 4;
+        if (CKPT && can_ckpt) {
+            slot = (f32x4 *)((char *)cc.ckpt + (size_t)CKPT_MAX_WGS * CKPT_HEADER_INTS * 4 + (size_t)blockIdx.x * CKPT_SLOT_BYTES) +
+                   (size_t)wave * MI * NI * 4 * 64;
+            if (kt0 > 0) {
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            f32x4 v = slot[((i * NI + j) * 4 + q) * 64 + lane];
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = v[e];
+                        }
+            }
+        }
+        int polled_stop = -1, polled_flag = 0;  // what lane 0 of wave 0 read one K-step ago
 
         const int wm = SPLITK ? 0 : wave / WGN, wn = SPLITK ? 0 : wave % WGN;
         auto frag = [&](int stage, int region_bytes, int row, int chunk) -> u32x4 {
@@ -248,12 +288,34 @@ struct PipeKernel {
             });
         };
         // k-tile kt: wait for its stage, start fetching stage kt+STAGES-1 (ISSUE) and multiply.
-        auto ktile = [&](int kt, bool tail, auto issue_c) {
+        auto ktile = [&](int kt, bool tail, auto issue_c) -> int {
             constexpr bool ISSUE = decltype(issue_c)::value != 0;
             // stage kt has landed once at most the loads of the younger in-flight stages remain
             if (!tail) wait_vmcnt<(STAGES - 2) * LPS>();
             else wait_vmcnt<0>();
+            int stop_now = 0, stop_word = 0;
+            if constexpr (CKPT) {
+                if (can_ckpt && tid == 0) {
+                    // publish last K-step's reads (they have landed: the wait above was for vmcnt 0)
+                    if (polled_flag != 0) atomicCAS(cc.stop_index, -1, cc.kernel_id);
+                    stopw[kt & 1] = (polled_stop != -1) | (polled_flag != 0);
+                }
+            }
             __syncthreads();  // everyone's part of stage kt is visible; stage kt-1's buffer is free
+            if constexpr (CKPT) {
+                if (can_ckpt) {
+                    stop_word = stopw[kt & 1];  // the same word for every wave: a uniform decision, looked at below
+                    if (tid == 0) {
+                        polled_stop = __hip_atomic_load(cc.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        // The flag is host memory: its read takes about as long as a K-step and the
+                        // next K-step's vmcnt(0) waits for it.  So eight workgroups take turns, each
+                        // reading it once in 16 K-steps: a read every second K-step overall, 6 %
+                        // of a K-step per polling workgroup.
+                        if (blockIdx.x < 8 && cc.flag && (kt & 15) == (int)blockIdx.x * 2)
+                            polled_flag = __hip_atomic_load(cc.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    }
+                }
+            }
             if (kt == 0) GP_PROBE(2);
             const int stage = kt % STAGES;
             StageAddr sa = {};
@@ -266,7 +328,7 @@ struct PipeKernel {
                 constexpr int LAST = (KSTEPS - 1) & 1;
                 read_frags(0, stage, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                if (kt > 0) {
+                if (kt > kt0) {
                     phase(LAST, issue_c, sa, IntC<0>{});  // last k-step of stage kt-1 (in registers)
                 } else if constexpr (ISSUE) {
                     static_for<0, NM>([&](auto qc) {  // first k-tile: phase 0 has loads but no MFMAs
@@ -283,6 +345,8 @@ struct PipeKernel {
                 });
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if constexpr (CKPT) stop_now = __builtin_amdgcn_readfirstlane(stop_word);
+            return stop_now;
         };
 
         // ---- output addressing; the lane's bias values are fetched before the main loop ---------
@@ -307,12 +371,20 @@ struct PipeKernel {
         __syncthreads();  // the previous tile of this workgroup may still be reading LDS
 #pragma unroll
         for (int s = 0; s < STAGES - 1; ++s)
-            if (s < KT) issue(s);
-        int kt = 0;
-        for (; kt + STAGES - 1 < KT; ++kt) ktile(kt, false, IntC<1>{});
-        for (; kt < KT; ++kt) ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
-        if (!SPLITK && KT > 0) mma_all((KSTEPS - 1) & 1);
+            if (kt0 + s < KT) issue(kt0 + s);
+        int kt = kt0, stopped = 0;
+        for (; kt + STAGES - 1 < KT; ++kt) {
+            stopped = ktile(kt, false, IntC<1>{});
+            if (CKPT && stopped) break;
+        }
+        if (!(CKPT && stopped))
+            for (; kt < KT; ++kt) ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
+        if (!SPLITK && KT > kt0) mma_all((KSTEPS - 1) & 1);
         GP_PROBE(3);
+        // When `stopped` (CKPT only), K-steps kt0..kt are in the accumulators and the "epilogue" below
+        // writes them to the checkpoint slot instead of finishing the tile.  The loads of step kt+1
+        // are still landing in LDS and must be waited for before the workgroup may go away.
+        if (CKPT && stopped) wait_vmcnt<0>();
 
         // ---- epilogue -------------------------------------------------------------------------
         // Accumulators go through LDS once so that each lane finishes four consecutive columns of
@@ -363,6 +435,10 @@ struct PipeKernel {
             }
         };
         float *red = (float *)lds_t;
+        // Every epilogue index is derived from these two laundered values: left to itself the compiler
+        // computes the output addresses before the main loop and keeps them in registers across it.
+        int lane_e = lane, tid_e = tid;
+        asm volatile("" : "+v"(lane_e), "+v"(tid_e));
         // (the empty asm pins the conversion here: hoisted next to the load it would wait for it)
         {
             typedef unsigned int raw_t __attribute__((ext_vector_type(sizeof(Vec4<T>) / 4)));
@@ -390,16 +466,26 @@ struct PipeKernel {
             constexpr int RPP = 64 / L4;     // rows per pass of the wave
             constexpr int PASSES = 32 / RPP;
             constexpr int G = PASSES < 4 ? PASSES : 4;
-            const int c4 = lane % L4, r_in = lane / L4;
+            const int c4 = lane_e % L4, r_in = lane_e / L4;
             const int j = c4 >> 3, col = (c4 & 7) * 4;
             const int n = n0 + wn * WN + j * 32 + col;
             __syncthreads();  // all waves are done reading the stage buffers
             static_for<0, MI>([&](auto ic) {
                 constexpr int i = ic;
+                if (CKPT && stopped) {  // (uniform) checkpoint: this strip's accumulators go to the slot as they are
+#pragma unroll
+                    for (int jj = 0; jj < NI; ++jj)
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            f32x4 v = {acc[i][jj][q * 4], acc[i][jj][q * 4 + 1], acc[i][jj][q * 4 + 2], acc[i][jj][q * 4 + 3]};
+                            slot[((i * NI + jj) * 4 + q) * 64 + lane_e] = v;
+                        }
+                    return;
+                }
 #pragma unroll
                 for (int jj = 0; jj < NI; ++jj)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) mine[(jj * 16 + v) * 64 + lane] = acc[i][jj][v];
+                    for (int v = 0; v < 16; ++v) mine[(jj * 16 + v) * 64 + lane_e] = acc[i][jj][v];
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // same wave reads other lanes' values next
 #pragma unroll 1
                 for (int p = 0; p < PASSES; p += G) {
@@ -423,7 +509,7 @@ struct PipeKernel {
             constexpr int RPP = NT / L4;     // rows per pass of the workgroup
             constexpr int PASSES = BM / RPP;
             constexpr int G = PASSES < 4 ? PASSES : 4;
-            const int c4 = tid % L4, r_in = tid / L4;
+            const int c4 = tid_e % L4, r_in = tid_e / L4;
             const int j = c4 >> 3, col = (c4 & 7) * 4;
             const int n = n0 + j * 32 + col;
             __syncthreads();  // all waves are done reading the stage buffers
@@ -432,7 +518,7 @@ struct PipeKernel {
 #pragma unroll
                 for (int jj = 0; jj < NI; ++jj)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + jj) * 16 + v) * 64 + lane] = acc[i][jj][v];
+                    for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + jj) * 16 + v) * 64 + lane_e] = acc[i][jj][v];
             __syncthreads();
 #pragma unroll 1
             for (int p = 0; p < PASSES; p += G) {
@@ -456,6 +542,16 @@ struct PipeKernel {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         GP_PROBE(5);
 #endif
+        if constexpr (CKPT) {
+            if (stopped) {
+                if (tid == 0) {
+                    int *hdr = (int *)cc.ckpt + (size_t)blockIdx.x * CKPT_HEADER_INTS;
+                    hdr[1] = cc.kernel_id; hdr[2] = tile_index; hdr[3] = kt + 1; hdr[0] = 1;
+                }
+                return true;
+            }
+        }
+        return false;
     }
 };
 

@@ -35,6 +35,7 @@ struct BlpArgs {
     int poll_mask;    // the claim numbered c reads the host flag when (c & poll_mask) == 0
     int groups;       // claim counters per kernel (>= 1); counter g sits at executed + g * COUNTER_STRIDE
     int order;        // tile order: 0 = x fastest (the reference's), 1 = y fastest
+    void *ckpt;       // checkpoint workspace of kernels that can leave a tile half-way, or nullptr
 };
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
@@ -64,6 +65,40 @@ __device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy, int orde
     return t;
 }
 
+// One claim by the workgroup's leader: -1 when the workgroup has to leave (stop requested or the
+// slice is handed out).
+//
+// The stop index (device memory) doubles as the device-side mirror of the flag: every claim
+// checks it, but only the workgroup about to make a claim whose number is a multiple of
+// poll_every reads the flag itself from host memory.  Reads of fine-grained host memory are
+// served one at a time (about 90 ns each on MI355X), so a poll per tile from every workgroup
+// would dominate short kernels.
+// The stop index is also sticky: once a kernel of this executor has been stopped, every later
+// kernel of the same submission leaves too until the host re-arms it, even if the flag has been
+// lowered in between; otherwise a kernel queued behind a stopped one could run to completion on
+// incomplete inputs.
+__device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_lo, int slice_n) {
+    int claim = -1;
+    int stop = __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
+    if (!stop) {
+        const int c = atomicAdd(b.executed + grp * COUNTER_STRIDE, 1);
+        if (c < slice_n) {
+            claim = slice_lo + c;
+            if (claim == b.inject_at && b.flag)
+                __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            // with several counters only the first four groups read the flag, unless it is read on
+            // every claim (poll_mask == 0: the flag is cheap device memory)
+            if ((grp < 4 || b.poll_mask == 0) && (c & b.poll_mask) == 0 && b.flag &&
+                __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
+                atomicCAS(b.stop_index, -1, b.kernel_id);
+            // the polling workgroup still owes the tile it has just claimed
+        }
+    } else {
+        atomicCAS(b.stop_index, -1, b.kernel_id);
+    }
+    return claim;
+}
+
 // Runs body(TileIdx) for every tile this workgroup obtains.  All threads of the workgroup must
 // call it; the body may use barriers freely.
 template <class Body>
@@ -82,43 +117,69 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
         if (!dynamic) {
             idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
         } else {
-            if (leader) {
-                // The stop index (device memory) doubles as the device-side mirror of the flag:
-                // every claim checks it, but only the workgroup about to make a claim whose number
-                // is a multiple of poll_every reads the flag itself from host memory.  Reads of
-                // fine-grained host memory are served one at a time (about 90 ns each on MI355X),
-                // so a poll per tile from every workgroup would dominate short kernels.
-                // The stop index is also sticky: once a kernel of this executor has been stopped,
-                // every later kernel of the same submission leaves too until the host re-arms it,
-                // even if the flag has been lowered in between; otherwise a kernel queued behind a
-                // stopped one could run to completion on incomplete inputs.
-                int claim = -1;
-                int stop = __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
-                if (!stop) {
-                    const int c = atomicAdd(b.executed + grp * COUNTER_STRIDE, 1);
-                    if (c >= slice_n) {
-                        claim = -1;
-                    } else {
-                        claim = slice_lo + c;
-                        if (claim == b.inject_at && b.flag)
-                            __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                        // with several counters only the first four groups read the flag, unless it
-                        // is read on every claim (poll_mask == 0: the flag is cheap device memory)
-                        if ((grp < 4 || b.poll_mask == 0) && (c & b.poll_mask) == 0 && b.flag &&
-                            __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
-                            atomicCAS(b.stop_index, -1, b.kernel_id);
-                        // the polling workgroup still owes the tile it has just claimed
-                    }
-                } else {
-                    atomicCAS(b.stop_index, -1, b.kernel_id);
-                }
-                mailbox[it & 1] = claim;
-            }
+            if (leader) mailbox[it & 1] = claim_tile(b, grp, slice_lo, slice_n);
             __syncthreads();
-            idx = mailbox[it & 1];
+            idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1]);  // wave-uniform: tile coordinates stay scalar
         }
         if (idx < 0) return;
         body(decode_tile(idx, b.sx, b.sy, b.order));
+    }
+}
+
+// ---- tiles that can be left half-way ------------------------------------------------------------
+// A tile whose K loop runs for hundreds of microseconds (a 256 x 256 tile over K = 8192 takes
+// about 200 us) makes "finish the tile you owe" too slow a way to leave.  Kernels built on
+// tile_loop_ckpt poll for the stop request inside the tile, and a workgroup that is asked to
+// leave writes its fp32 accumulators and its position in K to its own slot of a checkpoint
+// workspace; the relaunch (same grid) finds the slot, reloads the accumulators and continues
+// with the next K-step.  The accumulation order is unchanged, so the result stays bit-identical.
+//
+// Workspace layout (BlpArgs::ckpt): CKPT_MAX_WGS headers of 64 bytes, then one slot of
+// `ckpt_slot_bytes` per workgroup.  Header words: [0] valid, [1] kernel id, [2] tile index,
+// [3] K-step to continue with.
+constexpr int CKPT_MAX_WGS = 1024;
+constexpr int CKPT_HEADER_INTS = 16;
+
+// body(TileIdx, tile index, first K-step (0 = fresh tile)) returns true when it has left the tile
+// half-way (and written its checkpoint); the workgroup then leaves the kernel.
+template <class Body>
+__device__ __forceinline__ void tile_loop_ckpt(const BlpArgs &b, Body &&body) {
+    __shared__ int mailbox[2][2];
+    const bool dynamic = b.executed != nullptr;
+    const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    const int grp = wg_group((int)blockIdx.x, b.groups);
+    const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
+    const int slice_n = (b.groups > 1 ? group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) : b.total) - slice_lo;
+    for (int it = 0;; ++it) {
+        int idx, kt0 = 0;
+        if (!dynamic) {
+            idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
+        } else {
+            if (leader) {
+                int claim = -1, first = 0;
+                int *hdr = b.ckpt ? (int *)b.ckpt + (size_t)blockIdx.x * CKPT_HEADER_INTS : nullptr;
+                if (it == 0 && hdr && hdr[0] == 1 && hdr[1] == b.kernel_id) {
+                    // a tile this workgroup left half-way in an earlier launch comes first; it was
+                    // counted when it was claimed
+                    if (__hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == -1) {
+                        claim = hdr[2];
+                        first = hdr[3];
+                        hdr[0] = 0;
+                    } else {
+                        atomicCAS(b.stop_index, -1, b.kernel_id);
+                    }
+                } else {
+                    claim = claim_tile(b, grp, slice_lo, slice_n);
+                }
+                mailbox[it & 1][0] = claim;
+                mailbox[it & 1][1] = first;
+            }
+            __syncthreads();
+            idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1][0]);  // wave-uniform: tile coordinates and
+            kt0 = __builtin_amdgcn_readfirstlane(mailbox[it & 1][1]);  // K position stay scalar
+        }
+        if (idx < 0) return;
+        if (body(decode_tile(idx, b.sx, b.sy, b.order), idx, kt0)) return;
     }
 }
 

@@ -123,6 +123,7 @@ BLPExecutor::BLPExecutor() {}
 BLPExecutor::~BLPExecutor() {
     if (dpStopIndex) gp_free(dpStopIndex);
     if (executed) gp_free(executed);
+    if (ckpt) gp_free(ckpt);
     if (stop_host) gp_host_free(stop_host);
     if (left_host) gp_flag_destroy(left_host);
 }
@@ -158,6 +159,16 @@ Status BLPExecutor::init(std::string workload) {
     // GPREEMPT_SINGLE_COUNTER=1 selects the reference's one-counter-per-kernel layout (for A/B timing)
     const char *single = std::getenv("GPREEMPT_SINGLE_COUNTER");
     RETURN_STATUS(model->add_block_preemption_param(executed, (single && *single == '1') ? 1 : kCounterGroups));
+    // long GEMM tiles may be left half-way: one slot per workgroup for their accumulators
+    // (GPREEMPT_NO_CHECKPOINT=1 keeps the reference's "finish the tile you owe" for A/B timing)
+    const char *nock = std::getenv("GPREEMPT_NO_CHECKPOINT");
+    ckpt_bytes = (nock && *nock == '1') ? 0 : model->checkpoint_bytes_wanted();
+    if (ckpt_bytes > 0) {
+        CUDA_RETURN_STATUS(gp_malloc(&ckpt, ckpt_bytes));
+        CUDA_RETURN_STATUS(gp_ckpt_reset_async(ckpt, nullptr));
+        CUDA_RETURN_STATUS(gp_stream_sync(nullptr));
+        model->set_checkpoint_workspace(ckpt, ckpt_bytes);
+    }
     RETURN_STATUS(this->load_param(model_path));
     return Status::Succ;
 }
@@ -214,6 +225,7 @@ Status BLPExecutor::resume(GPUstream stream) {
 
 Status BLPExecutor::reset_counters(GPUstream stream) {
     CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride, stream));
+    if (ckpt) CUDA_RETURN_STATUS(gp_ckpt_reset_async(ckpt, stream));  // a fresh run has no tile to continue
     return Status::Succ;
 }
 

@@ -297,6 +297,16 @@ Status Model::add_block_preemption_param(GPUdeviceptr ptr, int counter_groups) {
     return Status::Succ;
 }
 
+size_t Model::checkpoint_bytes_wanted() const {
+    size_t want = 0;
+    for (const KernelInfo &k : kernel_infos) {
+        if (k.op != OpKind::Gemm || !k.preemptible) continue;
+        size_t b = 0;
+        if (gp_gemm_ckpt_bytes(&k.p.gemm, &b) == 0 && b > want) want = b;
+    }
+    return want;
+}
+
 Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
     if (idx >= kernel_infos.size()) return Status::OutOfRange;
     KernelInfo &k = kernel_infos[idx];
@@ -318,6 +328,8 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.max_workgroups = 0;
         ctx.poll_every = poll_every_;
         ctx.counter_groups = counter_groups_;
+        ctx.ckpt = ckpt_;
+        ctx.ckpt_bytes = ckpt_bytes_;
         pc = &ctx;
     }
     gp_launch_info info{};

@@ -116,6 +116,8 @@ private:
     int *stop_host = nullptr;            // pinned landing slot for the stop index
     volatile int *left_host = nullptr;   // fine-grained host word written by a program's last leaving workgroup
     void *left_dev = nullptr;
+    GPUdeviceptr ckpt = nullptr;         // owned: checkpoint workspace of long GEMM tiles, or null
+    size_t ckpt_bytes = 0;
     int inject_kernel = -1, inject_claim = -1;
     std::atomic<int> *lc_tasks = nullptr;
     std::atomic<int> *be_tasks = nullptr;

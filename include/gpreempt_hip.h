@@ -118,6 +118,13 @@ typedef struct gp_preempt_ctx {
                      /* word; the last workgroup to leave a launch stores that launch's number    */
                      /* (info->shape[1] of gp_program_launch) there, so the host learns that the  */
                      /* GPU has been vacated without a queue query                                */
+    void *ckpt;      /* may be NULL.  Workspace (gp_gemm_ckpt_bytes) that lets a long GEMM tile be   */
+                     /* left between two K-steps: the workgroup stores its fp32 accumulators and    */
+                     /* K position there and the relaunch (same grid) continues from them, still    */
+                     /* bit-identical.  Without it a workgroup finishes the tile it owes.  Clear it */
+                     /* with gp_ckpt_reset_async whenever the claim counters are cleared.  No       */
+                     /* counterpart in the reference, whose tiles are never long enough to matter.  */
+    unsigned long long ckpt_bytes;
 } gp_preempt_ctx;
 
 /* What a launch did: filled when the `info` argument of a launcher is non-NULL. */
@@ -156,6 +163,11 @@ typedef struct gp_gemm_params {
     int variant;        /* enum gp_mat_variant; 0 = chosen by the launcher */
 } gp_gemm_params;
 int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+/* Bytes of gp_preempt_ctx::ckpt workspace this GEMM can use (0: its tiles are short and always
+ * finished), and the reset of such a workspace.  Extension of the dispatcher that
+ * scripts/compile/convert_to_blp.py:40-69 generates (which can only stop between tiles). */
+int gp_gemm_ckpt_bytes(const gp_gemm_params *p, size_t *bytes);
+int gp_ckpt_reset_async(void *ckpt, gp_stream s);
 
 /* Implicit-GEMM convolution.  Activations are NHWC with a pixel stride (in elements) that may
  * exceed the channel count, so a layer can read or write a channel slice of a wider buffer

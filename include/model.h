@@ -121,6 +121,10 @@ public:
     // device-visible address of a host word that a program's last leaving workgroup sets to the
     // launch number returned by launch_program()
     void set_left_word(GPUdeviceptr p) { left_word_ = p; }
+    // workspace that lets long GEMM tiles be left between two K-steps (gp_preempt_ctx::ckpt)
+    void set_checkpoint_workspace(GPUdeviceptr p, size_t bytes) { ckpt_ = p; ckpt_bytes_ = bytes; }
+    // largest such workspace any kernel of the model can use (0: none can)
+    size_t checkpoint_bytes_wanted() const;
     int last_launch_tag() const { return last_launch_tag_; }
 
     // Whole-model program: all kernels as one persistent device kernel (the counterpart of the
@@ -146,6 +150,8 @@ private:
     int counter_groups_ = 1;
     int poll_every_ = 0;
     GPUdeviceptr left_word_ = nullptr;
+    GPUdeviceptr ckpt_ = nullptr;
+    size_t ckpt_bytes_ = 0;
     int last_launch_tag_ = 0;
     std::string workload_, dtype_;
     std::vector<StorageInfo> storage_infos;

@@ -220,3 +220,114 @@ def test_pipelined_gemm_preempt_resume_bit_exact(gp, dt, tile, variant):
         gp.launch("gp_launch_gemm", p, st.ctx())
         gp.check(gp.lib().gp_stream_sync(None))
         assert np.array_equal(dC.download(), base)
+
+
+# ---- long tiles left between two K-steps ---------------------------------------------------------
+def _ckpt_gemm(gp, dt, M, N, K, seed=5):
+    rng = np.random.default_rng(seed)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (N, K)).astype(np.float32)
+    bias = rng.uniform(-0.1, 0.1, N).astype(np.float32)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    dA, dB, db = gp.DevBuf.from_array(A, dtype), gp.DevBuf.from_array(B, dtype), gp.DevBuf.from_array(bias, dtype)
+    dC = gp.DevBuf(M * N * gp.DTYPE_SIZE[dtype])
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N,
+                      bias=db.ptr, alpha=1.0, act=gp.ACT_RELU, batch=1, tile_m=256, tile_n=256)
+    return p, (dA, dB, db, dC)
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+def test_long_tiles_are_left_mid_k_and_resumed_bit_exact(gp, dt):
+    """256 x 256 tiles over a long K: with a checkpoint workspace a stop request is honoured between
+    two K-steps (workgroups store accumulators + K position), not only between tiles; the relaunch
+    continues from the stored state and the result is bit-identical to the uninterrupted run."""
+    M, N, K = 1024, 1024, 8192 if dt != "f32" else 4096
+    p, bufs = _ckpt_gemm(gp, dt, M, N, K)
+    dC = bufs[3]
+    stream = gp.Stream(1)
+    gp.launch("gp_launch_gemm", p, None, stream)
+    stream.sync()
+    want = dC.download().copy()
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    assert st.enable_checkpoints(p) > 0
+    tiles = (M // 256) * (N // 256)
+    stops = 0
+    for inject in (0, 5, tiles - 1):
+        dC.fill32(0)
+        st.reset()
+        st.clear_stop()
+        flag.set(0)
+        gp.check(gp.lib().gp_ckpt_reset_async(gp.vp(st.ckpt.ptr), None))
+        info = gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0, inject_at=inject), stream)
+        stream.sync()
+        assert flag.get() == 1
+        assert info.grid == tiles  # every tile is claimed at once: only a mid-tile stop can interrupt
+        hdr = st.checkpoint_headers(info.grid)
+        n_ck = int(hdr[:, 0].sum())
+        if st.stop_index() == 0:
+            stops += 1
+            assert n_ck > 0
+            live = hdr[hdr[:, 0] == 1]
+            assert (live[:, 1] == 0).all() and (live[:, 3] > 0).all() and (live[:, 3] * (64 if dt != "f32" else 32) < K).all()
+            assert len(set(live[:, 2].tolist())) == len(live)  # distinct tiles
+            assert not np.array_equal(dC.download(), want)
+        # resume until complete (the flag is down, so one relaunch finishes)
+        flag.set(0)
+        st.clear_stop()
+        gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
+        stream.sync()
+        assert st.stop_index() == -1
+        assert int(st.checkpoint_headers(info.grid)[:, 0].sum()) == 0
+        assert np.array_equal(dC.download(), want), (dt, inject)
+    assert stops >= 2, "the stop request was never seen inside a tile"
+
+
+def test_long_tiles_stopped_twice_then_finished(gp):
+    """A tile can be left more than once; every relaunch continues where the last one stopped."""
+    M, N, K = 512, 512, 16384
+    p, bufs = _ckpt_gemm(gp, "bf16", M, N, K, seed=9)
+    dC = bufs[3]
+    stream = gp.Stream(1)
+    gp.launch("gp_launch_gemm", p, None, stream)
+    stream.sync()
+    want = dC.download().copy()
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    st.enable_checkpoints(p)
+    dC.fill32(0)
+    flag.set(0)
+    info = gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0, inject_at=0), stream)
+    stream.sync()
+    first = st.checkpoint_headers(info.grid)
+    assert st.stop_index() == 0 and first[:, 0].sum() > 0
+    # second launch with the flag still up: workgroups with a stored tile leave it where it is
+    st.clear_stop()
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
+    stream.sync()
+    second = st.checkpoint_headers(info.grid)
+    assert st.stop_index() == 0
+    assert (second[:, 0] == first[:, 0]).all() and (second[second[:, 0] == 1][:, 3] >= first[first[:, 0] == 1][:, 3]).all()
+    flag.set(0)
+    st.clear_stop()
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
+    stream.sync()
+    assert st.stop_index() == -1
+    assert np.array_equal(dC.download(), want)
+
+
+def test_without_workspace_long_tiles_are_finished(gp):
+    """No checkpoint workspace: the reference's behaviour, a workgroup finishes the tile it owes."""
+    p, bufs = _ckpt_gemm(gp, "bf16", 512, 512, 4096)
+    dC = bufs[3]
+    stream = gp.Stream(1)
+    gp.launch("gp_launch_gemm", p, None, stream)
+    stream.sync()
+    want = dC.download().copy()
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    dC.fill32(0)
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0, inject_at=0), stream)
+    stream.sync()
+    assert flag.get() == 1
+    assert np.array_equal(dC.download(), want)  # all four tiles were owed and finished
