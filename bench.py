@@ -140,31 +140,78 @@ def roofline(workload, iters, dt):
             "algorithmic_flop_per_launch": total_flop / launches, "algorithmic_bytes_per_launch": total_bytes / launches}
 
 
-def gemm_roofline(iters=10):
-    """BASELINE config 5's best-effort tenant alone: bf16 8192^3 GEMM (fp32 accumulate), preemptible."""
-    from gpreempt_amd import capi as gp
-    n = 8192
-    dA, dB, dC = gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2)
-    dA.fill32(0x3F803F80)
-    dB.fill32(0x3C003C00)
-    p = gp.GemmParams(dtype=gp.BF16, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=1, C=dC.ptr, ldc=n, alpha=1.0, batch=1)
-    flag = gp.Flag()
-    st = gp.BlpState(1, flag)
-    stream = gp.Stream(1)
+def _time_gemm(gp, p, stream, st, iters):
+    """median HIP-event time (s) of one launch; st = None launches without claim counters"""
     e0, e1 = gp.Event(), gp.Event()
     ms = []
+    info = None
     for i in range(iters + 2):
-        st.reset()
+        if st is not None:
+            st.reset()
         e0.record(stream)
-        info = gp.launch("gp_launch_gemm", p, st.ctx(), stream)
+        info = gp.launch("gp_launch_gemm", p, st.ctx() if st is not None else None, stream)
         e1.record(stream)
         e1.sync()
         if i >= 2:
             ms.append(e0.elapsed_ms(e1))
-    t = sorted(ms)[len(ms) // 2] * 1e-3
-    ach = 2.0 * n ** 3 / t / 1e12
+    return sorted(ms)[len(ms) // 2] * 1e-3, info
+
+
+def config1_gemm1024(iters=20):
+    """BASELINE config 1: C = relu(A B + bias), 1024^3 fp32, as a plain and as a preemptible launch
+    (the difference is what the dispatcher costs: SURVEY's flag-poll A/B)."""
+    import numpy as np
+    from gpreempt_amd import capi as gp
+    n = 1024
+    rng = np.random.default_rng(0xC0FFEE)
+    A = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    B = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    bias = rng.uniform(-0.1, 0.1, n).astype(np.float32)
+    dA, dB, db = gp.DevBuf.from_array(A, gp.F32), gp.DevBuf.from_array(np.ascontiguousarray(B.T), gp.F32), gp.DevBuf.from_array(bias, gp.F32)
+    dC = gp.DevBuf(n * n * 4)
+    p = gp.GemmParams(dtype=gp.F32, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=1, C=dC.ptr, ldc=n, bias=db.ptr,
+                      alpha=1.0, act=gp.ACT_RELU, batch=1)
+    stream = gp.Stream(1)
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    t_plain, info = _time_gemm(gp, p, stream, None, iters)
+    t_blp, info_b = _time_gemm(gp, p, stream, st, iters)
+    flop = 2.0 * n ** 3 + 2.0 * n * n
+    return {"bound": "mfma", "dtype": "f32", "algorithmic_flop": flop, "algorithmic_bytes": 4 * (3 * n * n + n),
+            "plain_us": t_plain * 1e6, "preemptible_us": t_blp * 1e6, "tiles": info.total_tiles, "grid_preemptible": info_b.grid,
+            "achieved": flop / t_blp / 1e12, "peak": PEAK["f32"], "unit": "TFLOP/s", "frac": flop / t_blp / 1e12 / PEAK["f32"],
+            "dispatcher_cost_us_per_tile": (t_blp - t_plain) * 1e6 / max(1, info.total_tiles),
+            "note": "a 1024^3 launch is 14 us of MFMA work at the fp32 peak; both forms are launch- and latency-bound"}
+
+
+def gemm_roofline(iters=10):
+    """BASELINE config 5's best-effort tenant alone: bf16 8192^3 GEMM (fp32 accumulate): launched
+    plainly, preemptibly (tiles are finished), and preemptibly with the checkpoint workspace that
+    lets a 256 x 256 tile be left between two K-steps."""
+    from gpreempt_amd import capi as gp
+    import numpy as np
+    n = 8192
+    # U[-1, 1) operands as the config asks (constant operands toggle fewer bits and run faster)
+    rng = np.random.default_rng(5)
+    dA, dB, dC = gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2)
+    for d in (dA, dB):
+        f = rng.random(n * n, dtype=np.float32) * 2.0 - 1.0
+        d.upload((f.view(np.uint32) >> 16).astype(np.uint16))  # bf16 by truncation: the values only need to be random
+    p = gp.GemmParams(dtype=gp.BF16, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=1, C=dC.ptr, ldc=n, alpha=1.0, batch=1)
+    flag = gp.Flag()
+    stream = gp.Stream(1)
+    st = gp.BlpState(1, flag)
+    t, info = _time_gemm(gp, p, stream, st, iters)
+    t_plain, _ = _time_gemm(gp, p, stream, None, iters)
+    st_ck = gp.BlpState(1, flag)
+    st_ck.enable_checkpoints(p)
+    t_ck, _ = _time_gemm(gp, p, stream, st_ck, iters)
+    flop = 2.0 * n ** 3
+    ach = flop / t / 1e12
     return {"bound": "mfma", "achieved": ach, "peak": PEAK["bf16"], "unit": "TFLOP/s", "frac": ach / PEAK["bf16"], "ms": t * 1e3,
-            "tiles": info.total_tiles, "grid": info.grid}
+            "tiles": info.total_tiles, "grid": info.grid,
+            "plain_launch": {"ms": t_plain * 1e3, "achieved": flop / t_plain / 1e12, "frac": flop / t_plain / 1e12 / PEAK["bf16"]},
+            "with_checkpoint_workspace": {"ms": t_ck * 1e3, "achieved": flop / t_ck / 1e12, "frac": flop / t_ck / 1e12 / PEAK["bf16"]}}
 
 
 def copy_calibration(mib=256, iters=10):
@@ -243,6 +290,7 @@ def main():
         out["roofline"] = roofline(args.be_model, 3, "f16")
     if args.only in ("", "gemm"):
         out["config5_gemm8192_bf16"] = gemm_roofline()
+        out["config1_gemm1024_f32"] = config1_gemm1024()
     if args.only == "copycal":
         out["copy_calibration"] = copy_calibration()
     if args.only in ("", "cpu"):

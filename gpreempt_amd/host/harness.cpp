@@ -15,7 +15,10 @@
 #include <chrono>
 #include <cmath>
 #include <cstring>
+#include <condition_variable>
+#include <memory>
 #include <mutex>
+#include <queue>
 #include <thread>
 
 #include "executor.h"
@@ -116,10 +119,79 @@ struct Stats {
 // Level p tenants obey flag word p-1, which is up while any tenant of a level < p is active
 // (the reference has two levels and one word, blpclient.cpp:185-195; the three-tenant
 // configuration needs one word per level).
+// Pre-preemption hints (reference src/cuda-clients/gpreemptclient.cpp:51-60, 203-219, 267-291):
+// a latency-critical client that knows its request will reach the GPU after `preprocess_time`
+// posts a hint on arrival; a daemon orders the hints by deadline and raises the flag words
+// `switch_us` before the kernels are due, so that the lower levels drain while the client is
+// still preprocessing on the CPU.  Whoever comes first, daemon or client, begins the request in
+// the PreemptDomain (exactly once); the client ends it.
+class HintDaemon {
+public:
+    struct Hint {
+        int64_t deadline_ns;
+        int priority;
+        std::shared_ptr<std::atomic<int>> state;  // 0 pending, 1 begun by the daemon, 2 begun by the client
+        bool operator>(const Hint &o) const { return deadline_ns > o.deadline_ns; }
+    };
+    explicit HintDaemon(PreemptDomain *d) : domain_(d), thread_([this] { run(); }) {}
+    ~HintDaemon() {
+        {
+            std::lock_guard<std::mutex> g(mu_);
+            quit_ = true;
+        }
+        cv_.notify_all();
+        thread_.join();
+    }
+    std::shared_ptr<std::atomic<int>> post(int64_t deadline_ns, int priority) {
+        auto st = std::make_shared<std::atomic<int>>(0);
+        {
+            std::lock_guard<std::mutex> g(mu_);
+            heap_.push(Hint{deadline_ns, priority, st});
+        }
+        cv_.notify_all();
+        return st;
+    }
+    long fired() const { return fired_.load(); }
+
+private:
+    void run() {
+        std::unique_lock<std::mutex> lk(mu_);
+        while (!quit_) {
+            if (heap_.empty()) { cv_.wait(lk); continue; }
+            Hint h = heap_.top();
+            int64_t now = now_ns();
+            if (now < h.deadline_ns) {
+                // sleep most of the way, spin the last stretch: a condition variable alone wakes tens of us late
+                int64_t left = h.deadline_ns - now;
+                if (left > 60000) cv_.wait_for(lk, std::chrono::nanoseconds(left - 50000));
+                else { lk.unlock(); spin_pause(); lk.lock(); }
+                continue;
+            }
+            heap_.pop();
+            int expect = 0;
+            if (h.state->compare_exchange_strong(expect, 1)) {
+                lk.unlock();
+                domain_->begin(h.priority);
+                fired_.fetch_add(1);
+                lk.lock();
+            }
+        }
+    }
+    PreemptDomain *domain_;
+    std::mutex mu_;
+    std::condition_variable cv_;
+    std::priority_queue<Hint, std::vector<Hint>, std::greater<Hint>> heap_;
+    bool quit_ = false;
+    std::atomic<long> fired_{0};
+    std::thread thread_;
+};
+
 struct Shared {
     std::string policy;
     int levels = 2;
     std::unique_ptr<PreemptDomain> domain;  // flag words and per-level request counts (gpreempt.h)
+    std::unique_ptr<HintDaemon> hints;      // null: no pre-preemption hints
+    int64_t hint_switch_us = 0;             // how long before the kernels are due the flag goes up
     std::atomic<int> on_gpu[kMaxLevels];    // preemptible tenants of this level with work in flight
     std::atomic<int> seq_waiting{0};        // "seq": latency-critical requests waiting for the lock
     std::mutex seq_mu;
@@ -385,8 +457,17 @@ void end_request(Tenant &t, Shared &sh) {
 // in the reference's clients, preprocess sleeps preprocess_time (blpclient.cpp:153-155).
 Status infer_once(Tenant &t, Shared &sh, double *total_us, double *infer_us) {
     int64_t t0 = now_ns();
-    if (t.preprocess_us > 0) std::this_thread::sleep_for(std::chrono::microseconds(t.preprocess_us));
-    begin_request(t, sh);
+    std::shared_ptr<std::atomic<int>> hint;
+    if (sh.hints && preempting_policy(sh) && t.preprocess_us > sh.hint_switch_us)
+        hint = sh.hints->post(t0 + (t.preprocess_us - sh.hint_switch_us) * 1000, t.priority);
+    if (t.preprocess_us > 0) {
+        // the reference sleeps (blpclient.cpp:153-155); a sleep overshoots by 50+ us, so the tail is spun
+        int64_t until = t0 + t.preprocess_us * 1000;
+        if (t.preprocess_us > 200) std::this_thread::sleep_for(std::chrono::microseconds(t.preprocess_us - 150));
+        while (now_ns() < until) spin_pause();
+    }
+    int expect = 0;
+    if (!hint || hint->compare_exchange_strong(expect, 2)) begin_request(t, sh);  // else the daemon has begun it
     struct Retire { Tenant &t; Shared &sh; ~Retire() { end_request(t, sh); } } retire{t, sh};
     // "resident_io": operands stay in device memory (a 8192^2 matrix is 134 MB: copied per
     // request it would be the whole request); the input is uploaded once, the output never read back
@@ -482,6 +563,9 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     const bool relay = cfg["flag_relay"].boolean(false);  // measured slower: a second resident kernel slows every launch
     sh.domain.reset(new PreemptDomain(sh.levels, relay));
     if (!sh.domain->ok()) return Status::Fail;
+    // "pre_preempt_hint_us" > 0: tenants with a preprocess_time longer than that post hints
+    sh.hint_switch_us = (int64_t)cfg["pre_preempt_hint_us"].number(0);
+    if (sh.hint_switch_us > 0) sh.hints.reset(new HintDaemon(sh.domain.get()));
     for (auto &t : tenants) RETURN_STATUS(init_tenant(*t, sh));
 
     // warm-up and stand-alone latency, one tenant at a time (benchmark.cpp:221-299)
@@ -558,8 +642,10 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     rep.set("hp_p99_vs_isolated") = hp_ratio;
     rep.set("be_throughput_kept") = n_be ? be_kept / n_be : 0.0;
     rep.set("preemptLatency(us)") = sh.preempt_latency.to_json();
+    rep.set("hints_fired") = (double)(sh.hints ? sh.hints->fired() : 0);
     report_text = rep.dump();
 
+    sh.hints.reset();         // joins the daemon before the domain goes
     sh.domain->stop_relay();  // frees below synchronise the device
     for (auto &t : tenants) {
         t->ex->clear();

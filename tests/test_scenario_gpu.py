@@ -58,3 +58,31 @@ def test_unknown_model_is_reported(gp):
     buf = C.create_string_buffer(1 << 16)
     rc = gx.lib().gpx_run_scenario(json.dumps(cfg).encode(), buf, C.c_size_t(len(buf)))
     assert rc != 0
+
+
+def _run_cfg(cfg):
+    from gpreempt_amd import executor as gx
+    buf = C.create_string_buffer(1 << 20)
+    rc = gx.lib().gpx_run_scenario(json.dumps(cfg).encode(), buf, C.c_size_t(len(buf)))
+    assert rc == 0, buf.value[:400]
+    return json.loads(buf.value.decode())
+
+
+def test_pre_preemption_hints_hide_the_drain(gp):
+    """gpreemptclient.cpp:203-219: a client that preprocesses for a while posts a hint, and the
+    daemon raises the flag shortly before the kernels are due; under the waiting policy ("wb") the
+    request then finds the GPU already vacated instead of waiting for the drain itself."""
+    def cfg(hint_us):
+        return {"time": 3.0, "policy": "wb", "hp_requests": 80, "warmups": 3, "standalone_runs": 20, "pre_preempt_hint_us": hint_us,
+                "tasks": [
+                    {"id": "hp", "load": {"type": "poisson", "frequency": 200, "seed": 11},
+                     "client": {"name": "hp", "model_name": "bert", "priority": 0, "use_cuda_graph": False, "launch_mode": "launch", "preprocess_time": 400}},
+                    {"id": "be", "load": {"type": "continuous"},
+                     "client": {"name": "be", "model_name": "resnet50", "priority": 1, "use_cuda_graph": True, "launch_mode": "program", "preprocess_time": 0}}]}
+    plain = _run_cfg(cfg(0))
+    hinted = _run_cfg(cfg(150))
+    assert plain["hints_fired"] == 0
+    assert hinted["hints_fired"] >= 0.9 * hinted["tasks"]["hp"]["requests"]
+    assert hinted["tasks"]["be"]["preemptions"] > 0
+    # the drain no longer sits inside the request's GPU phase
+    assert hinted["tasks"]["hp"]["inferLatency(us)"]["p50"] < plain["tasks"]["hp"]["inferLatency(us)"]["p50"] + 5.0
