@@ -38,14 +38,16 @@ template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool CONV, bool 
 using TK = TileKernel<T, BM, BN, BK, WGM, WGN, CONV, B_KN>;
 
 template <class K> struct K_is_ckpt { static constexpr bool value = false; };
-template <typename T> struct K_is_ckpt<PipeKernel<T, 256, 256, 2, false, false, true>> { static constexpr bool value = true; };
+template <typename T, int BM, int BN, int ST, bool CV> struct K_is_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true>> { static constexpr bool value = true; };
 template <class K> struct KernelOf { static constexpr auto fn = mat_kernel<K>; };
-template <typename T> struct KernelOf<PipeKernel<T, 256, 256, 2, false, false, true>> {
-    static constexpr auto fn = mat_kernel_ckpt<PipeKernel<T, 256, 256, 2, false, false, true>>;
+template <typename T, int BM, int BN, int ST, bool CV> struct KernelOf<PipeKernel<T, BM, BN, ST, CV, false, true>> {
+    static constexpr auto fn = mat_kernel_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true>>;
 };
 
 // bytes of checkpoint workspace a launch of body K needs (0: the body always finishes its tiles)
-static size_t ckpt_workspace_bytes(size_t slot_bytes) { return (size_t)CKPT_MAX_WGS * (CKPT_HEADER_INTS * 4 + slot_bytes); }
+static size_t ckpt_workspace_bytes(size_t slot_bytes, int workgroups) {
+    return (size_t)CKPT_MAX_WGS * CKPT_HEADER_INTS * 4 + (size_t)workgroups * slot_bytes;
+}
 
 template <class K>
 static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
@@ -64,7 +66,7 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     blp.order = pl.order;
     if constexpr (K_is_ckpt<K>::value) {
         // mid-tile checkpoints need the caller's workspace and a slot per workgroup
-        if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
+        if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES, grid) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(K::NT), K::LDS_BYTES, native(s), pl.g, blp);
     GP_HIP(hipGetLastError());
@@ -86,16 +88,23 @@ static int pipe_case(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, 
     if (pl.conv) return launch_mat<PipeKernel<T, TILE, TILE, STAGES, true, SPLITK>>(pl, ctx, s, info);
     return launch_mat<PipeKernel<T, TILE, TILE, STAGES, false, SPLITK>>(pl, ctx, s, info);
 }
+static size_t plan_ckpt_bytes(const MatPlan &pl);
+// the instantiation that can leave a tile between two K-steps, when the caller brought a workspace big enough for it
+template <typename T, int TILE, int STAGES>
+static int pipe_case_ckpt(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    if (!(ctx && ctx->ckpt && ctx->ckpt_bytes >= plan_ckpt_bytes(pl))) return pipe_case<T, TILE, STAGES, false>(pl, ctx, s, info);
+    if (pl.conv) return launch_mat<PipeKernel<T, TILE, TILE, STAGES, true, false, true>>(pl, ctx, s, info);
+    return launch_mat<PipeKernel<T, TILE, TILE, STAGES, false, false, true>>(pl, ctx, s, info);
+}
 
 template <typename T>
 static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
     switch (pl.body) {
         case MB_PIPE256:  // GEMM only: the gathered A operand of a convolution does not fit its register budget
-            // the checkpointing instantiation only when the caller brought a workspace
             if (ctx && ctx->ckpt) return launch_mat<PipeKernel<T, 256, 256, 2, false, false, true>>(pl, ctx, s, info);
             return launch_mat<PipeKernel<T, 256, 256, 2, false, false, false>>(pl, ctx, s, info);
-        case MB_PIPE128: return pipe_case<T, 128, GP_S128, false>(pl, ctx, s, info);
+        case MB_PIPE128: return pipe_case_ckpt<T, 128, GP_S128>(pl, ctx, s, info);
         case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
         case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
         case MB_PIPE32_SK: return pipe_case<T, 32, GP_S32, true>(pl, ctx, s, info);
@@ -125,7 +134,7 @@ int launch_mat_plan(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
 static size_t body_lds_bytes(int body, int dtype) {
     const size_t es = dtype == GP_F32 ? 4 : 2;
     switch (body) {
-        case MB_PIPE256: return 2 * (256 + 256) * 128 + 16;
+        case MB_PIPE256: return 2 * (256 + 256) * 128;
         case MB_PIPE128: return GP_S128 * (128 + 128) * 128;
         case MB_PIPE64: return GP_S64 * (64 + 64) * 128;
         case MB_PIPE64_SK: return GP_S64 * (64 + 64) * 128;   // at least the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4 = 64 KB)
@@ -269,13 +278,29 @@ extern "C" int gp_debug_tile_prof(unsigned long long *out, int n) {
 }
 #endif
 
-// Checkpoint workspace of the bodies that can leave a tile half-way (only the 256 x 256 GEMM body).
+// Checkpoint workspace of the bodies that can leave a tile half-way (the 256 x 256 and 128 x 128
+// bodies): headers plus one accumulator slot per resident workgroup.
+namespace gp {
+static size_t plan_ckpt_bytes(const MatPlan &pl) {
+    if (pl.body == MB_PIPE256) return ckpt_workspace_bytes(PipeKernel<float, 256, 256, 2, false, false, true>::CKPT_SLOT_BYTES, (int)device_cus());
+    if (pl.body == MB_PIPE128) return ckpt_workspace_bytes(PipeKernel<float, 128, 128, GP_S128, false, false, true>::CKPT_SLOT_BYTES, 2 * (int)device_cus());
+    return 0;
+}
+}  // namespace gp
 extern "C" int gp_gemm_ckpt_bytes(const gp_gemm_params *p, size_t *bytes) {
     GP_REQUIRE(bytes != nullptr, "null bytes");
     MatPlan pl;
     int rc = plan_gemm(p, &pl);
     if (rc) return rc;
-    *bytes = pl.body == MB_PIPE256 ? ckpt_workspace_bytes(PipeKernel<float, 256, 256, 2, false, false, true>::CKPT_SLOT_BYTES) : 0;
+    *bytes = plan_ckpt_bytes(pl);
+    return GP_SUCC;
+}
+extern "C" int gp_conv_ckpt_bytes(const gp_conv_params *p, size_t *bytes) {
+    GP_REQUIRE(bytes != nullptr, "null bytes");
+    MatPlan pl;
+    int rc = plan_conv2d(p, &pl);
+    if (rc) return rc;
+    *bytes = plan_ckpt_bytes(pl);
     return GP_SUCC;
 }
 

@@ -36,6 +36,15 @@ __device__ __forceinline__ void load_lds16(const void *gptr, unsigned lds_byte) 
                  : "memory", "m0");
 }
 
+// 4 bytes per lane: lane i's dword lands at lds_byte + 4*i.  Read past the caches (sc0 sc1): the
+// word is one that another workgroup or the host changes while this kernel runs.
+__device__ __forceinline__ void load_lds4(const void *gptr, unsigned lds_byte) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off sc0 sc1"
+                 :
+                 : "v"(gptr), "s"(lds_byte)
+                 : "memory", "m0");
+}
+
 #ifndef GP_LOAD_SPREAD
 #define GP_LOAD_SPREAD 0  // MFMAs between two loads of a stage; 0: chosen from the tile shape
 #endif
@@ -64,10 +73,13 @@ template <typename T> __device__ __forceinline__ void st_vec4(T *p, Vec4<T> o) {
     else st_out64(p, __builtin_bit_cast(unsigned long long, o));
 }
 
-// CKPT = true (two-stage GEMM bodies only): the tile can be left between two K-steps; see
-// tile_loop_ckpt in tile_loop.hpp.  One lane of the workgroup reads the stop index once per
-// K-step (and, in the first eight workgroups, now and then the host flag); the answer reaches the
-// other waves through an LDS word one K-step later, so nothing waits for the stop-index read.
+// CKPT = true (bodies with the waves tiled 2 x 2): the tile can be left between two K-steps; see
+// tile_loop_ckpt in tile_loop.hpp.  The stop index is read with the same direct-to-LDS loads as
+// the operands, one extra load per stage: it lands in an LDS word in order with the stage it
+// travels with, is covered by the same hand-placed vmcnt wait and barrier, and every wave then
+// reads the same word, so the decision to leave is uniform and nothing ever waits for the poll.
+// Eight workgroups take turns fetching the host flag the same way (each once in 8 polls: that
+// read takes about as long as a K-step) and pass it on through the stop index.
 struct CkptCtx {       // what a checkpointing body needs from the dispatcher, passed by value
     int *stop_index;   // nullptr: never leave a tile
     int *flag;
@@ -87,16 +99,21 @@ struct PipeKernel {
     static constexpr int A_BYTES = BM * RB, B_BYTES = BN * RB, STAGE_BYTES = A_BYTES + B_BYTES;
     static constexpr int A_PW = BM / 8 / WAVES, B_PW = BN / 8 / WAVES;  // load instructions per wave per stage
     static constexpr int LPS = A_PW + B_PW;
+    static constexpr int NLOADS = LPS + (CKPT ? 1 : 0);   // + the stop-word load of a checkpointing body
     static constexpr int WGM = SPLITK ? 1 : 2, WGN = SPLITK ? 1 : 2;
     static constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 32, NI = WN / 32;
     static constexpr size_t RED_BYTES = (size_t)WAVES * (SPLITK ? MI : 1) * NI * 16 * 64 * 4;  // epilogue staging
     static constexpr size_t RING_BYTES = (size_t)STAGES * STAGE_BYTES > RED_BYTES ? (size_t)STAGES * STAGE_BYTES : RED_BYTES;
-    static constexpr size_t LDS_BYTES = RING_BYTES + (CKPT ? 16 : 0);  // + the stop words of a checkpointing body
+    static constexpr size_t POLL_BYTES = CKPT ? (size_t)STAGES * WAVES * 256 : 0;  // a 256-byte landing slot per wave and stage
+    static constexpr size_t LDS_BYTES = RING_BYTES + POLL_BYTES;
     static constexpr size_t CKPT_SLOT_BYTES = (size_t)WAVES * MI * NI * 16 * 64 * 4;  // one workgroup's accumulators
     static constexpr bool ckpt = CKPT;
-    static_assert(!CKPT || (STAGES == 2 && !CONV && !SPLITK), "checkpointing is built for the two-stage GEMM body");
+    // The stop words are fetched with every stage (so that every wave issues the same number of
+    // loads) but looked at every POLL_EVERY-th K-step: about every 2.5 us for either tile size.
+    static constexpr int POLL_EVERY = BM >= 256 ? 2 : 4;
+    static_assert(!CKPT || !SPLITK, "checkpointing is built for the bodies without split K");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && A_PW >= 1 && B_PW >= 1, "tile shape");
-    static_assert(STAGES >= 2 && (STAGES - 2) * LPS < 64, "pipeline depth");
+    static_assert(STAGES >= 2 && (STAGES - 2) * NLOADS < 64, "pipeline depth");
 
     // Returns true when the tile was left half-way (CKPT only); kt0 > 0 continues such a tile.
     static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0},
@@ -119,6 +136,7 @@ struct PipeKernel {
         }
         const T *A = (const T *)g.A + offa, *B = (const T *)g.B + offb;
         const T *zero = (const T *)g_zero_page;
+        const bool can_ckpt = CKPT && cc.stop_index != nullptr && cc.ckpt != nullptr;
 
         // ---- loader slots -------------------------------------------------------------------
         // Slot j of a wave covers rows (wave*PW + j)*8 .. +7 of the operand block; lane -> (row in
@@ -152,19 +170,40 @@ struct PipeKernel {
                              B + (long)b_row0 * g.ldb + chunk_of(wave * B_PW + 1) * VEC};
         const bool conv_fast = CONV && (g.Cin % BK == 0);  // a K-step never straddles a filter tap
         const bool k_full = g.K % BK == 0;                 // no K-chunk of any stage lies past K
+        // Running source pointers.  Within one filter tap (conv) or along K (weights, GEMM rows) a
+        // slot's address only advances by BK elements per stage, so it is kept and bumped instead
+        // of rebuilt: a wave has one instruction stream, and twenty address instructions per load
+        // were more issue time than the MFMAs they feed.  `inc` is 0 for a slot parked on the zero
+        // page.  (Only bodies with few slots keep them for the B / GEMM-A side: registers.)
+        constexpr bool INCR = A_PW + B_PW <= 8;
+        const T *a_cur[A_PW], *b_cur[B_PW];
+        int a_inc[A_PW], b_inc[B_PW];
+#pragma unroll
+        for (int j = 0; j < A_PW; ++j) { a_cur[j] = zero; a_inc[j] = 0; }
+#pragma unroll
+        for (int j = 0; j < B_PW; ++j) { b_cur[j] = zero; b_inc[j] = 0; }
 
         // Loads of one stage: slot l < A_PW is an A slot, the rest are B slots.  `StageAddr` holds
         // the wave-uniform part, computed once per stage.
-        struct StageAddr { unsigned sbase; int k0, r_u, s_u, tap_off; };
+        struct StageAddr { unsigned sbase, sbase_poll; int k0, r_u, s_u, tap_off; bool new_tap, first; };
         // Stages are fetched in increasing order, so the filter tap (r, s) and channel offset of
         // the next stage advance incrementally instead of being divided out of k every time.
         int nx_r = 0, nx_s = 0, nx_ci = 0;
+        if (CKPT && CONV && kt0 > 0 && conv_fast) {  // a tile that is continued starts at K-step kt0
+            const int k = kt0 * BK, rs = k / g.Cin;
+            nx_ci = k - rs * g.Cin;
+            nx_r = rs / g.S;
+            nx_s = rs - nx_r * g.S;
+        }
         auto stage_addr = [&](int kt) {
             StageAddr sa;
             sa.sbase = lds0 + (unsigned)(kt % STAGES) * STAGE_BYTES;
+            sa.sbase_poll = lds0 + (unsigned)RING_BYTES + (unsigned)(kt % STAGES) * WAVES * 256;
             sa.k0 = kt * BK;
             sa.r_u = nx_r; sa.s_u = nx_s;
             sa.tap_off = (nx_r * g.W + nx_s) * (int)g.lda + nx_ci;  // elements from the window origin
+            sa.first = kt == kt0;                  // first stage fetched for this tile (or its continuation)
+            sa.new_tap = sa.first || nx_ci == 0;   // the running conv pointers have to be rebuilt
             if (conv_fast) {
                 nx_ci += BK;
                 if (nx_ci >= g.Cin) {
@@ -175,25 +214,49 @@ struct PipeKernel {
             return sa;
         };
         auto issue_one = [&](const StageAddr &sa, int l) {  // l is a compile-time constant at every call
-            if (l < A_PW) {
+            if (CKPT && l == LPS) {
+                // wave 0 fetches the stop index, wave 1 (when it is this workgroup's turn) the host
+                // flag, the others a zero: every wave issues the same number of loads per stage
+                const void *src = zero;
+                if (can_ckpt) {
+                    if (wave == 0) src = cc.stop_index;
+                    else if (wave == 1 && blockIdx.x < 8 && cc.flag && ((sa.k0 / BK) & (8 * POLL_EVERY - 1)) == (int)blockIdx.x * POLL_EVERY) src = cc.flag;
+                }
+                load_lds4(src, sa.sbase_poll + (unsigned)wave * 256);
+            } else if (l < A_PW) {
                 const int j = l;
                 const int kc = chunk_of(wave * A_PW + j) * VEC;
                 const T *src;
                 if (CONV) {
                     const int jj = CONV ? j : 0;
-                    int r, s2, off;
-                    bool ok = a_row0 + j * 8 < g.M;
                     if (conv_fast) {
-                        r = sa.r_u; s2 = sa.s_u; off = sa.tap_off + kc;
+                        if (sa.new_tap) {  // (uniform) rebuild: bounds of the tap, pointer or zero page
+                            const bool ok = (a_row0 + j * 8 < g.M) & ((unsigned)(a_h0[jj] + sa.r_u) < (unsigned)g.H) &
+                                            ((unsigned)(a_w0[jj] + sa.s_u) < (unsigned)g.W);
+                            a_cur[j] = ok ? a_org[jj] + (sa.tap_off + kc) : zero;
+                            a_inc[j] = ok ? BK : 0;
+                        } else {
+                            a_cur[j] += a_inc[j];
+                        }
+                        src = a_cur[j];
                     } else {
-                        int k = sa.k0 + kc, rs = k / g.Cin, ci = k - rs * g.Cin;
-                        r = rs / g.S; s2 = rs - r * g.S;
-                        off = (r * g.W + s2) * (int)g.lda + ci;
-                        ok = ok & (k < g.K);
+                        const int k = sa.k0 + kc, rs = k / g.Cin, ci = k - rs * g.Cin;
+                        const int r = rs / g.S, s2 = rs - r * g.S;
+                        const int off = (r * g.W + s2) * (int)g.lda + ci;
+                        // selects, not branches: every lane computes an address and picks it or the zero page
+                        const bool ok = (a_row0 + j * 8 < g.M) & (k < g.K) & ((unsigned)(a_h0[jj] + r) < (unsigned)g.H) &
+                                        ((unsigned)(a_w0[jj] + s2) < (unsigned)g.W);
+                        src = ok ? a_org[jj] + off : zero;
                     }
-                    // selects, not branches: every lane computes an address and picks it or the zero page
-                    ok = ok & ((unsigned)(a_h0[jj] + r) < (unsigned)g.H) & ((unsigned)(a_w0[jj] + s2) < (unsigned)g.W);
-                    src = ok ? a_org[jj] + off : zero;
+                } else if (INCR && k_full) {
+                    if (sa.first) {
+                        const bool ok = a_row0 + j * 8 < g.M;
+                        a_cur[j] = ok ? a_par[j & 1] + ((long)(j * 8) * g.lda + sa.k0) : zero;
+                        a_inc[j] = ok ? BK : 0;
+                    } else {
+                        a_cur[j] += a_inc[j];
+                    }
+                    src = a_cur[j];
                 } else {
                     const bool ok = (a_row0 + j * 8 < g.M) & (k_full | (sa.k0 + kc < g.K));
                     src = ok ? a_par[j & 1] + ((long)(j * 8) * g.lda + sa.k0) : zero;
@@ -202,15 +265,27 @@ struct PipeKernel {
             } else {
                 const int j = l - A_PW;
                 const int kc = chunk_of(wave * B_PW + j) * VEC;
-                const bool ok = (b_row0 + j * 8 < g.N) & (k_full | (sa.k0 + kc < g.K));
-                const T *src = ok ? b_par[j & 1] + ((long)(j * 8) * g.ldb + sa.k0) : zero;
+                const T *src;
+                if (INCR && k_full) {
+                    if (sa.first) {
+                        const bool ok = b_row0 + j * 8 < g.N;
+                        b_cur[j] = ok ? b_par[j & 1] + ((long)(j * 8) * g.ldb + sa.k0) : zero;
+                        b_inc[j] = ok ? BK : 0;
+                    } else {
+                        b_cur[j] += b_inc[j];
+                    }
+                    src = b_cur[j];
+                } else {
+                    const bool ok = (b_row0 + j * 8 < g.N) & (k_full | (sa.k0 + kc < g.K));
+                    src = ok ? b_par[j & 1] + ((long)(j * 8) * g.ldb + sa.k0) : zero;
+                }
                 load_lds16(src, sa.sbase + (unsigned)(A_BYTES + (wave * B_PW + j) * 8 * RB));
             }
         };
         auto issue = [&](int kt) {
             const StageAddr sa = stage_addr(kt);
 #pragma unroll
-            for (int l = 0; l < LPS; ++l) issue_one(sa, l);
+            for (int l = 0; l < NLOADS; ++l) issue_one(sa, l);
         };
 
         f32x16 acc[MI][NI];
@@ -221,11 +296,10 @@ struct PipeKernel {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
         // checkpointing state
-        const bool can_ckpt = CKPT && cc.stop_index != nullptr && cc.ckpt != nullptr;
         f32x4 *slot = nullptr;       // this wave's part of the workgroup's checkpoint slot
-        // two LDS words behind the ring, indexed by K-step parity
+        // landing slots of the stop-word loads, behind the ring: [stage][wave][64 dwords]
         typedef __attribute__((address_space(3))) volatile int lds_vint;
-        lds_vint *stopw = (lds_vint *)(__attribute__((address_space(3))) void *)lds_t + RING_BYTES / 4;
+        lds_vint *pollw = (lds_vint *)(__attribute__((address_space(3))) void *)lds_t + RING_BYTES / 4;
         if (CKPT && can_ckpt) {
             slot = (f32x4 *)((char *)cc.ckpt + (size_t)CKPT_MAX_WGS * CKPT_HEADER_INTS * 4 + (size_t)blockIdx.x * CKPT_SLOT_BYTES) +
                    (size_t)wave * MI * NI * 4 * 64;
@@ -237,12 +311,14 @@ struct PipeKernel {
 #pragma unroll
                         for (int q = 0; q < 4; ++q) {
                             f32x4 v = slot[((i * NI + j) * 4 + q) * 64 + lane];
+                            // (reading the value here makes the compiler wait for the load now: left
+                            // pending, it would put vmcnt waits in front of the MFMAs of every K-step)
+                            asm volatile("" : "+v"(v));
 #pragma unroll
                             for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = v[e];
                         }
             }
         }
-        int polled_stop = -1, polled_flag = 0;  // what lane 0 of wave 0 read one K-step ago
 
         const int wm = SPLITK ? 0 : wave / WGN, wn = SPLITK ? 0 : wave % WGN;
         auto frag = [&](int stage, int region_bytes, int row, int chunk) -> u32x4 {
@@ -271,19 +347,19 @@ struct PipeKernel {
         // SPREAD-th MFMA, so that their address arithmetic issues while the matrix pipe is busy
         // instead of in front of it, and the requests reach the memory system as a steady stream.
         constexpr int NM = MI * NI;
-        constexpr int EVEN = KSTEPS * NM / LPS > 0 ? KSTEPS * NM / LPS : 1;
+        constexpr int EVEN = KSTEPS * NM / NLOADS > 0 ? KSTEPS * NM / NLOADS : 1;
         constexpr int SPREAD = GP_LOAD_SPREAD > 0 ? GP_LOAD_SPREAD : (EVEN >= 4 ? EVEN - 1 : EVEN);  // measured: slightly front-loaded beats even for the 256x256 tile
-        static_assert(SPLITK || LPS <= KSTEPS * NM, "every load of a stage needs an MFMA slot");
+        static_assert(SPLITK || NLOADS <= KSTEPS * NM, "every load of a stage needs an MFMA slot");
         auto phase = [&](int buf, auto issue_c, const StageAddr &sa, auto p_c) {
             constexpr bool ISSUE = decltype(issue_c)::value != 0;
             constexpr int P = decltype(p_c)::value;
             static_for<0, NM>([&](auto qc) {
                 constexpr int q = decltype(qc)::value, slot = P * NM + q;
                 Elem<T>::mma(fa[buf][q / NI], fb[buf][q % NI], acc[q / NI][q % NI]);
-                if constexpr (ISSUE && slot % SPREAD == 0 && slot / SPREAD < LPS) issue_one(sa, slot / SPREAD);
+                if constexpr (ISSUE && slot % SPREAD == 0 && slot / SPREAD < NLOADS) issue_one(sa, slot / SPREAD);
                 // the slots cannot hold every load at this spacing: the rest follow the last MFMA
-                if constexpr (ISSUE && slot == KSTEPS * NM - 1 && slot / SPREAD + 1 < LPS)
-                    static_for<slot / SPREAD + 1, LPS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
+                if constexpr (ISSUE && slot == KSTEPS * NM - 1 && slot / SPREAD + 1 < NLOADS)
+                    static_for<slot / SPREAD + 1, NLOADS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
                 if constexpr (ISSUE) __builtin_amdgcn_sched_barrier(0);
             });
         };
@@ -291,29 +367,15 @@ struct PipeKernel {
         auto ktile = [&](int kt, bool tail, auto issue_c) -> int {
             constexpr bool ISSUE = decltype(issue_c)::value != 0;
             // stage kt has landed once at most the loads of the younger in-flight stages remain
-            if (!tail) wait_vmcnt<(STAGES - 2) * LPS>();
+            if (!tail) wait_vmcnt<(STAGES - 2) * NLOADS>();
             else wait_vmcnt<0>();
-            int stop_now = 0, stop_word = 0;
-            if constexpr (CKPT) {
-                if (can_ckpt && tid == 0) {
-                    // publish last K-step's reads (they have landed: the wait above was for vmcnt 0)
-                    if (polled_flag != 0) atomicCAS(cc.stop_index, -1, cc.kernel_id);
-                    stopw[kt & 1] = (polled_stop != -1) | (polled_flag != 0);
-                }
-            }
+            int stop_word = -1, flag_word = 0;
             __syncthreads();  // everyone's part of stage kt is visible; stage kt-1's buffer is free
             if constexpr (CKPT) {
-                if (can_ckpt) {
-                    stop_word = stopw[kt & 1];  // the same word for every wave: a uniform decision, looked at below
-                    if (tid == 0) {
-                        polled_stop = __hip_atomic_load(cc.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        // The flag is host memory: its read takes about as long as a K-step and the
-                        // next K-step's vmcnt(0) waits for it.  So eight workgroups take turns, each
-                        // reading it once in 16 K-steps: a read every second K-step overall, 6 %
-                        // of a K-step per polling workgroup.
-                        if (blockIdx.x < 8 && cc.flag && (kt & 15) == (int)blockIdx.x * 2)
-                            polled_flag = __hip_atomic_load(cc.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                    }
+                if (can_ckpt && (kt & (POLL_EVERY - 1)) == 0) {
+                    // the words that travelled with stage kt: the same two for every wave, looked at below
+                    stop_word = pollw[((kt % STAGES) * WAVES + 0) * 64];
+                    flag_word = pollw[((kt % STAGES) * WAVES + 1) * 64];
                 }
             }
             if (kt == 0) GP_PROBE(2);
@@ -322,7 +384,7 @@ struct PipeKernel {
             if constexpr (ISSUE) sa = stage_addr(kt + STAGES - 1);
             if constexpr (SPLITK) {
                 read_frags(0, stage, wave);  // the address arithmetic of the loads overlaps the LDS latency
-                if constexpr (ISSUE) static_for<0, LPS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
+                if constexpr (ISSUE) static_for<0, NLOADS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
                 mma_all(0);
             } else {
                 constexpr int LAST = (KSTEPS - 1) & 1;
@@ -333,7 +395,7 @@ struct PipeKernel {
                 } else if constexpr (ISSUE) {
                     static_for<0, NM>([&](auto qc) {  // first k-tile: phase 0 has loads but no MFMAs
                         constexpr int slot = decltype(qc)::value;
-                        if constexpr (slot % SPREAD == 0 && slot / SPREAD < LPS) issue_one(sa, slot / SPREAD);
+                        if constexpr (slot % SPREAD == 0 && slot / SPREAD < NLOADS) issue_one(sa, slot / SPREAD);
                     });
                 }
                 static_for<0, KSTEPS - 1>([&](auto kc) {
@@ -345,7 +407,12 @@ struct PipeKernel {
                 });
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if constexpr (CKPT) stop_now = __builtin_amdgcn_readfirstlane(stop_word);
+            int stop_now = 0;
+            if constexpr (CKPT) {
+                const int sw = __builtin_amdgcn_readfirstlane(stop_word), fw = __builtin_amdgcn_readfirstlane(flag_word);
+                if (fw != 0 && tid == 0) atomicCAS(cc.stop_index, -1, cc.kernel_id);  // pass the host flag on
+                stop_now = (sw != -1) | (fw != 0);
+            }
             return stop_now;
         };
 

@@ -163,8 +163,8 @@ typedef struct gp_gemm_params {
     int variant;        /* enum gp_mat_variant; 0 = chosen by the launcher */
 } gp_gemm_params;
 int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
-/* Bytes of gp_preempt_ctx::ckpt workspace this GEMM can use (0: its tiles are short and always
- * finished), and the reset of such a workspace.  Extension of the dispatcher that
+/* Bytes of gp_preempt_ctx::ckpt workspace this GEMM can use (0: it runs on a body whose tiles are
+ * short and always finished), and the reset of such a workspace.  Extension of the dispatcher that
  * scripts/compile/convert_to_blp.py:40-69 generates (which can only stop between tiles). */
 int gp_gemm_ckpt_bytes(const gp_gemm_params *p, size_t *bytes);
 int gp_ckpt_reset_async(void *ckpt, gp_stream s);
@@ -187,6 +187,8 @@ typedef struct gp_conv_params {
     int variant;
 } gp_conv_params;
 int gp_launch_conv2d(const gp_conv_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+/* As gp_gemm_ckpt_bytes, for a convolution (0 unless it runs on the 128 x 128 body). */
+int gp_conv_ckpt_bytes(const gp_conv_params *p, size_t *bytes);
 
 /* NCHW -> NHWC with zero padding of the channel count up to c_pad (input adapter: the
  * reference's "data" tensor is NCHW, src/tests/test-dnn.cpp:25-30). */

@@ -121,9 +121,12 @@ def test_config1_preempt_resume_bit_exact(gp, tile):
     base = dC.download(gp.F32, (1024, 1024)).copy()
     ref = O.gemm_bias_act(A, B, bias, act=O.ACT_RELU)
     assert rel_err(base, ref) < 1e-4
-    # uninterrupted, preemptible launch: same bits
+    # uninterrupted, preemptible launch: same bits.  The grid is capped below the tile count so
+    # that claims are spread over the kernel's run: with one workgroup per tile every claim is made
+    # in the first microsecond and whether one of them sees the injected flag is a race.
+    WGS = 16
     dC.fill32(0xFFFFFFFF)
-    info = gp.launch("gp_launch_gemm", p, st.ctx())
+    info = gp.launch("gp_launch_gemm", p, st.ctx(max_workgroups=WGS))
     gp.check(gp.lib().gp_stream_sync(None))
     total = info.total_tiles
     assert total == (1024 // tile) ** 2 and info.grid <= total
@@ -135,7 +138,7 @@ def test_config1_preempt_resume_bit_exact(gp, tile):
         st.reset()
         flag.set(0)
         dC.fill32(0xFFFFFFFF)
-        gp.launch("gp_launch_gemm", p, st.ctx(inject_at=k - 1))  # claim number k raises the flag
+        gp.launch("gp_launch_gemm", p, st.ctx(inject_at=k - 1, max_workgroups=WGS))  # claim number k raises the flag
         gp.check(gp.lib().gp_stream_sync(None))
         assert flag.get() == 1
         assert st.stop_index() == 0
@@ -148,7 +151,7 @@ def test_config1_preempt_resume_bit_exact(gp, tile):
         # host: *flag = 0; resume (executor.cpp:280-298): counters are NOT reset
         flag.set(0)
         st.clear_stop()
-        gp.launch("gp_launch_gemm", p, st.ctx())
+        gp.launch("gp_launch_gemm", p, st.ctx(max_workgroups=WGS))
         gp.check(gp.lib().gp_stream_sync(None))
         assert np.array_equal(dC.download(gp.F32, (1024, 1024)), base), f"resume after {frac:.0%} differs"
         assert st.stop_index() == -1

@@ -216,3 +216,47 @@ def test_every_op_resumes_bit_exact(gp):
         sync(gp)
         assert np.array_equal(do.download(), base), fn
         assert st.stop_index() == -1
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+def test_conv2d_long_tiles_left_mid_k_and_resumed_bit_exact(gp, dt):
+    """A deep 3x3 convolution on the 128 x 128 body (K = 9 * Cin): with the checkpoint workspace the
+    stop request is honoured between two K-steps, and the resumed result (bias, residual and ReLU
+    included) is bit-identical to the uninterrupted one."""
+    rng = np.random.default_rng(21)
+    N, H, Cin, Cout = 4, 16, 512 if dt == "f16" else 256, 256
+    x = rnd(rng, (N, Cin, H, H), dt)
+    w = rnd(rng, (Cout, Cin, 3, 3), dt, -0.05, 0.05)
+    b = rnd(rng, (Cout,), dt, -0.1, 0.1)
+    res = rnd(rng, (N, Cout, H, H), dt)
+    want, info0, (p, do, keep) = gpu_conv2d(gp, dt, x, w, b, 1, 1, res, gp.ACT_RELU, tile=128, variant=2)
+    ref = O.conv2d(x, w, b, 1, 1, residual=res, act=O.ACT_RELU) if hasattr(O, "ACT_RELU") else None
+    if ref is not None:
+        assert rel_err(want, O.round_to(ref, dt)) < TOL[dt]
+    raw_want = do.download().copy()
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    assert st.enable_checkpoints(p) > 0
+    stream = gp.Stream(1)
+    tiles = info0.total_tiles
+    stopped = 0
+    for inject in (0, tiles // 2):
+        do.fill32(0)
+        st.reset(); st.clear_stop(); flag.set(0)
+        gp.check(gp.lib().gp_ckpt_reset_async(gp.vp(st.ckpt.ptr), None))
+        info = gp.launch("gp_launch_conv2d", p, st.ctx(kernel_id=0, inject_at=inject), stream)
+        stream.sync()
+        assert flag.get() == 1
+        hdr = st.checkpoint_headers(info.grid)
+        if st.stop_index() == 0 and hdr[:, 0].sum() > 0:
+            stopped += 1
+            live = hdr[hdr[:, 0] == 1]
+            assert (live[:, 3] > 0).all() and len(set(live[:, 2].tolist())) == len(live)
+            assert not np.array_equal(do.download(), raw_want)
+        flag.set(0); st.clear_stop()
+        gp.launch("gp_launch_conv2d", p, st.ctx(kernel_id=0), stream)
+        stream.sync()
+        assert st.stop_index() == -1
+        assert int(st.checkpoint_headers(info.grid)[:, 0].sum()) == 0
+        assert np.array_equal(do.download(), raw_want), (dt, inject)
+    assert stopped >= 1, "the stop request was never seen inside a tile"
