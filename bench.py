@@ -214,6 +214,56 @@ def gemm_roofline(iters=10):
             "with_checkpoint_workspace": {"ms": t_ck * 1e3, "achieved": flop / t_ck / 1e12, "frac": flop / t_ck / 1e12 / PEAK["bf16"]}}
 
 
+def hbm_ops(iters=20):
+    """The memory-bound operators against the 8 TB/s HBM peak: achieved = algorithmic bytes (tensor in
+    + tensor out) / HIP-event time of one preemptible launch, at the shapes the two tenants use and at
+    a size large enough to leave the launch-latency regime."""
+    from gpreempt_amd import capi as gp
+    stream = gp.Stream(1)
+    flag = gp.Flag()
+    out = {}
+
+    def timed(fn, p, bytes_moved):
+        st = gp.BlpState(1, flag)
+        e0, e1 = gp.Event(), gp.Event()
+        ms = []
+        for i in range(iters + 2):
+            st.reset()
+            e0.record(stream)
+            gp.launch(fn, p, st.ctx(), stream)
+            e1.record(stream)
+            e1.sync()
+            if i >= 2:
+                ms.append(e0.elapsed_ms(e1))
+        t = sorted(ms)[len(ms) // 2] * 1e-3
+        return {"us": t * 1e6, "algorithmic_bytes": bytes_moved, "achieved": bytes_moved / t / 1e9, "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "frac": bytes_moved / t / 1e9 / HBM_PEAK_GBS}
+
+    def buf(n_bytes, pattern=0x3C003C00):
+        b = gp.DevBuf(n_bytes)
+        b.fill32(pattern)
+        return b
+
+    for tag, rows, cols in (("resnet152_b8_56x56x256", 8 * 56 * 56, 256), ("large", 1 << 18, 512)):
+        a, b2, o = buf(rows * cols * 2), buf(rows * cols * 2), buf(rows * cols * 2)
+        p = gp.EltwiseParams(dtype=gp.F16, rows=rows, cols=cols, a=a.ptr, a_stride=cols, b=b2.ptr, b_stride=cols, out=o.ptr, out_stride=cols, act=gp.ACT_RELU)
+        out["add_relu_f16_" + tag] = timed("gp_launch_eltwise", p, 3 * rows * cols * 2)
+    for tag, N, H, Cc in (("resnet152_b8_112x112x64", 8, 112, 64), ("large_b64", 64, 112, 64)):
+        Ho = (H + 2 - 3) // 2 + 1
+        x, o = buf(N * H * H * Cc * 2), buf(N * Ho * Ho * Cc * 2)
+        p = gp.PoolParams(dtype=gp.F16, N=N, H=H, W=H, C=Cc, R=3, S=3, stride=2, pad=1, mode=0, in_=x.ptr, in_pix_stride=Cc, out=o.ptr, out_pix_stride=Cc)
+        out["maxpool3x3s2_f16_" + tag] = timed("gp_launch_pool2d", p, (N * H * H * Cc + N * Ho * Ho * Cc) * 2)
+    for tag, rows, cols in (("bert_s128", 128, 768), ("large", 1 << 17, 768)):
+        x, r, g, be, o = buf(rows * cols * 2), buf(rows * cols * 2), buf(cols * 2), buf(cols * 2), buf(rows * cols * 2)
+        p = gp.LayernormParams(dtype=gp.F16, rows=rows, cols=cols, x=x.ptr, residual=r.ptr, gamma=g.ptr, beta=be.ptr, out=o.ptr, eps=1e-12)
+        out["residual_layernorm_f16_" + tag] = timed("gp_launch_layernorm", p, 3 * rows * cols * 2)
+    for tag, rows, cols in (("bert_s128_12heads", 12 * 128, 128), ("large", 1 << 19, 128)):
+        x, o = buf(rows * cols * 2), buf(rows * cols * 2)
+        p = gp.SoftmaxParams(dtype=gp.F16, rows=rows, cols=cols, x=x.ptr, out=o.ptr, scale=0.125)
+        out["softmax_f16_" + tag] = timed("gp_launch_softmax", p, 2 * rows * cols * 2)
+    return out
+
+
 def copy_calibration(mib=256, iters=10):
     """A plain device-to-device copy of known size (the runtime's copy kernel), used to scale
     the FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc runs."""
@@ -262,7 +312,7 @@ def main():
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
-    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | cpu | copycal")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | cpu | copycal")
     ap.add_argument("--cpu-requests", type=int, default=4)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -291,6 +341,8 @@ def main():
     if args.only in ("", "gemm"):
         out["config5_gemm8192_bf16"] = gemm_roofline()
         out["config1_gemm1024_f32"] = config1_gemm1024()
+    if args.only in ("", "hbm"):
+        out["hbm_bound_ops"] = hbm_ops()
     if args.only == "copycal":
         out["copy_calibration"] = copy_calibration()
     if args.only in ("", "cpu"):

@@ -48,10 +48,13 @@ inline size_t dtype_size(int dt) {
 // workgroup per tile.
 template <class Kernel>
 int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int sz,
-                const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info) {
-    long total = (long)sx * sy * sz;
-    GP_REQUIRE(total > 0 && total < (1L << 31), "tile count %ld out of range", total);
+                const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info, int batch = 1) {
+    long tiles = (long)sx * sy * sz;
+    GP_REQUIRE(tiles > 0 && tiles < (1L << 31), "tile count %ld out of range", tiles);
+    if (batch < 1) batch = 1;
+    long total = (tiles + batch - 1) / batch;  // claims
     blp->total = (int)total; blp->sx = sx; blp->sy = sy; blp->order = 0; blp->ckpt = nullptr;
+    blp->batch = batch; blp->tiles = (int)tiles;
     if (ctx) {
         GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
         blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;

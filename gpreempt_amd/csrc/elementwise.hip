@@ -1,3 +1,4 @@
+#include <algorithm>
 // Stand-alone launchers of the memory-bound operators (C ABI); the tile bodies live in
 // elementwise_bodies.hpp.
 #include "plans.hpp"
@@ -8,7 +9,10 @@ template <class Kernel, class Arg>
 static int launch_tiles(Kernel kern, int sx, int sy, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info, const Arg &arg) {
     BlpArgs blp;
     int grid = 0;
-    int rc = plan_launch(kern, NT, 0, sx, sy, 1, ctx, &blp, &grid, info);
+    // several tiles per claim once there are far more tiles than workgroups that could hold them
+    const long tiles = (long)sx * sy;
+    const int batch = (int)std::min<long>(16, std::max<long>(1, tiles / (32L * device_cus())));
+    int rc = plan_launch(kern, NT, 0, sx, sy, 1, ctx, &blp, &grid, info, batch);
     if (rc) return rc;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), 0, native(s), arg, blp);
     GP_HIP(hipGetLastError());
@@ -83,7 +87,10 @@ int plan_softmax(const gp_softmax_params *p, EltPlan *out) {
     GP_REQUIRE(p && p->x && p->out, "null softmax params");
     GP_REQUIRE(is_float(p->dtype), "softmax dtype %d", p->dtype);
     GP_REQUIRE(p->rows > 0 && p->cols > 0, "softmax shape");
-    long tiles = (p->rows + 3) / 4;
+    // rows made of whole 16-byte chunks are read as vectors
+    GP_REQUIRE(softmax_group(p->cols, vec_of(p->dtype)) == 0 || (al16(p->x) && al16(p->out)), "softmax: 16-byte alignment");
+    const int rpt = softmax_rows_per_tile(p->cols, vec_of(p->dtype));
+    long tiles = (p->rows + rpt - 1) / rpt;
     GP_REQUIRE(tiles < (1L << 31), "softmax: too many rows");
     *out = EltPlan{};
     out->op = OP_SOFTMAX; out->dtype = p->dtype; out->sx = (int)tiles; out->sy = 1;

@@ -230,23 +230,89 @@ __global__ __launch_bounds__(NT) void eltwise_kernel(EltwiseArgs a, BlpArgs blp)
 }
 
 // ---- softmax -------------------------------------------------------------------------------
-// one wavefront per row, 4 rows per tile; lane i reads elements i, i+64, ...
+// A row is held in registers by G lanes (16-byte chunks, C per lane): one read and one write per
+// element, reductions by xor-shuffles inside the lane group.  Short rows share a wavefront: with
+// G = 16 a wave handles 4 rows at once (BERT's 128-wide score rows are 16 chunks of fp16).
+// Rows whose length is not a multiple of the chunk, or longer than 256 chunks, take the scalar path.
+__host__ __device__ inline int softmax_group(int cols, int vec) {  // lanes per row; 0 = scalar path
+    if (cols % vec) return 0;
+    const int chunks = cols / vec;
+    return chunks <= 16 ? 16 : chunks <= 256 ? 64 : 0;
+}
+__host__ __device__ inline int softmax_rows_per_tile(int cols, int vec) {
+    const int g = softmax_group(cols, vec);
+    return g ? 4 * (64 / g) : 4;
+}
+
+template <typename T, int G, int C>
+__device__ __forceinline__ void softmax_rows_grouped(const gp_softmax_params &p, TileIdx t) {
+    constexpr int VEC = VecIO<T>::VEC;
+    const int lane = threadIdx.x & 63, sub = lane % G;
+    const long row = ((long)t.x * 4 + (threadIdx.x >> 6)) * (64 / G) + lane / G;
+    const int chunks = p.cols / VEC;
+    const bool live = row < p.rows;
+    const T *x = (const T *)p.x + (live ? row : 0) * p.cols;
+    float v[C][VEC];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        const int ch = sub + i * G;
+        if (live && ch < chunks) {
+            VecIO<T>::load(x + ch * VEC, v[i]);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) { v[i][j] *= p.scale; mx = fmaxf(mx, v[i][j]); }
+        }
+    }
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        const int ch = sub + i * G;
+        if (live && ch < chunks) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) { v[i][j] = __expf(v[i][j] - mx); sum += v[i][j]; }
+        }
+    }
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+    const float inv = 1.f / sum;
+    T *out = (T *)p.out + (live ? row : 0) * p.cols;
+#pragma unroll
+    for (int i = 0; i < C; ++i) {
+        const int ch = sub + i * G;
+        if (live && ch < chunks) {
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) v[i][j] *= inv;
+            VecIO<T>::store(out + ch * VEC, v[i]);
+        }
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ void softmax_tile(const gp_softmax_params &p, TileIdx t) {
-    
-        long row = (long)t.x * 4 + (threadIdx.x >> 6);
-        if (row >= p.rows) return;
-        const int lane = threadIdx.x & 63;
-        const T *x = (const T *)p.x + row * p.cols;
-        T *o = (T *)p.out + row * p.cols;
-        float mx = -INFINITY;
-        for (int c = lane; c < p.cols; c += 64) mx = fmaxf(mx, VecIO<T>::ld1(x + c) * p.scale);
-        mx = wave_max(mx);
-        float sum = 0.f;
-        for (int c = lane; c < p.cols; c += 64) sum += __expf(VecIO<T>::ld1(x + c) * p.scale - mx);
-        sum = wave_sum(sum);
-        float inv = 1.f / sum;
-        for (int c = lane; c < p.cols; c += 64) VecIO<T>::st1(o + c, __expf(VecIO<T>::ld1(x + c) * p.scale - mx) * inv);
+    constexpr int VEC = VecIO<T>::VEC;
+    const int g = softmax_group(p.cols, VEC);  // uniform
+    if (g == 16) { softmax_rows_grouped<T, 16, 1>(p, t); return; }
+    if (g == 64) {
+        if (p.cols / VEC <= 64) softmax_rows_grouped<T, 64, 1>(p, t);
+        else softmax_rows_grouped<T, 64, 4>(p, t);
+        return;
+    }
+    // scalar path: one wavefront per row, 4 rows per tile; lane i reads elements i, i+64, ...
+    long row = (long)t.x * 4 + (threadIdx.x >> 6);
+    if (row >= p.rows) return;
+    const int lane = threadIdx.x & 63;
+    const T *x = (const T *)p.x + row * p.cols;
+    T *o = (T *)p.out + row * p.cols;
+    float mx = -INFINITY;
+    for (int c = lane; c < p.cols; c += 64) mx = fmaxf(mx, VecIO<T>::ld1(x + c) * p.scale);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int c = lane; c < p.cols; c += 64) sum += __expf(VecIO<T>::ld1(x + c) * p.scale - mx);
+    sum = wave_sum(sum);
+    float inv = 1.f / sum;
+    for (int c = lane; c < p.cols; c += 64) VecIO<T>::st1(o + c, __expf(VecIO<T>::ld1(x + c) * p.scale - mx) * inv);
 }
 template <typename T>
 __global__ __launch_bounds__(NT) void softmax_kernel(gp_softmax_params p, BlpArgs blp) {

@@ -36,6 +36,8 @@ struct BlpArgs {
     int groups;       // claim counters per kernel (>= 1); counter g sits at executed + g * COUNTER_STRIDE
     int order;        // tile order: 0 = x fastest (the reference's), 1 = y fastest
     void *ckpt;       // checkpoint workspace of kernels that can leave a tile half-way, or nullptr
+    int batch;        // tiles per claim (>= 1): a claim of index u stands for tiles [u*batch, (u+1)*batch)
+    int tiles;        // number of tiles (total = ceil(tiles / batch) claims)
 };
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
@@ -122,7 +124,10 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
             idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1]);  // wave-uniform: tile coordinates stay scalar
         }
         if (idx < 0) return;
-        body(decode_tile(idx, b.sx, b.sy, b.order));
+        // Streaming kernels have tiles of a few KB; handing them out several at a time keeps the
+        // claim (an atomic and a barrier, 1-2 us) off their critical path.
+        const int first = idx * b.batch, last = first + b.batch < b.tiles ? first + b.batch : b.tiles;
+        for (int tile = first; tile < last; ++tile) body(decode_tile(tile, b.sx, b.sy, b.order));
     }
 }
 
