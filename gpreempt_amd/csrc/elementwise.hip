@@ -6,15 +6,16 @@
 namespace gp {
 
 template <class Kernel, class Arg>
-static int launch_tiles(Kernel kern, int sx, int sy, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info, const Arg &arg) {
+static int launch_tiles(Kernel kern, int sx, int sy, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info, const Arg &arg, size_t lds_bytes = 0) {
     BlpArgs blp;
     int grid = 0;
     // several tiles per claim once there are far more tiles than workgroups that could hold them
     const long tiles = (long)sx * sy;
     const int batch = (int)std::min<long>(16, std::max<long>(1, tiles / (32L * device_cus())));
-    int rc = plan_launch(kern, NT, 0, sx, sy, 1, ctx, &blp, &grid, info, batch);
+    if (lds_bytes > 48 * 1024) GP_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    int rc = plan_launch(kern, NT, lds_bytes, sx, sy, 1, ctx, &blp, &grid, info, batch);
     if (rc) return rc;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), 0, native(s), arg, blp);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds_bytes, native(s), arg, blp);
     GP_HIP(hipGetLastError());
     return GP_SUCC;
 }
@@ -130,6 +131,22 @@ int plan_embed(const gp_embed_params *p, EltPlan *out) {
     return GP_SUCC;
 }
 
+int plan_attention(const gp_attention_params *p, EltPlan *out) {
+    GP_REQUIRE(p && p->q && p->k && p->v && p->out, "null attention params");
+    GP_REQUIRE(p->dtype == GP_F16 || p->dtype == GP_BF16, "attention: fp16 or bf16 only (dtype %d)", p->dtype);
+    GP_REQUIRE(p->head_dim == ATT_D, "attention: head_dim must be %d", ATT_D);
+    GP_REQUIRE(p->batch > 0 && p->heads > 0 && p->seq > 0 && p->seq <= 512, "attention: seq must be 1..512");
+    GP_REQUIRE(p->ld_qkv % 8 == 0 && p->ld_out > 0, "attention: row strides must be multiples of 8 elements");
+    GP_REQUIRE(al16(p->q) && al16(p->k) && al16(p->v), "attention: 16-byte alignment");
+    *out = EltPlan{};
+    out->op = OP_ATTENTION; out->dtype = p->dtype;
+    out->sx = (p->seq + ATT_QB - 1) / ATT_QB; out->sy = p->batch * p->heads;
+    out->lds_bytes = attention_lds_bytes(attention_nb_class(p->seq));
+    out->u.attn = AttnArgs{*p};
+    if (out->u.attn.p.scale == 0.f) out->u.attn.p.scale = 1.f;
+    return GP_SUCC;
+}
+
 int plan_copy(const void *src, void *dst, long bytes, EltPlan *out) {
     GP_REQUIRE(src && dst && bytes > 0, "copy arguments");
     GP_REQUIRE(al16(src) && al16(dst), "copy: 16-byte alignment");
@@ -164,6 +181,15 @@ int launch_elt_plan(const EltPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
             break;
         case OP_EMBED: GP_BY_DTYPE(pl.dtype, launch_tiles(embed_kernel<T>, pl.sx, pl.sy, ctx, s, info, pl.u.embed)); break;
         case OP_COPY: return launch_tiles(copy_kernel<0>, pl.sx, pl.sy, ctx, s, info, pl.u.copy);
+        case OP_ATTENTION:
+            switch (attention_nb_class(pl.u.attn.p.seq) * 2 + (pl.dtype == GP_F16)) {
+#define GP_ATT(NB)                                                                                                            \
+    case NB * 2 + 1: return launch_tiles(attention_kernel<_Float16, NB>, pl.sx, pl.sy, ctx, s, info, pl.u.attn, pl.lds_bytes); \
+    case NB * 2: return launch_tiles(attention_kernel<__bf16, NB>, pl.sx, pl.sy, ctx, s, info, pl.u.attn, pl.lds_bytes);
+                GP_ATT(4) GP_ATT(8) GP_ATT(12) GP_ATT(16)
+#undef GP_ATT
+            }
+            return GP_OUTOFRANGE;
     }
     set_error("unsupported elementwise plan (op %d dtype %d)", pl.op, pl.dtype);
     return GP_OUTOFRANGE;
@@ -179,6 +205,7 @@ using namespace gp;
     return rc ? rc : launch_elt_plan(pl, ctx, s, info);
 
 extern "C" int gp_launch_nchw_to_nhwc(const gp_layout_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_layout(p, &pl)) }
+extern "C" int gp_launch_attention(const gp_attention_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_attention(p, &pl)) }
 extern "C" int gp_launch_pool2d(const gp_pool_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_pool2d(p, &pl)) }
 extern "C" int gp_launch_eltwise(const gp_eltwise_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_eltwise(p, &pl)) }
 extern "C" int gp_launch_softmax(const gp_softmax_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_softmax(p, &pl)) }

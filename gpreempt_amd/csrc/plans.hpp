@@ -4,6 +4,7 @@
 #pragma once
 #include "elementwise_bodies.hpp"
 #include "mma.hpp"
+#include "attention_bodies.hpp"
 
 namespace gp {
 
@@ -17,12 +18,14 @@ struct MatPlan {
     size_t lds_bytes;
 };
 
-enum EltOp { OP_MAT = 0, OP_LAYOUT, OP_POOL, OP_ELTWISE, OP_SOFTMAX, OP_LAYERNORM, OP_EMBED, OP_COPY };
+enum EltOp { OP_MAT = 0, OP_LAYOUT, OP_POOL, OP_ELTWISE, OP_SOFTMAX, OP_LAYERNORM, OP_EMBED, OP_COPY, OP_ATTENTION };
 
 struct EltPlan {
     int op, dtype, sub;  // sub: layout -> (dtype_in * 4 + dtype_out); layernorm -> chunks kept per lane (2, 8, 16)
     int sx, sy;
+    size_t lds_bytes;    // dynamic LDS of the body (attention only; 0 otherwise)
     union {
+        AttnArgs attn;
         LayoutArgs layout;
         PoolArgs pool;
         EltwiseArgs elt;
@@ -44,6 +47,7 @@ int plan_softmax(const gp_softmax_params *p, EltPlan *out);
 int plan_layernorm(const gp_layernorm_params *p, EltPlan *out);
 int plan_embed(const gp_embed_params *p, EltPlan *out);
 int plan_copy(const void *src, void *dst, long bytes, EltPlan *out);
+int plan_attention(const gp_attention_params *p, EltPlan *out);
 int launch_elt_plan(const EltPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
 
 }  // namespace gp

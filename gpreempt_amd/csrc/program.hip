@@ -51,6 +51,7 @@ struct LayerDesc {
         gp_layernorm_params ln;
         gp_embed_params embed;
         CopyArgs copy;
+        AttnArgs attn;
     } u;
 };
 
@@ -123,6 +124,9 @@ __device__ __forceinline__ void run_layer(const LayerDesc &d, TileIdx t, T *lds)
         }
         case OP_EMBED: { const gp_embed_params a = d.u.embed; embed_tile<T>(a, t); break; }
         case OP_COPY: { const CopyArgs a = d.u.copy; copy_tile(a, t); break; }
+        case OP_ATTENTION:
+            if constexpr (sizeof(T) == 2) { const AttnArgs a = d.u.attn; attention_tile<T, 4>(a, t, lds); }  // seq <= 128 only
+            break;
     }
 }
 
@@ -334,6 +338,7 @@ static int push_elt(gp_program pr, const EltPlan &pl) {
     memcpy(&d.u, &pl.u, sizeof(pl.u));
     pr->layers.push_back(d);
     if (d.total > pr->max_tiles) pr->max_tiles = d.total;
+    if (pl.lds_bytes > pr->lds_bytes) pr->lds_bytes = pl.lds_bytes;
     return GP_SUCC;
 }
 
@@ -379,6 +384,12 @@ extern "C" int gp_program_add_eltwise(gp_program pr, const gp_eltwise_params *p)
 extern "C" int gp_program_add_softmax(gp_program pr, const gp_softmax_params *p) { GP_ADD_ELT(plan_softmax(p, &pl)) }
 extern "C" int gp_program_add_layernorm(gp_program pr, const gp_layernorm_params *p) { GP_ADD_ELT(plan_layernorm(p, &pl)) }
 extern "C" int gp_program_add_embed(gp_program pr, const gp_embed_params *p) { GP_ADD_ELT(plan_embed(p, &pl)) }
+extern "C" int gp_program_add_attention(gp_program pr, const gp_attention_params *p) {
+    // the program kernel carries the 128-key body only: the longer classes keep up to 256 score
+    // registers per lane, which would push every layer of the program into scratch memory
+    GP_REQUIRE(p && p->seq <= 128, "program attention: seq must be <= 128 (use unfused layers beyond)");
+    GP_ADD_ELT(plan_attention(p, &pl))
+}
 extern "C" int gp_program_add_copy(gp_program pr, const void *src, void *dst, size_t bytes) { GP_ADD_ELT(plan_copy(src, dst, (long)bytes, &pl)) }
 
 template <typename T>

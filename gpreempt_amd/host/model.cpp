@@ -148,6 +148,7 @@ void Model::bind_pointers(KernelInfo &k) {
         case OpKind::Eltwise: k.p.eltwise.a = P(0); k.p.eltwise.b = P(1); k.p.eltwise.scale = P(2); k.p.eltwise.shift = P(3); k.p.eltwise.out = P(4); break;
         case OpKind::Softmax: k.p.softmax.x = P(0); k.p.softmax.out = P(1); break;
         case OpKind::Layernorm: k.p.layernorm.x = P(0); k.p.layernorm.residual = P(1); k.p.layernorm.gamma = P(2); k.p.layernorm.beta = P(3); k.p.layernorm.out = P(4); break;
+        case OpKind::Attention: k.p.attention.q = P(0); k.p.attention.k = P(1); k.p.attention.v = P(2); k.p.attention.out = P(3); break;
         case OpKind::Embed: k.p.embed.ids = (const int64_t *)P(0); k.p.embed.tok = P(1); k.p.embed.pos = P(2); k.p.embed.seg = P(3); k.p.embed.out = P(4); break;
     }
 }
@@ -348,6 +349,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         case OpKind::Softmax: rc = gp_launch_softmax(&k.p.softmax, pc, stream, &info); break;
         case OpKind::Layernorm: rc = gp_launch_layernorm(&k.p.layernorm, pc, stream, &info); break;
         case OpKind::Embed: rc = gp_launch_embed(&k.p.embed, pc, stream, &info); break;
+        case OpKind::Attention: rc = gp_launch_attention(&k.p.attention, pc, stream, &info); break;
         case OpKind::Nop: break;
     }
     CUDA_RETURN_STATUS(rc);
@@ -376,6 +378,7 @@ Status Model::build_program() {
             case OpKind::Softmax: rc = gp_program_add_softmax(pr, &k.p.softmax); break;
             case OpKind::Layernorm: rc = gp_program_add_layernorm(pr, &k.p.layernorm); break;
             case OpKind::Embed: rc = gp_program_add_embed(pr, &k.p.embed); break;
+            case OpKind::Attention: rc = gp_program_add_attention(pr, &k.p.attention); break;
         }
         if (rc != 0) {
             std::fprintf(stderr, "build_program: kernel %zu (%s): %s\n", i, k.name.c_str(), gp_last_error());

@@ -349,7 +349,8 @@ Status build_densenet201(Model &m, const Options &o) {
 
 // ---- BERT encoder -----------------------------------------------------------------------------
 // token + position + segment-0 embedding -> LayerNorm -> L x { fused QKV dense, per-head
-// softmax(Q K^T / sqrt(d)) V as two batched GEMMs over head slices of the QKV buffer, output
+// softmax(Q K^T / sqrt(d)) V (one fused kernel for 16-bit models, else two batched GEMMs over head
+// slices of the QKV buffer around a softmax), output
 // dense + residual, LayerNorm, FFN dense + erf-GELU, dense + residual, LayerNorm }; eps 1e-12.
 // "data" holds int64 token ids (reference src/tests/test-dnn.cpp:21-23); "heads" is the last
 // hidden state [batch*seq, hidden].
@@ -361,6 +362,9 @@ Status build_bert(Model &m, const Options &o) {
     int heads = o.geti("heads", 12), F = o.geti("ffn", 3072), vocab = o.geti("vocab", 30522), maxpos = o.geti("maxpos", 512);
     if (Hd % heads || S > maxpos) return Status::OutOfRange;
     int d = Hd / heads;
+    // 16-bit models with 64-wide heads use the fused attention kernel ("fused_attention=0" keeps
+    // the exported graph's batch_matmul / softmax / batch_matmul sequence)
+    const bool fused = o.geti("fused_attention", 1) != 0 && dt != "f32" && d == 64 && S <= 512;
     long T = (long)B * S;
     const float std_ = 0.02f;
     size_t es = g.es();
@@ -400,29 +404,39 @@ Status build_bert(Model &m, const Options &o) {
         std::string n = "layer" + std::to_string(l);
         size_t qkv = g.add_storage(n + ".qkv", (size_t)T * 3 * Hd, g.stype_);
         g.dense(n + ".attn.qkv", x, 0, T, Hd, Hd, 3 * Hd, GP_ACT_NONE, SIZE_MAX, qkv, 0, 3 * Hd, std_);
-        size_t sc = g.add_storage(n + ".scores", (size_t)B * heads * S * S, g.stype_);
-        {   // scores[b,h] = Q[b,h] K[b,h]^T / sqrt(d)
-            double flops = 2.0 * B * heads * (double)S * S * d;
-            KernelInfo &k = g.add_kernel("batch_matmul_qk", OpKind::Gemm, {GraphBuilder::ref(qkv, 0), GraphBuilder::ref(qkv, (size_t)Hd * es), GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(sc)},
-                                         flops, es * (2.0 * T * Hd + (double)B * heads * S * S));
-            gp_gemm_params &p = k.p.gemm;
-            p.dtype = g.gp_dtype(); p.M = S; p.N = S; p.K = d; p.lda = 3 * Hd; p.ldb = 3 * Hd; p.b_is_nk = 1; p.ldc = S;
-            p.alpha = 1.f / std::sqrt((float)d); p.act = GP_ACT_NONE; p.batch = B * heads; p.batch_inner = heads;
-            p.stride_a = d; p.stride_b = d; p.stride_c = (long)S * S;
-            p.stride_a_outer = (long)S * 3 * Hd; p.stride_b_outer = (long)S * 3 * Hd; p.stride_c_outer = (long)heads * S * S;
-        }
-        size_t pr = g.add_storage(n + ".probs", (size_t)B * heads * S * S, g.stype_);
-        g.softmax(sc, pr, (long)B * heads * S, S, 1.f);
         size_t ctx = g.add_storage(n + ".context", (size_t)T * Hd, g.stype_);
-        {   // context[b,:,h] = probs[b,h] V[b,h]
-            double flops = 2.0 * B * heads * (double)S * S * d;
-            KernelInfo &k = g.add_kernel("batch_matmul_pv", OpKind::Gemm, {GraphBuilder::ref(pr), GraphBuilder::ref(qkv, (size_t)2 * Hd * es), GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(ctx)},
-                                         flops, es * ((double)B * heads * S * S + 2.0 * T * Hd));
-            gp_gemm_params &p = k.p.gemm;
-            p.dtype = g.gp_dtype(); p.M = S; p.N = d; p.K = S; p.lda = S; p.ldb = 3 * Hd; p.b_is_nk = 0; p.ldc = Hd;
-            p.alpha = 1.f; p.act = GP_ACT_NONE; p.batch = B * heads; p.batch_inner = heads;
-            p.stride_a = (long)S * S; p.stride_b = d; p.stride_c = d;
-            p.stride_a_outer = (long)heads * S * S; p.stride_b_outer = (long)S * 3 * Hd; p.stride_c_outer = (long)S * Hd;
+        if (fused) {
+            // one kernel: softmax(Q K^T / sqrt(d)) V per head, scores never leave the chip
+            double flops = 4.0 * B * heads * (double)S * S * d;
+            KernelInfo &k = g.add_kernel("attention", OpKind::Attention, {GraphBuilder::ref(qkv, 0), GraphBuilder::ref(qkv, (size_t)Hd * es), GraphBuilder::ref(qkv, (size_t)2 * Hd * es), GraphBuilder::ref(ctx)},
+                                         flops, es * 4.0 * T * Hd);
+            gp_attention_params &p = k.p.attention;
+            p.dtype = g.gp_dtype(); p.batch = B; p.heads = heads; p.seq = S; p.head_dim = d;
+            p.ld_qkv = 3 * Hd; p.ld_out = Hd; p.scale = 1.f / std::sqrt((float)d);
+        } else {
+            size_t sc = g.add_storage(n + ".scores", (size_t)B * heads * S * S, g.stype_);
+            {   // scores[b,h] = Q[b,h] K[b,h]^T / sqrt(d)
+                double flops = 2.0 * B * heads * (double)S * S * d;
+                KernelInfo &k = g.add_kernel("batch_matmul_qk", OpKind::Gemm, {GraphBuilder::ref(qkv, 0), GraphBuilder::ref(qkv, (size_t)Hd * es), GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(sc)},
+                                             flops, es * (2.0 * T * Hd + (double)B * heads * S * S));
+                gp_gemm_params &p = k.p.gemm;
+                p.dtype = g.gp_dtype(); p.M = S; p.N = S; p.K = d; p.lda = 3 * Hd; p.ldb = 3 * Hd; p.b_is_nk = 1; p.ldc = S;
+                p.alpha = 1.f / std::sqrt((float)d); p.act = GP_ACT_NONE; p.batch = B * heads; p.batch_inner = heads;
+                p.stride_a = d; p.stride_b = d; p.stride_c = (long)S * S;
+                p.stride_a_outer = (long)S * 3 * Hd; p.stride_b_outer = (long)S * 3 * Hd; p.stride_c_outer = (long)heads * S * S;
+            }
+            size_t pr = g.add_storage(n + ".probs", (size_t)B * heads * S * S, g.stype_);
+            g.softmax(sc, pr, (long)B * heads * S, S, 1.f);
+            {   // context[b,:,h] = probs[b,h] V[b,h]
+                double flops = 2.0 * B * heads * (double)S * S * d;
+                KernelInfo &k = g.add_kernel("batch_matmul_pv", OpKind::Gemm, {GraphBuilder::ref(pr), GraphBuilder::ref(qkv, (size_t)2 * Hd * es), GraphBuilder::none(), GraphBuilder::none(), GraphBuilder::ref(ctx)},
+                                             flops, es * ((double)B * heads * S * S + 2.0 * T * Hd));
+                gp_gemm_params &p = k.p.gemm;
+                p.dtype = g.gp_dtype(); p.M = S; p.N = d; p.K = S; p.lda = S; p.ldb = 3 * Hd; p.b_is_nk = 0; p.ldc = Hd;
+                p.alpha = 1.f; p.act = GP_ACT_NONE; p.batch = B * heads; p.batch_inner = heads;
+                p.stride_a = (long)S * S; p.stride_b = d; p.stride_c = d;
+                p.stride_a_outer = (long)heads * S * S; p.stride_b_outer = (long)S * 3 * Hd; p.stride_c_outer = (long)S * Hd;
+            }
         }
         size_t ao = g.add_storage(n + ".attn.out", (size_t)T * Hd, g.stype_);
         g.dense(n + ".attn.proj", ctx, 0, T, Hd, Hd, Hd, GP_ACT_NONE, x, ao, 0, Hd, std_);   // + residual x

@@ -242,6 +242,21 @@ typedef struct gp_layernorm_params {
 } gp_layernorm_params;
 int gp_launch_layernorm(const gp_layernorm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
 
+/* Fused scaled-dot-product attention over the heads of packed Q / K / V activations: for every
+ * batch b and head h, out[b*seq + i, h*64 .. h*64+63] = sum_j softmax_j(scale * <Q_i, K_j>) V_j,
+ * where row t of Q (K, V) for head h is q (k, v) + t*ld_qkv + h*64.  Replaces the batch_matmul,
+ * softmax, batch_matmul sequence of the exported BERT graph (scripts/compile/compile-bert.py:76-77)
+ * and the two seq x seq tensors between them; the softmax runs in fp32 on unrounded scores.
+ * fp16 / bf16 only, head_dim = 64, seq <= 512, 16-byte aligned rows. */
+typedef struct gp_attention_params {
+    int dtype;
+    int batch, heads, seq, head_dim;
+    const void *q; const void *k; const void *v; long ld_qkv;
+    void *out; long ld_out;
+    float scale;
+} gp_attention_params;
+int gp_launch_attention(const gp_attention_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
 /* out[t,:] = tok[ids[t],:] + pos[t % seq,:] (+ seg[0,:]); ids are int64 (the reference feeds
  * BERT int64 token ids, src/tests/test-dnn.cpp:21-23). */
 typedef struct gp_embed_params {
@@ -277,6 +292,7 @@ int gp_program_add_pool2d(gp_program p, const gp_pool_params *params);
 int gp_program_add_eltwise(gp_program p, const gp_eltwise_params *params);
 int gp_program_add_softmax(gp_program p, const gp_softmax_params *params);
 int gp_program_add_layernorm(gp_program p, const gp_layernorm_params *params);
+int gp_program_add_attention(gp_program pr, const gp_attention_params *p);
 int gp_program_add_embed(gp_program p, const gp_embed_params *params);
 int gp_program_add_copy(gp_program p, const void *src, void *dst, size_t bytes); /* the reference's "nop" copy */
 int gp_program_finalize(gp_program p);

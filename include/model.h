@@ -38,7 +38,7 @@ struct ParamLayout {
     float init_a = 0.f, init_b = 0.f;
 };
 
-enum class OpKind { Nop, Gemm, Conv, Layout, Pool, Eltwise, Softmax, Layernorm, Embed };
+enum class OpKind { Nop, Gemm, Conv, Layout, Pool, Eltwise, Softmax, Layernorm, Embed, Attention };
 
 struct ArgRef {
     size_t storage = SIZE_MAX;  // SIZE_MAX = absent
@@ -53,6 +53,7 @@ public:
     union {
         gp_gemm_params gemm;
         gp_conv_params conv;
+        gp_attention_params attention;
         gp_layout_params layout;
         gp_pool_params pool;
         gp_eltwise_params eltwise;

@@ -93,9 +93,14 @@ def densenet(params, x, dt="f16", blocks=(6, 12, 48, 32), growth=32):
     return c.R(O.softmax(c.dense("classifier", gap)))
 
 
-def bert(params, ids, dt="f16", batch=1, seq=128, layers=12, hidden=768, heads=12):
+def bert(params, ids, dt="f16", batch=1, seq=128, layers=12, hidden=768, heads=12, fused_attention=None):
     """BERT encoder: embeddings + LayerNorm, then `layers` post-LN transformer blocks with
-    erf GELU and eps 1e-12; returns the last hidden state [batch*seq, hidden]."""
+    erf GELU and eps 1e-12; returns the last hidden state [batch*seq, hidden].
+    fused_attention (default: 16-bit dtypes): scores and probabilities are not rounded to the
+    storage dtype between the two products, as in a kernel that never writes them out."""
+    if fused_attention is None:
+        fused_attention = dt != "f32"
+    RA = (lambda a: a) if fused_attention else None
     c = _Ctx(params, dt)
     d = hidden // heads
     T = batch * seq
@@ -105,8 +110,9 @@ def bert(params, ids, dt="f16", batch=1, seq=128, layers=12, hidden=768, heads=1
         n = f"layer{l}"
         qkv = c.dense(n + ".attn.qkv", x)
         q, k, v = (qkv[:, i * hidden:(i + 1) * hidden].reshape(batch, seq, heads, d).transpose(0, 2, 1, 3).reshape(batch * heads, seq, d) for i in range(3))
-        scores = c.R(O.bmm(q, k, alpha=1.0 / np.sqrt(d), b_is_nk=True))
-        probs = c.R(O.softmax(scores))
+        RS = RA or c.R
+        scores = RS(O.bmm(q, k, alpha=1.0 / np.sqrt(d), b_is_nk=True))
+        probs = RS(O.softmax(scores))
         ctxv = c.R(O.bmm(probs, v))
         ctxv = ctxv.reshape(batch, heads, seq, d).transpose(0, 2, 1, 3).reshape(T, hidden)
         ao = c.dense(n + ".attn.proj", ctxv, residual=x)

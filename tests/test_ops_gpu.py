@@ -260,3 +260,59 @@ def test_conv2d_long_tiles_left_mid_k_and_resumed_bit_exact(gp, dt):
         assert int(st.checkpoint_headers(info.grid)[:, 0].sum()) == 0
         assert np.array_equal(do.download(), raw_want), (dt, inject)
     assert stopped >= 1, "the stop request was never seen inside a tile"
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", [(1, 12, 128), (2, 3, 77), (1, 2, 384), (1, 1, 512), (1, 4, 33)])
+def test_fused_attention_matches_composed_oracle(gp, dt, shape):
+    """softmax(Q K^T / sqrt(d)) V over the heads of a packed QKV buffer, against the oracle's
+    batched-matmul / softmax / batched-matmul composition (fp64 softmax on unrounded scores)."""
+    B, Hh, S = shape
+    d, Hd = 64, Hh * 64
+    rng = np.random.default_rng(S * 7 + Hh)
+    qkv = rnd(rng, (B * S, 3 * Hd), dt, -1.5, 1.5)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    es = gp.DTYPE_SIZE[dtype]
+    dq = gp.DevBuf.from_array(qkv, dtype)
+    do = gp.DevBuf(B * S * Hd * es)
+    do.fill32(0x7E007E00)
+    p = gp.AttentionParams(dtype=dtype, batch=B, heads=Hh, seq=S, head_dim=d, q=dq.ptr, k=dq.ptr + Hd * es, v=dq.ptr + 2 * Hd * es,
+                           ld_qkv=3 * Hd, out=do.ptr, ld_out=Hd, scale=1.0 / np.sqrt(d))
+    info = gp.launch("gp_launch_attention", p)
+    sync(gp)
+    got = do.download(dtype, (B, S, Hh, d))
+    x = qkv.astype(np.float64).reshape(B, S, 3, Hh, d)
+    q, k, v = x[:, :, 0], x[:, :, 1], x[:, :, 2]
+    sc = np.einsum("bihd,bjhd->bhij", q, k) / np.sqrt(d)
+    sc -= sc.max(-1, keepdims=True)
+    pr = np.exp(sc)
+    pr /= pr.sum(-1, keepdims=True)
+    ref = np.einsum("bhij,bjhd->bihd", pr, v)
+    assert info.total_tiles == -(-S // 128) * B * Hh
+    assert np.isfinite(got).all()
+    assert rel_err(got, ref) < TOL[dt], (dt, shape)
+
+
+def test_fused_attention_preempt_resume_bit_exact(gp):
+    B, Hh, S, d = 4, 12, 128, 64
+    Hd = Hh * d
+    rng = np.random.default_rng(3)
+    qkv = rnd(rng, (B * S, 3 * Hd), "f16", -1, 1)
+    dq = gp.DevBuf.from_array(qkv, gp.F16)
+    do = gp.DevBuf(B * S * Hd * 2)
+    p = gp.AttentionParams(dtype=gp.F16, batch=B, heads=Hh, seq=S, head_dim=d, q=dq.ptr, k=dq.ptr + Hd * 2, v=dq.ptr + 2 * Hd * 2,
+                           ld_qkv=3 * Hd, out=do.ptr, ld_out=Hd, scale=0.125)
+    gp.launch("gp_launch_attention", p)
+    sync(gp)
+    want = do.download().copy()
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    do.fill32(0)
+    gp.launch("gp_launch_attention", p, st.ctx(inject_at=10, max_workgroups=4))
+    sync(gp)
+    assert flag.get() == 1 and st.stop_index() == 0 and st.counters()[0] < B * Hh
+    flag.set(0)
+    st.clear_stop()
+    gp.launch("gp_launch_attention", p, st.ctx(max_workgroups=4))
+    sync(gp)
+    assert np.array_equal(do.download(), want)
