@@ -2,6 +2,7 @@
 // Stand-alone launchers of the memory-bound operators (C ABI); the tile bodies live in
 // elementwise_bodies.hpp.
 #include "plans.hpp"
+#include "stencil_bodies.hpp"
 
 namespace gp {
 
@@ -205,6 +206,24 @@ using namespace gp;
     return rc ? rc : launch_elt_plan(pl, ctx, s, info);
 
 extern "C" int gp_launch_nchw_to_nhwc(const gp_layout_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_layout(p, &pl)) }
+extern "C" int gp_launch_miniweather(const gp_miniweather_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    GP_REQUIRE(p && p->hydro, "null miniweather params");
+    GP_REQUIRE(p->kernel >= GP_MW_HALO_X && p->kernel <= GP_MW_UPDATE_Z, "miniweather kernel %d", p->kernel);
+    GP_REQUIRE(p->nx >= 4 && p->nz >= 4 && (long)p->nx * p->nz <= (1L << 27), "miniweather grid %d x %d", p->nx, p->nz);
+    GP_REQUIRE(p->dt > 0 && p->dx > 0 && p->dz > 0, "miniweather steps must be positive");
+    const bool update = p->kernel == GP_MW_UPDATE_X || p->kernel == GP_MW_UPDATE_Z;
+    const bool flux = p->kernel == GP_MW_FLUX_X || p->kernel == GP_MW_FLUX_Z;
+    GP_REQUIRE(p->state || p->kernel == GP_MW_UPDATE_X, "miniweather: state missing");
+    GP_REQUIRE(!(update || flux) || p->flux, "miniweather: flux missing");
+    GP_REQUIRE(!update || (p->state_init && p->state_out), "miniweather: update operands missing");
+    const int tiles = (int)((mw_ids(p->kernel, p->nx, p->nz) + MW_TILE - 1) / MW_TILE);
+    switch (p->kernel) {
+#define GP_MW(K) case K: return launch_tiles(miniweather_kernel<K>, tiles, 1, ctx, s, info, *p);
+        GP_MW(GP_MW_HALO_X) GP_MW(GP_MW_FLUX_X) GP_MW(GP_MW_UPDATE_X) GP_MW(GP_MW_HALO_Z) GP_MW(GP_MW_FLUX_Z) GP_MW(GP_MW_UPDATE_Z)
+#undef GP_MW
+    }
+    return GP_OUTOFRANGE;
+}
 extern "C" int gp_launch_attention(const gp_attention_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_attention(p, &pl)) }
 extern "C" int gp_launch_pool2d(const gp_pool_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_pool2d(p, &pl)) }
 extern "C" int gp_launch_eltwise(const gp_eltwise_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) { GP_PLAN_AND_LAUNCH(plan_eltwise(p, &pl)) }

@@ -15,7 +15,7 @@ vp = C.c_void_p
 SYMBOLS = """gpx_create gpx_destroy gpx_init gpx_set_input gpx_get_output gpx_get_data_size gpx_execute
 gpx_launch_kernel gpx_get_kernel_num gpx_capture_graph gpx_uses_program gpx_clear gpx_set_flag gpx_set_running gpx_resume
 gpx_get_stop_point gpx_last_stop_index gpx_inject_preempt gpx_read_counters gpx_reset_counters gpx_storage_num gpx_storage_info
-gpx_kernel_info gpx_read_storage gpx_run_scenario gpx_preempt_probe gpx_parse_params""".split()
+gpx_kernel_info gpx_read_storage gpx_miniweather_reductions gpx_run_scenario gpx_preempt_probe gpx_parse_params""".split()
 
 STATUS = ["Succ", "Fail", "Timeout", "NotFound", "OutOfRange", "Full"]
 _lib = None
@@ -132,6 +132,12 @@ class Executor:
         return raw
 
     # -- execution
+    def miniweather_reductions(self):
+        """(mass, total energy) of the "miniweather" workload's current state"""
+        m, t = C.c_double(), C.c_double()
+        _chk(lib().gpx_miniweather_reductions(self.h, C.byref(m), C.byref(t)), "miniweather_reductions")
+        return m.value, t.value
+
     def execute(self, stream=None):
         _chk(lib().gpx_execute(self.h, stream.h if stream else None), "execute")
 

@@ -2,6 +2,7 @@
 #include <cstring>
 #include "executor.h"
 #include "gpreempt_exec_c.h"
+#include "workloads/scicomput.h"
 #include "harness.h"
 
 using namespace foo;
@@ -86,6 +87,20 @@ int gpx_read_storage(gpx_executor e, const char *key, void *out, size_t len) {
 }
 
 }  // extern "C"
+
+extern "C" int gpx_miniweather_reductions(gpx_executor e, double *mass, double *te) {
+    auto m = H(e)->ex->get_model();
+    if (!m || m->get_kernel_num() == 0 || m->get_kernel_info(0).op != OpKind::Stencil) return Status::NotFound;
+    const gp_miniweather_params &p = m->get_kernel_info(0).p.miniweather;
+    const SciCompute::Grid g = SciCompute::make_grid(p.nx, p.nz);
+    std::vector<float> state(SciCompute::state_elems(g)), hydro(SciCompute::hydro_elems(g));
+    Status st = m->get("state", state.data(), state.size() * sizeof(float), nullptr);
+    if (st == Status::Succ) st = m->get("hydro", hydro.data(), hydro.size() * sizeof(float), nullptr);
+    if (st != Status::Succ) return st;
+    if (gp_stream_sync(nullptr) != 0) return Status::Fail;
+    SciCompute::reductions(g, state.data(), hydro.data(), *mass, *te);
+    return Status::Succ;
+}
 
 extern "C" int gpx_storage_info(gpx_executor e, size_t idx, char *name, size_t name_len, char *stype, size_t stype_len,
                                 size_t *bytes, int *is_param, size_t *disk_elems, int dims[8]) {

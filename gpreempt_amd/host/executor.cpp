@@ -9,7 +9,8 @@
 
 namespace foo {
 
-static const std::set<std::string> kNotBuilt = {"cc", "bfs", "pagerank", "sssp", "miniweather"};
+// the graph workloads need a dataset the reference does not ship (src/executor.cpp:12)
+static const std::set<std::string> kNotBuilt = {"cc", "bfs", "pagerank", "sssp"};
 
 static std::string model_root() {
     const char *e = std::getenv("GPREEMPT_MODEL_PATH");

@@ -130,6 +130,7 @@ Status Model::allocate_and_bind() {
             case ParamLayout::InitConst: for (float &v : host) v = L.init_a; break;
             case ParamLayout::InitUniform: for (float &v : host) v = rng.uniform(L.init_a, L.init_b); break;
             case ParamLayout::InitNormal: for (float &v : host) v = rng.normal() * L.init_a; break;
+            case ParamLayout::InitData: if (L.init_data && L.init_data->size() == host.size()) host = *L.init_data; break;
         }
         RETURN_STATUS(upload_param(i, host.data(), host.size()));
     }
@@ -149,6 +150,10 @@ void Model::bind_pointers(KernelInfo &k) {
         case OpKind::Softmax: k.p.softmax.x = P(0); k.p.softmax.out = P(1); break;
         case OpKind::Layernorm: k.p.layernorm.x = P(0); k.p.layernorm.residual = P(1); k.p.layernorm.gamma = P(2); k.p.layernorm.beta = P(3); k.p.layernorm.out = P(4); break;
         case OpKind::Attention: k.p.attention.q = P(0); k.p.attention.k = P(1); k.p.attention.v = P(2); k.p.attention.out = P(3); break;
+        case OpKind::Stencil:
+            k.p.miniweather.state = (float *)P(0); k.p.miniweather.flux = (float *)P(1); k.p.miniweather.state_init = (const float *)P(2);
+            k.p.miniweather.state_out = (float *)P(3); k.p.miniweather.hydro = (const float *)P(4);
+            break;
         case OpKind::Embed: k.p.embed.ids = (const int64_t *)P(0); k.p.embed.tok = P(1); k.p.embed.pos = P(2); k.p.embed.seg = P(3); k.p.embed.out = P(4); break;
     }
 }
@@ -350,6 +355,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         case OpKind::Layernorm: rc = gp_launch_layernorm(&k.p.layernorm, pc, stream, &info); break;
         case OpKind::Embed: rc = gp_launch_embed(&k.p.embed, pc, stream, &info); break;
         case OpKind::Attention: rc = gp_launch_attention(&k.p.attention, pc, stream, &info); break;
+        case OpKind::Stencil: rc = gp_launch_miniweather(&k.p.miniweather, pc, stream, &info); break;
         case OpKind::Nop: break;
     }
     CUDA_RETURN_STATUS(rc);
@@ -379,6 +385,10 @@ Status Model::build_program() {
             case OpKind::Layernorm: rc = gp_program_add_layernorm(pr, &k.p.layernorm); break;
             case OpKind::Embed: rc = gp_program_add_embed(pr, &k.p.embed); break;
             case OpKind::Attention: rc = gp_program_add_attention(pr, &k.p.attention); break;
+            case OpKind::Stencil:  // launched kernel by kernel only
+                std::fprintf(stderr, "build_program: the miniweather workload has no whole-model program\n");
+                gp_program_destroy(pr);
+                return Status::Fail;
         }
         if (rc != 0) {
             std::fprintf(stderr, "build_program: kernel %zu (%s): %s\n", i, k.name.c_str(), gp_last_error());

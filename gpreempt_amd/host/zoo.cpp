@@ -4,10 +4,12 @@
 // configurations name.  Activations are NHWC with 16-byte aligned channel counts; parameters are
 // declared in the reference's on-disk convention (fp32, OIHW) and re-laid-out at load time.
 #include "zoo.h"
+#include "workloads/scicomput.h"
 
 #include <cmath>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <sstream>
 
 namespace foo {
@@ -222,6 +224,52 @@ Status build_gemm(Model &m, const Options &o, int M, int N, int K, const std::st
     gp_gemm_params &p = k.p.gemm;
     p.dtype = g.gp_dtype(); p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = K; p.b_is_nk = 1; p.ldc = N; p.alpha = 1.f; p.act = act; p.batch = 1;
     p.tile_m = p.tile_n = tile;
+    return Status::Succ;
+}
+
+// ---- miniWeather ---------------------------------------------------------------------------------
+// One perform_timestep of the reference (src/workloads/miniweather.tr.cu:184-206) as a kernel list:
+// four direction sweeps (x, z, z, x), three Runge-Kutta stages each, three kernels per stage (halo
+// exchange, interface fluxes, state update) = 36 kernels, so the stop index of a preempted step is
+// the reference's `start_from` (= stage * 3 + kernel).  The state lives in the model's storages
+// and advances by two time steps of `dt` per execute().
+Status build_miniweather(Model &m, const Options &o) {
+    GraphBuilder g(m, "f32");
+    const int nx = o.geti("nx", 3200), nz = o.geti("nz", 1600), spec = o.geti("spec", SciCompute::Collision);
+    if (nx < 4 || nz < 4 || (long)nx * nz > (1L << 27)) return Status::OutOfRange;
+    if (spec != 1 && spec != 2 && spec != 3 && spec != 5 && spec != 6) return Status::OutOfRange;
+    const SciCompute::Grid grid = SciCompute::make_grid(nx, nz);
+    auto state0 = std::make_shared<std::vector<float>>();
+    auto hydro0 = std::make_shared<std::vector<float>>();
+    SciCompute::initial_state(grid, spec, *state0, *hydro0);
+    ParamLayout LS; LS.disk_elems = state0->size(); LS.init = ParamLayout::InitData; LS.init_data = state0;
+    ParamLayout LH; LH.disk_elems = hydro0->size(); LH.init = ParamLayout::InitData; LH.init_data = hydro0;
+    const size_t state = g.add_param("state", state0->size(), LS);
+    const size_t state_tmp = g.add_param("state_tmp", state0->size(), LS);
+    const size_t hydro = g.add_param("hydro", hydro0->size(), LH);
+    const size_t flux = g.add_storage("flux", SciCompute::flux_elems(grid), "float32");
+    static const char *names[6] = {"set_halo_values_x", "compute_tendencies_x", "compute_tendencies_x_r",
+                                   "set_halo_values_z", "compute_tendencies_z", "compute_tendencies_z_r"};
+    const double cells = (double)nx * nz;
+    for (int kid = 0; kid < 36; ++kid) {
+        const int step = kid / 3, sub = kid % 3, sweep = step / 3, stage = step % 3;
+        const bool dir_z = sweep == 1 || sweep == 2;
+        const size_t forcing = stage == 0 ? state : state_tmp, out = stage == 2 ? state : state_tmp;
+        const int kernel = (dir_z ? 3 : 0) + sub;
+        // algorithmic traffic: fluxes read the 4 state fields and write 4 flux fields; updates read
+        // 4 flux fields and 4 state fields (+ density for gravity) and write 4 state fields
+        double bytes = 0, flops = 0;
+        if (sub == 0) bytes = 4.0 * 4 * 4 * 2 * (dir_z ? nx + 4 : nz);
+        else if (sub == 1) { bytes = 4.0 * 8 * cells; flops = 60 * cells; }
+        else { bytes = 4.0 * (12 + (dir_z ? 1 : 0)) * cells; flops = 4 * 4 * cells; }
+        KernelInfo &k = g.add_kernel(names[kernel], OpKind::Stencil,
+                                     {GraphBuilder::ref(forcing), GraphBuilder::ref(flux), GraphBuilder::ref(state), GraphBuilder::ref(out), GraphBuilder::ref(hydro)},
+                                     flops, bytes);
+        gp_miniweather_params &p = k.p.miniweather;
+        p.kernel = kernel; p.nx = nx; p.nz = nz;
+        p.dt = stage == 0 ? grid.dt / 3 : stage == 1 ? grid.dt / 2 : grid.dt / 1;
+        p.dx = grid.dx; p.dz = grid.dz;
+    }
     return Status::Succ;
 }
 
@@ -486,7 +534,8 @@ Status zoo_build(Model &m, const std::string &workload) {
     if (n == "densenet" || n == "densenet201") return build_densenet201(m, o);
     if (n == "bert") return build_bert(m, o);
     if (n == "toy") return build_toy(m, o);
-    std::fprintf(stderr, "unknown workload '%s' (known: gemm1024 gemm8192 resnet50 resnet101 resnet152 vgg16 densenet201 bert toy)\n", n.c_str());
+    if (n == "miniweather") return build_miniweather(m, o);
+    std::fprintf(stderr, "unknown workload '%s' (known: gemm1024 gemm8192 resnet50 resnet101 resnet152 vgg16 densenet201 bert miniweather toy)\n", n.c_str());
     return Status::NotFound;
 }
 

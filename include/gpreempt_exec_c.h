@@ -48,6 +48,10 @@ int gpx_kernel_info(gpx_executor e, size_t idx, char *name, size_t name_len, dou
                     int *total_blocks, int *grid);
 int gpx_read_storage(gpx_executor e, const char *key, void *out, size_t len); /* blocking Model::get */
 
+/* "miniweather" workload only: domain mass and total energy of the current state
+ * (SciComputeBlp::reductions, reference src/workloads/miniweather.tr.cu:906-932); blocking. */
+int gpx_miniweather_reductions(gpx_executor e, double *mass, double *te);
+
 /* Multi-tenant scenario runner: the role of the reference's client executables
  * (src/cuda-clients/blpclient.cpp main() and the programs under src/common-clients) over a DISB task file
  * (config/A.json schema) with an extra "policy" key: "wb" (block-level preemption, HP waits for

@@ -257,6 +257,28 @@ typedef struct gp_attention_params {
 } gp_attention_params;
 int gp_launch_attention(const gp_attention_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
 
+/* One kernel of the miniWeather workload (2-D stratified compressible flow; the reference's non-DNN
+ * preemptible workload).  Replaces the six kernels of src/workloads/miniweather.tr.cu:
+ * set_halo_values_x :504-520, compute_tendencies_x :283-349, compute_tendencies_x_r :351-393,
+ * set_halo_values_z :523-552, compute_tendencies_z :399-468, compute_tendencies_z_r :470-502.
+ * A tile is 256 consecutive element ids, as a thread block of the reference.
+ *   state      forcing state, 4 x (nz+4) x (nx+4) fp32 (halo kernels write its halo cells)
+ *   flux       4 x (nz+1) x (nx+1) fp32
+ *   state_init / state_out   update kernels: out = init + dt * tendency(flux[, state])
+ *   hydro      hydrostatic background in one buffer: cell density, cell density*theta (nz+4 each),
+ *              interface density, density*theta, pressure (nz+1 each), 4 boundary density ratios
+ * dt is the stage's step (dt/3, dt/2, dt of the Runge-Kutta stages). */
+enum gp_mw_kernel { GP_MW_HALO_X = 0, GP_MW_FLUX_X = 1, GP_MW_UPDATE_X = 2, GP_MW_HALO_Z = 3, GP_MW_FLUX_Z = 4, GP_MW_UPDATE_Z = 5 };
+typedef struct gp_miniweather_params {
+    int kernel;
+    int nx, nz;
+    float dt, dx, dz;
+    float *state; float *flux;
+    const float *state_init; float *state_out;
+    const float *hydro;
+} gp_miniweather_params;
+int gp_launch_miniweather(const gp_miniweather_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
 /* out[t,:] = tok[ids[t],:] + pos[t % seq,:] (+ seg[0,:]); ids are int64 (the reference feeds
  * BERT int64 token ids, src/tests/test-dnn.cpp:21-23). */
 typedef struct gp_embed_params {

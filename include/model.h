@@ -34,11 +34,12 @@ struct ParamLayout {
     size_t disk_elems = 0;                      // fp32 values expected on disk
     bool is_param = false;
     // seeded initial value when no parameter file is given
-    enum Init { InitZero, InitNormal /* N(0, a) */, InitUniform /* U[a, b] */, InitConst /* a */ } init = InitZero;
+    enum Init { InitZero, InitNormal /* N(0, a) */, InitUniform /* U[a, b] */, InitConst /* a */, InitData /* *init_data */ } init = InitZero;
     float init_a = 0.f, init_b = 0.f;
+    std::shared_ptr<std::vector<float>> init_data;  // InitData: disk_elems values computed by the builder
 };
 
-enum class OpKind { Nop, Gemm, Conv, Layout, Pool, Eltwise, Softmax, Layernorm, Embed, Attention };
+enum class OpKind { Nop, Gemm, Conv, Layout, Pool, Eltwise, Softmax, Layernorm, Embed, Attention, Stencil };
 
 struct ArgRef {
     size_t storage = SIZE_MAX;  // SIZE_MAX = absent
@@ -60,6 +61,7 @@ public:
         gp_softmax_params softmax;
         gp_layernorm_params layernorm;
         gp_embed_params embed;
+        gp_miniweather_params miniweather;
     } p;
     std::vector<size_t> args_index;       // storage index per pointer slot (SIZE_MAX = absent)
     std::vector<ArgRef> refs;             // same slots with byte offsets into the storage

@@ -1,0 +1,199 @@
+"""miniWeather on the GPU (gp_launch_miniweather and the "miniweather" workload of the executor)
+against the CPU oracle, and the preempt-then-resume protocol on its non-idempotent kernels
+(reference src/workloads/miniweather.tr.cu; BLPExecutor::execute / resume, src/executor.cpp:211-298).
+
+Tolerances: halo and update kernels are bit-exact (adds, multiplies and correctly rounded divides,
+no fused multiply-add on either side); the flux kernels call pow / powf, whose device and host
+implementations differ in the last bit, so they are compared to 1e-6 (fp64 pow, result rounded to
+fp32) and 2e-5 (fp32 powf on pressures that nearly cancel against the background) of the field's
+magnitude; whole time steps to 1e-4 of each field's magnitude."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from oracle import miniweather as MW
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ex_mod(gp):
+    from gpreempt_amd import executor
+    return executor
+
+
+def f32(raw):
+    return np.frombuffer(raw.tobytes(), np.float32).copy()
+
+
+def random_sim(nx, nz, seed):
+    """a developed flow plus noise, so that no term of the scheme is zero"""
+    s = MW.Sim(nx, nz, MW.COLLISION)
+    for _ in range(3):
+        s.timestep()
+    rng = np.random.default_rng(seed)
+    s.state += rng.normal(0, 1e-3, s.state.shape).astype(np.float32) * np.array([1, 10, 10, 100], np.float32)[:, None, None]
+    s.state_tmp[:] = s.state + rng.normal(0, 1e-3, s.state.shape).astype(np.float32)
+    s.flux[:] = rng.normal(0, 1, s.flux.shape).astype(np.float32)
+    return s
+
+
+def launch_kernel(gp, sim, kid, ctx=None):
+    """runs kernel `kid` of the time step on copies of sim's arrays; returns (state, state_tmp, flux)"""
+    kernel = MW.kernel_of(kid)
+    stage = (kid // 3) % 3
+    bufs = {"state": gp.DevBuf.from_array(sim.state), "state_tmp": gp.DevBuf.from_array(sim.state_tmp),
+            "flux": gp.DevBuf.from_array(sim.flux), "hydro": gp.DevBuf.from_array(sim.hydro)}
+    forcing = bufs["state"] if stage == 0 else bufs["state_tmp"]
+    out = bufs["state"] if stage == 2 else bufs["state_tmp"]
+    dt = np.float32(sim.dt) / np.float32([3, 2, 1][stage])
+    p = gp.MiniweatherParams(kernel, sim.nx, sim.nz, float(dt), float(sim.dx), float(sim.dz),
+                             forcing.ptr, bufs["flux"].ptr, bufs["state"].ptr, out.ptr, bufs["hydro"].ptr)
+    info = gp.launch("gp_launch_miniweather", p, ctx)
+    gp.check(gp.lib().gp_stream_sync(None))
+    got = tuple(bufs[k].download(np_dtype=np.float32).reshape(getattr(sim, k).shape) for k in ("state", "state_tmp", "flux"))
+    return got, info
+
+
+@pytest.mark.parametrize("kid", [0, 1, 2, 3, 4, 5, 8, 9, 10, 11, 12, 13, 14, 17, 35])
+@pytest.mark.parametrize("preemptible", [False, True])
+def test_each_kernel_matches_oracle(gp, kid, preemptible):
+    sim = random_sim(200, 100, kid)
+    ctx = None
+    if preemptible:
+        blp = gp.BlpState(1, gp.Flag())
+        ctx = blp.ctx(0)
+    got, info = launch_kernel(gp, sim, kid, ctx)
+    want = sim.copy()
+    want.run_kernel(kid)
+    kind = MW.kernel_of(kid)
+    assert info.total_tiles == MW.kernel_tiles(kind, 200, 100)
+    for g, w, name in zip(got, (want.state, want.state_tmp, want.flux), ("state", "state_tmp", "flux")):
+        if kind in (MW.FLUX_X, MW.FLUX_Z) and name == "flux":
+            tol = 1e-6 if kind == MW.FLUX_X else 2e-5
+            for v in range(4):
+                assert np.abs(g[v] - w[v]).max() <= tol * np.abs(w[v]).max(), (name, v)
+        else:
+            assert np.array_equal(g, w), name
+
+
+def test_bad_arguments_are_refused(gp):
+    sim = MW.Sim(16, 8)
+    st = gp.DevBuf.from_array(sim.state)
+    p = gp.MiniweatherParams(7, 16, 8, 0.1, 1.0, 1.0, st.ptr, st.ptr, st.ptr, st.ptr, st.ptr)
+    with pytest.raises(gp.GpError):
+        gp.launch("gp_launch_miniweather", p)
+    p = gp.MiniweatherParams(MW.FLUX_X, 16, 8, 0.1, 1.0, 1.0, st.ptr, None, st.ptr, st.ptr, st.ptr)
+    with pytest.raises(gp.GpError):
+        gp.launch("gp_launch_miniweather", p)
+    p = gp.MiniweatherParams(MW.FLUX_X, 2, 8, 0.1, 1.0, 1.0, st.ptr, st.ptr, st.ptr, st.ptr, st.ptr)
+    with pytest.raises(gp.GpError):
+        gp.launch("gp_launch_miniweather", p)
+
+
+def test_workload_matches_oracle_over_time_steps(gp, ex_mod):
+    nx, nz = 200, 100
+    ex = ex_mod.Executor(f"miniweather@nx={nx},nz={nz}")
+    assert ex.kernel_num() == 36
+    names = [k["name"] for k in ex.kernels()]
+    assert names[:3] == ["set_halo_values_x", "compute_tendencies_x", "compute_tendencies_x_r"]
+    assert names[9:12] == ["set_halo_values_z", "compute_tendencies_z", "compute_tendencies_z_r"]
+    sim = MW.Sim(nx, nz, MW.COLLISION)
+    state0 = f32(ex.read_storage("state")).reshape(sim.state.shape)
+    hydro0 = f32(ex.read_storage("hydro"))
+    # the host library's own set-up against the oracle's (both restate sci_init)
+    assert np.abs(state0 - sim.state).max() <= 1e-6 * np.abs(sim.state).max()
+    assert np.allclose(hydro0, sim.hydro, rtol=1e-6)
+    sim.state[:] = state0
+    sim.state_tmp[:] = state0
+    sim.hydro[:] = hydro0
+    m0, e0 = ex.miniweather_reductions()
+    assert (m0, e0) == pytest.approx(sim.reductions(), rel=1e-12)
+    for _ in range(4):
+        ex.execute()
+        sim.timestep()
+    got = f32(ex.read_storage("state")).reshape(sim.state.shape)
+    for v in range(4):
+        inner = (slice(MW.HS, -MW.HS), slice(MW.HS, -MW.HS))
+        assert np.abs(got[v][inner] - sim.state[v][inner]).max() <= 1e-4 * np.abs(sim.state[v][inner]).max(), v
+    m1, e1 = ex.miniweather_reductions()
+    assert abs(m1 - m0) / m0 < 1e-6 and abs(e1 - e0) / e0 < 1e-3
+
+
+def _arrays(ex):
+    return [f32(ex.read_storage(k)) for k in ("state", "state_tmp", "flux")]
+
+
+# (kernel, claim): first halo; mid flux; the in-place third-stage updates (8: x, 17: z); the z
+# update whose forcing state is its output (14); the very last kernel
+INJECTIONS = [(0, 0), (1, 700), (8, 3000), (14, 5000), (17, 1234), (22, 10), (35, 8000)]
+
+
+def test_preempt_resume_is_bit_exact(gp, ex_mod):
+    wl = "miniweather@nx=1024,nz=512"
+    base = ex_mod.Executor(wl)
+    ex = ex_mod.Executor(wl, blp=True)
+    flag = gp.Flag()
+    ex.set_flag(flag)
+    stream = gp.Stream(1)
+    base.execute()
+    ex.execute(stream)
+    ex.set_running(True)
+    stream.sync()
+    assert ex.stop_point(stream) == -1
+    for a, b in zip(_arrays(base), _arrays(ex)):
+        assert np.array_equal(a, b)  # preemptible launches alone change nothing
+    stopped = 0
+    for kernel, claim in INJECTIONS:
+        base.execute()
+        flag.set(0)
+        ex.inject_preempt(kernel, claim)
+        ex.execute(stream)
+        ex.set_running(True)
+        stream.sync()
+        assert flag.get() == 1, (kernel, claim)
+        cnt = ex.counters()
+        assert (cnt[kernel + 3:] == 0).all(), (kernel, cnt)
+        part = _arrays(ex)
+        ex.inject_preempt(-1, -1)
+        flag.set(0)
+        ex.resume(stream)
+        stream.sync()
+        si = ex.last_stop_index()
+        if si != -1:
+            stopped += 1
+            assert kernel <= si <= kernel + 2, (si, kernel)
+            # the stopped step really was incomplete
+            assert any(not np.array_equal(a, b) for a, b in zip(_arrays(base), part)), (kernel, claim)
+        else:
+            assert kernel >= 33
+        for a, b, name in zip(_arrays(base), _arrays(ex), ("state", "state_tmp", "flux")):
+            assert np.array_equal(a, b), (kernel, claim, name)
+    assert stopped >= len(INJECTIONS) - 1
+
+
+def test_full_size_conservation_with_host_timed_preemption(gp, ex_mod):
+    """The reference's size (3200 x 1600 cells): mass is conserved to rounding and total energy
+    nearly, across time steps that the host interrupts whenever its store happens to land."""
+    ex = ex_mod.Executor("miniweather", blp=True)
+    flag = gp.Flag()
+    ex.set_flag(flag)
+    stream = gp.Stream(1)
+    m0, e0 = ex.miniweather_reductions()
+    stops = []
+    for _ in range(6):
+        ex.execute(stream)
+        ex.set_running(True)
+        flag.set(1)
+        stream.sync()
+        flag.set(0)
+        ex.resume(stream)
+        stops.append(ex.last_stop_index())
+        stream.sync()
+    m1, e1 = ex.miniweather_reductions()
+    assert any(s != -1 for s in stops), stops
+    assert abs(m1 - m0) / m0 < 1e-7
+    assert abs(e1 - e0) / e0 < 1e-5
+    w = f32(ex.read_storage("state")).reshape(4, 1604, 3204)[2]
+    assert np.isfinite(w).all() and np.abs(w).max() > 1e-3  # the bubbles have started to move

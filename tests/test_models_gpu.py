@@ -106,7 +106,7 @@ def test_executor_error_paths(gp, ex_mod, tmp_path):
         ex_mod.Executor("no_such_model", model_root=str(tmp_path))
     assert e.value.status == 3  # NotFound
     with pytest.raises(ex_mod.StatusError) as e:
-        ex_mod.Executor("miniweather", model_root=str(tmp_path))  # reference workload outside this build
+        ex_mod.Executor("pagerank", model_root=str(tmp_path))  # reference workload outside this build (needs a graph dataset)
     assert e.value.status == 3
     ex = ex_mod.Executor("toy", model_root=str(tmp_path))
     with pytest.raises(ex_mod.StatusError) as e:
