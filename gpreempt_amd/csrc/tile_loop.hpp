@@ -95,9 +95,10 @@ __device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_l
                 atomicCAS(b.stop_index, -1, b.kernel_id);
             // the polling workgroup still owes the tile it has just claimed
         }
-    } else {
-        atomicCAS(b.stop_index, -1, b.kernel_id);
     }
+    // (a workgroup that finds the stop index set has nothing to record: the first writer won.
+    // An atomic on that one word from every leaving workgroup would serialise the exit of a
+    // 2000-workgroup grid into 80 us.)
     return claim;
 }
 
@@ -170,8 +171,6 @@ __device__ __forceinline__ void tile_loop_ckpt(const BlpArgs &b, Body &&body) {
                         claim = hdr[2];
                         first = hdr[3];
                         hdr[0] = 0;
-                    } else {
-                        atomicCAS(b.stop_index, -1, b.kernel_id);
                     }
                 } else {
                     claim = claim_tile(b, grp, slice_lo, slice_n);
