@@ -264,6 +264,41 @@ def hbm_ops(iters=20):
     return out
 
 
+def miniweather(steps=50):
+    """The reference's non-DNN workload at its own size (3200 x 1600 cells): one execute() = 36
+    preemptible kernels = two time steps.  Achieved bandwidth = algorithmic bytes of the kernel
+    list / HIP-event time, against the 8 TB/s HBM peak; mass / energy drift over the run is the
+    workload's own self-check; the CPU figure is the oracle on a 400 x 200 grid scaled by cells."""
+    from gpreempt_amd import capi as gp, executor as E
+    from oracle import miniweather as MW
+    ex = E.Executor("miniweather", blp=True)
+    ex.set_flag(gp.Flag())
+    stream = gp.Stream(1)
+    m0, e0 = ex.miniweather_reductions()
+    for _ in range(3):
+        ex.execute(stream)
+    a, b = gp.Event(), gp.Event()
+    a.record(stream)
+    for _ in range(steps):
+        ex.execute(stream)
+    b.record(stream)
+    b.sync()
+    ms = a.elapsed_ms(b) / steps
+    m1, e1 = ex.miniweather_reductions()
+    nbytes = sum(k["bytes"] for k in ex.kernels())
+    sim = MW.Sim(400, 200)
+    sim.timestep()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        sim.timestep()
+    cpu_ms = (time.perf_counter() - t0) / 5 * 1e3 * (3200 * 1600) / (400 * 200)
+    ex.destroy()
+    return {"workload": "miniweather 3200x1600 fp32, collision test case, 36 kernels per execute", "ms_per_execute": ms,
+            "algorithmic_MB": nbytes / 1e6, "achieved_GBps": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / 8000.0,
+            "mass_drift": abs(m1 - m0) / m0, "energy_drift": abs(e1 - e0) / e0, "executes": steps + 3,
+            "cpu_oracle_ms_per_execute_scaled": cpu_ms, "cpu_cores": 1}
+
+
 def copy_calibration(mib=256, iters=10):
     """A plain device-to-device copy of known size (the runtime's copy kernel), used to scale
     the FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc runs."""
@@ -312,7 +347,7 @@ def main():
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
-    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | cpu | copycal")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | cpu | copycal")
     ap.add_argument("--cpu-requests", type=int, default=4)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -343,6 +378,8 @@ def main():
         out["config1_gemm1024_f32"] = config1_gemm1024()
     if args.only in ("", "hbm"):
         out["hbm_bound_ops"] = hbm_ops()
+    if args.only in ("", "miniweather"):
+        out["miniweather"] = miniweather()
     if args.only == "copycal":
         out["copy_calibration"] = copy_calibration()
     if args.only in ("", "cpu"):

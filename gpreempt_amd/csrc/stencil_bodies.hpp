@@ -48,18 +48,175 @@ __device__ __forceinline__ void mw_reconstruct(const float (&s)[4], float hv_coe
     d3 = (-s[0] + 3 * (s[1] - s[2]) + s[3]) * hv_coef;
 }
 
+// Pointers into the hydrostatic background buffer: cell density, cell density*theta (nz+4 each),
+// interface density, density*theta, pressure (nz+1 each), four boundary density ratios.
+struct MwHydro {
+    const float *dens_cell, *dens_theta_cell, *dens_int, *dens_theta_int, *pressure_int, *cell_const;
+    __device__ __forceinline__ MwHydro(const float *h, int nz) {
+        dens_cell = h;
+        dens_theta_cell = dens_cell + nz + 2 * MW_HS;
+        dens_int = dens_theta_cell + nz + 2 * MW_HS;
+        dens_theta_int = dens_int + nz + 1;
+        pressure_int = dens_theta_int + nz + 1;
+        cell_const = pressure_int + nz + 1;
+    }
+};
+
+// What one element id reads, split from what it computes and writes so that a lane can have the
+// loads of several ids in flight before the first result is needed (an id alone keeps 12-72 bytes
+// in flight per lane, too few to cover HBM latency at 32 waves per CU).
+template <int KIND> struct MwOperands;
+
+template <> struct MwOperands<GP_MW_UPDATE_X> { long c; float f0, f1, init; };
+template <> struct MwOperands<GP_MW_UPDATE_Z> { long c; int ll; float f0, f1, init, d0, d1, dinit; };
+template <> struct MwOperands<GP_MW_FLUX_X> { int k, i; float s[MW_VARS][4], h0, h1; };
+template <> struct MwOperands<GP_MW_FLUX_Z> { int k, i; float s[MW_VARS][4], h0, h1, h2; };
+
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_UPDATE_X> &o) {
+    const MwView v{p.nx, p.nz};
+    const int nx = p.nx, nz = p.nz;
+    const int k = (int)((id / nx) % nz), i = (int)(id % nx), ll = (int)(id / nx / nz);
+    if (ll >= MW_VARS) return false;
+    o.c = v.st(ll, k + MW_HS, i + MW_HS);
+    o.f0 = p.flux[v.fx(ll, k, i)];
+    o.f1 = p.flux[v.fx(ll, k, i + 1)];
+    o.init = p.state_init[o.c];
+    return true;
+}
+__device__ __forceinline__ void mw_finish(const gp_miniweather_params &p, const MwOperands<GP_MW_UPDATE_X> &o) {
+#pragma clang fp contract(off)
+    const float tend = -(o.f1 - o.f0) / p.dx;
+    p.state_out[o.c] = o.init + p.dt * tend;
+}
+
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_UPDATE_Z> &o) {
+    const MwView v{p.nx, p.nz};
+    const int nx = p.nx, nz = p.nz;
+    const int i = (int)(id % nx), k = (int)((id / nx) % nz), ll = (int)(id / nx / nz);
+    if (ll >= MW_VARS) return false;
+    o.ll = ll;
+    o.c = v.st(ll, k + MW_HS, i + MW_HS);
+    o.f0 = p.flux[v.fx(ll, k, i)];
+    o.f1 = p.flux[v.fx(ll, k + 1, i)];
+    o.init = p.state_init[o.c];
+    o.d0 = o.d1 = o.dinit = 0.f;
+    if (ll == MW_WMOM) {
+        // Gravity acts on the density of the forcing state.  When the forcing state is also the
+        // output (second Runge-Kutta stage) other lanes overwrite that density in this very
+        // kernel; in element order the density ids come first, so the value defined for this read
+        // is the UPDATED one, which is recomputed from operands the kernel never writes instead
+        // of being read while it changes.
+        const long cd = v.st(MW_DENS, k + MW_HS, i + MW_HS);
+        if (p.state == p.state_out) {
+            o.d0 = p.flux[v.fx(MW_DENS, k, i)];
+            o.d1 = p.flux[v.fx(MW_DENS, k + 1, i)];
+            o.dinit = p.state_init[cd];
+        } else {
+            o.dinit = p.state[cd];
+        }
+    }
+    return true;
+}
+__device__ __forceinline__ void mw_finish(const gp_miniweather_params &p, const MwOperands<GP_MW_UPDATE_Z> &o) {
+#pragma clang fp contract(off)
+    float tend = -(o.f1 - o.f0) / p.dz;
+    if (o.ll == MW_WMOM) {
+        float dens = o.dinit;
+        if (p.state == p.state_out) {
+            const float td = -(o.d1 - o.d0) / p.dz;
+            dens = o.dinit + p.dt * td;
+        }
+        tend = tend - dens * MW_GRAV;
+    }
+    p.state_out[o.c] = o.init + p.dt * tend;
+}
+
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_FLUX_X> &o) {
+    const MwView v{p.nx, p.nz};
+    const MwHydro hy(p.hydro, p.nz);
+    const int nx = p.nx;
+    o.k = (int)(id / (nx + 1));
+    o.i = (int)(id % (nx + 1));
+    if (o.k >= p.nz) return false;
+#pragma unroll
+    for (int ll = 0; ll < MW_VARS; ++ll) {
+        const float *c = p.state + v.st(ll, o.k + MW_HS, o.i);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) o.s[ll][s] = c[s];
+    }
+    o.h0 = hy.dens_cell[o.k + MW_HS];
+    o.h1 = hy.dens_theta_cell[o.k + MW_HS];
+    return true;
+}
+__device__ __forceinline__ void mw_finish(const gp_miniweather_params &p, const MwOperands<GP_MW_FLUX_X> &o) {
+#pragma clang fp contract(off)
+    const MwView v{p.nx, p.nz};
+    const float hv_coef = -MW_HV_BETA * p.dx / (16 * p.dt);
+    float vals[MW_VARS], d3[MW_VARS];
+#pragma unroll
+    for (int ll = 0; ll < MW_VARS; ++ll) mw_reconstruct(o.s[ll], hv_coef, vals[ll], d3[ll]);
+    const double r = vals[MW_DENS] + o.h0;
+    const double u = vals[MW_UMOM] / r;
+    const double w = vals[MW_WMOM] / r;
+    const double th = (vals[MW_RHOT] + o.h1) / r;
+    // (rho theta)^gamma as exp(gamma log(.)): the argument is positive and the result is rounded to
+    // fp32 when the flux is stored, 8 decimal digits above what the fp64 exp/log pair loses, and
+    // the pair costs a third of a general pow (which made this kernel ALU-bound: 60 us of fp64
+    // work against 35 us of memory traffic)
+    const double pr = MW_C0 * exp((double)MW_GAMMA * log(r * th));
+    p.flux[v.fx(MW_DENS, o.k, o.i)] = (float)(r * u - d3[MW_DENS]);
+    p.flux[v.fx(MW_UMOM, o.k, o.i)] = (float)(r * u * u + pr - d3[MW_UMOM]);
+    p.flux[v.fx(MW_WMOM, o.k, o.i)] = (float)(r * u * w - d3[MW_WMOM]);
+    p.flux[v.fx(MW_RHOT, o.k, o.i)] = (float)(r * u * th - d3[MW_RHOT]);
+}
+
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_FLUX_Z> &o) {
+    const MwView v{p.nx, p.nz};
+    const MwHydro hy(p.hydro, p.nz);
+    const int nx = p.nx;
+    o.i = (int)(id % nx);
+    o.k = (int)(id / nx);
+    if (o.k >= p.nz + 1) return false;
+    const long row = nx + 2 * MW_HS;
+#pragma unroll
+    for (int ll = 0; ll < MW_VARS; ++ll) {
+        const float *c = p.state + v.st(ll, o.k, o.i + MW_HS);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) o.s[ll][s] = c[s * row];
+    }
+    o.h0 = hy.dens_int[o.k];
+    o.h1 = hy.dens_theta_int[o.k];
+    o.h2 = hy.pressure_int[o.k];
+    return true;
+}
+__device__ __forceinline__ void mw_finish(const gp_miniweather_params &p, const MwOperands<GP_MW_FLUX_Z> &o) {
+#pragma clang fp contract(off)
+    const MwView v{p.nx, p.nz};
+    const float hv_coef = -MW_HV_BETA * p.dz / (16 * p.dt);
+    float vals[MW_VARS], d3[MW_VARS];
+#pragma unroll
+    for (int ll = 0; ll < MW_VARS; ++ll) mw_reconstruct(o.s[ll], hv_coef, vals[ll], d3[ll]);
+    const float r = vals[MW_DENS] + o.h0;
+    const float u = vals[MW_UMOM] / r;
+    float w = vals[MW_WMOM] / r;
+    const float th = (vals[MW_RHOT] + o.h1) / r;
+    const float pr = MW_C0 * powf(r * th, MW_GAMMA) - o.h2;
+    if (o.k == 0 || o.k == p.nz) {  // no flow through the bottom and top faces, exact mass conservation
+        w = 0.f;
+        d3[MW_DENS] = 0.f;
+    }
+    p.flux[v.fx(MW_DENS, o.k, o.i)] = r * w - d3[MW_DENS];
+    p.flux[v.fx(MW_UMOM, o.k, o.i)] = r * w * u - d3[MW_UMOM];
+    p.flux[v.fx(MW_WMOM, o.k, o.i)] = r * w * w + pr - d3[MW_WMOM];
+    p.flux[v.fx(MW_RHOT, o.k, o.i)] = r * w * th - d3[MW_RHOT];
+}
+
+// halo kernels: a few thousand ids, nothing to overlap
 template <int KIND>
-__device__ __forceinline__ void mw_tile(const gp_miniweather_params &p, TileIdx t) {
+__device__ __forceinline__ void mw_halo(const gp_miniweather_params &p, long id) {
 #pragma clang fp contract(off)
     const MwView v{p.nx, p.nz};
     const int nx = p.nx, nz = p.nz;
-    const long id = (long)t.x * MW_TILE + threadIdx.x;
-    // hydrostatic background, one buffer: cell density, cell density*theta (nz+4 each), interface
-    // density, density*theta, pressure (nz+1 each), four boundary density ratios
-    const float *hy_dens_cell = p.hydro, *hy_dens_theta_cell = hy_dens_cell + nz + 2 * MW_HS;
-    const float *hy_dens_int = hy_dens_theta_cell + nz + 2 * MW_HS, *hy_dens_theta_int = hy_dens_int + nz + 1;
-    const float *hy_pressure_int = hy_dens_theta_int + nz + 1, *hy_cell_const = hy_pressure_int + nz + 1;
-
     if constexpr (KIND == GP_MW_HALO_X) {  // periodic in x
         const int ll = (int)(id / nz), k = (int)(id % nz);
         if (ll < MW_VARS) {
@@ -67,7 +224,8 @@ __device__ __forceinline__ void mw_tile(const gp_miniweather_params &p, TileIdx 
             const float a = row[nx + MW_HS - 2], b = row[nx + MW_HS - 1], c = row[MW_HS], d = row[MW_HS + 1];
             row[0] = a; row[1] = b; row[nx + MW_HS] = c; row[nx + MW_HS + 1] = d;
         }
-    } else if constexpr (KIND == GP_MW_HALO_Z) {  // solid walls: no flow through, momentum scaled by the density ratio
+    } else {  // solid walls: no flow through, horizontal momentum scaled by the density ratio
+        const MwHydro hy(p.hydro, nz);
         const int i = (int)(id % (nx + 2 * MW_HS)), ll = (int)(id / (nx + 2 * MW_HS));
         if (ll < MW_VARS) {
             float *s = p.state;
@@ -77,95 +235,39 @@ __device__ __forceinline__ void mw_tile(const gp_miniweather_params &p, TileIdx 
             } else {
                 const float lo = s[v.st(ll, MW_HS, i)], hi = s[v.st(ll, nz + MW_HS - 1, i)];
                 const bool um = ll == MW_UMOM;
-                s[v.st(ll, 0, i)] = um ? lo * hy_cell_const[0] : lo;
-                s[v.st(ll, 1, i)] = um ? lo * hy_cell_const[1] : lo;
-                s[v.st(ll, nz + MW_HS, i)] = um ? hi * hy_cell_const[2] : hi;
-                s[v.st(ll, nz + MW_HS + 1, i)] = um ? hi * hy_cell_const[3] : hi;
+                s[v.st(ll, 0, i)] = um ? lo * hy.cell_const[0] : lo;
+                s[v.st(ll, 1, i)] = um ? lo * hy.cell_const[1] : lo;
+                s[v.st(ll, nz + MW_HS, i)] = um ? hi * hy.cell_const[2] : hi;
+                s[v.st(ll, nz + MW_HS + 1, i)] = um ? hi * hy.cell_const[3] : hi;
             }
         }
-    } else if constexpr (KIND == GP_MW_FLUX_X) {
-        const int k = (int)(id / (nx + 1)), i = (int)(id % (nx + 1));
-        if (k < nz) {
-            const float hv_coef = -MW_HV_BETA * p.dx / (16 * p.dt);
-            float vals[MW_VARS], d3[MW_VARS];
+    }
+}
+
+// Tiles [first, last) of one claim: U tiles at a time, all loads first.  The ids of different
+// tiles never touch the same output element, and an update reads the element it writes only
+// through its own lane, so issuing the loads of U tiles ahead of their stores changes nothing.
+template <int KIND>
+__device__ __forceinline__ void mw_span(const gp_miniweather_params &p, int first, int last) {
+    if constexpr (KIND == GP_MW_HALO_X || KIND == GP_MW_HALO_Z) {
+        for (int t = first; t < last; ++t) mw_halo<KIND>(p, (long)t * MW_TILE + threadIdx.x);
+    } else {
+        constexpr int U = (KIND == GP_MW_UPDATE_X || KIND == GP_MW_UPDATE_Z) ? 4 : 2;
+        for (int t = first; t < last; t += U) {
+            MwOperands<KIND> op[U];
+            bool ok[U];
 #pragma unroll
-            for (int ll = 0; ll < MW_VARS; ++ll) {
-                const float *c = p.state + v.st(ll, k + MW_HS, i);
-                const float s[4] = {c[0], c[1], c[2], c[3]};
-                mw_reconstruct(s, hv_coef, vals[ll], d3[ll]);
-            }
-            const double r = vals[MW_DENS] + hy_dens_cell[k + MW_HS];
-            const double u = vals[MW_UMOM] / r;
-            const double w = vals[MW_WMOM] / r;
-            const double th = (vals[MW_RHOT] + hy_dens_theta_cell[k + MW_HS]) / r;
-            const double pr = MW_C0 * pow(r * th, (double)MW_GAMMA);
-            p.flux[v.fx(MW_DENS, k, i)] = (float)(r * u - d3[MW_DENS]);
-            p.flux[v.fx(MW_UMOM, k, i)] = (float)(r * u * u + pr - d3[MW_UMOM]);
-            p.flux[v.fx(MW_WMOM, k, i)] = (float)(r * u * w - d3[MW_WMOM]);
-            p.flux[v.fx(MW_RHOT, k, i)] = (float)(r * u * th - d3[MW_RHOT]);
-        }
-    } else if constexpr (KIND == GP_MW_FLUX_Z) {
-        const int i = (int)(id % nx), k = (int)(id / nx);
-        if (k < nz + 1) {
-            const float hv_coef = -MW_HV_BETA * p.dz / (16 * p.dt);
-            float vals[MW_VARS], d3[MW_VARS];
+            for (int j = 0; j < U; ++j) ok[j] = t + j < last && mw_load(p, (long)(t + j) * MW_TILE + threadIdx.x, op[j]);
 #pragma unroll
-            for (int ll = 0; ll < MW_VARS; ++ll) {
-                const float *c = p.state + v.st(ll, k, i + MW_HS);
-                const long row = nx + 2 * MW_HS;
-                const float s[4] = {c[0], c[row], c[2 * row], c[3 * row]};
-                mw_reconstruct(s, hv_coef, vals[ll], d3[ll]);
-            }
-            const float r = vals[MW_DENS] + hy_dens_int[k];
-            const float u = vals[MW_UMOM] / r;
-            float w = vals[MW_WMOM] / r;
-            const float th = (vals[MW_RHOT] + hy_dens_theta_int[k]) / r;
-            const float pr = MW_C0 * powf(r * th, MW_GAMMA) - hy_pressure_int[k];
-            if (k == 0 || k == nz) {  // no flow through the bottom and top faces, exact mass conservation
-                w = 0.f;
-                d3[MW_DENS] = 0.f;
-            }
-            p.flux[v.fx(MW_DENS, k, i)] = r * w - d3[MW_DENS];
-            p.flux[v.fx(MW_UMOM, k, i)] = r * w * u - d3[MW_UMOM];
-            p.flux[v.fx(MW_WMOM, k, i)] = r * w * w + pr - d3[MW_WMOM];
-            p.flux[v.fx(MW_RHOT, k, i)] = r * w * th - d3[MW_RHOT];
-        }
-    } else if constexpr (KIND == GP_MW_UPDATE_X) {
-        const int k = (int)((id / nx) % nz), i = (int)(id % nx), ll = (int)(id / nx / nz);
-        if (ll < MW_VARS) {
-            const float tend = -(p.flux[v.fx(ll, k, i + 1)] - p.flux[v.fx(ll, k, i)]) / p.dx;
-            const long c = v.st(ll, k + MW_HS, i + MW_HS);
-            p.state_out[c] = p.state_init[c] + p.dt * tend;
-        }
-    } else {  // GP_MW_UPDATE_Z
-        const int i = (int)(id % nx), k = (int)((id / nx) % nz), ll = (int)(id / nx / nz);
-        if (ll < MW_VARS) {
-            float tend = -(p.flux[v.fx(ll, k + 1, i)] - p.flux[v.fx(ll, k, i)]) / p.dz;
-            if (ll == MW_WMOM) {
-                // Gravity acts on the density of the forcing state.  When the forcing state is also
-                // the output (second Runge-Kutta stage) other lanes overwrite that density in this
-                // very kernel; in element order the density ids come first, so the value defined
-                // for this read is the UPDATED one, which is recomputed here from operands the
-                // kernel never writes instead of being read while it changes.
-                const long cd = v.st(MW_DENS, k + MW_HS, i + MW_HS);
-                float dens;
-                if (p.state == p.state_out) {
-                    const float td = -(p.flux[v.fx(MW_DENS, k + 1, i)] - p.flux[v.fx(MW_DENS, k, i)]) / p.dz;
-                    dens = p.state_init[cd] + p.dt * td;
-                } else {
-                    dens = p.state[cd];
-                }
-                tend = tend - dens * MW_GRAV;
-            }
-            const long c = v.st(ll, k + MW_HS, i + MW_HS);
-            p.state_out[c] = p.state_init[c] + p.dt * tend;
+            for (int j = 0; j < U; ++j)
+                if (ok[j]) mw_finish(p, op[j]);
         }
     }
 }
 
 template <int KIND>
 __global__ __launch_bounds__(MW_TILE) void miniweather_kernel(gp_miniweather_params p, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { mw_tile<KIND>(p, t); });
+    tile_loop_span(blp, [&](int first, int last) { mw_span<KIND>(p, first, last); });
 }
 
 }  // namespace gp

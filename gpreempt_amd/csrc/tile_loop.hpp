@@ -132,6 +132,32 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     }
 }
 
+// The same dispatcher for one-dimensional streaming kernels that want a claim's tiles all at once
+// (to keep the loads of several tiles in flight together): body(first_tile, last_tile) is called
+// once per claim with the half-open range of tile numbers the claim stands for.
+template <class Body>
+__device__ __forceinline__ void tile_loop_span(const BlpArgs &b, Body &&body) {
+    __shared__ int mailbox[2];
+    const bool dynamic = b.executed != nullptr;
+    const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    const int grp = wg_group((int)blockIdx.x, b.groups);
+    const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
+    const int slice_n = (b.groups > 1 ? group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) : b.total) - slice_lo;
+    for (int it = 0;; ++it) {
+        int idx;
+        if (!dynamic) {
+            idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
+        } else {
+            if (leader) mailbox[it & 1] = claim_tile(b, grp, slice_lo, slice_n);
+            __syncthreads();
+            idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1]);
+        }
+        if (idx < 0) return;
+        const int first = idx * b.batch;
+        body(first, first + b.batch < b.tiles ? first + b.batch : b.tiles);
+    }
+}
+
 // ---- tiles that can be left half-way ------------------------------------------------------------
 // A tile whose K loop runs for hundreds of microseconds (a 256 x 256 tile over K = 8192 takes
 // about 200 us) makes "finish the tile you owe" too slow a way to leave.  Kernels built on
