@@ -83,6 +83,12 @@ class MiniweatherParams(C.Structure):
                 ("state", vp), ("flux", vp), ("state_init", vp), ("state_out", vp), ("hydro", vp)]
 
 
+class GraphParams(C.Structure):
+    _fields_ = [("kernel", C.c_int), ("level", C.c_uint), ("vertex_count", C.c_ulonglong), ("vertex_list", vp), ("edge_list", vp),
+                ("weight_list", vp), ("label", vp), ("active", vp), ("next_active", vp), ("comp", vp), ("delta", vp), ("residual", vp),
+                ("value", vp), ("alpha", C.c_float), ("tolerance", C.c_float), ("cost", vp), ("new_cost", vp), ("changed", vp)]
+
+
 class EmbedParams(C.Structure):
     _fields_ = [("dtype", C.c_int), ("tokens", C.c_long), ("seq", C.c_int), ("hidden", C.c_int), ("vocab", C.c_long),
                 ("ids", vp), ("tok", vp), ("pos", vp), ("seg", vp), ("out", vp)]
@@ -94,7 +100,7 @@ gp_stream_query gp_stream_priority gp_stream_native gp_event_create gp_event_des
 gp_event_sync gp_event_query gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free gp_memcpy_h2d gp_memcpy_d2h
 gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_flag_relay_start
 gp_launch_gemm gp_gemm_ckpt_bytes gp_conv_ckpt_bytes gp_ckpt_reset_async gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
-gp_launch_layernorm gp_launch_attention gp_launch_miniweather gp_launch_embed gp_launch_gate gp_launch_noop gp_graph_begin gp_graph_end gp_graph_launch
+gp_launch_layernorm gp_launch_attention gp_launch_miniweather gp_launch_graph gp_launch_embed gp_launch_gate gp_launch_noop gp_graph_begin gp_graph_end gp_graph_launch
 gp_graph_destroy gp_program_create gp_program_destroy gp_program_add_gemm gp_program_add_conv2d
 gp_program_add_nchw_to_nhwc gp_program_add_pool2d gp_program_add_eltwise gp_program_add_softmax gp_program_add_layernorm
 gp_program_add_attention gp_program_add_embed gp_program_add_copy gp_program_finalize gp_program_launch gp_program_layers gp_program_read_state""".split()

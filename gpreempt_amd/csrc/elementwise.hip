@@ -3,6 +3,7 @@
 // elementwise_bodies.hpp.
 #include "plans.hpp"
 #include "stencil_bodies.hpp"
+#include "graph_bodies.hpp"
 
 namespace gp {
 
@@ -221,6 +222,29 @@ extern "C" int gp_launch_miniweather(const gp_miniweather_params *p, const gp_pr
 #define GP_MW(K) case K: return launch_tiles(miniweather_kernel<K>, tiles, 1, ctx, s, info, *p);
         GP_MW(GP_MW_HALO_X) GP_MW(GP_MW_FLUX_X) GP_MW(GP_MW_UPDATE_X) GP_MW(GP_MW_HALO_Z) GP_MW(GP_MW_FLUX_Z) GP_MW(GP_MW_UPDATE_Z)
 #undef GP_MW
+    }
+    return GP_OUTOFRANGE;
+}
+extern "C" int gp_launch_graph(const gp_graph_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    GP_REQUIRE(p && p->vertex_list, "null graph params");
+    GP_REQUIRE(p->kernel >= GP_GRAPH_BFS_STEP && p->kernel <= GP_GRAPH_SSSP_UPDATE, "graph kernel %d", p->kernel);
+    GP_REQUIRE(p->vertex_count > 0 && p->vertex_count < (1ULL << 32), "graph: vertex count out of range");
+    GP_REQUIRE(p->changed || p->kernel == GP_GRAPH_PR_INIT || p->kernel == GP_GRAPH_PR_PUSH || p->kernel == GP_GRAPH_SSSP_RELAX, "graph: changed word missing");
+    GP_REQUIRE(!graph_kernel_is_edge_parallel(p->kernel) || p->edge_list, "graph: edge list missing");
+    switch (p->kernel) {
+        case GP_GRAPH_BFS_STEP: GP_REQUIRE(p->label, "bfs: label missing"); break;
+        case GP_GRAPH_CC_STEP: GP_REQUIRE(p->active && p->next_active && p->comp, "cc: operands missing"); break;
+        case GP_GRAPH_PR_INIT: case GP_GRAPH_PR_PUSH: case GP_GRAPH_PR_UPDATE:
+            GP_REQUIRE(p->active && p->delta && p->residual && p->value, "pagerank: operands missing"); break;
+        case GP_GRAPH_SSSP_RELAX: GP_REQUIRE(p->weight_list && p->active && p->new_cost, "sssp: operands missing"); break;
+        case GP_GRAPH_SSSP_UPDATE: GP_REQUIRE(p->active && p->cost && p->new_cost, "sssp: operands missing"); break;
+    }
+    const int tiles = (int)graph_kernel_tiles(p->kernel, p->vertex_count);
+    switch (p->kernel) {
+#define GP_GR(K) case K: return launch_tiles(graph_kernel<K>, tiles, 1, ctx, s, info, *p);
+        GP_GR(GP_GRAPH_BFS_STEP) GP_GR(GP_GRAPH_CC_STEP) GP_GR(GP_GRAPH_PR_INIT) GP_GR(GP_GRAPH_PR_PUSH)
+        GP_GR(GP_GRAPH_PR_UPDATE) GP_GR(GP_GRAPH_SSSP_RELAX) GP_GR(GP_GRAPH_SSSP_UPDATE)
+#undef GP_GR
     }
     return GP_OUTOFRANGE;
 }

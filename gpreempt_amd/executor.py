@@ -15,7 +15,8 @@ vp = C.c_void_p
 SYMBOLS = """gpx_create gpx_destroy gpx_init gpx_set_input gpx_get_output gpx_get_data_size gpx_execute
 gpx_launch_kernel gpx_get_kernel_num gpx_capture_graph gpx_uses_program gpx_clear gpx_set_flag gpx_set_running gpx_resume
 gpx_get_stop_point gpx_last_stop_index gpx_inject_preempt gpx_read_counters gpx_reset_counters gpx_storage_num gpx_storage_info
-gpx_kernel_info gpx_read_storage gpx_miniweather_reductions gpx_run_scenario gpx_preempt_probe gpx_parse_params""".split()
+gpx_kernel_info gpx_read_storage gpx_miniweather_reductions gpx_graph_info gpx_graph_result_bytes gpx_graph_result
+gpx_graph_inject_preempt gpx_set_lc_tasks gpx_set_graph_path gpx_write_synthetic_graph gpx_run_scenario gpx_preempt_probe gpx_parse_params""".split()
 
 STATUS = ["Succ", "Fail", "Timeout", "NotFound", "OutOfRange", "Full"]
 _lib = None
@@ -32,6 +33,7 @@ def lib():
         _lib.gpx_get_data_size.restype = C.c_size_t
         _lib.gpx_get_kernel_num.restype = C.c_size_t
         _lib.gpx_storage_num.restype = C.c_size_t
+        _lib.gpx_graph_result_bytes.restype = C.c_size_t
         _lib.gpx_destroy.restype = None
         _lib.gpx_clear.restype = None
     return _lib
@@ -62,11 +64,13 @@ def write_params(path, params):
 
 
 class Executor:
-    def __init__(self, workload, blp=False, model_root=None):
+    def __init__(self, workload, blp=False, model_root=None, graph_path=None):
         if model_root is not None:
             os.environ["GPREEMPT_MODEL_PATH"] = model_root
         self.blp = blp
         self.h = vp(lib().gpx_create(int(blp)))
+        if graph_path:
+            _chk(lib().gpx_set_graph_path(self.h, graph_path.encode()), "set_graph_path")
         _chk(lib().gpx_init(self.h, workload.encode()), f"init({workload})")
 
     # -- introspection
@@ -132,6 +136,23 @@ class Executor:
         return raw
 
     # -- execution
+    # -- graph workloads
+    def graph_info(self):
+        v = (C.c_ulonglong * 5)()
+        _chk(lib().gpx_graph_info(self.h, v), "graph_info")
+        return dict(vertices=v[0], edges=v[1], iterations=v[2], preemptions=v[3], kernels_launched=v[4])
+
+    def graph_result(self, key, np_dtype):
+        raw = np.empty(lib().gpx_graph_result_bytes(self.h, key.encode()), np.uint8)
+        _chk(lib().gpx_graph_result(self.h, key.encode(), raw.ctypes.data_as(vp), C.c_size_t(raw.nbytes)), f"graph_result({key})")
+        return raw.view(np_dtype)
+
+    def graph_inject_preempt(self, iteration, kernel, claim):
+        _chk(lib().gpx_graph_inject_preempt(self.h, iteration, kernel, claim), "graph_inject_preempt")
+
+    def set_lc_tasks(self, n):
+        _chk(lib().gpx_set_lc_tasks(self.h, int(n)), "set_lc_tasks")
+
     def miniweather_reductions(self):
         """(mass, total energy) of the "miniweather" workload's current state"""
         m, t = C.c_double(), C.c_double()

@@ -1,4 +1,5 @@
 // extern "C" forwarding layer over foo::Executor / foo::BLPExecutor (include/gpreempt_exec_c.h).
+#include <atomic>
 #include <cstring>
 #include "executor.h"
 #include "gpreempt_exec_c.h"
@@ -11,6 +12,7 @@ namespace {
 struct Handle {
     std::unique_ptr<Executor> ex;
     BLPExecutor *blp = nullptr;
+    std::atomic<int> lc_tasks{0}, be_tasks{1};  // handed to BLPExecutor::set_lc_be_tasks
 };
 Handle *H(gpx_executor e) { return static_cast<Handle *>(e); }
 void copy_str(char *dst, size_t n, const std::string &s) {
@@ -24,7 +26,7 @@ extern "C" {
 
 gpx_executor gpx_create(int blp) {
     Handle *h = new Handle();
-    if (blp) { h->blp = new BLPExecutor(); h->ex.reset(h->blp); }
+    if (blp) { h->blp = new BLPExecutor(); h->ex.reset(h->blp); h->blp->set_lc_be_tasks(h->lc_tasks, h->be_tasks); }
     else h->ex.reset(new BaseExecutor());
     return h;
 }
@@ -87,6 +89,33 @@ int gpx_read_storage(gpx_executor e, const char *key, void *out, size_t len) {
 }
 
 }  // extern "C"
+
+extern "C" int gpx_graph_info(gpx_executor e, unsigned long long info[5]) {
+    GraphCompute::Workload *w = H(e)->ex->graph_workload();
+    if (!w) return Status::NotFound;
+    info[0] = w->vertex_count(); info[1] = w->edge_count(); info[2] = (unsigned long long)w->iterations();
+    info[3] = (unsigned long long)w->preemptions(); info[4] = (unsigned long long)w->kernels_launched();
+    return Status::Succ;
+}
+extern "C" size_t gpx_graph_result_bytes(gpx_executor e, const char *key) {
+    GraphCompute::Workload *w = H(e)->ex->graph_workload();
+    return w ? w->result_bytes(key) : 0;
+}
+extern "C" int gpx_graph_result(gpx_executor e, const char *key, void *out, size_t len) {
+    GraphCompute::Workload *w = H(e)->ex->graph_workload();
+    return w ? w->read_result(key, out, len) : Status::NotFound;
+}
+extern "C" int gpx_graph_inject_preempt(gpx_executor e, int iteration, int kernel, int claim) {
+    if (!H(e)->blp) return Status::Fail;
+    H(e)->blp->inject_preempt_graph(iteration, kernel, claim);
+    return Status::Succ;
+}
+extern "C" int gpx_set_lc_tasks(gpx_executor e, int n) { H(e)->lc_tasks.store(n); return Status::Succ; }
+extern "C" int gpx_set_graph_path(gpx_executor e, const char *base) { return H(e)->ex->set_graph_path(base ? base : ""); }
+extern "C" int gpx_write_synthetic_graph(const char *base, unsigned long long vertices, unsigned degree, unsigned long long seed) {
+    if (!base || vertices < 2 || vertices >= (1ULL << 28) || degree < 1 || degree > 256) return Status::OutOfRange;
+    return GraphCompute::write_graph(base, GraphCompute::synthetic_graph(vertices, degree, seed));
+}
 
 extern "C" int gpx_miniweather_reductions(gpx_executor e, double *mass, double *te) {
     auto m = H(e)->ex->get_model();

@@ -6,11 +6,29 @@
 #include <algorithm>
 #include <cstdlib>
 #include <set>
+#include <thread>
 
 namespace foo {
 
-// the graph workloads need a dataset the reference does not ship (src/executor.cpp:12)
-static const std::set<std::string> kNotBuilt = {"cc", "bfs", "pagerank", "sssp"};
+static const std::set<std::string> kGraphCompute = {"cc", "bfs", "pagerank", "sssp"};  // reference executor.cpp:13
+
+static void split_workload(const std::string &workload, std::string &name, std::string &options) {
+    size_t at = workload.find('@');
+    name = workload.substr(0, at);
+    options = at == std::string::npos ? "" : workload.substr(at + 1);
+}
+static long option_int(const std::string &options, const std::string &key, long fallback) {
+    size_t pos = 0;
+    while (pos < options.size()) {
+        size_t end = options.find(',', pos);
+        if (end == std::string::npos) end = options.size();
+        const std::string kv = options.substr(pos, end - pos);
+        size_t eq = kv.find('=');
+        if (eq != std::string::npos && kv.substr(0, eq) == key) return std::atol(kv.c_str() + eq + 1);
+        pos = end + 1;
+    }
+    return fallback;
+}
 
 static std::string model_root() {
     const char *e = std::getenv("GPREEMPT_MODEL_PATH");
@@ -27,11 +45,29 @@ Executor::~Executor() {
 }
 
 // reference executor.cpp:23-45 (dnn branch)
-Status Executor::init(std::string workload) {
-    if (kNotBuilt.count(workload)) {
-        std::fprintf(stderr, "workload '%s' is not part of this build\n", workload.c_str());
-        return Status::NotFound;
+// reference executor.cpp:26-34 (graph branch).  The reference reads its dataset from a fixed
+// directory (:12) that does not ship with it; here the graph comes from set_graph_path(),
+// $GPREEMPT_GRAPH_PATH or, by default, a seeded random graph.
+Status Executor::init_graph(const std::string &kind, const std::string &options) {
+    type = "graph";
+    GraphCompute::CsrGraph g;
+    const char *env = std::getenv("GPREEMPT_GRAPH_PATH");
+    std::string base = !graph_path.empty() ? graph_path : (env && *env ? std::string(env) : std::string());
+    if (!base.empty()) {
+        RETURN_STATUS(GraphCompute::read_graph(base, g, kind == "sssp"));
+    } else {
+        long n = option_int(options, "n", 1 << 20), deg = option_int(options, "deg", 8), seed = option_int(options, "seed", 1);
+        if (n < 2 || n >= (1L << 28) || deg < 1 || deg > 256) return Status::OutOfRange;
+        g = GraphCompute::synthetic_graph((uint64_t)n, (unsigned)deg, (uint64_t)seed);
     }
+    graph_compute = GraphCompute::Workload::create(kind, g);
+    return graph_compute ? Status::Succ : Status::Fail;
+}
+
+Status Executor::init(std::string workload) {
+    std::string name, options;
+    split_workload(workload, name, options);
+    if (kGraphCompute.count(name)) return init_graph(name, options);
     type = "dnn";
     RETURN_STATUS(this->load_model(model_root() + "/" + workload));
     RETURN_STATUS(this->load_param(model_root() + "/" + workload));
@@ -74,6 +110,7 @@ Status Executor::load_param(std::string model_path) { return model->load_param((
 
 // reference executor.cpp:119-134
 Status Executor::execute(GPUstream stream) {
+    if (graph_compute) return graph_compute->compute(stream, nullptr);
     if (use_program) return model->launch_program(stream, true);
     if (use_cuda_graph) {
         CUDA_RETURN_STATUS(gp_graph_launch(graph_exec, stream));
@@ -95,6 +132,7 @@ static bool want_hipgraph() {
 }
 
 void Executor::capture_graph(GPUstream stream) {
+    if (graph_compute) return;  // a host loop cannot be captured (the reference records one iteration's launches, executor.cpp:183-186)
     if (graph_exec) { gp_graph_destroy(graph_exec); graph_exec = nullptr; }
     use_cuda_graph = false;
     use_program = false;
@@ -137,9 +175,18 @@ bool BLPExecutor::program_vacated() const {
 // one counter per kernel, append (flag, stop index) by reference to every kernel and the
 // per-kernel preemption arguments, then load parameters.
 Status BLPExecutor::init(std::string workload) {
-    if (kNotBuilt.count(workload)) {
-        std::fprintf(stderr, "workload '%s' is not part of this build\n", workload.c_str());
-        return Status::NotFound;
+    std::string name, options;
+    split_workload(workload, name, options);
+    if (kGraphCompute.count(name)) {
+        // reference executor.cpp:304-316: stop index and three counters, then the workload
+        RETURN_STATUS(init_graph(name, options));
+        CUDA_RETURN_STATUS(gp_malloc(&dpStopIndex, sizeof(int)));
+        CUDA_RETURN_STATUS(gp_fill32_async(dpStopIndex, 0xFFFFFFFFu, 1, nullptr));
+        const size_t counter_ints = 3 * (size_t)kCounterGroups * kCounterStride;
+        CUDA_RETURN_STATUS(gp_malloc(&executed, sizeof(int) * counter_ints));
+        CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, counter_ints, nullptr));
+        CUDA_RETURN_STATUS(gp_stream_sync(nullptr));
+        return Status::Succ;
     }
     type = "dnn";
     model = std::make_shared<Model>();
@@ -183,6 +230,26 @@ Status BLPExecutor::launch_kernel(size_t kernel_offset, GPUstream stream) {
 // reference executor.cpp:211-232: zero every tile counter, then launch (or replay the graph).
 // The counters are cleared by a fill kernel outside the captured graph.
 Status BLPExecutor::execute(GPUstream stream) {
+    if (graph_compute) {
+        // reference executor.cpp:226-228: the workload's own loop, handed the flag, the counters
+        // and the two task counts; it returns when the algorithm has converged
+        GraphCompute::PreemptEnv env;
+        env.flag = dpStop; env.stop_index = dpStopIndex; env.executed = executed;
+        env.counter_groups = kCounterGroups; env.counter_stride = kCounterStride; env.poll_every = poll_every;
+        std::atomic<int> *lc = lc_tasks, *be = be_tasks;
+        if (lc) env.higher_priority_active = [lc, be]() {
+            // waits here while a latency-critical task is active; meanwhile this workload is not
+            // counted as running (the be_tasks.fetch_sub / fetch_add pair around the reference's
+            // wait loops, graphcompute.tr.cu:163-165)
+            if (lc->load() == 0) return false;
+            if (be) be->fetch_sub(1);
+            while (lc->load() != 0) std::this_thread::yield();
+            if (be) be->fetch_add(1);
+            return false;
+        };
+        env.inject_iteration = inject_iteration; env.inject_kernel = inject_kernel; env.inject_claim = inject_claim;
+        return graph_compute->compute(stream, dpStop ? &env : nullptr);
+    }
     model->set_poll_every(poll_every);
     if (use_program) return model->launch_program(stream, true, inject_kernel, inject_claim);
     RETURN_STATUS(reset_counters(stream));
@@ -202,6 +269,7 @@ void BLPExecutor::clear() {
 
 // reference executor.cpp:269-278
 Status BLPExecutor::getStopPoint(GPUstream stream) {
+    if (graph_compute) { stopIndex = -1; return Status::Succ; }  // the workload's loop resumes itself
     CUDA_RETURN_STATUS(gp_memcpy_d2h_async(stop_host, dpStopIndex, sizeof(int), stream));
     CUDA_RETURN_STATUS(gp_stream_sync(stream));
     stopIndex = *stop_host;
@@ -214,7 +282,7 @@ Status BLPExecutor::getStopPoint(GPUstream stream) {
 // the one at the stop index continues from its counter, later ones start from zero claims.
 // Always launch-by-launch, never through the captured graph.
 Status BLPExecutor::resume(GPUstream stream) {
-    if (!running) return Status::Succ;
+    if (!running || graph_compute) return Status::Succ;
     RETURN_STATUS(getStopPoint(stream));
     if (stopIndex == -1) return Status::Succ;
     // the program continues from its own per-layer counters; per-kernel mode relaunches one by one
@@ -225,12 +293,14 @@ Status BLPExecutor::resume(GPUstream stream) {
 }
 
 Status BLPExecutor::reset_counters(GPUstream stream) {
+    if (graph_compute) return Status::Succ;
     CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride, stream));
     if (ckpt) CUDA_RETURN_STATUS(gp_ckpt_reset_async(ckpt, stream));  // a fresh run has no tile to continue
     return Status::Succ;
 }
 
 Status BLPExecutor::read_counters(std::vector<int> &out) {
+    if (graph_compute) { out.clear(); return Status::Succ; }
     if (use_program) {
         std::vector<int> done;
         int error = 0;

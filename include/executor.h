@@ -3,15 +3,16 @@
 //
 // Interface of the reference's include/executor.h:14-84: same class names, method names,
 // argument meaning, public data members (BLPExecutor::dpStop, BLPExecutor::running) and Status
-// results.  Workload names select natively built graphs; the reference's graph-analytics and
-// miniWeather workloads ("cc", "bfs", "pagerank", "sssp", "miniweather") are not part of this
-// build and init() answers Status::NotFound for them.
+// results.  Workload names select natively built models ("resnet152", "bert", "miniweather", ...)
+// or one of the graph workloads ("cc", "bfs", "pagerank", "sssp"), which run a host loop of their
+// own inside execute() as in the reference (src/executor.cpp:125-130, :226-228).
 #pragma once
 #include <atomic>
 #include <memory>
 #include <string>
 #include <vector>
 #include "model.h"
+#include "workloads/graphcompute.h"
 
 namespace foo {
 
@@ -48,6 +49,8 @@ public:
     std::shared_ptr<Model> get_model() const { return model; }
     bool uses_graph() const { return use_cuda_graph; }
     bool uses_program() const { return use_program; }
+    // the graph workload behind a "cc" / "bfs" / "pagerank" / "sssp" executor (else null)
+    GraphCompute::Workload *graph_workload() const { return graph_compute.get(); }
 
 protected:
     std::shared_ptr<Model> model;
@@ -56,6 +59,10 @@ protected:
     bool use_program = false;     // ... and it is the persistent program
     GPUgraphExec graph_exec = nullptr;
     std::string graph_path;
+    std::unique_ptr<GraphCompute::Workload> graph_compute;
+    // "cc@n=..,deg=..,seed=.." builds a seeded random graph; set_graph_path() (or
+    // $GPREEMPT_GRAPH_PATH) names <base> of <base>.col/.dst/.val files instead
+    Status init_graph(const std::string &kind, const std::string &options);
 };
 
 class BaseExecutor : public Executor {
@@ -87,6 +94,8 @@ public:
     // Arms deterministic preemption: the workgroup whose claim on kernel `kernel` returns
     // `claim` raises the flag itself.  Applies to the next execute()/resume(); -1 disarms.
     void inject_preempt(int kernel, int claim) { inject_kernel = kernel; inject_claim = claim; }
+    // graph workloads: the same hook for iteration `iteration` of the host loop (-1 = set-up kernels)
+    void inject_preempt_graph(int iteration, int kernel, int claim) { inject_iteration = iteration; inject_kernel = kernel; inject_claim = claim; }
     Status read_counters(std::vector<int> &out);
     // Zeroes every tile counter on `stream` (what execute() does first), for callers that
     // launch kernel by kernel.
@@ -118,7 +127,7 @@ private:
     void *left_dev = nullptr;
     GPUdeviceptr ckpt = nullptr;         // owned: checkpoint workspace of long GEMM tiles, or null
     size_t ckpt_bytes = 0;
-    int inject_kernel = -1, inject_claim = -1;
+    int inject_kernel = -1, inject_claim = -1, inject_iteration = -2;
     std::atomic<int> *lc_tasks = nullptr;
     std::atomic<int> *be_tasks = nullptr;
 };

@@ -48,6 +48,21 @@ int gpx_kernel_info(gpx_executor e, size_t idx, char *name, size_t name_len, dou
                     int *total_blocks, int *grid);
 int gpx_read_storage(gpx_executor e, const char *key, void *out, size_t len); /* blocking Model::get */
 
+/* Graph workloads ("cc", "bfs", "pagerank", "sssp"; GraphCompute classes of the reference's
+ * include/workloads/graphcompute.h).  info = {vertices, edges, iterations of the last execute,
+ * preemptions so far, kernels launched so far}; result keys: "comp" (u64 per vertex), "label" (u32),
+ * "value" (f32), "cost" (u32).  gpx_set_lc_tasks sets the count of active latency-critical tasks
+ * that the executor's loop waits on when it has been stopped (BLPExecutor::set_lc_be_tasks is
+ * called with counters the handle owns). */
+int gpx_graph_info(gpx_executor e, unsigned long long info[5]);
+size_t gpx_graph_result_bytes(gpx_executor e, const char *key);
+int gpx_graph_result(gpx_executor e, const char *key, void *out, size_t len);
+int gpx_graph_inject_preempt(gpx_executor e, int iteration, int kernel, int claim); /* BLPExecutor::inject_preempt_graph */
+int gpx_set_lc_tasks(gpx_executor e, int n);
+int gpx_set_graph_path(gpx_executor e, const char *base);           /* Executor::set_graph_path (before gpx_init) */
+/* Writes a seeded random graph as <base>.col / .dst / .val in the reference's file format. */
+int gpx_write_synthetic_graph(const char *base, unsigned long long vertices, unsigned degree, unsigned long long seed);
+
 /* "miniweather" workload only: domain mass and total energy of the current state
  * (SciComputeBlp::reductions, reference src/workloads/miniweather.tr.cu:906-932); blocking. */
 int gpx_miniweather_reductions(gpx_executor e, double *mass, double *te);

@@ -279,6 +279,39 @@ typedef struct gp_miniweather_params {
 } gp_miniweather_params;
 int gp_launch_miniweather(const gp_miniweather_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
 
+/* One kernel of the graph workloads over a CSR graph (vertex_list: vertex_count+1 offsets,
+ * edge_list: neighbour ids, both 64-bit as in the reference's files; weight_list: 32-bit edge
+ * weights for SSSP).  Replaces the kernels of src/workloads/graphcompute.tr.cu: cc_kernel_coalesce
+ * :59-127, bfs_kernel_coalesce :190-241, pr_initialize :298-335, pr_kernel_coalesce :338-384,
+ * pr_update :386-425, sssp_kernel_coalesce :511-561, sssp_update :564-603.
+ *   BFS_STEP     vertices with label == level give label level+1 to unlabelled (0xFFFFFFFF) neighbours
+ *   CC_STEP      active vertices exchange component labels with their neighbours (smaller wins);
+ *                the end that changed is marked in next_active
+ *   PR_INIT      value = 1-alpha, delta = (1-alpha)*alpha/degree, residual = 0, active = 1
+ *   PR_PUSH      active vertices add delta to the residual of every neighbour, then go inactive
+ *   PR_UPDATE    residual > tolerance: value += residual, delta = residual*alpha/degree, residual = 0, active
+ *   SSSP_RELAX   active vertices offer new_cost[v] + weight to every neighbour (atomic min), then go inactive
+ *   SSSP_UPDATE  new_cost < cost: cost = new_cost, active
+ * *changed is set to 1 by any kernel that changed something (the host clears it). */
+enum gp_graph_kernel { GP_GRAPH_BFS_STEP = 0, GP_GRAPH_CC_STEP = 1, GP_GRAPH_PR_INIT = 2, GP_GRAPH_PR_PUSH = 3,
+                       GP_GRAPH_PR_UPDATE = 4, GP_GRAPH_SSSP_RELAX = 5, GP_GRAPH_SSSP_UPDATE = 6 };
+typedef struct gp_graph_params {
+    int kernel;
+    unsigned int level;                      /* BFS */
+    unsigned long long vertex_count;
+    const unsigned long long *vertex_list;
+    const unsigned long long *edge_list;
+    const unsigned int *weight_list;         /* SSSP */
+    unsigned int *label;                     /* BFS: level per vertex */
+    unsigned char *active, *next_active;     /* CC: current / next frontier; PageRank, SSSP: active */
+    unsigned long long *comp;                /* CC: component label per vertex */
+    float *delta, *residual, *value;         /* PageRank */
+    float alpha, tolerance;
+    unsigned int *cost, *new_cost;           /* SSSP */
+    unsigned int *changed;
+} gp_graph_params;
+int gp_launch_graph(const gp_graph_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+
 /* out[t,:] = tok[ids[t],:] + pos[t % seq,:] (+ seg[0,:]); ids are int64 (the reference feeds
  * BERT int64 token ids, src/tests/test-dnn.cpp:21-23). */
 typedef struct gp_embed_params {

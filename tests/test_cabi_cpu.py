@@ -41,15 +41,15 @@ def test_struct_sizes_match_header():
     import subprocess
     import tempfile
     from gpreempt_amd import capi
-    src = '#include <stdio.h>\n#include "gpreempt_hip.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",' \
+    src = '#include <stdio.h>\n#include "gpreempt_hip.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu %zu\\n",' \
           'sizeof(gp_preempt_ctx),sizeof(gp_launch_info),sizeof(gp_gemm_params),sizeof(gp_conv_params),sizeof(gp_layout_params),' \
-          'sizeof(gp_pool_params),sizeof(gp_eltwise_params),sizeof(gp_softmax_params),sizeof(gp_layernorm_params),sizeof(gp_embed_params),sizeof(gp_attention_params),sizeof(gp_miniweather_params));}'
+          'sizeof(gp_pool_params),sizeof(gp_eltwise_params),sizeof(gp_softmax_params),sizeof(gp_layernorm_params),sizeof(gp_embed_params),sizeof(gp_attention_params),sizeof(gp_miniweather_params),sizeof(gp_graph_params));}'
     with tempfile.TemporaryDirectory() as d:
         open(os.path.join(d, "s.c"), "w").write(src)
         subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), os.path.join(d, "s.c"), "-o", os.path.join(d, "s")])
         sizes = [int(v) for v in subprocess.check_output([os.path.join(d, "s")]).split()]
     mirrors = [capi.PreemptCtx, capi.LaunchInfo, capi.GemmParams, capi.ConvParams, capi.LayoutParams, capi.PoolParams,
-               capi.EltwiseParams, capi.SoftmaxParams, capi.LayernormParams, capi.EmbedParams, capi.AttentionParams, capi.MiniweatherParams]
+               capi.EltwiseParams, capi.SoftmaxParams, capi.LayernormParams, capi.EmbedParams, capi.AttentionParams, capi.MiniweatherParams, capi.GraphParams]
     assert sizes == [C.sizeof(m) for m in mirrors]
 
 
