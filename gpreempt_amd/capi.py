@@ -86,7 +86,7 @@ class MiniweatherParams(C.Structure):
 class GraphParams(C.Structure):
     _fields_ = [("kernel", C.c_int), ("level", C.c_uint), ("vertex_count", C.c_ulonglong), ("vertex_list", vp), ("edge_list", vp),
                 ("weight_list", vp), ("label", vp), ("active", vp), ("next_active", vp), ("comp", vp), ("delta", vp), ("residual", vp),
-                ("value", vp), ("alpha", C.c_float), ("tolerance", C.c_float), ("cost", vp), ("new_cost", vp), ("changed", vp)]
+                ("value", vp), ("alpha", C.c_float), ("tolerance", C.c_float), ("cost", vp), ("new_cost", vp), ("changed", vp), ("lanes_per_vertex", C.c_int)]
 
 
 class EmbedParams(C.Structure):

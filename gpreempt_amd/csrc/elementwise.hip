@@ -227,23 +227,27 @@ extern "C" int gp_launch_miniweather(const gp_miniweather_params *p, const gp_pr
 }
 extern "C" int gp_launch_graph(const gp_graph_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     GP_REQUIRE(p && p->vertex_list, "null graph params");
-    GP_REQUIRE(p->kernel >= GP_GRAPH_BFS_STEP && p->kernel <= GP_GRAPH_SSSP_UPDATE, "graph kernel %d", p->kernel);
+    GP_REQUIRE(p->kernel >= GP_GRAPH_BFS_STEP && p->kernel <= GP_GRAPH_CC_INIT, "graph kernel %d", p->kernel);
     GP_REQUIRE(p->vertex_count > 0 && p->vertex_count < (1ULL << 32), "graph: vertex count out of range");
-    GP_REQUIRE(p->changed || p->kernel == GP_GRAPH_PR_INIT || p->kernel == GP_GRAPH_PR_PUSH || p->kernel == GP_GRAPH_SSSP_RELAX, "graph: changed word missing");
+    GP_REQUIRE(p->changed || p->kernel == GP_GRAPH_CC_INIT || p->kernel == GP_GRAPH_PR_INIT || p->kernel == GP_GRAPH_PR_PUSH || p->kernel == GP_GRAPH_SSSP_RELAX, "graph: changed word missing");
     GP_REQUIRE(!graph_kernel_is_edge_parallel(p->kernel) || p->edge_list, "graph: edge list missing");
     switch (p->kernel) {
         case GP_GRAPH_BFS_STEP: GP_REQUIRE(p->label, "bfs: label missing"); break;
-        case GP_GRAPH_CC_STEP: GP_REQUIRE(p->active && p->next_active && p->comp, "cc: operands missing"); break;
+        case GP_GRAPH_CC_STEP: case GP_GRAPH_CC_INIT: GP_REQUIRE(p->active && p->next_active && p->comp, "cc: operands missing"); break;
         case GP_GRAPH_PR_INIT: case GP_GRAPH_PR_PUSH: case GP_GRAPH_PR_UPDATE:
             GP_REQUIRE(p->active && p->delta && p->residual && p->value, "pagerank: operands missing"); break;
         case GP_GRAPH_SSSP_RELAX: GP_REQUIRE(p->weight_list && p->active && p->new_cost, "sssp: operands missing"); break;
         case GP_GRAPH_SSSP_UPDATE: GP_REQUIRE(p->active && p->cost && p->new_cost, "sssp: operands missing"); break;
     }
-    const int tiles = (int)graph_kernel_tiles(p->kernel, p->vertex_count);
-    switch (p->kernel) {
-#define GP_GR(K) case K: return launch_tiles(graph_kernel<K>, tiles, 1, ctx, s, info, *p);
-        GP_GR(GP_GRAPH_BFS_STEP) GP_GR(GP_GRAPH_CC_STEP) GP_GR(GP_GRAPH_PR_INIT) GP_GR(GP_GRAPH_PR_PUSH)
-        GP_GR(GP_GRAPH_PR_UPDATE) GP_GR(GP_GRAPH_SSSP_RELAX) GP_GR(GP_GRAPH_SSSP_UPDATE)
+    GP_REQUIRE(p->lanes_per_vertex == 0 || p->lanes_per_vertex == 16 || p->lanes_per_vertex == 32 || p->lanes_per_vertex == 64, "graph: lanes_per_vertex must be 0, 16, 32 or 64");
+    const int lanes = graph_kernel_is_edge_parallel(p->kernel) ? graph_lanes(p->lanes_per_vertex) : 64;
+    const int tiles = (int)graph_kernel_tiles(p->kernel, p->vertex_count, lanes);
+    switch (p->kernel * 100 + lanes) {
+#define GP_GR(K, L) case K * 100 + L: return launch_tiles(graph_kernel<K, L>, tiles, 1, ctx, s, info, *p);
+#define GP_GR_EDGE(K) GP_GR(K, 16) GP_GR(K, 32) GP_GR(K, 64)
+        GP_GR_EDGE(GP_GRAPH_BFS_STEP) GP_GR_EDGE(GP_GRAPH_CC_STEP) GP_GR_EDGE(GP_GRAPH_PR_PUSH) GP_GR_EDGE(GP_GRAPH_SSSP_RELAX)
+        GP_GR(GP_GRAPH_PR_INIT, 64) GP_GR(GP_GRAPH_PR_UPDATE, 64) GP_GR(GP_GRAPH_SSSP_UPDATE, 64) GP_GR(GP_GRAPH_CC_INIT, 64)
+#undef GP_GR_EDGE
 #undef GP_GR
     }
     return GP_OUTOFRANGE;

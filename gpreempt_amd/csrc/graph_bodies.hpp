@@ -4,10 +4,11 @@
 // bfs_kernel_coalesce :218-241, pr_initialize :327-335, pr_kernel_coalesce :367-384, pr_update
 // :416-425, sssp_kernel_coalesce :540-561, sssp_update :592-603; derived from EMOGI).
 //
-// Edge-parallel kernels give one vertex to one wavefront: its 64 lanes walk the vertex's
-// neighbour list from the 128-byte boundary at or below its first edge, so every wave access is
-// a run of whole cache lines (the reference does the same with 32-lane warps).  A tile is 256
-// threads = 4 vertices.  Vertex-parallel kernels give one vertex to one lane, 256 per tile.
+// Edge-parallel kernels give one vertex to a group of 16, 32 or 64 lanes of a wavefront (the
+// caller picks the width nearest the average degree; the reference always uses a 32-lane warp):
+// the group walks the vertex's neighbour list from the 128-byte boundary at or below its first
+// edge, so every access of a group is a run of whole cache lines.  A tile is 256 threads = 4 to
+// 16 vertices.  Vertex-parallel kernels give one vertex to one lane, 256 per tile.
 //
 // The reference wraps these kernels by hand with a reduced dispatcher (no stop index, no kernel
 // id) and a host loop of `goto resume`; here they run under the same dispatcher as every other
@@ -28,18 +29,23 @@ constexpr unsigned int GR_INF = 0xFFFFFFFFu;
 __host__ __device__ inline bool graph_kernel_is_edge_parallel(int k) {
     return k == GP_GRAPH_BFS_STEP || k == GP_GRAPH_CC_STEP || k == GP_GRAPH_PR_PUSH || k == GP_GRAPH_SSSP_RELAX;
 }
-__host__ __device__ inline long graph_kernel_tiles(int k, unsigned long long vertex_count) {
-    const unsigned long long per_tile = graph_kernel_is_edge_parallel(k) ? GR_WAVES : GR_TILE;
+__host__ __device__ inline int graph_lanes(int lanes_per_vertex) { return lanes_per_vertex == 16 || lanes_per_vertex == 32 ? lanes_per_vertex : 64; }
+__host__ __device__ inline long graph_kernel_tiles(int k, unsigned long long vertex_count, int lanes) {
+    const unsigned long long per_tile = graph_kernel_is_edge_parallel(k) ? GR_TILE / lanes : GR_TILE;
     return (long)((vertex_count + per_tile - 1) / per_tile);
 }
 
-template <int KIND>
+template <int KIND, int LANES>
 __device__ __forceinline__ void graph_tile(const gp_graph_params &p, TileIdx t) {
     typedef unsigned long long u64;
-    if constexpr (KIND == GP_GRAPH_PR_INIT || KIND == GP_GRAPH_PR_UPDATE || KIND == GP_GRAPH_SSSP_UPDATE) {
+    if constexpr (KIND == GP_GRAPH_PR_INIT || KIND == GP_GRAPH_PR_UPDATE || KIND == GP_GRAPH_SSSP_UPDATE || KIND == GP_GRAPH_CC_INIT) {
         const u64 v = (u64)t.x * GR_TILE + threadIdx.x;
         if (v >= p.vertex_count) return;
-        if constexpr (KIND == GP_GRAPH_PR_INIT) {
+        if constexpr (KIND == GP_GRAPH_CC_INIT) {  // CC::compute's upload of 0..n-1 and its two memsets (graphcompute.tr.cu:143-148)
+            p.comp[v] = v;
+            p.active[v] = 1;
+            p.next_active[v] = 0;
+        } else if constexpr (KIND == GP_GRAPH_PR_INIT) {
             const u64 deg = p.vertex_list[v + 1] - p.vertex_list[v];
             p.value[v] = 1.0f - p.alpha;
             p.delta[v] = deg ? (1.0f - p.alpha) * p.alpha / (float)deg : 0.f;  // a sink has nobody to push to
@@ -64,8 +70,8 @@ __device__ __forceinline__ void graph_tile(const gp_graph_params &p, TileIdx t) 
             }
         }
     } else {
-        const u64 v = (u64)t.x * GR_WAVES + (threadIdx.x >> 6);
-        const unsigned lane = threadIdx.x & 63;
+        const u64 v = (u64)t.x * (GR_TILE / LANES) + threadIdx.x / LANES;
+        const unsigned lane = threadIdx.x % LANES;
         if (v >= p.vertex_count) return;
         if constexpr (KIND == GP_GRAPH_BFS_STEP) {
             if (p.label[v] != p.level) return;
@@ -75,7 +81,7 @@ __device__ __forceinline__ void graph_tile(const gp_graph_params &p, TileIdx t) 
         const u64 start = p.vertex_list[v], end = p.vertex_list[v + 1];
         const u64 from = start & GR_ALIGN;
         if constexpr (KIND == GP_GRAPH_BFS_STEP) {
-            for (u64 i = from + lane; i < end; i += 64) {
+            for (u64 i = from + lane; i < end; i += LANES) {
                 if (i < start) continue;
                 const u64 next = p.edge_list[i];
                 if (p.label[next] == GR_INF) {
@@ -84,7 +90,7 @@ __device__ __forceinline__ void graph_tile(const gp_graph_params &p, TileIdx t) 
                 }
             }
         } else if constexpr (KIND == GP_GRAPH_CC_STEP) {
-            for (u64 i = from + lane; i < end; i += 64) {
+            for (u64 i = from + lane; i < end; i += LANES) {
                 if (i < start) continue;
                 const u64 comp_src = p.comp[v];
                 const u64 next = p.edge_list[i];
@@ -100,14 +106,14 @@ __device__ __forceinline__ void graph_tile(const gp_graph_params &p, TileIdx t) 
             }
         } else if constexpr (KIND == GP_GRAPH_PR_PUSH) {
             const float d = p.delta[v];
-            for (u64 i = from + lane; i < end; i += 64) {
+            for (u64 i = from + lane; i < end; i += LANES) {
                 if (i < start) continue;
                 atomicAdd(&p.residual[p.edge_list[i]], d);
             }
             if (lane == 0) p.active[v] = 0;
         } else {  // GP_GRAPH_SSSP_RELAX
             const unsigned int c = p.new_cost[v];
-            for (u64 i = from + lane; i < end; i += 64) {
+            for (u64 i = from + lane; i < end; i += LANES) {
                 if (i < start) continue;
                 const u64 next = p.edge_list[i];
                 const unsigned int via = c + p.weight_list[i];
@@ -118,9 +124,9 @@ __device__ __forceinline__ void graph_tile(const gp_graph_params &p, TileIdx t) 
     }
 }
 
-template <int KIND>
+template <int KIND, int LANES>
 __global__ __launch_bounds__(GR_TILE) void graph_kernel(gp_graph_params p, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { graph_tile<KIND>(p, t); });
+    tile_loop(blp, [&](TileIdx t) { graph_tile<KIND, LANES>(p, t); });
 }
 
 }  // namespace gp

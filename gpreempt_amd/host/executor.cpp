@@ -237,7 +237,8 @@ Status BLPExecutor::execute(GPUstream stream) {
         env.flag = dpStop; env.stop_index = dpStopIndex; env.executed = executed;
         env.counter_groups = kCounterGroups; env.counter_stride = kCounterStride; env.poll_every = poll_every;
         std::atomic<int> *lc = lc_tasks, *be = be_tasks;
-        if (lc) env.higher_priority_active = [lc, be]() {
+        if (wait_for_turn) env.higher_priority_active = [this]() { wait_for_turn(); return false; };
+        else if (lc) env.higher_priority_active = [lc, be]() {
             // waits here while a latency-critical task is active; meanwhile this workload is not
             // counted as running (the be_tasks.fetch_sub / fetch_add pair around the reference's
             // wait loops, graphcompute.tr.cu:163-165)

@@ -113,6 +113,9 @@ std::unique_ptr<Workload> Workload::create(const std::string &kind, const CsrGra
     w->kind_ = kind;
     w->n_ = g.vertex_count;
     w->m_ = g.edge_count;
+    // lanes per neighbour list: the width nearest the average degree keeps most lanes busy
+    const double avg_degree = (double)g.edge_count / (double)g.vertex_count;
+    w->lanes_ = avg_degree <= 24 ? 16 : avg_degree <= 48 ? 32 : 64;
     const size_t n = g.vertex_count;
     auto dev = [](GPUdeviceptr *p, size_t bytes) { return gp_malloc(p, bytes ? bytes : 4) == 0; };
     auto up = [&](GPUdeviceptr *p, const void *src, size_t bytes) { return dev(p, bytes) && (bytes == 0 || gp_memcpy_h2d(*p, src, bytes) == 0); };
@@ -121,8 +124,6 @@ std::unique_ptr<Workload> Workload::create(const std::string &kind, const CsrGra
     if (kind == "bfs") ok = ok && dev(&w->label_, n * 4);
     if (kind == "cc") {
         ok = ok && dev(&w->comp_, n * 8) && dev(&w->active_, round4(n)) && dev(&w->next_active_, round4(n));
-        w->identity_.resize(n);
-        for (size_t i = 0; i < n; ++i) w->identity_[i] = i;
     }
     if (kind == "pagerank") ok = ok && dev(&w->active_, round4(n)) && dev(&w->delta_, n * 4) && dev(&w->residual_, n * 4) && dev(&w->value_, n * 4);
     if (kind == "sssp")
@@ -150,11 +151,6 @@ Status Workload::begin(GPUstream stream) {
         GC_CHECK(gp_stream_sync(stream));
         GC_CHECK(gp_memcpy_h2d(label_, &zero, 4));  // source = vertex 0 (graphcompute.tr.cu:255)
         level_ = 0;
-    } else if (kind_ == "cc") {
-        GC_CHECK(gp_fill32_async(active_, 0x01010101u, round4(n) / 4, stream));
-        GC_CHECK(gp_fill32_async(next_active_, 0, round4(n) / 4, stream));
-        GC_CHECK(gp_stream_sync(stream));
-        GC_CHECK(gp_memcpy_h2d(comp_, identity_.data(), n * 8));
     } else if (kind_ == "sssp") {
         GC_CHECK(gp_fill32_async(cost_, 0xFFFFFFFFu, n, stream));
         GC_CHECK(gp_fill32_async(new_cost_, 0xFFFFFFFFu, n, stream));
@@ -194,6 +190,7 @@ Status Workload::run_kernels(const std::vector<int> &kernels, GPUstream stream, 
             p.alpha = 0.85f; p.tolerance = 0.001f;  // graphcompute.h:83-84
             p.cost = (unsigned int *)cost_; p.new_cost = (unsigned int *)new_cost_;
             p.changed = (unsigned int *)changed_;
+            p.lanes_per_vertex = lanes_;
             if (env) {
                 gp_preempt_ctx ctx;
                 std::memset(&ctx, 0, sizeof(ctx));
@@ -240,7 +237,12 @@ Status Workload::compute(GPUstream stream, const PreemptEnv *env) {
     std::vector<int> loop;
     int max_iter = 1 << 30;
     if (kind_ == "bfs") loop = {GP_GRAPH_BFS_STEP};
-    else if (kind_ == "cc") loop = {GP_GRAPH_CC_STEP};
+    else if (kind_ == "cc") {
+        loop = {GP_GRAPH_CC_STEP};
+        // labels and frontier are set up by a kernel (the reference uploads 8 bytes per vertex
+        // from the host on every run, graphcompute.tr.cu:143-146)
+        RETURN_STATUS(run_kernels({GP_GRAPH_CC_INIT}, stream, env, -1, &changed));
+    }
     else if (kind_ == "sssp") loop = {GP_GRAPH_SSSP_RELAX, GP_GRAPH_SSSP_UPDATE};
     else {
         loop = {GP_GRAPH_PR_PUSH, GP_GRAPH_PR_UPDATE};

@@ -239,7 +239,7 @@ void fill_input(Tenant &t) {
     numeric::Rng rng(0xDA7A + std::hash<std::string>()(t.id) % 1000);
     auto m = t.ex->get_model();
     size_t idx = 0;
-    if (m->find_storage_idx("data", idx) != Status::Succ) return;  // a workload without input (miniweather)
+    if (!m || m->find_storage_idx("data", idx) != Status::Succ) return;  // a workload without input (miniweather)
     const std::string &st = m->get_storage_info(idx).stype;
     if (st == "int64") { int64_t *p = (int64_t *)t.input; for (size_t i = 0; i < t.input_size / 8; ++i) p[i] = (int64_t)(rng.next() % 30522); }
     else if (st == "float32") { float *p = (float *)t.input; for (size_t i = 0; i < t.input_size / 4; ++i) p[i] = rng.normal(); }
@@ -400,6 +400,25 @@ Status infer(Tenant &t, Shared &sh) {
     if (!t.blp) {
         st = t.ex->execute(t.stream);
         if (st == Status::Succ) st = drain(t.stream);
+    } else if (t.ex->graph_workload()) {
+        // graph workloads drive their own loop inside execute() (graphcompute.tr.cu:142-174);
+        // when stopped they come back here through wait_for_turn
+        while (sh.active_above(p) > 0) spin_pause();
+        t.blp->wait_for_turn = [&t, &sh, p]() {
+            int64_t drained = now_ns();
+            sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
+            int64_t raised = sh.domain->raised_ns(p);
+            if (sh.active_above(p) > 0 && raised > 0 && drained >= raised) {
+                std::lock_guard<std::mutex> g(sh.stats_mu);
+                sh.preempt_latency.add((drained - raised) / 1e3);
+            }
+            while (sh.active_above(p) > 0) spin_pause();
+            sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
+            ++t.preemptions;
+        };
+        sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
+        st = t.blp->execute(t.stream);
+        sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
     } else if (is_chunked(pol)) {
         while (sh.active_above(p) > 0) spin_pause();
         st = infer_chunked(t, sh, p);

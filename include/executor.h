@@ -8,6 +8,7 @@
 // own inside execute() as in the reference (src/executor.cpp:125-130, :226-228).
 #pragma once
 #include <atomic>
+#include <functional>
 #include <memory>
 #include <string>
 #include <vector>
@@ -117,6 +118,10 @@ public:
     // How often kernels read *dpStop: the claim numbered c reads it when c % poll_every == 0
     // (a power of two; 0 = the device layer's default, 8).  Use 1 when dpStop is device memory.
     int poll_every = 0;
+    // Graph workloads: called by the workload's loop when it has been stopped; returns when the
+    // workload may go back to the GPU.  Unset: the loop waits for *lc_tasks == 0 as in the
+    // reference (set_lc_be_tasks).
+    std::function<void()> wait_for_turn;
 
 private:
     GPUdeviceptr dpStopIndex = nullptr;  // owned

@@ -287,6 +287,7 @@ int gp_launch_miniweather(const gp_miniweather_params *p, const gp_preempt_ctx *
  *   BFS_STEP     vertices with label == level give label level+1 to unlabelled (0xFFFFFFFF) neighbours
  *   CC_STEP      active vertices exchange component labels with their neighbours (smaller wins);
  *                the end that changed is marked in next_active
+ *   CC_INIT      comp = own vertex id, active = 1, next_active = 0
  *   PR_INIT      value = 1-alpha, delta = (1-alpha)*alpha/degree, residual = 0, active = 1
  *   PR_PUSH      active vertices add delta to the residual of every neighbour, then go inactive
  *   PR_UPDATE    residual > tolerance: value += residual, delta = residual*alpha/degree, residual = 0, active
@@ -294,7 +295,7 @@ int gp_launch_miniweather(const gp_miniweather_params *p, const gp_preempt_ctx *
  *   SSSP_UPDATE  new_cost < cost: cost = new_cost, active
  * *changed is set to 1 by any kernel that changed something (the host clears it). */
 enum gp_graph_kernel { GP_GRAPH_BFS_STEP = 0, GP_GRAPH_CC_STEP = 1, GP_GRAPH_PR_INIT = 2, GP_GRAPH_PR_PUSH = 3,
-                       GP_GRAPH_PR_UPDATE = 4, GP_GRAPH_SSSP_RELAX = 5, GP_GRAPH_SSSP_UPDATE = 6 };
+                       GP_GRAPH_PR_UPDATE = 4, GP_GRAPH_SSSP_RELAX = 5, GP_GRAPH_SSSP_UPDATE = 6, GP_GRAPH_CC_INIT = 7 };
 typedef struct gp_graph_params {
     int kernel;
     unsigned int level;                      /* BFS */
@@ -309,6 +310,7 @@ typedef struct gp_graph_params {
     float alpha, tolerance;
     unsigned int *cost, *new_cost;           /* SSSP */
     unsigned int *changed;
+    int lanes_per_vertex;                    /* edge-parallel kernels: 16, 32 or 64 lanes walk one neighbour list (0 = 64); pick ~ the average degree */
 } gp_graph_params;
 int gp_launch_graph(const gp_graph_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
 

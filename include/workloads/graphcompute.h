@@ -74,6 +74,7 @@ private:
     uint64_t n_ = 0, m_ = 0;
     int iterations_ = 0, preemptions_ = 0, launches_ = 0;
     uint32_t level_ = 0;
+    int lanes_ = 64;
     bool injected_ = false, flag_to_lower_ = false;  // test hook state (PreemptEnv::inject_*)
     // device arrays (owned)
     GPUdeviceptr vertex_list_ = nullptr, edge_list_ = nullptr, weight_list_ = nullptr;
@@ -81,7 +82,6 @@ private:
     GPUdeviceptr delta_ = nullptr, residual_ = nullptr, value_ = nullptr, cost_ = nullptr, new_cost_ = nullptr;
     GPUdeviceptr changed_ = nullptr;
     int *host_words_ = nullptr;  // pinned: [0] stop index, [1] changed
-    std::vector<uint64_t> identity_;
 };
 
 }  // namespace GraphCompute

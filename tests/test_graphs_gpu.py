@@ -85,10 +85,10 @@ def test_synthetic_default_and_bad_names(gp, ex_mod):
 
 
 # (iteration, kernel, claim): -1 = PageRank's set-up kernel
-INJECT = {"bfs": [(0, 0, 0), (2, 0, 900), (4, 0, 3000)],
-          "cc": [(0, 0, 2500), (1, 0, 10), (2, 0, 7000)],
-          "sssp": [(1, 0, 100), (3, 1, 60), (6, 0, 4000)],
-          "pagerank": [(-1, 0, 50), (0, 0, 3000), (1, 1, 20), (5, 0, 6000)]}
+INJECT = {"bfs": [(0, 0, 0), (2, 0, 900), (4, 0, 1500)],
+          "cc": [(-1, 0, 5), (0, 0, 1500), (1, 0, 10), (2, 0, 1800)],
+          "sssp": [(1, 0, 100), (3, 1, 60), (6, 0, 1700)],
+          "pagerank": [(-1, 0, 50), (0, 0, 1000), (1, 1, 20), (5, 0, 1600)]}
 
 
 @pytest.mark.parametrize("kind", ["bfs", "cc", "sssp", "pagerank"])
@@ -125,7 +125,7 @@ def test_pagerank_push_runs_every_tile_exactly_once(gp):
                 residual=gp.DevBuf.from_array(np.zeros(n, np.float32)), value=gp.DevBuf.from_array(np.zeros(n, np.float32)),
                 changed=gp.DevBuf.from_array(np.zeros(1, np.uint32)))
     p = gp.GraphParams(3, 0, n, bufs["vl"].ptr, bufs["el"].ptr, None, None, bufs["active"].ptr, None, None,
-                       bufs["delta"].ptr, bufs["residual"].ptr, bufs["value"].ptr, 0.85, 0.001, None, None, bufs["changed"].ptr)
+                       bufs["delta"].ptr, bufs["residual"].ptr, bufs["value"].ptr, 0.85, 0.001, None, None, bufs["changed"].ptr, 0)
     flag = gp.Flag()
     st = gp.BlpState(1, flag)
     info = gp.launch("gp_launch_graph", p, st.ctx(0, inject_at=40))
@@ -141,6 +141,29 @@ def test_pagerank_push_runs_every_tile_exactly_once(gp):
     assert st.stop_index() == -1
     assert np.array_equal(bufs["residual"].download(np_dtype=np.float32), want)
     assert not bufs["active"].download(np_dtype=np.uint8).any()
+
+
+@pytest.mark.parametrize("lanes", [16, 32, 64])
+def test_bfs_step_lane_widths(gp, graph, lanes):
+    """one BFS level through the C ABI at each lane-group width, against the oracle's frontier"""
+    _, indptr, indices, _ = graph
+    label = np.full(N, G.INF, np.uint32)
+    label[0] = 0
+    want, _ = G.bfs(indptr, indices)
+    bufs = dict(vl=gp.DevBuf.from_array(indptr.astype(np.uint64)), el=gp.DevBuf.from_array(indices.astype(np.uint64)),
+                label=gp.DevBuf.from_array(label), changed=gp.DevBuf.from_array(np.zeros(1, np.uint32)))
+    for level in range(3):
+        p = gp.GraphParams(0, level, N, bufs["vl"].ptr, bufs["el"].ptr, None, bufs["label"].ptr, None, None, None,
+                           None, None, None, 0, 0, None, None, bufs["changed"].ptr, lanes)
+        info = gp.launch("gp_launch_graph", p)
+        assert info.total_tiles == (N + 256 // lanes - 1) // (256 // lanes)
+    gp.check(gp.lib().gp_stream_sync(None))
+    got = bufs["label"].download(np_dtype=np.uint32)
+    assert np.array_equal(got[want <= 3], want[want <= 3]) and (got[want > 3] == G.INF).all()
+    p = gp.GraphParams(0, 0, N, bufs["vl"].ptr, bufs["el"].ptr, None, bufs["label"].ptr, None, None, None,
+                       None, None, None, 0, 0, None, None, bufs["changed"].ptr, 8)
+    with pytest.raises(gp.GpError):
+        gp.launch("gp_launch_graph", p)
 
 
 @pytest.mark.parametrize("kind", ["cc", "pagerank"])
