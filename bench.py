@@ -299,6 +299,45 @@ def miniweather(steps=50):
             "cpu_oracle_ms_per_execute_scaled": cpu_ms, "cpu_cores": 1}
 
 
+def graph_workloads(runs=5):
+    """The reference's graph workloads on a seeded random graph (2^20 vertices, 16.8 M directed
+    edges; the reference's dataset does not ship with it): wall time of one execute() to
+    convergence, preemptible launches; bytes = per iteration, every edge id (8 B) and its
+    endpoint's word once, an upper bound that frontier-driven iterations stay well below, so the
+    bandwidth figure is indicative only.  CPU figure: the numpy oracle on a 2^16-vertex graph of the
+    same degree, scaled by edges."""
+    import ctypes as C
+    import os
+    import tempfile
+    from gpreempt_amd import capi as gp, executor as E
+    from oracle import graphs as G
+    out = {"graph": "synthetic, 1048576 vertices, degree 8 per direction, seed 1"}
+    d = tempfile.mkdtemp()
+    small = os.path.join(d, "small")
+    E.lib().gpx_write_synthetic_graph(small.encode(), C.c_ulonglong(1 << 16), 8, C.c_ulonglong(1))
+    indptr, indices, w = G.read_graph(small, weights=True)
+    cpu = {"bfs": lambda: G.bfs(indptr, indices), "cc": lambda: G.cc(indptr, indices),
+           "sssp": lambda: G.sssp(indptr, indices, w), "pagerank": lambda: G.pagerank(indptr, indices)}
+    for kind in ("bfs", "cc", "sssp", "pagerank"):
+        ex = E.Executor(f"{kind}@n=1048576,deg=8,seed=1", blp=True)
+        ex.set_flag(gp.Flag())
+        stream = gp.Stream(1)
+        ex.execute(stream)
+        t0 = time.perf_counter()
+        for _ in range(runs):
+            ex.execute(stream)
+        dt = (time.perf_counter() - t0) / runs
+        info = ex.graph_info()
+        t0 = time.perf_counter()
+        cpu[kind]()
+        cpu_s = (time.perf_counter() - t0) * info["edges"] / len(indices)
+        out[kind] = {"ms_per_execute": dt * 1e3, "iterations": info["iterations"], "edges": info["edges"],
+                     "edge_visits_per_s_upper_bound": info["edges"] * info["iterations"] / dt,
+                     "cpu_oracle_ms_scaled": cpu_s * 1e3, "cpu_cores": 1}
+        ex.destroy()
+    return out
+
+
 def copy_calibration(mib=256, iters=10):
     """A plain device-to-device copy of known size (the runtime's copy kernel), used to scale
     the FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc runs."""
@@ -347,7 +386,7 @@ def main():
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
-    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | cpu | copycal")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal")
     ap.add_argument("--cpu-requests", type=int, default=4)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -380,6 +419,8 @@ def main():
         out["hbm_bound_ops"] = hbm_ops()
     if args.only in ("", "miniweather"):
         out["miniweather"] = miniweather()
+    if args.only in ("", "graphs"):
+        out["graph_workloads"] = graph_workloads()
     if args.only == "copycal":
         out["copy_calibration"] = copy_calibration()
     if args.only in ("", "cpu"):

@@ -8,12 +8,12 @@
 namespace gp {
 
 template <class Kernel, class Arg>
-static int launch_tiles(Kernel kern, int sx, int sy, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info, const Arg &arg, size_t lds_bytes = 0) {
+static int launch_tiles(Kernel kern, int sx, int sy, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info, const Arg &arg, size_t lds_bytes = 0, int max_batch = 16) {
     BlpArgs blp;
     int grid = 0;
     // several tiles per claim once there are far more tiles than workgroups that could hold them
     const long tiles = (long)sx * sy;
-    const int batch = (int)std::min<long>(16, std::max<long>(1, tiles / (32L * device_cus())));
+    const int batch = (int)std::min<long>(max_batch, std::max<long>(1, tiles / (32L * device_cus())));
     if (lds_bytes > 48 * 1024) GP_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     int rc = plan_launch(kern, NT, lds_bytes, sx, sy, 1, ctx, &blp, &grid, info, batch);
     if (rc) return rc;
@@ -242,8 +242,11 @@ extern "C" int gp_launch_graph(const gp_graph_params *p, const gp_preempt_ctx *c
     GP_REQUIRE(p->lanes_per_vertex == 0 || p->lanes_per_vertex == 16 || p->lanes_per_vertex == 32 || p->lanes_per_vertex == 64, "graph: lanes_per_vertex must be 0, 16, 32 or 64");
     const int lanes = graph_kernel_is_edge_parallel(p->kernel) ? graph_lanes(p->lanes_per_vertex) : 64;
     const int tiles = (int)graph_kernel_tiles(p->kernel, p->vertex_count, lanes);
+    // a tile of an edge-parallel kernel is a few hundred scattered accesses or atomics (microseconds):
+    // claims stay small so that a stop is honoured quickly
+    const int max_batch = graph_kernel_is_edge_parallel(p->kernel) ? 4 : 16;
     switch (p->kernel * 100 + lanes) {
-#define GP_GR(K, L) case K * 100 + L: return launch_tiles(graph_kernel<K, L>, tiles, 1, ctx, s, info, *p);
+#define GP_GR(K, L) case K * 100 + L: return launch_tiles(graph_kernel<K, L>, tiles, 1, ctx, s, info, *p, 0, max_batch);
 #define GP_GR_EDGE(K) GP_GR(K, 16) GP_GR(K, 32) GP_GR(K, 64)
         GP_GR_EDGE(GP_GRAPH_BFS_STEP) GP_GR_EDGE(GP_GRAPH_CC_STEP) GP_GR_EDGE(GP_GRAPH_PR_PUSH) GP_GR_EDGE(GP_GRAPH_SSSP_RELAX)
         GP_GR(GP_GRAPH_PR_INIT, 64) GP_GR(GP_GRAPH_PR_UPDATE, 64) GP_GR(GP_GRAPH_SSSP_UPDATE, 64) GP_GR(GP_GRAPH_CC_INIT, 64)

@@ -210,7 +210,13 @@ Status Workload::run_kernels(const std::vector<int> &kernels, GPUstream stream, 
         host_words_[0] = -1;
         if (env) GC_CHECK(gp_memcpy_d2h_async(&host_words_[0], env->stop_index, sizeof(int), stream));
         GC_CHECK(gp_memcpy_d2h_async(&host_words_[1], changed_, sizeof(int), stream));
-        GC_CHECK(gp_stream_sync(stream));
+        // polled, not a blocking wait: a blocked thread wakes up tens of microseconds late, which
+        // is paid once per iteration and on every preemption
+        for (;;) {
+            int idle = 0;
+            GC_CHECK(gp_stream_query(stream, &idle));
+            if (idle) break;
+        }
         const int stop = host_words_[0];
         if (!env || stop < 0) break;
         // stopped in kernel `stop`: stay off the GPU while a higher priority needs it

@@ -105,9 +105,6 @@ def test_executor_error_paths(gp, ex_mod, tmp_path):
     with pytest.raises(ex_mod.StatusError) as e:
         ex_mod.Executor("no_such_model", model_root=str(tmp_path))
     assert e.value.status == 3  # NotFound
-    with pytest.raises(ex_mod.StatusError) as e:
-        ex_mod.Executor("pagerank", model_root=str(tmp_path))  # reference workload outside this build (needs a graph dataset)
-    assert e.value.status == 3
     ex = ex_mod.Executor("toy", model_root=str(tmp_path))
     with pytest.raises(ex_mod.StatusError) as e:
         ex.set_input("data", np.zeros(8, np.float32))  # shorter than the storage: OutOfRange (model.cpp:319)

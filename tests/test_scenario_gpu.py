@@ -54,7 +54,7 @@ def test_non_preempting_policies_complete(gp, policy):
 def test_unknown_model_is_reported(gp):
     from gpreempt_amd import executor as gx
     cfg = {"time": 1.0, "policy": "wb", "tasks": [{"id": "x", "load": {"type": "continuous"},
-           "client": {"name": "x", "model_name": "pagerank", "priority": 0}}]}
+           "client": {"name": "x", "model_name": "no_such_model", "priority": 0}}]}
     buf = C.create_string_buffer(1 << 16)
     rc = gx.lib().gpx_run_scenario(json.dumps(cfg).encode(), buf, C.c_size_t(len(buf)))
     assert rc != 0
@@ -86,3 +86,20 @@ def test_pre_preemption_hints_hide_the_drain(gp):
     assert hinted["tasks"]["be"]["preemptions"] > 0
     # the drain no longer sits inside the request's GPU phase
     assert hinted["tasks"]["hp"]["inferLatency(us)"]["p50"] < plain["tasks"]["hp"]["inferLatency(us)"]["p50"] + 5.0
+
+
+def test_graph_and_stencil_tenants_under_a_latency_critical_model(gp):
+    """the reference's configs Y and Z in small: a periodic high-priority DNN over a miniWeather
+    tenant and a graph tenant, all of which must make progress and be preempted"""
+    cfg = {"time": 1.5, "policy": "wb-chunk-async", "tasks": [
+        {"id": "hp", "load": {"type": "periodic", "frequency": 200},
+         "client": {"name": "hp", "model_name": "toy", "priority": 0, "launch_mode": "launch"}},
+        {"id": "mw", "load": {"type": "continuous"},
+         "client": {"name": "mw", "model_name": "miniweather@nx=800,nz=400", "priority": 1, "launch_mode": "launch"}},
+        {"id": "cc", "load": {"type": "continuous"},
+         "client": {"name": "cc", "model_name": "cc@n=200000,deg=6,seed=2", "priority": 1, "launch_mode": "launch"}}]}
+    rep = _run_cfg(cfg)
+    t = rep["tasks"]
+    assert t["hp"]["requests"] >= 250
+    assert t["mw"]["requests"] > 50 and t["cc"]["requests"] > 50
+    assert t["mw"]["preemptions"] + t["cc"]["preemptions"] > 20
