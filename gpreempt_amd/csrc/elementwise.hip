@@ -51,7 +51,7 @@ int plan_pool2d(const gp_pool_params *p, EltPlan *out) {
     GP_REQUIRE(is_float(p->dtype), "pool dtype %d", p->dtype);
     const int vec = vec_of(p->dtype);
     GP_REQUIRE(p->N > 0 && p->H > 0 && p->W > 0 && p->C > 0 && p->C % vec == 0, "pool: C must be a positive multiple of %d", vec);
-    GP_REQUIRE(p->mode >= 0 && p->mode <= 2, "pool mode %d", p->mode);
+    GP_REQUIRE(p->mode >= 0 && p->mode <= 3, "pool mode %d", p->mode);
     GP_REQUIRE(p->in_pix_stride % vec == 0 && p->out_pix_stride % vec == 0 && p->in_pix_stride >= p->C && p->out_pix_stride >= p->C, "pool pixel strides");
     GP_REQUIRE(al16(p->in) && al16(p->out), "pool: 16-byte alignment");
     int Ho = 1, Wo = 1;

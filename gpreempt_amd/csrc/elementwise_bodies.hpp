@@ -170,7 +170,8 @@ __device__ __forceinline__ void pool_tile(const PoolArgs &a, TileIdx t) {
                 ++cnt;
             }
         }
-        if (p.mode == 1) {
+        if (p.mode == 1 || p.mode == 3) {
+            if (p.mode == 3) cnt = p.R * p.S;  // padding counts as zeros
             float inv = 1.f / (float)(cnt > 0 ? cnt : 1);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) acc[j] *= inv;

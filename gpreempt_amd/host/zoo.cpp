@@ -78,22 +78,27 @@ public:
     // conv + folded-BN bias + optional residual + activation; writes into `into` when given
     Tensor conv(const std::string &name, const Tensor &in, int cout, int k, int stride, int pad, int act,
                 const Tensor *residual = nullptr, const Tensor *into = nullptr, int cin_logical = -1, float init_gain = 1.f) {
-        int Ho = (in.H + 2 * pad - k) / stride + 1, Wo = (in.W + 2 * pad - k) / stride + 1;
+        return conv_hw(name, in, cout, k, k, stride, pad, pad, act, residual, into, cin_logical, init_gain);
+    }
+    // the same with a kh x kw filter and separate vertical / horizontal padding (Inception's 1x7 and 7x1)
+    Tensor conv_hw(const std::string &name, const Tensor &in, int cout, int kh, int kw, int stride, int ph, int pw, int act,
+                   const Tensor *residual = nullptr, const Tensor *into = nullptr, int cin_logical = -1, float init_gain = 1.f) {
+        int Ho = (in.H + 2 * ph - kh) / stride + 1, Wo = (in.W + 2 * pw - kw) / stride + 1;
         int cin = cin_logical > 0 ? cin_logical : in.C;
         ParamLayout L;
-        L.kind = ParamLayout::ConvOIHW; L.o = cout; L.i = cin; L.r = k; L.s = k; L.i_pad = in.C;
-        L.disk_elems = (size_t)cout * cin * k * k;
-        L.init = ParamLayout::InitNormal; L.init_a = init_gain * std::sqrt(2.f / (float)(cin * k * k));  // He-normal
-        size_t w = add_param(name + ".weight", (size_t)cout * k * k * in.C, L);
+        L.kind = ParamLayout::ConvOIHW; L.o = cout; L.i = cin; L.r = kh; L.s = kw; L.i_pad = in.C;
+        L.disk_elems = (size_t)cout * cin * kh * kw;
+        L.init = ParamLayout::InitNormal; L.init_a = init_gain * std::sqrt(2.f / (float)(cin * kh * kw));  // He-normal
+        size_t w = add_param(name + ".weight", (size_t)cout * kh * kw * in.C, L);
         ParamLayout LB; LB.disk_elems = cout; LB.init = ParamLayout::InitZero;
         size_t b = add_param(name + ".bias", cout, LB);
         Tensor out = into ? *into : activation(name + ".out", in.N, Ho, Wo, cout);
-        double flops = 2.0 * in.N * Ho * Wo * cout * (double)cin * k * k;
-        double bytes = es_ * ((double)in.N * in.H * in.W * cin + (double)cout * cin * k * k + cout + (double)in.N * Ho * Wo * cout * (residual ? 2 : 1));
+        double flops = 2.0 * in.N * Ho * Wo * cout * (double)cin * kh * kw;
+        double bytes = es_ * ((double)in.N * in.H * in.W * cin + (double)cout * cin * kh * kw + cout + (double)in.N * Ho * Wo * cout * (residual ? 2 : 1));
         KernelInfo &ki = add_kernel("conv2d", OpKind::Conv, {ref(in), ref(w), ref(b), residual ? ref(*residual) : none(), ref(out)}, flops, bytes);
         gp_conv_params &p = ki.p.conv;
-        p.dtype = gp_dt_; p.N = in.N; p.H = in.H; p.W = in.W; p.Cin = in.C; p.Cout = cout; p.R = k; p.S = k;
-        p.stride_h = p.stride_w = stride; p.pad_h = p.pad_w = pad;
+        p.dtype = gp_dt_; p.N = in.N; p.H = in.H; p.W = in.W; p.Cin = in.C; p.Cout = cout; p.R = kh; p.S = kw;
+        p.stride_h = p.stride_w = stride; p.pad_h = ph; p.pad_w = pw;
         p.in_pix_stride = in.ps; p.res_pix_stride = residual ? residual->ps : 0; p.out_pix_stride = out.ps; p.act = act;
         Tensor o = out; o.N = in.N; o.H = Ho; o.W = Wo; o.C = cout;
         return o;
@@ -224,6 +229,118 @@ Status build_gemm(Model &m, const Options &o, int M, int N, int K, const std::st
     gp_gemm_params &p = k.p.gemm;
     p.dtype = g.gp_dtype(); p.M = M; p.N = N; p.K = K; p.lda = K; p.ldb = K; p.b_is_nk = 1; p.ldc = N; p.alpha = 1.f; p.act = act; p.batch = 1;
     p.tile_m = p.tile_n = tile;
+    return Status::Succ;
+}
+
+// ---- Inception-v3 ------------------------------------------------------------------------------
+// The architecture of relay.testing.inception_v3 (the reference's "inception" model,
+// scripts/compile/compile.py:36-38): 299x299 input, a five-convolution stem, three A blocks
+// (35x35), a reducing B block, four C blocks (17x17, factorised 7x7), a reducing D block, two E
+// blocks (8x8), global average pool, FC 1000, softmax.  Every convolution carries a folded
+// batch-norm and a ReLU.  Branch outputs are written straight into their channel slice of the
+// block's output (no concatenation kernel); average pools count the padding, as relay's do.
+Status build_inception_v3(Model &m, const Options &o) {
+    std::string dt = o.gets("dtype", "f16");
+    if (!valid_dtype(dt)) return Status::OutOfRange;
+    GraphBuilder g(m, dt);
+    const int N = o.geti("b", 1), HW = o.geti("hw", 299), classes = o.geti("classes", 1000);
+    if (HW < 75) return Status::OutOfRange;  // below that the 8x8 stage has no pixel left
+    auto cv = [&](const std::string &n, const Tensor &in, int cout, int kh, int kw, int stride, int ph, int pw, const Tensor *into = nullptr) {
+        return g.conv_hw(n, in, cout, kh, kw, stride, ph, pw, GP_ACT_RELU, nullptr, into);
+    };
+    auto out_size = [](int h, int k, int s, int p) { return (h + 2 * p - k) / s + 1; };
+    Tensor x = g.input_nchw(N, 3, HW, HW);
+    x = g.conv_hw("conv", x, 32, 3, 3, 2, 0, 0, GP_ACT_RELU, nullptr, nullptr, 3);
+    x = cv("conv_1", x, 32, 3, 3, 1, 0, 0);
+    x = cv("conv_2", x, 64, 3, 3, 1, 1, 1);
+    x = g.pool("pool", x, 3, 2, 0, 0);
+    x = cv("conv_3", x, 80, 1, 1, 1, 0, 0);
+    x = cv("conv_4", x, 192, 3, 3, 1, 0, 0);
+    x = g.pool("pool1", x, 3, 2, 0, 0);
+    int idx = 0;
+    auto block_name = [&]() { return "mixed" + std::to_string(idx++); };
+    // A: 1x1 | 1x1 -> 5x5 | 1x1 -> 3x3 -> 3x3 | avgpool -> 1x1
+    for (int proj : {32, 64, 64}) {
+        const std::string n = block_name();
+        Tensor out = g.activation(n + ".out", N, x.H, x.W, 64 + 64 + 96 + proj);
+        Tensor s0 = GraphBuilder::slice(out, 0, 64), s1 = GraphBuilder::slice(out, 64, 64), s2 = GraphBuilder::slice(out, 128, 96), s3 = GraphBuilder::slice(out, 224, proj);
+        cv(n + ".1x1", x, 64, 1, 1, 1, 0, 0, &s0);
+        Tensor t = cv(n + ".5x5_r", x, 48, 1, 1, 1, 0, 0);
+        cv(n + ".5x5", t, 64, 5, 5, 1, 2, 2, &s1);
+        t = cv(n + ".3x3_r", x, 64, 1, 1, 1, 0, 0);
+        t = cv(n + ".3x3_1", t, 96, 3, 3, 1, 1, 1);
+        cv(n + ".3x3_2", t, 96, 3, 3, 1, 1, 1, &s2);
+        t = g.pool(n + ".pool", x, 3, 1, 1, 3);
+        cv(n + ".proj", t, proj, 1, 1, 1, 0, 0, &s3);
+        x = out;
+    }
+    {   // B: 3x3/2 | 1x1 -> 3x3 -> 3x3/2 | maxpool/2
+        const std::string n = block_name();
+        const int H = out_size(x.H, 3, 2, 0);
+        Tensor out = g.activation(n + ".out", N, H, H, 384 + 96 + x.C);
+        Tensor s0 = GraphBuilder::slice(out, 0, 384), s1 = GraphBuilder::slice(out, 384, 96), s2 = GraphBuilder::slice(out, 480, x.C);
+        cv(n + ".3x3", x, 384, 3, 3, 2, 0, 0, &s0);
+        Tensor t = cv(n + ".d3x3_r", x, 64, 1, 1, 1, 0, 0);
+        t = cv(n + ".d3x3_1", t, 96, 3, 3, 1, 1, 1);
+        cv(n + ".d3x3_2", t, 96, 3, 3, 2, 0, 0, &s1);
+        g.pool(n + ".pool", x, 3, 2, 0, 0, &s2);
+        x = out;
+    }
+    // C: 1x1 | 1x1 -> 1x7 -> 7x1 | 1x1 -> 7x1 -> 1x7 -> 7x1 -> 1x7 | avgpool -> 1x1
+    for (int c7 : {128, 160, 160, 192}) {
+        const std::string n = block_name();
+        Tensor out = g.activation(n + ".out", N, x.H, x.W, 192 * 4);
+        Tensor s0 = GraphBuilder::slice(out, 0, 192), s1 = GraphBuilder::slice(out, 192, 192), s2 = GraphBuilder::slice(out, 384, 192), s3 = GraphBuilder::slice(out, 576, 192);
+        cv(n + ".1x1", x, 192, 1, 1, 1, 0, 0, &s0);
+        Tensor t = cv(n + ".7_r", x, c7, 1, 1, 1, 0, 0);
+        t = cv(n + ".7_1", t, c7, 1, 7, 1, 0, 3);
+        cv(n + ".7_2", t, 192, 7, 1, 1, 3, 0, &s1);
+        t = cv(n + ".d7_r", x, c7, 1, 1, 1, 0, 0);
+        t = cv(n + ".d7_1", t, c7, 7, 1, 1, 3, 0);
+        t = cv(n + ".d7_2", t, c7, 1, 7, 1, 0, 3);
+        t = cv(n + ".d7_3", t, c7, 7, 1, 1, 3, 0);
+        cv(n + ".d7_4", t, 192, 1, 7, 1, 0, 3, &s2);
+        t = g.pool(n + ".pool", x, 3, 1, 1, 3);
+        cv(n + ".proj", t, 192, 1, 1, 1, 0, 0, &s3);
+        x = out;
+    }
+    {   // D: 1x1 -> 3x3/2 | 1x1 -> 1x7 -> 7x1 -> 3x3/2 | maxpool/2
+        const std::string n = block_name();
+        const int H = out_size(x.H, 3, 2, 0);
+        Tensor out = g.activation(n + ".out", N, H, H, 320 + 192 + x.C);
+        Tensor s0 = GraphBuilder::slice(out, 0, 320), s1 = GraphBuilder::slice(out, 320, 192), s2 = GraphBuilder::slice(out, 512, x.C);
+        Tensor t = cv(n + ".3x3_r", x, 192, 1, 1, 1, 0, 0);
+        cv(n + ".3x3", t, 320, 3, 3, 2, 0, 0, &s0);
+        t = cv(n + ".7x3_r", x, 192, 1, 1, 1, 0, 0);
+        t = cv(n + ".7x3_1", t, 192, 1, 7, 1, 0, 3);
+        t = cv(n + ".7x3_2", t, 192, 7, 1, 1, 3, 0);
+        cv(n + ".7x3_3", t, 192, 3, 3, 2, 0, 0, &s1);
+        g.pool(n + ".pool", x, 3, 2, 0, 0, &s2);
+        x = out;
+    }
+    // E: 1x1 | 1x1 -> {1x3, 3x1} | 1x1 -> 3x3 -> {1x3, 3x1} | pool -> 1x1 (average, then max)
+    for (int pool_mode : {3, 0}) {
+        const std::string n = block_name();
+        Tensor out = g.activation(n + ".out", N, x.H, x.W, 320 + 768 + 768 + 192);
+        Tensor s0 = GraphBuilder::slice(out, 0, 320), s1a = GraphBuilder::slice(out, 320, 384), s1b = GraphBuilder::slice(out, 704, 384);
+        Tensor s2a = GraphBuilder::slice(out, 1088, 384), s2b = GraphBuilder::slice(out, 1472, 384), s3 = GraphBuilder::slice(out, 1856, 192);
+        cv(n + ".1x1", x, 320, 1, 1, 1, 0, 0, &s0);
+        Tensor t = cv(n + ".3_r", x, 384, 1, 1, 1, 0, 0);
+        cv(n + ".3_a", t, 384, 1, 3, 1, 0, 1, &s1a);
+        cv(n + ".3_b", t, 384, 3, 1, 1, 1, 0, &s1b);
+        t = cv(n + ".d3_r", x, 448, 1, 1, 1, 0, 0);
+        t = cv(n + ".d3_1", t, 384, 3, 3, 1, 1, 1);
+        cv(n + ".d3_a", t, 384, 1, 3, 1, 0, 1, &s2a);
+        cv(n + ".d3_b", t, 384, 3, 1, 1, 1, 0, &s2b);
+        t = g.pool(n + ".pool", x, 3, 1, 1, pool_mode);
+        cv(n + ".proj", t, 192, 1, 1, 1, 0, 0, &s3);
+        x = out;
+    }
+    Tensor gap = g.pool("global_pool", x, 0, 1, 0, 2);
+    size_t logits = g.add_storage("fc1.out", (size_t)N * classes, g.stype_);
+    g.dense("fc1", gap.st, 0, N, gap.C, gap.C, classes, GP_ACT_NONE, SIZE_MAX, logits, 0, classes, 0.01f);
+    size_t heads = g.add_storage("heads", (size_t)N * classes, g.stype_);
+    g.softmax(logits, heads, N, classes, 1.f);
     return Status::Succ;
 }
 
@@ -532,10 +649,11 @@ Status zoo_build(Model &m, const std::string &workload) {
     if (n == "resnet152" || n == "resnet") return build_resnet(m, o, r152, 8, "f16");
     if (n == "vgg" || n == "vgg16") return build_vgg16(m, o);
     if (n == "densenet" || n == "densenet201") return build_densenet201(m, o);
+    if (n == "inception" || n == "inception_v3") return build_inception_v3(m, o);
     if (n == "bert") return build_bert(m, o);
     if (n == "toy") return build_toy(m, o);
     if (n == "miniweather") return build_miniweather(m, o);
-    std::fprintf(stderr, "unknown workload '%s' (known: gemm1024 gemm8192 resnet50 resnet101 resnet152 vgg16 densenet201 bert miniweather toy)\n", n.c_str());
+    std::fprintf(stderr, "unknown workload '%s' (known: gemm1024 gemm8192 resnet50 resnet101 resnet152 vgg16 densenet201 inception bert miniweather toy; graph workloads: cc bfs pagerank sssp)\n", n.c_str());
     return Status::NotFound;
 }
 

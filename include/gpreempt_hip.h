@@ -200,7 +200,8 @@ typedef struct gp_layout_params {
 int gp_launch_nchw_to_nhwc(const gp_layout_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
 
 /* Pooling on NHWC.  mode 0 = max, 1 = average (padding excluded from the count),
- * 2 = global average (R,S,stride,pad ignored; output N x 1 x 1 x C). */
+ * 2 = global average (R,S,stride,pad ignored; output N x 1 x 1 x C), 3 = average with the
+ * padding counted as zeros (divisor R*S; relay's count_include_pad, used by Inception-v3). */
 typedef struct gp_pool_params {
     int dtype;
     int N, H, W, C, R, S, stride, pad, mode;

@@ -93,6 +93,69 @@ def densenet(params, x, dt="f16", blocks=(6, 12, 48, 32), growth=32):
     return c.R(O.softmax(c.dense("classifier", gap)))
 
 
+def inception_v3(params, x, dt="f16"):
+    """Inception-v3 as relay.testing.inception_v3 lays it out: stem, 3 x A, B, 4 x C, D, 2 x E,
+    global average pool, FC, softmax; every convolution with folded batch-norm and ReLU; average
+    pools count their padding."""
+    c = _Ctx(params, dt)
+
+    def cv(name, t, stride=1, pad=0):
+        return c.conv(name, t, stride, pad, O.ACT_RELU)
+
+    x = c.R(x)
+    x = cv("conv", x, 2)
+    x = cv("conv_1", x)
+    x = cv("conv_2", x, 1, 1)
+    x = O.pool2d(x, 3, 2, 0, "max")
+    x = cv("conv_3", x)
+    x = cv("conv_4", x)
+    x = O.pool2d(x, 3, 2, 0, "max")
+    i = 0
+    for _ in range(3):
+        n = f"mixed{i}"
+        i += 1
+        b0 = cv(n + ".1x1", x)
+        b1 = cv(n + ".5x5", cv(n + ".5x5_r", x), 1, 2)
+        b2 = cv(n + ".3x3_2", cv(n + ".3x3_1", cv(n + ".3x3_r", x), 1, 1), 1, 1)
+        b3 = cv(n + ".proj", c.R(O.pool2d(x, 3, 1, 1, "avg_pad")))
+        x = np.concatenate([b0, b1, b2, b3], axis=1)
+    n = f"mixed{i}"
+    i += 1
+    b0 = cv(n + ".3x3", x, 2)
+    b1 = cv(n + ".d3x3_2", cv(n + ".d3x3_1", cv(n + ".d3x3_r", x), 1, 1), 2)
+    x = np.concatenate([b0, b1, O.pool2d(x, 3, 2, 0, "max")], axis=1)
+    for _ in range(4):
+        n = f"mixed{i}"
+        i += 1
+        b0 = cv(n + ".1x1", x)
+        b1 = cv(n + ".7_2", cv(n + ".7_1", cv(n + ".7_r", x), 1, (0, 3)), 1, (3, 0))
+        t = cv(n + ".d7_r", x)
+        t = cv(n + ".d7_1", t, 1, (3, 0))
+        t = cv(n + ".d7_2", t, 1, (0, 3))
+        t = cv(n + ".d7_3", t, 1, (3, 0))
+        b2 = cv(n + ".d7_4", t, 1, (0, 3))
+        b3 = cv(n + ".proj", c.R(O.pool2d(x, 3, 1, 1, "avg_pad")))
+        x = np.concatenate([b0, b1, b2, b3], axis=1)
+    n = f"mixed{i}"
+    i += 1
+    b0 = cv(n + ".3x3", cv(n + ".3x3_r", x), 2)
+    t = cv(n + ".7x3_2", cv(n + ".7x3_1", cv(n + ".7x3_r", x), 1, (0, 3)), 1, (3, 0))
+    b1 = cv(n + ".7x3_3", t, 2)
+    x = np.concatenate([b0, b1, O.pool2d(x, 3, 2, 0, "max")], axis=1)
+    for mode in ("avg_pad", "max"):
+        n = f"mixed{i}"
+        i += 1
+        b0 = cv(n + ".1x1", x)
+        t = cv(n + ".3_r", x)
+        b1 = np.concatenate([cv(n + ".3_a", t, 1, (0, 1)), cv(n + ".3_b", t, 1, (1, 0))], axis=1)
+        t = cv(n + ".d3_1", cv(n + ".d3_r", x), 1, 1)
+        b2 = np.concatenate([cv(n + ".d3_a", t, 1, (0, 1)), cv(n + ".d3_b", t, 1, (1, 0))], axis=1)
+        b3 = cv(n + ".proj", c.R(O.pool2d(x, 3, 1, 1, mode)))
+        x = np.concatenate([b0, b1, b2, b3], axis=1)
+    gap = c.R(O.global_avgpool(x))
+    return c.R(O.softmax(c.dense("fc1", gap)))
+
+
 def bert(params, ids, dt="f16", batch=1, seq=128, layers=12, hidden=768, heads=12, fused_attention=None):
     """BERT encoder: embeddings + LayerNorm, then `layers` post-LN transformer blocks with
     erf GELU and eps 1e-12; returns the last hidden state [batch*seq, hidden].

@@ -80,13 +80,13 @@ def conv2d(x, w, bias=None, stride=1, pad=0, residual=None, act=ACT_NONE):
 
 
 def pool2d(x, k, stride, pad, mode):
-    """mode: 'max' | 'avg' (count_include_pad False)."""
+    """mode: 'max' | 'avg' (count_include_pad False) | 'avg_pad' (padding counted as zeros)."""
     x = _f(x)
     N, Cc, H, W = x.shape
     Ho, Wo = (H + 2 * pad - k) // stride + 1, (W + 2 * pad - k) // stride + 1
     out = np.empty((N, Cc, Ho, Wo), np.float32)
     lib().orc_pool2d_nchw(*(C.c_int(v) for v in (N, Cc, H, W, k, k, stride, stride, pad, pad,
-                                                 0 if mode == "max" else 1)), _p(x), _p(out))
+                                                 {"max": 0, "avg": 1, "avg_pad": 3}[mode])), _p(x), _p(out))
     return out
 
 

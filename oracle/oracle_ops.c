@@ -146,6 +146,7 @@ void orc_pool2d_nchw(int N, int C, int H, int W, int R, int S, int sh, int sw, i
                         sum += v;
                         ++cnt;
                     }
+                if (mode == 3) cnt = R * S; /* padding counted as zeros */
                 out[((size_t)nc * Ho + ho) * Wo + wo] = (float)(mode == 0 ? best : sum / (cnt ? cnt : 1));
             }
 }

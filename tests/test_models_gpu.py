@@ -79,6 +79,17 @@ def test_densenet_matches_oracle(gp, ex_mod, tmp_path):
     assert rel_err(got, OM.densenet(params, x, "f16", (2, 4, 5, 3))) < TOL["f16"]
 
 
+def test_inception_v3_matches_oracle(gp, ex_mod, tmp_path):
+    # full widths, 107 x 107 input (the 8 x 8 stage of the 299 x 299 network becomes 1 x 1)
+    wl = "inception@b=1,hw=107"
+    ex, params = make_model(ex_mod, tmp_path, wl, "cnn", 8)
+    assert ex.kernel_num() > 100
+    x = O.round_to(np.random.default_rng(9).normal(0, 1, (1, 3, 107, 107)).astype(np.float32), "f16")
+    got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (1, 1000))
+    assert np.isfinite(got).all() and abs(got.sum() - 1) < 2e-2
+    assert rel_err(got, OM.inception_v3(params, x, "f16")) < TOL["f16"]
+
+
 @pytest.mark.parametrize("workload,kw", [
     ("bert", dict(batch=1, seq=128, layers=12)),                       # config 3's high-priority tenant, full size
     ("bert@b=2,s=48,layers=2,dtype=f32", dict(batch=2, seq=48, layers=2)),

@@ -79,7 +79,7 @@ def test_nchw_to_nhwc(gp, dt_in, dt_out):
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("cfg", [(3, 2, 1, "max"), (2, 2, 0, "max"), (2, 2, 0, "avg"), (3, 1, 1, "avg"), (7, 1, 0, "gap")])
+@pytest.mark.parametrize("cfg", [(3, 2, 1, "max"), (2, 2, 0, "max"), (2, 2, 0, "avg"), (3, 1, 1, "avg"), (3, 1, 1, "avg_pad"), (7, 1, 0, "gap")])
 def test_pool2d(gp, dt, cfg):
     k, stride, pad, mode = cfg
     rng = np.random.default_rng(k * 10 + stride)
@@ -96,7 +96,7 @@ def test_pool2d(gp, dt, cfg):
         ref = O.pool2d(x, k, stride, pad, mode)
         Ho, Wo = ref.shape[2:]
     do = gp.DevBuf(N * Ho * Wo * Cc * gp.DTYPE_SIZE[dtype])
-    p = gp.PoolParams(dtype, N, H, W, Cc, k, k, stride, pad, {"max": 0, "avg": 1, "gap": 2}[mode], di.ptr, Cc, do.ptr, Cc)
+    p = gp.PoolParams(dtype, N, H, W, Cc, k, k, stride, pad, {"max": 0, "avg": 1, "gap": 2, "avg_pad": 3}[mode], di.ptr, Cc, do.ptr, Cc)
     gp.launch("gp_launch_pool2d", p)
     sync(gp)
     got = nhwc_to_nchw(do.download(dtype, (N, Ho, Wo, Cc)))

@@ -97,6 +97,7 @@ def test_pooling_vs_torch():
     assert np.array_equal(O.pool2d(x, 2, 2, 0, "max"), F.max_pool2d(tx, 2, 2, 0).numpy())
     assert np.allclose(O.pool2d(x, 2, 2, 0, "avg"), F.avg_pool2d(tx, 2, 2, 0).numpy(), atol=1e-6)
     assert np.allclose(O.pool2d(x, 3, 1, 1, "avg"), F.avg_pool2d(tx, 3, 1, 1, count_include_pad=False).numpy(), atol=1e-6)
+    assert np.allclose(O.pool2d(x, 3, 1, 1, "avg_pad"), F.avg_pool2d(tx, 3, 1, 1, count_include_pad=True).numpy(), atol=1e-6)
     assert np.allclose(O.global_avgpool(x), x.mean(axis=(2, 3)), atol=1e-6)
     # all-negative input: padding must never win a max
     assert (O.pool2d(-np.abs(x) - 1, 3, 2, 1, "max") < 0).all()
@@ -154,3 +155,14 @@ def test_rounding_matches_library_types():
     x = np.concatenate([r.normal(size=1000) * 10.0 ** r.integers(-6, 6, 1000), [0.0, -0.0, 1.0, 65504.0]]).astype(np.float32)
     assert np.array_equal(O.round_bf16(x), torch.from_numpy(x).to(torch.bfloat16).float().numpy())
     assert np.array_equal(O.round_f16(x), torch.from_numpy(x).to(torch.float16).float().numpy())
+
+
+def test_conv_with_a_1x7_and_a_7x1_filter_vs_torch():
+    r = rng(11)
+    x = r.normal(size=(1, 5, 9, 10)).astype(np.float32)
+    for (kh, kw, ph, pw) in ((1, 7, 0, 3), (7, 1, 3, 0), (1, 3, 0, 1), (3, 1, 1, 0)):
+        w = r.normal(size=(4, 5, kh, kw)).astype(np.float32)
+        b = r.normal(size=4).astype(np.float32)
+        got = O.conv2d(x, w, b, 1, (ph, pw), None, O.ACT_RELU)
+        t = F.relu(F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), torch.from_numpy(b).double(), 1, (ph, pw))).numpy()
+        assert got.shape == (1, 4, 9, 10) and np.allclose(got, t, atol=1e-5)
