@@ -51,6 +51,9 @@ struct Load {
     uint64_t seed = 1;
     int64_t next = 0, end = 0;
     numeric::Rng rng{1};
+    std::vector<int64_t> trace_ms;  // "trace": arrival times in milliseconds from the start (load.cpp:239-248)
+    size_t next_trace = 0;
+    int64_t begin = 0;
 
     int64_t gap_ns() {
         if (type == "poisson") {  // exponential gaps: -ln(u) / frequency (load.cpp:230-237)
@@ -60,9 +63,11 @@ struct Load {
         }
         return (int64_t)(1e9 / frequency);
     }
-    void start(int64_t begin, int64_t end_) {
-        next = begin; end = end_;
+    void start(int64_t begin_, int64_t end_) {
+        next = begin = begin_; end = end_;
         rng = numeric::Rng(seed);
+        next_trace = 0;
+        std::sort(trace_ms.begin(), trace_ms.end());
     }
     // Returns false when the run is over.  A launch whose successor is already due is given up,
     // as in DISB ("always choose the newest frame", load.cpp:196-222).  *scheduled receives the
@@ -72,6 +77,22 @@ struct Load {
         if (type == "continuous") {
             *scheduled = now;
             return now < end;
+        }
+        if (type == "trace") {
+            // the arrival whose successor is already due is given up (load.cpp:258-296)
+            if (next_trace >= trace_ms.size()) return false;
+            int64_t launch = begin + trace_ms[next_trace] * 1000000;
+            size_t nn = next_trace + 1;
+            while (nn < trace_ms.size() && begin + trace_ms[nn] * 1000000 < now) { launch = begin + trace_ms[nn] * 1000000; ++nn; }
+            next_trace = nn;
+            if (launch >= end) return false;
+            while (now_ns() < launch) {
+                int64_t left = launch - now_ns();
+                if (left > 200000) std::this_thread::sleep_for(std::chrono::nanoseconds(left - 100000));
+                else spin_pause();
+            }
+            *scheduled = launch;
+            return true;
         }
         if (frequency <= 0) return false;
         int64_t nn = next + gap_ns();
@@ -572,6 +593,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         t->load.type = l["type"].string("continuous");
         t->load.frequency = l["frequency"].number(0);
         t->load.seed = (uint64_t)l["seed"].number(1 + (double)tenants.size());
+        for (const json::Value &v : l["trace"].arr) t->load.trace_ms.push_back((int64_t)v.number(0));
         if (sh.policy == "lco" && t->priority != 0) continue;  // rtonlyclient.cpp:120-141: keep the real-time tasks only
         max_prio = std::max(max_prio, t->priority);
         tenants.push_back(std::move(t));

@@ -103,3 +103,18 @@ def test_graph_and_stencil_tenants_under_a_latency_critical_model(gp):
     assert t["hp"]["requests"] >= 250
     assert t["mw"]["requests"] > 50 and t["cc"]["requests"] > 50
     assert t["mw"]["preemptions"] + t["cc"]["preemptions"] > 20
+
+
+def test_trace_load_serves_the_newest_arrival(gp):
+    """DISB's "trace" load (third_party/disb/src/load.cpp:239-296): arrival times in milliseconds;
+    an arrival whose successor is already due is skipped."""
+    trace = [0, 5, 10, 200, 200, 200, 201, 400, 405, 410, 415, 1600]  # the last one falls past the end
+    cfg = {"time": 1.0, "policy": "wb-chunk-async", "tasks": [
+        {"id": "hp", "load": {"type": "trace", "trace": trace},
+         "client": {"name": "hp", "model_name": "toy", "priority": 0, "launch_mode": "launch"}},
+        {"id": "be", "load": {"type": "continuous"},
+         "client": {"name": "be", "model_name": "resnet50", "priority": 1, "launch_mode": "launch"}}]}
+    rep = _run_cfg(cfg)
+    n = rep["tasks"]["hp"]["requests"]
+    assert 7 <= n <= 11, n  # the burst at 200 ms collapses; nothing is served after the end
+    assert rep["tasks"]["be"]["requests"] > 10
