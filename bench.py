@@ -113,6 +113,7 @@ def roofline(workload, iters, dt):
         empty.append(a.elapsed_ms(b))
     bracket_ms = sorted(empty)[len(empty) // 2]
     total_ms, total_flop, total_bytes, launches = 0.0, 0.0, 0.0, 0
+    roof_ms, hbm_bound_layers = 0.0, 0
     for _ in range(iters):
         # one pass through the reference's launch_kernel API, events around each convolution
         ex.reset_counters(stream)
@@ -131,13 +132,21 @@ def roofline(workload, iters, dt):
             total_flop += kernels[i]["flops"]
             total_bytes += kernels[i]["bytes"]
             launches += 1
+            # the layer's own roofline: whichever of the two peaks bounds it
+            t_mfma, t_hbm = kernels[i]["flops"] / (PEAK[dt] * 1e12), kernels[i]["bytes"] / 8e12
+            roof_ms += max(t_mfma, t_hbm) * 1e3
+            hbm_bound_layers += t_hbm > t_mfma
     ex.destroy()
     achieved = total_flop / (total_ms * 1e-3) / 1e12
     return {"bound": "mfma", "kernel": "mat_kernel<PipeKernel<f16,conv>> (implicit-GEMM conv2d of " + workload + ", preemptible launches)",
             "achieved": achieved, "peak": PEAK[dt], "unit": "TFLOP/s", "frac": achieved / PEAK[dt],
             "traffic": HBM_TRAFFIC_PER_LAUNCH.get((workload, dt)),
             "launches": launches, "avg_launch_us": total_ms * 1e3 / launches, "event_bracket_us": bracket_ms * 1e3,
-            "algorithmic_flop_per_launch": total_flop / launches, "algorithmic_bytes_per_launch": total_bytes / launches}
+            "algorithmic_flop_per_launch": total_flop / launches, "algorithmic_bytes_per_launch": total_bytes / launches,
+            # every layer against the peak that bounds IT (8 TB/s HBM or the MFMA peak): sum of the
+            # layers' roofline times over the sum of their measured times
+            "per_layer_roofline_frac": roof_ms / total_ms, "layers_hbm_bound": hbm_bound_layers / launches,
+            "achieved_GBps": total_bytes / (total_ms * 1e-3) / 1e9}
 
 
 def _time_gemm(gp, p, stream, st, iters):
