@@ -109,6 +109,11 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     __shared__ int mailbox[2];
     const bool dynamic = b.executed != nullptr;
     const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    // As many workgroups as claims: a counter's slice is as long as the number of workgroups that
+    // serve it (util/slice_map.h), so nobody can get a second claim, on a first launch or on a
+    // relaunch, and the claim that would only report "nothing left" (an atomic and a barrier at
+    // the tail of every small kernel) is skipped.
+    const bool single = (int)gridDim.x >= b.total;
     // which counter this workgroup serves and the slice of the tile order that counter owns
     const int grp = wg_group((int)blockIdx.x, b.groups);
     const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
@@ -129,6 +134,7 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
         // claim (an atomic and a barrier, 1-2 us) off their critical path.
         const int first = idx * b.batch, last = first + b.batch < b.tiles ? first + b.batch : b.tiles;
         for (int tile = first; tile < last; ++tile) body(decode_tile(tile, b.sx, b.sy, b.order));
+        if (single) return;
     }
 }
 
@@ -155,6 +161,7 @@ __device__ __forceinline__ void tile_loop_span(const BlpArgs &b, Body &&body) {
         if (idx < 0) return;
         const int first = idx * b.batch;
         body(first, first + b.batch < b.tiles ? first + b.batch : b.tiles);
+        if ((int)gridDim.x >= b.total) return;  // one claim per workgroup at most (see tile_loop)
     }
 }
 
@@ -210,6 +217,9 @@ __device__ __forceinline__ void tile_loop_ckpt(const BlpArgs &b, Body &&body) {
         }
         if (idx < 0) return;
         if (body(decode_tile(idx, b.sx, b.sy, b.order), idx, kt0)) return;
+        // one claim per workgroup at most (see tile_loop); a relaunch may continue a stored tile and
+        // then still owe its slice a claim, so the shortcut holds on the fresh path only
+        if ((int)gridDim.x >= b.total && kt0 == 0 && !(it == 0 && b.ckpt)) return;
     }
 }
 
