@@ -89,8 +89,8 @@ def probe(workload, trials):
 
 
 def roofline(workload, iters, dt):
-    """Times every launch of the model's MFMA convolution kernel with HIP events on the stream
-    the kernel runs on; achieved = algorithmic flop of those launches / their summed duration."""
+    """Times the launches of the model's MFMA convolution kernel with HIP events on the stream the
+    kernel runs on; achieved = algorithmic flop of those launches / their summed duration."""
     from gpreempt_amd import capi as gp
     from gpreempt_amd import executor as gx
     ex = gx.Executor(workload, blp=True)
@@ -101,34 +101,30 @@ def roofline(workload, iters, dt):
     conv = [i for i, k in enumerate(kernels) if k["name"] == "conv2d"]
     ex.execute(stream)  # warm-up, also resolves launch geometry
     stream.sync()
-    ev = [(gp.Event(), gp.Event()) for _ in conv]
-    # what an event pair reads with nothing between its two records: subtracted from every bracket
-    # below, so that the figure is the kernel's own duration, as a kernel trace reports it
+    e0, e1 = gp.Event(), gp.Event()
+    # what an event pair reads with nothing between its two records; subtracted once per pass
     empty = []
-    for a, b in ev[:64]:
-        a.record(stream)
-        b.record(stream)
-    stream.sync()
-    for a, b in ev[:64]:
-        empty.append(a.elapsed_ms(b))
+    for _ in range(16):
+        e0.record(stream)
+        e1.record(stream)
+        e1.sync()
+        empty.append(e0.elapsed_ms(e1))
     bracket_ms = sorted(empty)[len(empty) // 2]
     total_ms, total_flop, total_bytes, launches = 0.0, 0.0, 0.0, 0
     roof_ms, hbm_bound_layers = 0.0, 0
     for _ in range(iters):
-        # one pass through the reference's launch_kernel API, events around each convolution
+        # one pass through the reference's launch_kernel API over the convolutions alone, back to
+        # back inside one event pair: a launch's duration then is what a kernel trace reports for it
+        # (brackets around single launches read up to 3 us less than the trace: part of the bracket's
+        # own cost overlaps with the kernel, by an amount that depends on how the kernel ends)
         ex.reset_counters(stream)
-        j = 0
-        for i in range(len(kernels)):
-            if j < len(conv) and conv[j] == i:
-                ev[j][0].record(stream)
-                ex.launch_kernel(i, stream)
-                ev[j][1].record(stream)
-                j += 1
-            else:
-                ex.launch_kernel(i, stream)
-        stream.sync()
-        for (a, b), i in zip(ev, conv):
-            total_ms += max(a.elapsed_ms(b) - bracket_ms, 1e-4)
+        e0.record(stream)
+        for i in conv:
+            ex.launch_kernel(i, stream)
+        e1.record(stream)
+        e1.sync()
+        total_ms += e0.elapsed_ms(e1) - bracket_ms
+        for i in conv:
             total_flop += kernels[i]["flops"]
             total_bytes += kernels[i]["bytes"]
             launches += 1
@@ -420,7 +416,7 @@ def main():
                     out["other_policies"][pol] = summarize(scenario(max(200, args.steps // 2), args.warmup, pol, args.hp_rate, args.be_model, args.hp_model))
             out["config2_resnet50_fp32_b1"] = probe("resnet50", 300)
     if args.only in ("", "roofline"):
-        out["roofline"] = roofline(args.be_model, 3, "f16")
+        out["roofline"] = roofline(args.be_model, 10, "f16")
     if args.only in ("", "gemm"):
         out["config5_gemm8192_bf16"] = gemm_roofline()
         out["config1_gemm1024_f32"] = config1_gemm1024()
