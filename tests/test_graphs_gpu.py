@@ -203,3 +203,16 @@ def test_host_timed_preemption(gp, ex_mod, kind):
             assert np.abs(got - want).max() < 2 * PR_TOL
         preempted = ex.graph_info()["preemptions"]
     assert preempted > 0
+
+
+def test_golden_graph_on_the_gpu(gp, ex_mod):
+    """tests/golden/tiny_graph (10 vertices, answers worked out by hand) through the executors"""
+    import json
+    import os
+    base = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tiny_graph")
+    want = json.load(open(base + ".expected.json"))
+    for kind, key, dt, field in (("bfs", "label", np.uint32, "bfs_levels"), ("cc", "comp", np.uint64, "components"), ("sssp", "cost", np.uint32, "distances")):
+        ex = ex_mod.Executor(kind, blp=True, graph_path=base)
+        ex.set_flag(gp.Flag())
+        ex.execute()
+        assert ex.graph_result(key, dt).tolist() == want[field], kind

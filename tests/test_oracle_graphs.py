@@ -130,3 +130,32 @@ def test_graph_files_round_trip(tmp_path):
     assert lib.gpx_write_synthetic_graph((base + "2").encode(), C.c_ulonglong(500), 4, C.c_ulonglong(9)) == 0
     assert open(base + ".dst", "rb").read() == open(base + "2.dst", "rb").read()
     assert lib.gpx_write_synthetic_graph(base.encode(), C.c_ulonglong(1), 4, C.c_ulonglong(9)) != 0
+
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def test_golden_graph_by_hand():
+    """the hand-worked answers of tests/golden/tiny_graph against the oracle"""
+    import json
+    indptr, indices, w = G.read_graph(os.path.join(GOLDEN, "tiny_graph"), weights=True)
+    want = json.load(open(os.path.join(GOLDEN, "tiny_graph.expected.json")))
+    assert len(indptr) == 11 and len(indices) == 20
+    assert G.bfs(indptr, indices)[0].tolist() == want["bfs_levels"]
+    assert G.cc(indptr, indices)[0].tolist() == want["components"]
+    assert G.sssp(indptr, indices, w)[0].tolist() == want["distances"]
+    value, _ = G.pagerank(indptr, indices, tolerance=1e-7, max_iter=1000)
+    assert np.allclose(value, G.pagerank_exact(indptr, indices), atol=1e-4)
+
+
+def test_golden_param_file():
+    from gpreempt_amd import executor
+    lib = executor.lib()
+    lib.gpx_parse_params.restype = C.c_long
+    path = os.path.join(GOLDEN, "tiny.mod.params").encode()
+    out = np.zeros(8, np.float32)
+    n = C.c_size_t(0)
+    assert lib.gpx_parse_params(path, b"p0", out.ctypes.data_as(C.c_void_p), C.c_size_t(8), C.byref(n)) == 2
+    assert n.value == 6 and out[:6].tolist() == [1.0, -2.5, 3.25, 0.0, np.float32(1e-3), 65504.0]
+    assert lib.gpx_parse_params(path, b"fc.bias", out.ctypes.data_as(C.c_void_p), C.c_size_t(8), C.byref(n)) == 2
+    assert n.value == 2 and out[:2].tolist() == [0.5, -0.5]
