@@ -113,7 +113,7 @@ extern "C" int gpx_graph_inject_preempt(gpx_executor e, int iteration, int kerne
 extern "C" int gpx_set_lc_tasks(gpx_executor e, int n) { H(e)->lc_tasks.store(n); return Status::Succ; }
 extern "C" int gpx_set_graph_path(gpx_executor e, const char *base) { return H(e)->ex->set_graph_path(base ? base : ""); }
 extern "C" int gpx_write_synthetic_graph(const char *base, unsigned long long vertices, unsigned degree, unsigned long long seed) {
-    if (!base || vertices < 2 || vertices >= (1ULL << 28) || degree < 1 || degree > 256) return Status::OutOfRange;
+    if (!base || vertices < 2 || vertices >= (1ULL << 28) || degree < 1 || degree > 256 || vertices * degree > (1ULL << 27)) return Status::OutOfRange;
     return GraphCompute::write_graph(base, GraphCompute::synthetic_graph(vertices, degree, seed));
 }
 

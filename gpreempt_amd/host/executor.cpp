@@ -57,7 +57,7 @@ Status Executor::init_graph(const std::string &kind, const std::string &options)
         RETURN_STATUS(GraphCompute::read_graph(base, g, kind == "sssp"));
     } else {
         long n = option_int(options, "n", 1 << 20), deg = option_int(options, "deg", 8), seed = option_int(options, "seed", 1);
-        if (n < 2 || n >= (1L << 28) || deg < 1 || deg > 256) return Status::OutOfRange;
+        if (n < 2 || n >= (1L << 28) || deg < 1 || deg > 256 || n * deg > (1L << 27)) return Status::OutOfRange;  // at most 2^28 directed edges
         g = GraphCompute::synthetic_graph((uint64_t)n, (unsigned)deg, (uint64_t)seed);
     }
     graph_compute = GraphCompute::Workload::create(kind, g);

@@ -3,6 +3,7 @@
 #include "workloads/graphcompute.h"
 
 #include <algorithm>
+#include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <thread>
@@ -226,8 +227,13 @@ Status Workload::run_kernels(const std::vector<int> &kernels, GPUstream stream, 
             GC_CHECK(gp_stream_sync(stream));
             flag_to_lower_ = false;
         }
-        if (env->higher_priority_active)
+        if (env->higher_priority_active) {
             while (env->higher_priority_active()) std::this_thread::yield();
+        } else {
+            // nobody to ask: give whoever raised the flag time to lower it instead of relaunching
+            // kernels that would leave at once
+            std::this_thread::sleep_for(std::chrono::microseconds(50));
+        }
         GC_CHECK(gp_fill32_async(env->stop_index, 0xFFFFFFFFu, 1, stream));
         from = stop < K ? stop : K - 1;
     }
