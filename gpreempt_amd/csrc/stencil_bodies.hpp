@@ -72,10 +72,11 @@ template <> struct MwOperands<GP_MW_UPDATE_Z> { long c; int ll; float f0, f1, in
 template <> struct MwOperands<GP_MW_FLUX_X> { int k, i; float s[MW_VARS][4], h0, h1; };
 template <> struct MwOperands<GP_MW_FLUX_Z> { int k, i; float s[MW_VARS][4], h0, h1, h2; };
 
-__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_UPDATE_X> &o) {
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, unsigned id, MwOperands<GP_MW_UPDATE_X> &o) {
     const MwView v{p.nx, p.nz};
-    const int nx = p.nx, nz = p.nz;
-    const int k = (int)((id / nx) % nz), i = (int)(id % nx), ll = (int)(id / nx / nz);
+    const unsigned nx = p.nx, nz = p.nz;
+    const unsigned row = id / nx;  // 32-bit: ids stay below 2^29 (the launcher bounds nx * nz)
+    const int i = (int)(id - row * nx), ll = (int)(row / nz), k = (int)(row - (unsigned)ll * nz);
     if (ll >= MW_VARS) return false;
     o.c = v.st(ll, k + MW_HS, i + MW_HS);
     o.f0 = p.flux[v.fx(ll, k, i)];
@@ -89,10 +90,11 @@ __device__ __forceinline__ void mw_finish(const gp_miniweather_params &p, const 
     p.state_out[o.c] = o.init + p.dt * tend;
 }
 
-__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_UPDATE_Z> &o) {
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, unsigned id, MwOperands<GP_MW_UPDATE_Z> &o) {
     const MwView v{p.nx, p.nz};
-    const int nx = p.nx, nz = p.nz;
-    const int i = (int)(id % nx), k = (int)((id / nx) % nz), ll = (int)(id / nx / nz);
+    const unsigned nx = p.nx, nz = p.nz;
+    const unsigned row = id / nx;
+    const int i = (int)(id - row * nx), ll = (int)(row / nz), k = (int)(row - (unsigned)ll * nz);
     if (ll >= MW_VARS) return false;
     o.ll = ll;
     o.c = v.st(ll, k + MW_HS, i + MW_HS);
@@ -131,12 +133,12 @@ __device__ __forceinline__ void mw_finish(const gp_miniweather_params &p, const 
     p.state_out[o.c] = o.init + p.dt * tend;
 }
 
-__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_FLUX_X> &o) {
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, unsigned id, MwOperands<GP_MW_FLUX_X> &o) {
     const MwView v{p.nx, p.nz};
     const MwHydro hy(p.hydro, p.nz);
-    const int nx = p.nx;
-    o.k = (int)(id / (nx + 1));
-    o.i = (int)(id % (nx + 1));
+    const unsigned w = p.nx + 1;
+    o.k = (int)(id / w);
+    o.i = (int)(id - (unsigned)o.k * w);
     if (o.k >= p.nz) return false;
 #pragma unroll
     for (int ll = 0; ll < MW_VARS; ++ll) {
@@ -170,12 +172,12 @@ __device__ __forceinline__ void mw_finish(const gp_miniweather_params &p, const 
     p.flux[v.fx(MW_RHOT, o.k, o.i)] = (float)(r * u * th - d3[MW_RHOT]);
 }
 
-__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, long id, MwOperands<GP_MW_FLUX_Z> &o) {
+__device__ __forceinline__ bool mw_load(const gp_miniweather_params &p, unsigned id, MwOperands<GP_MW_FLUX_Z> &o) {
     const MwView v{p.nx, p.nz};
     const MwHydro hy(p.hydro, p.nz);
     const int nx = p.nx;
-    o.i = (int)(id % nx);
-    o.k = (int)(id / nx);
+    o.k = (int)(id / (unsigned)nx);
+    o.i = (int)(id - (unsigned)o.k * (unsigned)nx);
     if (o.k >= p.nz + 1) return false;
     const long row = nx + 2 * MW_HS;
 #pragma unroll
@@ -257,7 +259,7 @@ __device__ __forceinline__ void mw_span(const gp_miniweather_params &p, int firs
             MwOperands<KIND> op[U];
             bool ok[U];
 #pragma unroll
-            for (int j = 0; j < U; ++j) ok[j] = t + j < last && mw_load(p, (long)(t + j) * MW_TILE + threadIdx.x, op[j]);
+            for (int j = 0; j < U; ++j) ok[j] = t + j < last && mw_load(p, (unsigned)(t + j) * MW_TILE + threadIdx.x, op[j]);
 #pragma unroll
             for (int j = 0; j < U; ++j)
                 if (ok[j]) mw_finish(p, op[j]);
