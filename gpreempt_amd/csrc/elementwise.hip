@@ -62,7 +62,7 @@ int plan_pool2d(const gp_pool_params *p, EltPlan *out) {
         GP_REQUIRE(Ho > 0 && Wo > 0, "pool: empty output");
     }
     long items = (long)p->N * Ho * Wo * (p->C / vec);
-    GP_REQUIRE((items + NT - 1) / NT < (1L << 31), "pool: too large");
+    GP_REQUIRE(items < (1L << 31), "pool: too large (2^31 16-byte items at most)");
     *out = EltPlan{};
     out->op = OP_POOL; out->dtype = p->dtype;
     out->sx = (int)((items + NT - 1) / NT); out->sy = 1;
@@ -79,7 +79,7 @@ int plan_eltwise(const gp_eltwise_params *p, EltPlan *out) {
     GP_REQUIRE(al16(p->a) && al16(p->out) && al16(p->b) && al16(p->scale) && al16(p->shift), "eltwise: 16-byte alignment");
     long items = p->rows * (p->cols / vec);
     long tiles = (items + (long)NT * ELT_PER - 1) / ((long)NT * ELT_PER);
-    GP_REQUIRE(tiles < (1L << 31), "eltwise: too large");
+    GP_REQUIRE(items < (1L << 31), "eltwise: too large (2^31 16-byte items at most)");
     *out = EltPlan{};
     out->op = OP_ELTWISE; out->dtype = p->dtype; out->sx = (int)tiles; out->sy = 1;
     out->u.elt = EltwiseArgs{*p, items};

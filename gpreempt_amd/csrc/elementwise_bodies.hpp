@@ -8,6 +8,7 @@
 #pragma once
 #include "common.hpp"
 #include "out_store.hpp"
+#include "mma.hpp"
 
 namespace gp {
 
@@ -127,10 +128,13 @@ __device__ __forceinline__ void pool_tile(const PoolArgs &a, TileIdx t) {
     constexpr int VEC = VecIO<T>::VEC;
     const int chunks = p.C / VEC;
     
-        long item = (long)t.x * NT + threadIdx.x;
-        if (item >= items) return;
-        int ch = (int)(item % chunks);
-        long pix = item / chunks;
+        // 32-bit index arithmetic (the planner bounds the item count): a 64-bit division is a
+        // subroutine of a hundred instructions, and five of them per item made this kernel ALU-bound
+        const unsigned item = (unsigned)t.x * NT + threadIdx.x;
+        if (item >= (unsigned)items) return;
+        const unsigned upix = item / (unsigned)chunks;
+        const int ch = (int)(item - upix * (unsigned)chunks);
+        const long pix = upix;
         const T *in = (const T *)p.in;
         T *out = (T *)p.out;
         float acc[VEC];
@@ -150,13 +154,39 @@ __device__ __forceinline__ void pool_tile(const PoolArgs &a, TileIdx t) {
             VecIO<T>::store(out + pix * p.out_pix_stride + ch * VEC, acc);
             return;
         }
-        int wo = (int)(pix % Wo);
-        long q = pix / Wo;
-        int ho = (int)(q % Ho);
-        long n = q / Ho;
+        const unsigned q = upix / (unsigned)Wo;
+        const int wo = (int)(upix - q * (unsigned)Wo);
+        const long n = q / (unsigned)Ho;
+        const int ho = (int)(q - (unsigned)n * (unsigned)Ho);
 #pragma unroll
         for (int i = 0; i < VEC; ++i) acc[i] = p.mode == 0 ? -INFINITY : 0.f;
         int cnt = 0;
+        // The usual windows are unrolled so that all their loads are in flight together; with the
+        // window size known only at run time every tap would wait for the one before.
+        auto window = [&](auto RC, auto SC) {
+            constexpr int R = decltype(RC)::value, S = decltype(SC)::value;
+            float f[R * S][VEC];
+            bool in_range[R * S];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+#pragma unroll
+                for (int s = 0; s < S; ++s) {
+                    const int hi = ho * p.stride - p.pad + r, wi = wo * p.stride - p.pad + s;
+                    in_range[r * S + s] = (unsigned)hi < (unsigned)p.H && (unsigned)wi < (unsigned)p.W;
+                    if (in_range[r * S + s]) VecIO<T>::load(in + ((n * p.H + hi) * p.W + wi) * p.in_pix_stride + ch * VEC, f[r * S + s]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < R * S; ++i) {
+                if (!in_range[i]) continue;
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) acc[j] = p.mode == 0 ? fmaxf(acc[j], f[i][j]) : acc[j] + f[i][j];
+                ++cnt;
+            }
+        };
+        if (p.R == 3 && p.S == 3) window(IntC<3>{}, IntC<3>{});
+        else if (p.R == 2 && p.S == 2) window(IntC<2>{}, IntC<2>{});
+        else
         for (int r = 0; r < p.R; ++r) {
             int hi = ho * p.stride - p.pad + r;
             if ((unsigned)hi >= (unsigned)p.H) continue;
@@ -196,10 +226,11 @@ __device__ __forceinline__ void eltwise_tile(const EltwiseArgs &a, TileIdx t) {
     
 #pragma unroll
         for (int u = 0; u < ELT_PER; ++u) {
-            long item = ((long)t.x * ELT_PER + u) * NT + threadIdx.x;
-            if (item >= items) continue;
-            int ch = (int)(item % chunks);
-            long row = item / chunks;
+            const unsigned item = ((unsigned)t.x * ELT_PER + u) * NT + threadIdx.x;  // 32-bit: see pool_tile
+            if (item >= (unsigned)items) continue;
+            const unsigned urow = item / (unsigned)chunks;
+            const int ch = (int)(item - urow * (unsigned)chunks);
+            const long row = urow;
             float a[VEC];
             VecIO<T>::load((const T *)p.a + row * p.a_stride + ch * VEC, a);
             if (p.b) {
