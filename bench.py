@@ -415,6 +415,12 @@ def main():
                 if pol != args.policy:
                     out["other_policies"][pol] = summarize(scenario(max(200, args.steps // 2), args.warmup, pol, args.hp_rate, args.be_model, args.hp_model))
             out["config2_resnet50_fp32_b1"] = probe("resnet50", 300)
+            # the high-priority tenant alone under the same arrival process (the reference's
+            # real-time-only client, rtonlyclient.cpp): `value` divides by back-to-back isolated
+            # runs, which are a little faster than requests that arrive every few milliseconds
+            alone = scenario(max(200, args.steps // 2), args.warmup, "lco", args.hp_rate, args.be_model, args.hp_model)["tasks"]["hp"]
+            out["hp_alone_same_arrivals_ms"] = {k: alone["totalLatency(us)"][k] / 1e3 for k in ("mean", "p50", "p99")}
+            out["hp_p99_vs_alone_same_arrivals"] = out["hp_corun_ms"]["p99"] / out["hp_alone_same_arrivals_ms"]["p99"]
     if args.only in ("", "roofline"):
         out["roofline"] = roofline(args.be_model, 10, "f16")
     if args.only in ("", "gemm"):
