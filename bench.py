@@ -178,7 +178,7 @@ def config1_gemm1024(iters=20):
                       alpha=1.0, act=gp.ACT_RELU, batch=1)
     stream = gp.Stream(1)
     flag = gp.Flag()
-    st = gp.BlpState(1, flag)
+    st = gp.BlpState(1, flag, 32)
     t_plain, info = _time_gemm(gp, p, stream, None, iters)
     t_blp, info_b = _time_gemm(gp, p, stream, st, iters)
     flop = 2.0 * n ** 3 + 2.0 * n * n
@@ -205,10 +205,10 @@ def gemm_roofline(iters=10):
     p = gp.GemmParams(dtype=gp.BF16, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=1, C=dC.ptr, ldc=n, alpha=1.0, batch=1)
     flag = gp.Flag()
     stream = gp.Stream(1)
-    st = gp.BlpState(1, flag)
+    st = gp.BlpState(1, flag, 32)
     t, info = _time_gemm(gp, p, stream, st, iters)
     t_plain, _ = _time_gemm(gp, p, stream, None, iters)
-    st_ck = gp.BlpState(1, flag)
+    st_ck = gp.BlpState(1, flag, 32)
     st_ck.enable_checkpoints(p)
     t_ck, _ = _time_gemm(gp, p, stream, st_ck, iters)
     flop = 2.0 * n ** 3
@@ -229,7 +229,7 @@ def hbm_ops(iters=20):
     out = {}
 
     def timed(fn, p, bytes_moved):
-        st = gp.BlpState(1, flag)
+        st = gp.BlpState(1, flag, 32)
         e0, e1 = gp.Event(), gp.Event()
         ms = []
         for i in range(iters + 2):

@@ -281,21 +281,27 @@ class BlpState:
     """stop_index (one int, -1) and executed[n] counters in device memory
     (BLPExecutor::init, reference src/executor.cpp:328-334)."""
 
-    def __init__(self, n_kernels, flag):
+    COUNTER_STRIDE = 16  # ints between the counters of one kernel when it has several (64-byte lines)
+
+    def __init__(self, n_kernels, flag, counter_groups=1):
+        """counter_groups = 1 is the reference's layout (one int per kernel); BLPExecutor uses 32
+        counters per kernel, each on its own line (gp_preempt_ctx::counter_groups)."""
         self.n = n_kernels
         self.flag = flag
+        self.groups = counter_groups
+        self.ints_per_kernel = 1 if counter_groups <= 1 else counter_groups * self.COUNTER_STRIDE
         self.stop = DevBuf(4)
-        self.executed = DevBuf(4 * n_kernels)
+        self.executed = DevBuf(4 * n_kernels * self.ints_per_kernel)
         self.stop.upload(np.array([-1], np.int32))
         self.reset()
 
     def reset(self):
-        self.executed.upload(np.zeros(self.n, np.int32))
+        self.executed.upload(np.zeros(self.n * self.ints_per_kernel, np.int32))
 
     def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0):
         ck = getattr(self, "ckpt", None)
-        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id, kernel_id, inject_at, max_workgroups, poll_every, 0, None,
-                          ck.ptr if ck else None, ck.nbytes if ck else 0)
+        return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id * self.ints_per_kernel, kernel_id, inject_at, max_workgroups,
+                          poll_every, self.groups if self.groups > 1 else 0, None, ck.ptr if ck else None, ck.nbytes if ck else 0)
 
     def enable_checkpoints(self, params):
         """Allocates the workspace that lets the GEMM `params` leave its tiles half-way (if it can)."""
