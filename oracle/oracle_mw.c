@@ -8,7 +8,9 @@
  * analytic profiles :689-775, reductions :906-932.
  *
  * Arithmetic types are the reference's: the state is fp32, the x flux is formed in fp64, the z
- * flux in fp32.  A "tile" is 256 consecutive element ids of a kernel (the reference's thread
+ * flux in fp32.  The reference is C++: a math call whose arguments are all float resolves to the
+ * float overload there, so this C file names powf / expf / sqrtf / cosf in exactly those places.
+ * A "tile" is 256 consecutive element ids of a kernel (the reference's thread
  * block), processed in increasing id order.
  *
  * One reference quirk is settled deliberately: in the second Runge-Kutta stage of a z sweep the
@@ -239,22 +241,22 @@ static void hydro_const_theta(real z, real *r, real *t) { /* :744-753 */
     real p, exner, rt;
     *t = theta0;
     exner = exner0 - grav * z / (cp * theta0);
-    p = p0 * pow(exner, (cp / rd));
-    rt = pow((p / C0), (1. / gamm));
+    p = p0 * powf(exner, (cp / rd));   /* all-float arguments: the C++ overload the reference compiles to */
+    rt = pow((p / C0), (1. / gamm));   /* a double exponent: double pow */
     *r = rt / *t;
 }
 static void hydro_const_bvfreq(real z, real bv_freq0, real *r, real *t) { /* :756-765 */
     const real theta0 = 300., exner0 = 1.;
     real p, exner, rt;
-    *t = theta0 * exp(bv_freq0 * bv_freq0 / grav * z);
+    *t = theta0 * expf(bv_freq0 * bv_freq0 / grav * z);
     exner = exner0 - grav * grav / (cp * bv_freq0 * bv_freq0) * (*t - theta0) / (*t * theta0);
-    p = p0 * pow(exner, (cp / rd));
+    p = p0 * powf(exner, (cp / rd));
     rt = pow((p / C0), (1. / gamm));
     *r = rt / *t;
 }
 static real sample_ellipse_cosine(real x, real z, real amp, real x0, real z0, real xrad, real zrad) { /* :768-775 */
-    real dist = sqrt(((x - x0) / xrad) * ((x - x0) / xrad) + ((z - z0) / zrad) * ((z - z0) / zrad)) * pi / 2.;
-    if (dist <= pi / 2.) return amp * pow(cos(dist), 2.);
+    real dist = sqrtf(((x - x0) / xrad) * ((x - x0) / xrad) + ((z - z0) / zrad) * ((z - z0) / zrad)) * pi / 2.;
+    if (dist <= pi / 2.) return amp * pow(cosf(dist), 2.);
     return 0.;
 }
 /* data_spec: 1 collision, 2 thermal, 3 gravity waves, 5 density current, 6 injection (:689-741) */
@@ -311,7 +313,7 @@ void mw_init(int nx, int nz, int spec, real *state, real *hydro) {
         profile(spec, 0., z, &r, &u, &w, &t, &hr, &ht);
         hy_dens_int[k] = hr;
         hy_dens_theta_int[k] = hr * ht;
-        hy_pressure_int[k] = C0 * pow((hr * ht), gamm);
+        hy_pressure_int[k] = C0 * powf((hr * ht), gamm);
     }
     cell_const[0] = hy_dens_cell[0] / hy_dens_cell[HS]; /* :679-683 */
     cell_const[1] = hy_dens_cell[1] / hy_dens_cell[HS];

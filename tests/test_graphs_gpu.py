@@ -216,3 +216,49 @@ def test_golden_graph_on_the_gpu(gp, ex_mod):
         ex.set_flag(gp.Flag())
         ex.execute()
         assert ex.graph_result(key, dt).tolist() == want[field], kind
+
+
+def test_ragged_graph_with_sinks_and_isolated_vertices(gp, ex_mod, tmp_path):
+    """directed edges, a sink (no out-edges), an isolated vertex, a self-contained pair, and a
+    vertex whose neighbour list is longer than a wavefront"""
+    import os
+    import struct
+    n = 200
+    adj = {v: [] for v in range(n)}
+    for v in range(1, 150):
+        adj[0].append(v)          # a hub with 149 out-edges
+    for v in range(1, 100):
+        adj[v].append(v + 1)      # a directed chain 1 -> 2 -> ... -> 100
+    adj[150].append(151)
+    adj[151].append(150)          # a pair on its own
+    # 100..149 are sinks; 152..199 are isolated
+    indptr, indices = [0], []
+    for v in range(n):
+        indices += sorted(adj[v])
+        indptr.append(len(indices))
+    w = [1 + (i * 7) % 13 for i in range(len(indices))]
+    base = str(tmp_path / "ragged")
+    for ext, arr, fmt, size in ((".col", indptr, "Q", 8), (".dst", indices, "Q", 8), (".val", w, "I", 4)):
+        with open(base + ext, "wb") as f:
+            f.write(struct.pack("<QQ", len(arr), size))
+            f.write(struct.pack("<%d%s" % (len(arr), fmt), *arr))
+    ip, ix, ww = G.read_graph(base, weights=True)
+    for kind, key, dt, want in (("bfs", "label", np.uint32, G.bfs(ip, ix)[0]), ("cc", "comp", np.uint64, G.cc(ip, ix)[0]),
+                                ("sssp", "cost", np.uint32, G.sssp(ip, ix, ww)[0])):
+        ex = ex_mod.Executor(kind, blp=True, graph_path=base)
+        ex.set_flag(gp.Flag())
+        ex.execute()
+        assert np.array_equal(ex.graph_result(key, dt), want), kind
+    ex = ex_mod.Executor("pagerank", blp=True, graph_path=base)
+    ex.set_flag(gp.Flag())
+    ex.execute()
+    value = ex.graph_result("value", np.float32)
+    ref, _ = G.pagerank(ip, ix)
+    assert np.isfinite(value).all() and np.abs(value - ref).max() < 5e-3
+    assert np.allclose(value[152:], 0.15)  # nobody points at the isolated vertices
+    # a malformed file is refused, not launched
+    with open(base + ".dst", "r+b") as f:
+        f.seek(16)
+        f.write(struct.pack("<Q", 10 ** 6))
+    with pytest.raises(ex_mod.StatusError):
+        ex_mod.Executor("bfs", graph_path=base)
