@@ -142,6 +142,137 @@ __device__ __forceinline__ void attention_tile(const AttnArgs &a, TileIdx t, T *
         }
 }
 
+// ---- longer sequences: 64 queries per tile, the keys split between two wavefronts -----------------
+// Beyond 128 keys a (batch, head) pair has too few 128-query tiles to fill the GPU and a wavefront
+// too long a chain of work (12 heads x 3 tiles at 384 keys).  Here a tile is 64 queries; waves 0 and
+// 1 take the first half of the key blocks for query rows 0-31 and 32-63, waves 2 and 3 the second
+// half.  Each wave runs the same S^T / softmax / P V sequence on its keys with its own running
+// maximum (probabilities left unnormalised), the second pair parks its partial result in LDS and
+// the first pair merges: O = (a1 O1 + a2 O2) / (a1 sum1 + a2 sum2), a_i = exp(m_i - max(m1, m2)).
+constexpr int ATT_QB_SPLIT = 64;
+__host__ __device__ inline size_t attention_vt_bytes(int nb) { return (attention_lds_bytes(nb) + 15) / 16 * 16; }
+__host__ __device__ inline size_t attention_split_lds_bytes(int nb) { return attention_vt_bytes(nb) + 2 * (32 * ATT_D + 64) * sizeof(float); }
+
+template <typename T, int NB>
+__device__ __forceinline__ void attention_tile_split(const AttnArgs &a, TileIdx t, T *vt) {
+    static_assert(NB % 2 == 0, "key blocks are halved");
+    constexpr int NBH = NB / 2;
+    const gp_attention_params &p = a.p;
+    constexpr int SP = NB * 32 + 4;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, half = lane >> 5;
+    const int qg = wave & 1, kh = wave >> 1;  // query group, key half (wave-uniform)
+    const int S = p.seq;
+    const int head = t.y % p.heads, bat = t.y / p.heads;
+    const long tok0 = (long)bat * S;
+    const T *Q = (const T *)p.q + tok0 * p.ld_qkv + (long)head * ATT_D;
+    const T *K = (const T *)p.k + tok0 * p.ld_qkv + (long)head * ATT_D;
+    const T *V = (const T *)p.v + tok0 * p.ld_qkv + (long)head * ATT_D;
+    T *O = (T *)p.out + tok0 * p.ld_out + (long)head * ATT_D;
+    const u32x4 zero4 = {0, 0, 0, 0};
+    float *merge = (float *)((char *)vt + attention_vt_bytes(NB)) + qg * (32 * ATT_D + 64);  // O2[32][64], m2[32], sum2[32]
+
+    const int q = t.x * ATT_QB_SPLIT + qg * 32 + l32;
+    u32x4 bq[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) bq[ks] = q < S ? *(const u32x4 *)(Q + (long)q * p.ld_qkv + ks * 16 + half * 8) : zero4;
+
+    __syncthreads();  // the previous tile of this workgroup may still be reading vt or the merge area
+    for (int idx = tid; idx < NB * 32 * (ATT_D / 8); idx += 256) {
+        const int key = idx % (NB * 32), dc = idx / (NB * 32);
+        u32x4 raw = key < S ? *(const u32x4 *)(V + (long)key * p.ld_qkv + dc * 8) : zero4;
+        const unsigned short *e = (const unsigned short *)&raw;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ((unsigned short *)vt)[(dc * 8 + j) * SP + key] = e[j];
+    }
+    __syncthreads();
+
+    const int nb0 = kh * NBH;
+    f32x16 s[NBH];
+#pragma unroll
+    for (int i = 0; i < NBH; ++i) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[i][v] = 0.f;
+        const int key = (nb0 + i) * 32 + l32;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const u32x4 a_k = key < S ? *(const u32x4 *)(K + (long)key * p.ld_qkv + ks * 16 + half * 8) : zero4;
+            Elem<T>::mma(a_k, bq[ks], s[i]);
+        }
+    }
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NBH; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = (nb0 + i) * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+            s[i][v] = key < S ? s[i][v] * p.scale : -INFINITY;
+            m = fmaxf(m, s[i][v]);
+        }
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+    const float mm = m == -INFINITY ? 0.f : m;  // a half with no valid key contributes nothing (and no NaN)
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < NBH; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            s[i][v] = __expf(s[i][v] - mm);
+            sum += s[i][v];
+        }
+    sum += __shfl_xor(sum, 32, 64);
+
+    f32x16 o[2];
+#pragma unroll
+    for (int db = 0; db < 2; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NBH; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            typedef T tx8 __attribute__((ext_vector_type(8)));
+            tx8 pa;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pa[e] = Elem<T>::from_f(s[i][8 * j + e]);
+            const int kbase = (nb0 + i) * 32 + 16 * j + 4 * half;
+#pragma unroll
+            for (int db = 0; db < 2; ++db) {
+                const unsigned short *row = (const unsigned short *)vt + (db * 32 + l32) * SP + kbase;
+                const unsigned long long lo = *(const unsigned long long *)row, hi = *(const unsigned long long *)(row + 8);
+                u32x4 bv = {(unsigned)lo, (unsigned)(lo >> 32), (unsigned)hi, (unsigned)(hi >> 32)};
+                Elem<T>::mma(__builtin_bit_cast(u32x4, pa), bv, o[db]);
+            }
+        }
+    // ---- merge the two key halves ------------------------------------------------------------------
+    if (kh == 1) {
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) merge[(8 * (v / 4) + 4 * half + (v % 4)) * ATT_D + db * 32 + l32] = o[db][v];
+        if (half == 0) {
+            merge[32 * ATT_D + l32] = m;
+            merge[32 * ATT_D + 32 + l32] = sum;
+        }
+    }
+    __syncthreads();
+    if (kh == 0) {
+        const float m2 = merge[32 * ATT_D + l32], sum2 = merge[32 * ATT_D + 32 + l32];
+        const float M = fmaxf(mm, m2);
+        const float a1 = __expf(mm - M), a2 = m2 == -INFINITY ? 0.f : __expf(m2 - M);
+        const float den = a1 * sum + a2 * sum2;
+        const float f1 = a1 / den, f2 = a2 / den;  // this lane's query (row l32 of the group)
+        const int q0 = t.x * ATT_QB_SPLIT + qg * 32;
+#pragma unroll
+        for (int db = 0; db < 2; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = 8 * (v / 4) + 4 * half + (v % 4);  // the accumulator's query row: its factors sit in lane r
+                const float g1 = __shfl(f1, r, 64), g2 = __shfl(f2, r, 64);
+                const float val = g1 * o[db][v] + g2 * merge[r * ATT_D + db * 32 + l32];
+                if (q0 + r < S) st_elem<T>(O + (long)(q0 + r) * p.ld_out + db * 32 + l32, Elem<T>::from_f(val));
+            }
+    }
+}
+
 // Key blocks the body is instantiated for: seq <= 128 / 256 / 384 / 512 keys.
 __host__ __device__ inline int attention_nb_class(int seq) {
     const int nb = attention_key_blocks(seq);
@@ -153,7 +284,16 @@ __host__ __device__ inline int attention_nb_class(int seq) {
 template <typename T, int NB>
 __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a, BlpArgs blp) {
     extern __shared__ __attribute__((aligned(16))) unsigned char att_lds[];
-    tile_loop(blp, [&](TileIdx t) { attention_tile<T, NB>(a, t, reinterpret_cast<T *>(att_lds)); });
+    tile_loop(blp, [&](TileIdx t) {
+        if constexpr (NB <= 4) attention_tile<T, NB>(a, t, reinterpret_cast<T *>(att_lds));
+        else attention_tile_split<T, NB>(a, t, reinterpret_cast<T *>(att_lds));
+    });
+}
+// queries per tile and LDS bytes of the class a sequence length falls into
+__host__ __device__ inline int attention_queries_per_tile(int seq) { return attention_nb_class(seq) <= 4 ? ATT_QB : ATT_QB_SPLIT; }
+__host__ __device__ inline size_t attention_class_lds_bytes(int seq) {
+    const int nb = attention_nb_class(seq);
+    return nb <= 4 ? attention_lds_bytes(nb) : attention_split_lds_bytes(nb);
 }
 
 }  // namespace gp

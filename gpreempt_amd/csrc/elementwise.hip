@@ -142,8 +142,9 @@ int plan_attention(const gp_attention_params *p, EltPlan *out) {
     GP_REQUIRE(al16(p->q) && al16(p->k) && al16(p->v), "attention: 16-byte alignment");
     *out = EltPlan{};
     out->op = OP_ATTENTION; out->dtype = p->dtype;
-    out->sx = (p->seq + ATT_QB - 1) / ATT_QB; out->sy = p->batch * p->heads;
-    out->lds_bytes = attention_lds_bytes(attention_nb_class(p->seq));
+    const int qb = attention_queries_per_tile(p->seq);
+    out->sx = (p->seq + qb - 1) / qb; out->sy = p->batch * p->heads;
+    out->lds_bytes = attention_class_lds_bytes(p->seq);
     out->u.attn = AttnArgs{*p};
     if (out->u.attn.p.scale == 0.f) out->u.attn.p.scale = 1.f;
     return GP_SUCC;

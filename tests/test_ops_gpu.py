@@ -263,7 +263,7 @@ def test_conv2d_long_tiles_left_mid_k_and_resumed_bit_exact(gp, dt):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-@pytest.mark.parametrize("shape", [(1, 12, 128), (2, 3, 77), (1, 2, 384), (1, 1, 512), (1, 4, 33)])
+@pytest.mark.parametrize("shape", [(1, 12, 128), (2, 3, 77), (1, 2, 384), (1, 1, 512), (1, 4, 33), (1, 2, 129), (2, 2, 200), (1, 3, 257), (1, 2, 300), (1, 1, 385), (1, 1, 450)])
 def test_fused_attention_matches_composed_oracle(gp, dt, shape):
     """softmax(Q K^T / sqrt(d)) V over the heads of a packed QKV buffer, against the oracle's
     batched-matmul / softmax / batched-matmul composition (fp64 softmax on unrounded scores)."""
@@ -288,7 +288,7 @@ def test_fused_attention_matches_composed_oracle(gp, dt, shape):
     pr = np.exp(sc)
     pr /= pr.sum(-1, keepdims=True)
     ref = np.einsum("bhij,bjhd->bihd", pr, v)
-    assert info.total_tiles == -(-S // 128) * B * Hh
+    assert info.total_tiles == -(-S // (128 if S <= 128 else 64)) * B * Hh  # longer sequences: 64 queries per tile, keys split over two waves
     assert np.isfinite(got).all()
     assert rel_err(got, ref) < TOL[dt], (dt, shape)
 
