@@ -142,9 +142,9 @@ __device__ __forceinline__ void attention_tile(const AttnArgs &a, TileIdx t, T *
         }
 }
 
-// ---- longer sequences: 64 queries per tile, the keys split between two wavefronts -----------------
-// Beyond 128 keys a (batch, head) pair has too few 128-query tiles to fill the GPU and a wavefront
-// too long a chain of work (12 heads x 3 tiles at 384 keys).  Here a tile is 64 queries; waves 0 and
+// ---- the stand-alone kernel: 64 queries per tile, the keys split between two wavefronts -----------
+// A (batch, head) pair has too few 128-query tiles to fill the GPU and a wavefront too long a chain
+// of work (12 heads x 1 tile at 128 keys, x 3 at 384).  Here a tile is 64 queries; waves 0 and
 // 1 take the first half of the key blocks for query rows 0-31 and 32-63, waves 2 and 3 the second
 // half.  Each wave runs the same S^T / softmax / P V sequence on its keys with its own running
 // maximum (probabilities left unnormalised), the second pair parks its partial result in LDS and
@@ -285,15 +285,15 @@ template <typename T, int NB>
 __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a, BlpArgs blp) {
     extern __shared__ __attribute__((aligned(16))) unsigned char att_lds[];
     tile_loop(blp, [&](TileIdx t) {
-        if constexpr (NB <= 4) attention_tile<T, NB>(a, t, reinterpret_cast<T *>(att_lds));
+        if constexpr (NB < 4) attention_tile<T, NB>(a, t, reinterpret_cast<T *>(att_lds));
         else attention_tile_split<T, NB>(a, t, reinterpret_cast<T *>(att_lds));
     });
 }
 // queries per tile and LDS bytes of the class a sequence length falls into
-__host__ __device__ inline int attention_queries_per_tile(int seq) { return attention_nb_class(seq) <= 4 ? ATT_QB : ATT_QB_SPLIT; }
+__host__ __device__ inline int attention_queries_per_tile(int seq) { return attention_nb_class(seq) < 4 ? ATT_QB : ATT_QB_SPLIT; }
 __host__ __device__ inline size_t attention_class_lds_bytes(int seq) {
     const int nb = attention_nb_class(seq);
-    return nb <= 4 ? attention_lds_bytes(nb) : attention_split_lds_bytes(nb);
+    return nb < 4 ? attention_lds_bytes(nb) : attention_split_lds_bytes(nb);
 }
 
 }  // namespace gp

@@ -125,7 +125,7 @@ __device__ __forceinline__ void run_layer(const LayerDesc &d, TileIdx t, T *lds)
         case OP_EMBED: { const gp_embed_params a = d.u.embed; embed_tile<T>(a, t); break; }
         case OP_COPY: { const CopyArgs a = d.u.copy; copy_tile(a, t); break; }
         case OP_ATTENTION:
-            if constexpr (sizeof(T) == 2) { const AttnArgs a = d.u.attn; attention_tile<T, 4>(a, t, lds); }  // seq <= 128 only
+            if constexpr (sizeof(T) == 2) { const AttnArgs a = d.u.attn; attention_tile_split<T, 4>(a, t, lds); }  // seq <= 128 only; the same body as the stand-alone kernel, so that both paths give the same bits
             break;
     }
 }
