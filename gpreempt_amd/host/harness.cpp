@@ -17,6 +17,7 @@
 #include <cstring>
 #include <condition_variable>
 #include <memory>
+#include <map>
 #include <mutex>
 #include <queue>
 #include <thread>
@@ -54,6 +55,8 @@ struct Load {
     std::vector<int64_t> trace_ms;  // "trace": arrival times in milliseconds from the start (load.cpp:239-248)
     size_t next_trace = 0;
     int64_t begin = 0;
+    int load_priority = 0;      // the load's own "priority" key: only loads with 0 are staggered (load.cpp:58-61)
+    int64_t launch_delay = 0;   // "periodic": set by the coordinator (load.cpp:47-69)
 
     int64_t gap_ns() {
         if (type == "poisson") {  // exponential gaps: -ln(u) / frequency (load.cpp:230-237)
@@ -64,7 +67,8 @@ struct Load {
         return (int64_t)(1e9 / frequency);
     }
     void start(int64_t begin_, int64_t end_) {
-        next = begin = begin_; end = end_;
+        begin = begin_; end = end_;
+        next = begin + (type == "periodic" ? launch_delay : 0);
         rng = numeric::Rng(seed);
         next_trace = 0;
         std::sort(trace_ms.begin(), trace_ms.end());
@@ -594,6 +598,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         t->load.frequency = l["frequency"].number(0);
         t->load.seed = (uint64_t)l["seed"].number(1 + (double)tenants.size());
         for (const json::Value &v : l["trace"].arr) t->load.trace_ms.push_back((int64_t)v.number(0));
+        t->load.load_priority = (int)l["priority"].number(0);
         if (sh.policy == "lco" && t->priority != 0) continue;  // rtonlyclient.cpp:120-141: keep the real-time tasks only
         max_prio = std::max(max_prio, t->priority);
         tenants.push_back(std::move(t));
@@ -623,6 +628,20 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         sh.preempt_latency = Stats();
     }
     sh.hp_busy_ns = 0;
+    // DISB's load coordinator (load.cpp:47-69): periodic loads of one frequency do not all fire at
+    // the same instant; each starts later than the one before by the sum of that one's stand-alone
+    // latencies ("stagger": false keeps them aligned)
+    if (cfg["stagger"].boolean(true)) {
+        std::map<long, int64_t> delay_by_freq;
+        for (auto &t : tenants) {
+            if (t->load.type != "periodic" || t->load.load_priority > 0) continue;
+            const long f = (long)t->load.frequency;
+            t->load.launch_delay = delay_by_freq[f];
+            double sum_us = 0;
+            for (double v : t->standalone.v) sum_us += v;
+            delay_by_freq[f] += (int64_t)(sum_us * 1e3);
+        }
+    }
 
     // co-run
     for (auto &t : tenants) if (t->priority == 0) sh.hp_unfinished.fetch_add(1);
