@@ -85,7 +85,7 @@ def probe(workload, trials):
             "isolated_ms": r["isolated(us)"]["mean"] / 1e3,
             "preemption_latency_us": {k: r["preemptLatency(us)"][k] for k in ("mean", "p50", "p99", "max")},
             "resume_call_us": {k: r["resumeCall(us)"][k] for k in ("mean", "p99", "max")},
-            "slowest_kernels": [{"kernel": k["kernel"], "name": k["name"], "tiles": k["tiles"], "preempt_max_us": k["preempt_max(us)"]} for k in worst]}
+            "slowest_kernels": [{"kernel": k["kernel"], "name": k["name"], "preempt_max_us": k["preempt_max(us)"]} for k in worst]}
 
 
 def roofline(workload, iters, dt):

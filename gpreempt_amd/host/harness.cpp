@@ -789,7 +789,8 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
         json::Value o = json::Value::object();
         o.set("kernel") = i;
         o.set("name") = model->get_kernel_info(i).name;
-        o.set("tiles") = model->get_kernel_info(i).total_blocks;
+        // known once the kernel has been launched on its own (not when the whole model runs as one program)
+        if (model->get_kernel_info(i).total_blocks > 0) o.set("tiles") = model->get_kernel_info(i).total_blocks;
         o.set("samples") = per_kernel[i].v.size();
         o.set("preempt_mean(us)") = per_kernel[i].mean();
         o.set("preempt_max(us)") = per_kernel[i].max();
