@@ -58,7 +58,6 @@ GPUdeviceptr PreemptDomain::flag_for(int priority) const {
 
 // word j is up while any request of a level <= j is active
 void PreemptDomain::update() {
-    std::lock_guard<std::mutex> g(mu_);
     int run = 0;
     for (int j = 0; j + 1 < levels_; ++j) {
         run += active_[j].load();
@@ -73,6 +72,12 @@ void PreemptDomain::update() {
 void PreemptDomain::begin(int priority) {
     int p = std::min(priority, levels_ - 1);
     if (p + 1 >= levels_) return;  // the lowest level preempts nobody
+    std::lock_guard<std::mutex> g(mu_);
+    // the time stamp goes first: whoever sees the request counted must not pair it with the
+    // stamp of an earlier raise
+    const int64_t now = steady_ns();
+    for (int j = p; j + 1 < levels_; ++j)
+        if (*host_[j] == 0) raised_[j].store(now);
     active_[p].fetch_add(1, std::memory_order_acq_rel);
     update();
 }
@@ -80,6 +85,7 @@ void PreemptDomain::begin(int priority) {
 void PreemptDomain::end(int priority) {
     int p = std::min(priority, levels_ - 1);
     if (p + 1 >= levels_) return;
+    std::lock_guard<std::mutex> g(mu_);
     active_[p].fetch_sub(1, std::memory_order_acq_rel);
     update();
 }

@@ -222,7 +222,20 @@ struct Shared {
     std::mutex seq_mu;
     std::mutex stats_mu;
     Stats preempt_latency;                  // flag store -> lower-priority stream drained
-    std::atomic<int64_t> hp_busy_ns{0};
+    // busy_above[L]: time during which at least one request of a level above L (a smaller number)
+    // was being served: what a continuous tenant of level L could not have used
+    std::mutex busy_mu;
+    int serving_above[kMaxLevels] = {};
+    int64_t busy_since[kMaxLevels] = {};
+    int64_t busy_above[kMaxLevels] = {};
+    void serving(int p, int delta) {
+        const int64_t now = now_ns();
+        std::lock_guard<std::mutex> g(busy_mu);
+        for (int l = p + 1; l < levels; ++l) {
+            if (delta > 0 && serving_above[l]++ == 0) busy_since[l] = now;
+            if (delta < 0 && --serving_above[l] == 0) busy_above[l] += now - busy_since[l];
+        }
+    }
     std::atomic<int> cores{0};
     long hp_requests = 0;                   // > 0: the run ends once every priority-0 tenant served this many
     std::atomic<int> hp_unfinished{0};
@@ -409,15 +422,15 @@ Status infer(Tenant &t, Shared &sh) {
     }
     if (!is_wb(pol)) {  // "np", "lco" and anything unknown
         // baseclient.cpp: every tenant submits on its own stream, nothing is preempted
-        int64_t t0 = now_ns();
-        RETURN_STATUS(t.ex->execute(t.stream));
-        RETURN_STATUS(drain(t.stream));
-        if (p == 0) sh.hp_busy_ns.fetch_add(now_ns() - t0);
-        return Status::Succ;
+        sh.serving(p, +1);
+        Status st = t.ex->execute(t.stream);
+        if (st == Status::Succ) st = drain(t.stream);
+        sh.serving(p, -1);
+        return st;
     }
     // ---- "wb": cooperative block-level preemption ------------------------------------------
     // (the request was announced by begin_request(): the flag words of every lower level are up)
-    int64_t t0 = now_ns();
+    sh.serving(p, +1);
     // "wb" / "wb-chunk": wait until lower-priority work has left the GPU (blpclient.cpp:189);
     // "wb-async" submits at once and lets the hardware start workgroups as the others retire.
     if (!is_async(pol)) while (sh.on_gpu_below(p) > 0) spin_pause();
@@ -477,7 +490,7 @@ Status infer(Tenant &t, Shared &sh) {
         t.blp->running = false;
         sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
     }
-    if (p == 0) sh.hp_busy_ns.fetch_add(now_ns() - t0);
+    sh.serving(p, -1);
     return st;
 }
 
@@ -627,7 +640,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         std::lock_guard<std::mutex> g(sh.stats_mu);
         sh.preempt_latency = Stats();
     }
-    sh.hp_busy_ns = 0;
+    for (int l = 0; l < kMaxLevels; ++l) sh.serving_above[l] = 0, sh.busy_above[l] = 0;
     // DISB's load coordinator (load.cpp:47-69): periodic loads of one frequency do not all fire at
     // the same instant; each starts later than the one before by the sum of that one's stand-alone
     // latencies ("stagger": false keeps them aligned)
@@ -660,7 +673,8 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     jt = json::Value::object();
     double hp_ratio = 0, be_kept = 0;
     int n_hp = 0, n_be = 0;
-    double busy_frac = std::min(1.0, sh.hp_busy_ns.load() / 1e9 / std::max(wall_s, 1e-9));
+    auto busy_fraction = [&](int level) { return std::min(1.0, sh.busy_above[std::min(std::max(level, 1), sh.levels - 1)] / 1e9 / std::max(wall_s, 1e-9)); };
+    double busy_frac = busy_fraction(1);
     Status result = Status::Succ;
     for (auto &t : tenants) {
         json::Value &o = jt.set(t->id);
@@ -689,8 +703,9 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
             ++n_hp;
         } else if (t->load.type == "continuous") {
             // throughput the idle gaps allow = isolated throughput x fraction of time without a
-            // high-priority request on the GPU
-            double allowed = alone_thr * (1.0 - busy_frac);
+            // request of a higher level being served
+            double allowed = alone_thr * (1.0 - busy_fraction(t->priority));
+            o.set("higher_levels_busy_fraction") = busy_fraction(t->priority);
             double kept = allowed > 0 ? thr / allowed : 0;
             o.set("throughput_kept") = kept;
             be_kept += kept;
