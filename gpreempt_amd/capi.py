@@ -22,12 +22,12 @@ vp = C.c_void_p
 
 class PreemptCtx(C.Structure):
     _fields_ = [("flag", vp), ("stop_index", vp), ("executed", vp), ("kernel_id", C.c_int),
-                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("left_host", vp),
+                ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("fresh", C.c_int), ("left_host", vp),
                 ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong)]
 
 
 class LaunchInfo(C.Structure):
-    _fields_ = [("total_tiles", C.c_int), ("shape", C.c_int * 3), ("grid", C.c_int), ("block", C.c_int)]
+    _fields_ = [("total_tiles", C.c_int), ("shape", C.c_int * 3), ("grid", C.c_int), ("block", C.c_int), ("fixed_claims", C.c_int)]
 
 
 class GemmParams(C.Structure):
@@ -298,10 +298,10 @@ class BlpState:
     def reset(self):
         self.executed.upload(np.zeros(self.n * self.ints_per_kernel, np.int32))
 
-    def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0):
+    def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0, fresh=0):
         ck = getattr(self, "ckpt", None)
         return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id * self.ints_per_kernel, kernel_id, inject_at, max_workgroups,
-                          poll_every, self.groups if self.groups > 1 else 0, None, ck.ptr if ck else None, ck.nbytes if ck else 0)
+                          poll_every, self.groups if self.groups > 1 else 0, fresh, None, ck.ptr if ck else None, ck.nbytes if ck else 0)
 
     def enable_checkpoints(self, params):
         """Allocates the workspace that lets the GEMM `params` leave its tiles half-way (if it can)."""

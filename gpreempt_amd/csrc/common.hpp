@@ -59,6 +59,7 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
         blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;
         blp->kernel_id = ctx->kernel_id; blp->inject_at = ctx->inject_at;
+        blp->fresh = ctx->fresh != 0;
         int pe = ctx->poll_every > 0 ? ctx->poll_every : 8;
         GP_REQUIRE((pe & (pe - 1)) == 0, "poll_every must be a power of two");
         blp->poll_mask = pe - 1;
@@ -74,12 +75,13 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         if (*grid < blp->groups) *grid = blp->groups;  // every counter needs a workgroup to serve its slice
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
-        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1;
+        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0;
         *grid = (int)total;
     }
     if (info) {
         info->total_tiles = (int)total; info->shape[0] = sx; info->shape[1] = sy; info->shape[2] = sz;
         info->grid = *grid; info->block = block;
+        info->fixed_claims = fixed_claims(ctx != nullptr, blp->groups, *grid, (int)total);
     }
     return GP_SUCC;
 }

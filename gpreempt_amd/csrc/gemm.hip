@@ -65,6 +65,7 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     if (rc) return rc;
     blp.order = pl.order;
     if constexpr (K_is_ckpt<K>::value) {
+        if (info) info->fixed_claims = 0;  // tile_loop_ckpt always claims through the counters
         // mid-tile checkpoints need the caller's workspace and a slot per workgroup
         if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES, grid) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
     }
@@ -273,7 +274,9 @@ extern "C" int gp_launch_conv2d(const gp_conv_params *p, const gp_preempt_ctx *c
 #ifdef GP_TILE_PROF
 extern "C" int gp_debug_tile_prof(unsigned long long *out, int n) {
     GP_HIP(hipDeviceSynchronize());
-    GP_HIP(hipMemcpyFromSymbol(out, HIP_SYMBOL(gp::g_tile_prof), sizeof(unsigned long long) * (size_t)n));
+    const int body = n < 256 * 8 ? n : 256 * 8;
+    GP_HIP(hipMemcpyFromSymbol(out, HIP_SYMBOL(gp::g_tile_prof), sizeof(unsigned long long) * (size_t)body));
+    if (n > body) GP_HIP(hipMemcpyFromSymbol(out + body, HIP_SYMBOL(gp::g_disp_prof), sizeof(unsigned long long) * (size_t)std::min(n - body, 256 * 8)));
     return GP_SUCC;
 }
 #endif

@@ -24,6 +24,18 @@
 
 namespace gp {
 
+// Optional timestamps of the dispatcher's steps in the first workgroups (compile with
+// -DGP_TILE_PROF; gp_debug_tile_prof returns them after the bodies' own slots).
+#ifdef GP_TILE_PROF
+static __device__ unsigned long long g_disp_prof[256 * 8];
+#define GP_DISP_PROBE(p)                                                             \
+    do {                                                                             \
+        if (threadIdx.x == 0 && blockIdx.x < 256) g_disp_prof[blockIdx.x * 8 + (p)] = __builtin_amdgcn_s_memtime(); \
+    } while (0)
+#else
+#define GP_DISP_PROBE(p) do { } while (0)
+#endif
+
 struct BlpArgs {
     int *flag;        // nullptr: never preempted
     int *stop_index;
@@ -38,6 +50,7 @@ struct BlpArgs {
     void *ckpt;       // checkpoint workspace of kernels that can leave a tile half-way, or nullptr
     int batch;        // tiles per claim (>= 1): a claim of index u stands for tiles [u*batch, (u+1)*batch)
     int tiles;        // number of tiles (total = ceil(tiles / batch) claims)
+    int fresh;        // the host vouches that no claim of this kernel has been made since its counters were cleared
 };
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
@@ -102,6 +115,39 @@ __device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_l
     return claim;
 }
 
+// ---- one claim per workgroup: fixed claims ------------------------------------------------------
+// When a launch has at least as many workgroups as claims, nobody needs to be told which claim is
+// next: workgroup b takes claim xcd_contiguous(b, total), the mapping of launches without
+// counters.  What a relaunch has to know is which of these were made before, so words 1..15 of
+// the 64-byte line of the workgroup's counter hold a bit per workgroup of that group, and word 0
+// keeps counting claims for the host.  On a kernel's first launch after its counters were cleared
+// (BlpArgs::fresh) every bit is known to be clear: the bit is set and the count raised without
+// waiting for the old values.  No slice boundaries are needed either; computing them cost more
+// than the claim itself (2 us of scalar arithmetic and instruction fetch in front of the first
+// operand load of every launch).
+static_assert(kFixedClaimBits == (COUNTER_STRIDE - 1) * 32, "a bit per workgroup in ints 1..15 of the counter's line");
+
+__device__ __forceinline__ int claim_fixed(const BlpArgs &b, int grp) {
+    if ((int)blockIdx.x >= b.total) return -1;
+    if (__hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1) return -1;
+    const int j = (int)blockIdx.x >> log2_pow2(b.groups);  // this workgroup's rank among those of its group
+    int *line = b.executed + grp * COUNTER_STRIDE;
+    const int bit = 1 << (j & 31);
+    if (b.fresh) {
+        __hip_atomic_fetch_or(line + 1 + (j >> 5), bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else if (__hip_atomic_fetch_or(line + 1 + (j >> 5), bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & bit) {
+        return -1;  // made in an earlier launch
+    }
+    __hip_atomic_fetch_add(line, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int claim = xcd_contiguous((int)blockIdx.x, b.total);
+    if (claim == b.inject_at && b.flag)
+        __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+    if ((grp < 4 || b.poll_mask == 0) && (j & b.poll_mask) == 0 && b.flag &&
+        __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
+        atomicCAS(b.stop_index, -1, b.kernel_id);
+    return claim;
+}
+
 // Runs body(TileIdx) for every tile this workgroup obtains.  All threads of the workgroup must
 // call it; the body may use barriers freely.
 template <class Body>
@@ -113,11 +159,16 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     // serve it (util/slice_map.h), so nobody can get a second claim, on a first launch or on a
     // relaunch, and the claim that would only report "nothing left" (an atomic and a barrier at
     // the tail of every small kernel) is skipped.
+    GP_DISP_PROBE(0);
     const bool single = (int)gridDim.x >= b.total;
+    const bool fixed = fixed_claims(dynamic, b.groups, (int)gridDim.x, b.total);
     // which counter this workgroup serves and the slice of the tile order that counter owns
     const int grp = wg_group((int)blockIdx.x, b.groups);
-    const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
-    const int slice_n = (b.groups > 1 ? group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) : b.total) - slice_lo;
+    int slice_lo = 0, slice_n = b.total;
+    if (b.groups > 1 && !fixed) {
+        slice_lo = group_slice_begin(b.total, grp, b.groups, (int)gridDim.x);
+        slice_n = group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) - slice_lo;
+    }
     // One loop and one call site for both modes, so that the body is inlined into the kernel and
     // the kernel arguments stay in scalar registers.
     for (int it = 0;; ++it) {
@@ -125,10 +176,13 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
         if (!dynamic) {
             idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
         } else {
-            if (leader) mailbox[it & 1] = claim_tile(b, grp, slice_lo, slice_n);
+            if (it == 0) GP_DISP_PROBE(1);
+            if (leader) mailbox[it & 1] = fixed ? claim_fixed(b, grp) : claim_tile(b, grp, slice_lo, slice_n);
+            if (it == 0) GP_DISP_PROBE(2);
             __syncthreads();
             idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1]);  // wave-uniform: tile coordinates stay scalar
         }
+        if (it == 0) GP_DISP_PROBE(3);
         if (idx < 0) return;
         // Streaming kernels have tiles of a few KB; handing them out several at a time keeps the
         // claim (an atomic and a barrier, 1-2 us) off their critical path.
@@ -147,14 +201,18 @@ __device__ __forceinline__ void tile_loop_span(const BlpArgs &b, Body &&body) {
     const bool dynamic = b.executed != nullptr;
     const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
     const int grp = wg_group((int)blockIdx.x, b.groups);
-    const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
-    const int slice_n = (b.groups > 1 ? group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) : b.total) - slice_lo;
+    const bool fixed = fixed_claims(dynamic, b.groups, (int)gridDim.x, b.total);
+    int slice_lo = 0, slice_n = b.total;
+    if (b.groups > 1 && !fixed) {
+        slice_lo = group_slice_begin(b.total, grp, b.groups, (int)gridDim.x);
+        slice_n = group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) - slice_lo;
+    }
     for (int it = 0;; ++it) {
         int idx;
         if (!dynamic) {
             idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
         } else {
-            if (leader) mailbox[it & 1] = claim_tile(b, grp, slice_lo, slice_n);
+            if (leader) mailbox[it & 1] = fixed ? claim_fixed(b, grp) : claim_tile(b, grp, slice_lo, slice_n);
             __syncthreads();
             idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1]);
         }

@@ -142,6 +142,7 @@ void Executor::capture_graph(GPUstream stream) {
         return;
     }
     if (gp_graph_begin(stream) != 0) return;
+    model->counters_cleared(false);
     bool ok = true;
     for (size_t i = 0; i < get_kernel_num() && ok; i++) ok = launch_kernel(i, stream) == Status::Succ;
     gp_graph g = nullptr;
@@ -297,6 +298,8 @@ Status BLPExecutor::reset_counters(GPUstream stream) {
     if (graph_compute) return Status::Succ;
     CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride, stream));
     if (ckpt) CUDA_RETURN_STATUS(gp_ckpt_reset_async(ckpt, stream));  // a fresh run has no tile to continue
+    // launches recorded into a graph are replayed with the arguments of the recording: never fresh
+    model->counters_cleared(!use_cuda_graph);
     return Status::Succ;
 }
 
@@ -320,6 +323,11 @@ Status BLPExecutor::read_counters(std::vector<int> &out) {
         if (model->counter_groups() == 1) { out[i] = raw[i]; continue; }
         // slices follow the workgroup distribution of the last launch (device layer, tile_loop.hpp)
         const long grid = std::max<long>(1, model->get_kernel_info(i).launch_params[0]);
+        if (model->get_kernel_info(i).fixed_claims) {  // int 0 of every line is an exact count
+            for (int g = 0; g < kCounterGroups; ++g) sum += raw[(i * kCounterGroups + g) * kCounterStride];
+            out[i] = (int)sum;
+            continue;
+        }
         auto begin = [&](int g) { return (long)gp::group_slice_begin((int)total, g, kCounterGroups, (int)grid); };
         for (int g = 0; g < kCounterGroups; ++g) {
             long size = begin(g + 1) - begin(g);

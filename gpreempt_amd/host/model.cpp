@@ -339,6 +339,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.max_workgroups = 0;
         ctx.poll_every = poll_every_;
         ctx.counter_groups = counter_groups_;
+        ctx.fresh = idx < fresh_.size() && fresh_[idx];
         ctx.ckpt = ckpt_;
         ctx.ckpt_bytes = ckpt_bytes_;
         pc = &ctx;
@@ -358,8 +359,10 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         case OpKind::Stencil: rc = gp_launch_miniweather(&k.p.miniweather, pc, stream, &info); break;
         case OpKind::Nop: break;
     }
+    if (idx < fresh_.size()) fresh_[idx] = 0;  // launched (or refused): from here on only its counters know
     CUDA_RETURN_STATUS(rc);
     k.total_blocks = info.total_tiles;
+    k.fixed_claims = info.fixed_claims != 0;
     k.launch_params[0] = (uint32_t)info.grid; k.launch_params[1] = 1; k.launch_params[2] = 1;
     k.launch_params[3] = (uint32_t)info.block; k.launch_params[4] = 1; k.launch_params[5] = 1;
     return Status::Succ;

@@ -114,6 +114,11 @@ typedef struct gp_preempt_ctx {
                      /* n > 1: executed points at n counters spaced 16 ints (64 bytes) apart;     */
                      /* workgroup w claims from counter w % n, which owns a contiguous slice of   */
                      /* the tiles.  Spreads the claim atomics, which serialise on one address.   */
+    int fresh;       /* nonzero: the caller vouches that this kernel has not been launched since its    */
+                     /* counters were last cleared.  With counter_groups > 1 a launch of at least as   */
+                     /* many workgroups as claims then records its claims (a bit per workgroup in      */
+                     /* ints 1..15 of each counter's 64 bytes, the count in int 0) without waiting     */
+                     /* for the old values; 0 is always safe.  Clear all 16 ints of every counter.     */
     int *left_host;  /* programs only, may be NULL: device-visible address of a gp_flag_create    */
                      /* word; the last workgroup to leave a launch stores that launch's number    */
                      /* (info->shape[1] of gp_program_launch) there, so the host learns that the  */
@@ -133,6 +138,8 @@ typedef struct gp_launch_info {
     int shape[3];       /* = dim3 shape of the reference (tile grid)          */
     int grid;           /* workgroups launched                                */
     int block;          /* threads per workgroup                              */
+    int fixed_claims;   /* 1: claims were fixed by workgroup index and recorded as bits (see  */
+                        /* gp_preempt_ctx::fresh); 0: handed out through the counters          */
 } gp_launch_info;
 
 /* ---- operators ---------------------------------------------------------------------------

@@ -70,6 +70,7 @@ public:
     // block-level preemption arguments (reference model.cpp:366-396)
     bool preemptible = false;
     int total_blocks = 0;
+    bool fixed_claims = false;            // how the last launch recorded its claims (gp_launch_info)
     GPUdeviceptr executed = nullptr;
     int kernel_id = 0;
     double flops = 0, bytes = 0;          // algorithmic work of one launch
@@ -121,6 +122,10 @@ public:
     // arguments added with batchAddParam.  inject_at is a test hook (-1 = off).
     Status launch(size_t idx, GPUstream stream, int inject_at = -1);
     void set_poll_every(int n) { poll_every_ = n; }
+    // The claim counters have just been cleared (or are about to be, earlier on the same stream):
+    // until its next launch every kernel is known to have made no claim (gp_preempt_ctx::fresh).
+    // `on` = false withdraws that for all kernels (launches that are recorded and replayed).
+    void counters_cleared(bool on) { fresh_.assign(kernel_infos.size(), on ? 1 : 0); }
     // device-visible address of a host word that a program's last leaving workgroup sets to the
     // launch number returned by launch_program()
     void set_left_word(GPUdeviceptr p) { left_word_ = p; }
@@ -152,6 +157,7 @@ private:
     gp_program program_ = nullptr;
     int counter_groups_ = 1;
     int poll_every_ = 0;
+    std::vector<char> fresh_;
     GPUdeviceptr left_word_ = nullptr;
     GPUdeviceptr ckpt_ = nullptr;
     size_t ckpt_bytes_ = 0;

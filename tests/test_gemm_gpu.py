@@ -189,6 +189,86 @@ def test_flag_set_before_launch(gp):
         gp.launch("gp_launch_gemm", p, st.ctx(poll_every=3))
 
 
+def test_fixed_claims_of_a_one_claim_per_workgroup_launch(gp):
+    """With several counters per kernel and at least as many workgroups as claims, a workgroup's
+    claim is fixed by its index and a bit per workgroup (ints 1..15 of the counter's line) says
+    whether it was made; int 0 counts.  A first launch (fresh) sets them without looking; a relaunch
+    runs exactly the claims whose bits are clear."""
+    A, B, bias, p, dC, keep = _config1(gp, 64)
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    base = dC.download(gp.F32, (1024, 1024)).copy()
+    flag = gp.Flag()
+    G = 32
+    st = gp.BlpState(1, flag, G)
+
+    def lines():
+        return st.counters().reshape(G, 16).copy()
+
+    def popcount(a):
+        return int(np.unpackbits(a.view(np.uint8)).sum())
+
+    def tiles_written():
+        c = dC.download(gp.F32, (1024, 1024)).reshape(16, 64, 16, 64)
+        return int((~np.isnan(c).any(axis=(1, 3))).sum())
+
+    dC.fill32(0xFFFFFFFF)
+    info = gp.launch("gp_launch_gemm", p, st.ctx(fresh=1))
+    gp.check(gp.lib().gp_stream_sync(None))
+    total = info.total_tiles
+    assert total == 256 and info.grid >= total, "the launch must have a workgroup per claim for this test"
+    assert np.array_equal(dC.download(gp.F32, (1024, 1024)), base)
+    full = lines()
+    assert full[:, 0].sum() == total and popcount(full[:, 1:]) == total and st.stop_index() == -1
+    # a second launch finds every claim made
+    dC.fill32(0xFFFFFFFF)
+    gp.launch("gp_launch_gemm", p, st.ctx())
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert tiles_written() == 0 and np.array_equal(lines(), full)
+    # a random half of the claims marked as made: the relaunch runs the others, once each
+    rng = np.random.default_rng(5)
+    bits = np.unpackbits(full[:, 1:].copy().view(np.uint8).reshape(G, -1), axis=1)
+    keep_mask = (rng.random(bits.shape) < 0.5).astype(np.uint8)
+    made = bits & keep_mask
+    state = np.zeros_like(full)
+    state[:, 1:] = np.packbits(made, axis=1).view(np.int32).reshape(G, 15)
+    state[:, 0] = made.sum(axis=1)
+    n_made = int(made.sum())
+    assert 0 < n_made < total
+    st.executed.upload(state.reshape(-1))
+    gp.launch("gp_launch_gemm", p, st.ctx())
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert tiles_written() == total - n_made
+    assert np.array_equal(lines(), full)
+    # ... and the complement fills in the rest: every claim stands for a tile of its own
+    rest = bits & (1 - keep_mask)
+    state[:, 1:] = np.packbits(rest, axis=1).view(np.int32).reshape(G, 15)
+    state[:, 0] = rest.sum(axis=1)
+    st.executed.upload(state.reshape(-1))
+    gp.launch("gp_launch_gemm", p, st.ctx())
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert np.array_equal(dC.download(gp.F32, (1024, 1024)), base)
+    # a stop recorded by an earlier kernel: nothing is claimed, fresh or not
+    st.reset()
+    st.stop.upload(np.array([7], np.int32))
+    dC.fill32(0xFFFFFFFF)
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0, fresh=1))
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert tiles_written() == 0 and not lines().any() and st.stop_index() == 7
+    # the flag up at launch: the polling workgroups record the stop, a relaunch completes the work
+    st.clear_stop()
+    flag.set(1)
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0, fresh=1))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert st.stop_index() == 0
+    flag.set(0)
+    st.clear_stop()
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert np.array_equal(dC.download(gp.F32, (1024, 1024)), base) and np.array_equal(lines(), full)
+
+
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("tile,variant", [(128, 2), (64, 2), (64, 3), (32, 3)])
 def test_pipelined_gemm_preempt_resume_bit_exact(gp, dt, tile, variant):
