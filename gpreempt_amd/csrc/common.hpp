@@ -73,9 +73,15 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         if (ctx->max_workgroups > 0 && resident > ctx->max_workgroups) resident = ctx->max_workgroups;
         *grid = (int)(total < resident ? total : resident);
         if (*grid < blp->groups) *grid = blp->groups;  // every counter needs a workgroup to serve its slice
+        // a launch with fixed claims gets four workgroups more, which only read the flag (tile_loop.hpp)
+        blp->spare = 0;
+        if (ctx->flag && blp->poll_mask != 0 && fixed_claims(true, ng, *grid, (int)total) && fixed_claims(true, ng, *grid + 4, (int)total)) {
+            blp->spare = 4;
+            *grid += 4;
+        }
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
-        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0;
+        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0; blp->spare = 0;
         *grid = (int)total;
     }
     if (info) {

@@ -66,6 +66,7 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     blp.order = pl.order;
     if constexpr (K_is_ckpt<K>::value) {
         if (info) info->fixed_claims = 0;  // tile_loop_ckpt always claims through the counters
+        if (blp.spare) { grid -= blp.spare; blp.spare = 0; if (info) info->grid = grid; }
         // mid-tile checkpoints need the caller's workspace and a slot per workgroup
         if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES, grid) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
     }

@@ -17,7 +17,10 @@
 //  * *stop_index is claimed with a compare-and-swap instead of a test followed by a store, and a
 //    workgroup also leaves when *stop_index is already set (see "Sticky" below);
 //  * with executed == nullptr the same kernel runs non-preemptibly, one workgroup per tile
-//    (the reference builds a second, untransformed module for that: mod.cubin vs mod.tr.cubin).
+//    (the reference builds a second, untransformed module for that: mod.cubin vs mod.tr.cubin);
+//  * a launch that has a workgroup for every claim does not hand claims out through the counter
+//    at all (see "fixed claims" below): the counter keeps counting, a bit per workgroup says
+//    which claims were made.
 #pragma once
 #include <hip/hip_runtime.h>
 #include "../../include/util/slice_map.h"
@@ -51,6 +54,7 @@ struct BlpArgs {
     int batch;        // tiles per claim (>= 1): a claim of index u stands for tiles [u*batch, (u+1)*batch)
     int tiles;        // number of tiles (total = ceil(tiles / batch) claims)
     int fresh;        // the host vouches that no claim of this kernel has been made since its counters were cleared
+    int spare;        // fixed claims only: the last `spare` workgroups of the grid have no claim and read the flag
 };
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
@@ -142,10 +146,22 @@ __device__ __forceinline__ int claim_fixed(const BlpArgs &b, int grp) {
     const int claim = xcd_contiguous((int)blockIdx.x, b.total);
     if (claim == b.inject_at && b.flag)
         __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-    if ((grp < 4 || b.poll_mask == 0) && (j & b.poll_mask) == 0 && b.flag &&
+    // (with spare workgroups the flag is theirs to read: nobody's tile waits for host memory)
+    if (b.spare == 0 && (grp < 4 || b.poll_mask == 0) && (j & b.poll_mask) == 0 && b.flag &&
         __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
         atomicCAS(b.stop_index, -1, b.kernel_id);
     return claim;
+}
+
+// A spare workgroup of a launch with fixed claims: reads the flag once on behalf of the launch and
+// leaves.  The read of host memory (1-2 us) then delays nobody's tile, where a poll after the
+// first claims made four workgroups, and with them the kernel, finish that much later.
+__device__ __forceinline__ bool spare_workgroup(const BlpArgs &b, bool fixed, bool leader) {
+    if (!fixed || b.spare == 0 || (int)blockIdx.x < (int)gridDim.x - b.spare) return false;
+    if (leader && b.flag && __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0 &&
+        __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == -1)
+        atomicCAS(b.stop_index, -1, b.kernel_id);
+    return true;
 }
 
 // Runs body(TileIdx) for every tile this workgroup obtains.  All threads of the workgroup must
@@ -169,6 +185,7 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
         slice_lo = group_slice_begin(b.total, grp, b.groups, (int)gridDim.x);
         slice_n = group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) - slice_lo;
     }
+    if (spare_workgroup(b, fixed, leader)) return;
     // One loop and one call site for both modes, so that the body is inlined into the kernel and
     // the kernel arguments stay in scalar registers.
     for (int it = 0;; ++it) {
@@ -207,6 +224,7 @@ __device__ __forceinline__ void tile_loop_span(const BlpArgs &b, Body &&body) {
         slice_lo = group_slice_begin(b.total, grp, b.groups, (int)gridDim.x);
         slice_n = group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) - slice_lo;
     }
+    if (spare_workgroup(b, fixed, leader)) return;
     for (int it = 0;; ++it) {
         int idx;
         if (!dynamic) {

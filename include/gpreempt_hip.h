@@ -109,7 +109,9 @@ typedef struct gp_preempt_ctx {
     int max_workgroups; /* 0 = occupancy-sized persistent grid; >0 caps it                      */
     int poll_every;  /* the claim numbered c reads the host flag when c % poll_every == 0; a power */
                      /* of two; 0 = default (8).  All claims check *stop_index (device memory),   */
-                     /* which the polling workgroup sets, so 1 reproduces a poll per tile         */
+                     /* which the polling workgroup sets, so 1 reproduces a poll per tile.  A      */
+                     /* launch with fixed claims (gp_launch_info) and poll_every != 1 instead gets */
+                     /* four workgroups more that own no claim and read the flag at launch         */
     int counter_groups; /* 0 or 1: *executed is one int (the reference's layout).  A power of two */
                      /* n > 1: executed points at n counters spaced 16 ints (64 bytes) apart;     */
                      /* workgroup w claims from counter w % n, which owns a contiguous slice of   */
