@@ -18,11 +18,12 @@
 
 namespace gp {
 
-template <class TK>
+// LOOP: which dispatcher loop the instantiation is built around (tile_loop.hpp)
+template <class TK, int LOOP>
 __global__ __launch_bounds__(TK::NT) void mat_kernel(MatArgs g, BlpArgs blp) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     auto *lds = reinterpret_cast<typename TK::elem *>(lds_raw);
-    tile_loop(blp, [&](TileIdx t) { TK::run(g, t, lds); });
+    tiles<LOOP>(blp, [&](TileIdx t) { TK::run(g, t, lds); });
 }
 
 // bodies that can leave a tile between two K-steps (tile_loop_ckpt)
@@ -39,9 +40,15 @@ using TK = TileKernel<T, BM, BN, BK, WGM, WGN, CONV, B_KN>;
 
 template <class K> struct K_is_ckpt { static constexpr bool value = false; };
 template <typename T, int BM, int BN, int ST, bool CV> struct K_is_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true>> { static constexpr bool value = true; };
-template <class K> struct KernelOf { static constexpr auto fn = mat_kernel<K>; };
+template <class K> struct KernelOf {
+    static constexpr auto fn = mat_kernel<K, LOOP_ANY>;
+    static constexpr auto plain = mat_kernel<K, LOOP_PLAIN>;
+    static constexpr auto fixed = mat_kernel<K, LOOP_FIXED>;
+};
 template <typename T, int BM, int BN, int ST, bool CV> struct KernelOf<PipeKernel<T, BM, BN, ST, CV, false, true>> {
     static constexpr auto fn = mat_kernel_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true>>;
+    static constexpr auto plain = fn;
+    static constexpr auto fixed = fn;
 };
 
 // bytes of checkpoint workspace a launch of body K needs (0: the body always finishes its tiles)
@@ -53,11 +60,13 @@ template <class K>
 static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     BlpArgs blp;
     int grid = 0;
-    auto kern = KernelOf<K>::fn;
+    auto kern = KernelOf<K>::fn;  // the launch is planned for the general form; the others need no more resources
     if (K::LDS_BYTES > 48 * 1024) {
         static bool once = false;  // benign race: idempotent attribute
         if (!once) {
-            GP_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES));
+            GP_HIP(hipFuncSetAttribute((const void *)KernelOf<K>::fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES));
+            GP_HIP(hipFuncSetAttribute((const void *)KernelOf<K>::plain, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES));
+            GP_HIP(hipFuncSetAttribute((const void *)KernelOf<K>::fixed, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES));
             once = true;
         }
     }
@@ -70,6 +79,9 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
         // mid-tile checkpoints need the caller's workspace and a slot per workgroup
         if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES, grid) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
     }
+    // one tile per claim here (plan_launch's default), which is what the two special forms assume
+    if (!ctx) kern = KernelOf<K>::plain;
+    else if (fixed_claims(true, blp.groups, grid, blp.total)) kern = KernelOf<K>::fixed;  // (not for checkpointing bodies: theirs is fn)
     hipLaunchKernelGGL(kern, dim3(grid), dim3(K::NT), K::LDS_BYTES, native(s), pl.g, blp);
     GP_HIP(hipGetLastError());
     return GP_SUCC;
