@@ -281,10 +281,10 @@ __host__ __device__ inline int attention_nb_class(int seq) {
 
 // One kernel per class: the score registers of the longest class (256 per lane) would otherwise set
 // the register budget, and the scratch memory, of the short sequences too.
-template <typename T, int NB>
+template <typename T, int NB, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(256) void attention_kernel(AttnArgs a, BlpArgs blp) {
     extern __shared__ __attribute__((aligned(16))) unsigned char att_lds[];
-    tile_loop(blp, [&](TileIdx t) {
+    tiles<LOOP>(blp, [&](TileIdx t) {
         if constexpr (NB < 4) attention_tile<T, NB>(a, t, reinterpret_cast<T *>(att_lds));
         else attention_tile_split<T, NB>(a, t, reinterpret_cast<T *>(att_lds));
     });

@@ -7,16 +7,31 @@
 
 namespace gp {
 
+// the three instantiations of one kernel: general dispatcher loop, no counters, fixed claims
+template <class Kernel> struct KernelSet { Kernel any, plain, fixed; };
+template <class Kernel> static KernelSet<Kernel> kernel_set(Kernel a, Kernel p, Kernel f) { return {a, p, f}; }
+#define GP_KSET(...) kernel_set(__VA_ARGS__, LOOP_ANY>, __VA_ARGS__, LOOP_PLAIN>, __VA_ARGS__, LOOP_FIXED>)
+
 template <class Kernel, class Arg>
-static int launch_tiles(Kernel kern, int sx, int sy, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info, const Arg &arg, size_t lds_bytes = 0, int max_batch = 16) {
+static int launch_tiles(KernelSet<Kernel> ks, int sx, int sy, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info, const Arg &arg, size_t lds_bytes = 0, int max_batch = 16) {
     BlpArgs blp;
     int grid = 0;
     // several tiles per claim once there are far more tiles than workgroups that could hold them
     const long tiles = (long)sx * sy;
     const int batch = (int)std::min<long>(max_batch, std::max<long>(1, tiles / (32L * device_cus())));
-    if (lds_bytes > 48 * 1024) GP_HIP(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    int rc = plan_launch(kern, NT, lds_bytes, sx, sy, 1, ctx, &blp, &grid, info, batch);
+    if (lds_bytes > 48 * 1024) {
+        GP_HIP(hipFuncSetAttribute((const void *)ks.any, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        GP_HIP(hipFuncSetAttribute((const void *)ks.plain, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+        GP_HIP(hipFuncSetAttribute((const void *)ks.fixed, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    }
+    // planned for the general form; the special ones need no more resources
+    int rc = plan_launch(ks.any, NT, lds_bytes, sx, sy, 1, ctx, &blp, &grid, info, batch);
     if (rc) return rc;
+    Kernel kern = ks.any;
+    if (batch == 1) {  // the special forms call the body once: one tile per claim only
+        if (!ctx) kern = ks.plain;
+        else if (fixed_claims(true, blp.groups, grid, blp.total)) kern = ks.fixed;
+    }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds_bytes, native(s), arg, blp);
     GP_HIP(hipGetLastError());
     return GP_SUCC;
@@ -165,7 +180,7 @@ int launch_elt_plan(const EltPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
     switch (pl.op) {
         case OP_LAYOUT: {
             const int di = pl.sub / 4, dout = pl.sub % 4;
-#define L(TI, TO) launch_tiles(nchw_to_nhwc_kernel<TI, TO>, pl.sx, pl.sy, ctx, s, info, pl.u.layout)
+#define L(TI, TO) launch_tiles(GP_KSET(nchw_to_nhwc_kernel<TI, TO), pl.sx, pl.sy, ctx, s, info, pl.u.layout)
             if (di == GP_F32 && dout == GP_F32) return L(float, float);
             if (di == GP_F32 && dout == GP_F16) return L(float, _Float16);
             if (di == GP_F32 && dout == GP_BF16) return L(float, __bf16);
@@ -174,21 +189,21 @@ int launch_elt_plan(const EltPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
 #undef L
             break;
         }
-        case OP_POOL: GP_BY_DTYPE(pl.dtype, launch_tiles(pool_kernel<T>, pl.sx, pl.sy, ctx, s, info, pl.u.pool)); break;
-        case OP_ELTWISE: GP_BY_DTYPE(pl.dtype, launch_tiles(eltwise_kernel<T>, pl.sx, pl.sy, ctx, s, info, pl.u.elt)); break;
-        case OP_SOFTMAX: GP_BY_DTYPE(pl.dtype, launch_tiles(softmax_kernel<T>, pl.sx, pl.sy, ctx, s, info, pl.u.softmax)); break;
+        case OP_POOL: GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(pool_kernel<T), pl.sx, pl.sy, ctx, s, info, pl.u.pool)); break;
+        case OP_ELTWISE: GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(eltwise_kernel<T), pl.sx, pl.sy, ctx, s, info, pl.u.elt)); break;
+        case OP_SOFTMAX: GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(softmax_kernel<T), pl.sx, pl.sy, ctx, s, info, pl.u.softmax)); break;
         case OP_LAYERNORM:
-            if (pl.sub == 2) { GP_BY_DTYPE(pl.dtype, launch_tiles(layernorm_kernel<T, 2>, pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
-            else if (pl.sub == 8) { GP_BY_DTYPE(pl.dtype, launch_tiles(layernorm_kernel<T, 8>, pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
-            else { GP_BY_DTYPE(pl.dtype, launch_tiles(layernorm_kernel<T, 16>, pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
+            if (pl.sub == 2) { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 2), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
+            else if (pl.sub == 8) { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 8), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
+            else { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 16), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
             break;
-        case OP_EMBED: GP_BY_DTYPE(pl.dtype, launch_tiles(embed_kernel<T>, pl.sx, pl.sy, ctx, s, info, pl.u.embed)); break;
-        case OP_COPY: return launch_tiles(copy_kernel<0>, pl.sx, pl.sy, ctx, s, info, pl.u.copy);
+        case OP_EMBED: GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(embed_kernel<T), pl.sx, pl.sy, ctx, s, info, pl.u.embed)); break;
+        case OP_COPY: return launch_tiles(GP_KSET(copy_kernel<0), pl.sx, pl.sy, ctx, s, info, pl.u.copy);
         case OP_ATTENTION:
             switch (attention_nb_class(pl.u.attn.p.seq) * 2 + (pl.dtype == GP_F16)) {
 #define GP_ATT(NB)                                                                                                            \
-    case NB * 2 + 1: return launch_tiles(attention_kernel<_Float16, NB>, pl.sx, pl.sy, ctx, s, info, pl.u.attn, pl.lds_bytes); \
-    case NB * 2: return launch_tiles(attention_kernel<__bf16, NB>, pl.sx, pl.sy, ctx, s, info, pl.u.attn, pl.lds_bytes);
+    case NB * 2 + 1: return launch_tiles(GP_KSET(attention_kernel<_Float16, NB), pl.sx, pl.sy, ctx, s, info, pl.u.attn, pl.lds_bytes); \
+    case NB * 2: return launch_tiles(GP_KSET(attention_kernel<__bf16, NB), pl.sx, pl.sy, ctx, s, info, pl.u.attn, pl.lds_bytes);
                 GP_ATT(4) GP_ATT(8) GP_ATT(12) GP_ATT(16)
 #undef GP_ATT
             }
@@ -220,7 +235,7 @@ extern "C" int gp_launch_miniweather(const gp_miniweather_params *p, const gp_pr
     GP_REQUIRE(!update || (p->state_init && p->state_out), "miniweather: update operands missing");
     const int tiles = (int)((mw_ids(p->kernel, p->nx, p->nz) + MW_TILE - 1) / MW_TILE);
     switch (p->kernel) {
-#define GP_MW(K) case K: return launch_tiles(miniweather_kernel<K>, tiles, 1, ctx, s, info, *p);
+#define GP_MW(K) case K: return launch_tiles(GP_KSET(miniweather_kernel<K), tiles, 1, ctx, s, info, *p);
         GP_MW(GP_MW_HALO_X) GP_MW(GP_MW_FLUX_X) GP_MW(GP_MW_UPDATE_X) GP_MW(GP_MW_HALO_Z) GP_MW(GP_MW_FLUX_Z) GP_MW(GP_MW_UPDATE_Z)
 #undef GP_MW
     }
@@ -247,7 +262,7 @@ extern "C" int gp_launch_graph(const gp_graph_params *p, const gp_preempt_ctx *c
     // claims stay small so that a stop is honoured quickly
     const int max_batch = graph_kernel_is_edge_parallel(p->kernel) ? 4 : 16;
     switch (p->kernel * 100 + lanes) {
-#define GP_GR(K, L) case K * 100 + L: return launch_tiles(graph_kernel<K, L>, tiles, 1, ctx, s, info, *p, 0, max_batch);
+#define GP_GR(K, L) case K * 100 + L: return launch_tiles(GP_KSET(graph_kernel<K, L), tiles, 1, ctx, s, info, *p, 0, max_batch);
 #define GP_GR_EDGE(K) GP_GR(K, 16) GP_GR(K, 32) GP_GR(K, 64)
         GP_GR_EDGE(GP_GRAPH_BFS_STEP) GP_GR_EDGE(GP_GRAPH_CC_STEP) GP_GR_EDGE(GP_GRAPH_PR_PUSH) GP_GR_EDGE(GP_GRAPH_SSSP_RELAX)
         GP_GR(GP_GRAPH_PR_INIT, 64) GP_GR(GP_GRAPH_PR_UPDATE, 64) GP_GR(GP_GRAPH_SSSP_UPDATE, 64) GP_GR(GP_GRAPH_CC_INIT, 64)

@@ -112,9 +112,10 @@ __device__ __forceinline__ void layout_tile(const LayoutArgs &a, TileIdx t) {
             VecIO<TO>::st1(dst + c, v);
         }
 }
-template <typename TI, typename TO>
+// (LOOP: which dispatcher form the instantiation is built around, tile_loop.hpp)
+template <typename TI, typename TO, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void nchw_to_nhwc_kernel(LayoutArgs a, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { layout_tile<TI, TO>(a, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { layout_tile<TI, TO>(a, t); });
 }
 
 // ---- pooling, NHWC -------------------------------------------------------------------------
@@ -208,9 +209,9 @@ __device__ __forceinline__ void pool_tile(const PoolArgs &a, TileIdx t) {
         }
         VecIO<T>::store(out + pix * p.out_pix_stride + ch * VEC, acc);
 }
-template <typename T>
+template <typename T, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void pool_kernel(PoolArgs a, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { pool_tile<T>(a, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { pool_tile<T>(a, t); });
 }
 
 // ---- elementwise ---------------------------------------------------------------------------
@@ -256,9 +257,9 @@ __device__ __forceinline__ void eltwise_tile(const EltwiseArgs &a, TileIdx t) {
             VecIO<T>::store((T *)p.out + row * p.out_stride + ch * VEC, a);
         }
 }
-template <typename T>
+template <typename T, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void eltwise_kernel(EltwiseArgs a, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { eltwise_tile<T>(a, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { eltwise_tile<T>(a, t); });
 }
 
 // ---- softmax -------------------------------------------------------------------------------
@@ -346,9 +347,9 @@ __device__ __forceinline__ void softmax_tile(const gp_softmax_params &p, TileIdx
     float inv = 1.f / sum;
     for (int c = lane; c < p.cols; c += 64) VecIO<T>::st1(o + c, __expf(VecIO<T>::ld1(x + c) * p.scale - mx) * inv);
 }
-template <typename T>
+template <typename T, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void softmax_kernel(gp_softmax_params p, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { softmax_tile<T>(p, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { softmax_tile<T>(p, t); });
 }
 
 // ---- layer norm ----------------------------------------------------------------------------
@@ -406,9 +407,9 @@ __device__ __forceinline__ void layernorm_tile(const gp_layernorm_params &p, Til
             }
         }
 }
-template <typename T, int MAXC>
+template <typename T, int MAXC, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void layernorm_kernel(gp_layernorm_params p, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { layernorm_tile<T, MAXC>(p, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { layernorm_tile<T, MAXC>(p, t); });
 }
 
 // ---- embedding -----------------------------------------------------------------------------
@@ -441,9 +442,9 @@ __device__ __forceinline__ void embed_tile(const gp_embed_params &p, TileIdx t) 
             VecIO<T>::store(o + ch * VEC, a);
         }
 }
-template <typename T>
+template <typename T, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void embed_kernel(gp_embed_params p, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { embed_tile<T>(p, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { embed_tile<T>(p, t); });
 }
 
 
@@ -462,9 +463,9 @@ __device__ __forceinline__ void copy_tile(const CopyArgs &a, TileIdx t) {
         else for (long i = off; i < a.bytes; ++i) st_out8(d + i, (unsigned char)s[i]);
     }
 }
-template <int UNUSED = 0>
+template <int UNUSED = 0, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void copy_kernel(CopyArgs a, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { copy_tile(a, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { copy_tile(a, t); });
 }
 
 }  // namespace gp

@@ -124,9 +124,9 @@ __device__ __forceinline__ void graph_tile(const gp_graph_params &p, TileIdx t) 
     }
 }
 
-template <int KIND, int LANES>
+template <int KIND, int LANES, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(GR_TILE) void graph_kernel(gp_graph_params p, BlpArgs blp) {
-    tile_loop(blp, [&](TileIdx t) { graph_tile<KIND, LANES>(p, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { graph_tile<KIND, LANES>(p, t); });
 }
 
 }  // namespace gp

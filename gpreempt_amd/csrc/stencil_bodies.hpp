@@ -267,9 +267,9 @@ __device__ __forceinline__ void mw_span(const gp_miniweather_params &p, int firs
     }
 }
 
-template <int KIND>
+template <int KIND, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(MW_TILE) void miniweather_kernel(gp_miniweather_params p, BlpArgs blp) {
-    tile_loop_span(blp, [&](int first, int last) { mw_span<KIND>(p, first, last); });
+    spans<LOOP>(blp, [&](int first, int last) { mw_span<KIND>(p, first, last); });
 }
 
 }  // namespace gp
