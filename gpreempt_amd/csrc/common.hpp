@@ -72,6 +72,10 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         long resident = (long)per_cu * device_cus();
         if (ctx->max_workgroups > 0 && resident > ctx->max_workgroups) resident = ctx->max_workgroups;
         *grid = (int)(total < resident ? total : resident);
+        // Up to a few waves of workgroups, a workgroup per claim (fixed claims, started by the
+        // hardware as others retire) beats a persistent grid that claims through the counters.
+        if (ng > 1 && ctx->max_workgroups == 0 && total > resident && total <= 4 * resident && total + 4 <= (long)ng * kFixedClaimBits)
+            *grid = (int)total;
         if (*grid < blp->groups) *grid = blp->groups;  // every counter needs a workgroup to serve its slice
         // a launch with fixed claims gets four workgroups more, which only read the flag (tile_loop.hpp)
         blp->spare = 0;
