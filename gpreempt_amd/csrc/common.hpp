@@ -48,7 +48,7 @@ inline size_t dtype_size(int dt) {
 // workgroup per tile.
 template <class Kernel>
 int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int sz,
-                const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info, int batch = 1) {
+                const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info, int batch = 1, int waves = 1) {
     long tiles = (long)sx * sy * sz;
     GP_REQUIRE(tiles > 0 && tiles < (1L << 31), "tile count %ld out of range", tiles);
     if (batch < 1) batch = 1;
@@ -72,14 +72,19 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         long resident = (long)per_cu * device_cus();
         if (ctx->max_workgroups > 0 && resident > ctx->max_workgroups) resident = ctx->max_workgroups;
         *grid = (int)(total < resident ? total : resident);
-        // Up to a few waves of workgroups, a workgroup per claim (fixed claims, started by the
-        // hardware as others retire) beats a persistent grid that claims through the counters.
-        if (ng > 1 && ctx->max_workgroups == 0 && total > resident && total <= 4 * resident && total + 4 <= (long)ng * kFixedClaimBits)
+        // Up to `waves` times the resident workgroups, a workgroup per claim (fixed claims, started
+        // by the hardware as others retire) beats a persistent grid that claims through the
+        // counters: 4 % on ResNet-152 b8.  The caller allows it where tiles are short; with
+        // VGG-16 b16's 128 x 128 tiles it lengthened the drain (p99 130 -> 178 us).
+        if (ng > 1 && ctx->max_workgroups == 0 && total > resident && total <= (long)waves * resident && total + 4 <= (long)ng * kFixedClaimBits)
             *grid = (int)total;
         if (*grid < blp->groups) *grid = blp->groups;  // every counter needs a workgroup to serve its slice
         // a launch with fixed claims gets four workgroups more, which only read the flag (tile_loop.hpp)
         blp->spare = 0;
-        if (ctx->flag && blp->poll_mask != 0 && fixed_claims(true, ng, *grid, (int)total) && fixed_claims(true, ng, *grid + 4, (int)total)) {
+        // (only when the whole grid starts at once: the last workgroups of a longer grid start last,
+        // and a flag read at the end of a kernel stops nothing; there every eighth workgroup of the
+        // first four groups reads it after its claim, as in the general loop)
+        if (ctx->flag && blp->poll_mask != 0 && *grid <= resident && fixed_claims(true, ng, *grid, (int)total) && fixed_claims(true, ng, *grid + 4, (int)total)) {
             blp->spare = 4;
             *grid += 4;
         }

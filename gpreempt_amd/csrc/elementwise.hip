@@ -25,7 +25,7 @@ static int launch_tiles(KernelSet<Kernel> ks, int sx, int sy, const gp_preempt_c
         GP_HIP(hipFuncSetAttribute((const void *)ks.fixed, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
     }
     // planned for the general form; the special ones need no more resources
-    int rc = plan_launch(ks.any, NT, lds_bytes, sx, sy, 1, ctx, &blp, &grid, info, batch);
+    int rc = plan_launch(ks.any, NT, lds_bytes, sx, sy, 1, ctx, &blp, &grid, info, batch, batch == 1 ? 4 : 1);
     if (rc) return rc;
     Kernel kern = ks.any;
     if (batch == 1) {  // the special forms call the body once: one tile per claim only

@@ -70,7 +70,7 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
             once = true;
         }
     }
-    int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info);
+    int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info, 1, K::LDS_BYTES <= 64 * 1024 ? 4 : 1);
     if (rc) return rc;
     blp.order = pl.order;
     if constexpr (K_is_ckpt<K>::value) {
