@@ -218,6 +218,48 @@ def test_every_op_resumes_bit_exact(gp):
         assert st.stop_index() == -1
 
 
+def test_conv2d_fixed_claims_beyond_the_resident_grid(gp):
+    """ResNet's 56 x 56 1x1 layer at batch 8 on the 64 x 64 body: 1568 tiles, more than the
+    workgroups the GPU holds at once, still a workgroup per claim (gp_launch_info::fixed_claims).
+    Claims marked as made are skipped by a relaunch, the others run exactly once, and a first
+    launch that is told so (fresh) marks every claim without looking."""
+    rng = np.random.default_rng(33)
+    N, H, Cin, Cout = 8, 56, 64, 256
+    x = rnd(rng, (N, Cin, H, H), "f16")
+    w = rnd(rng, (Cout, Cin, 1, 1), "f16", -0.2, 0.2)
+    b = rnd(rng, (Cout,), "f16", -0.1, 0.1)
+    want, info0, (p, do, keep) = gpu_conv2d(gp, "f16", x, w, b, 1, 0, None, gp.ACT_RELU, tile=64, variant=2)
+    raw_want = do.download().copy()
+    G = 32
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag, G)
+    do.fill32(0xFFFFFFFF)
+    info = gp.launch("gp_launch_conv2d", p, st.ctx(fresh=1))
+    sync(gp)
+    total = info.total_tiles
+    assert total == 1568 and info.fixed_claims == 1 and total <= info.grid <= total + 4
+    assert np.array_equal(do.download(), raw_want)
+    full = st.counters().reshape(G, 16).copy()
+    popcount = lambda a: int(np.unpackbits(np.ascontiguousarray(a).view(np.uint8)).sum())
+    assert full[:, 0].sum() == total and popcount(full[:, 1:]) == total
+    bits = np.unpackbits(np.ascontiguousarray(full[:, 1:]).view(np.uint8).reshape(G, -1), axis=1)
+    keep_mask = (rng.random(bits.shape) < 0.5).astype(np.uint8)
+    def relaunch_with(made):
+        state = np.zeros_like(full)
+        state[:, 1:] = np.packbits(made, axis=1).view(np.int32).reshape(G, 15)
+        state[:, 0] = made.sum(axis=1)
+        st.executed.upload(state.reshape(-1))
+        gp.launch("gp_launch_conv2d", p, st.ctx())
+        sync(gp)
+        assert np.array_equal(st.counters().reshape(G, 16), full)
+
+    do.fill32(0xFFFFFFFF)
+    relaunch_with(bits & keep_mask)          # a random half marked as made: the other half runs
+    assert not np.array_equal(do.download(), raw_want)
+    relaunch_with(bits & (1 - keep_mask))    # the complement fills in the rest
+    assert np.array_equal(do.download(), raw_want)
+
+
 @pytest.mark.parametrize("dt", ["f16", "f32"])
 def test_conv2d_long_tiles_left_mid_k_and_resumed_bit_exact(gp, dt):
     """A deep 3x3 convolution on the 128 x 128 body (K = 9 * Cin): with the checkpoint workspace the
