@@ -342,10 +342,10 @@ Status drain(GPUstream s) {
 // "wb-chunk" / "wb-chunk-async": the best-effort model is submitted launch by launch
 // (Executor::launch_kernel, the reference's own launch loop, src/executor.cpp:222-225) but never
 // more than two chunks of kernels ahead of the GPU.  A preempted model then has at most two chunks
-// of queued kernels to flush (each leaves at its first look at the stop index, about 6 us apiece
+// of queued kernels to flush (each leaves at its first look at the stop index, about 4 us apiece
 // on MI355X) instead of the rest of the network, while every kernel keeps its own occupancy.
-// Measured with BERT over ResNet-152: chunks of 6 / 3 / 2 / 1 kernels drain in 88 / 55 / 44 / 32 us
-// (mean) and cost 0 / 3 / 6 / 14 % of the best-effort throughput; the default is 2
+// Measured with BERT over ResNet-152: chunks of 6 / 3 / 2 / 1 kernels drain in 44 / 32 / 28 / 23 us
+// (mean) and cost 0 / 3 / 7 / 16 % of the best-effort throughput; the default is 2
 // (environment variable GPREEMPT_CHUNK overrides it).
 static int chunk_size() {
     static const int v = [] { const char *e = getenv("GPREEMPT_CHUNK"); int c = e ? atoi(e) : 2; return c < 1 ? 1 : c; }();
