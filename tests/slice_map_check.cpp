@@ -53,6 +53,28 @@ int main() {
             last[b % 8] = u;
         }
     }
+    // fixed claims: workgroup b records its claim as bit (b / groups) of counter wg_group(b); the
+    // pairs must be distinct over a grid and the bit must fit the 15 spare ints of a counter's line
+    for (int groups : {8, 16, 32, 64})
+        for (int grid : {groups, 100, 392, 396, 1572, 2048, groups * gp::kFixedClaimBits}) {
+            if (grid < groups) continue;
+            if (!gp::fixed_claims(true, groups, grid, grid) || gp::fixed_claims(true, groups, grid, grid + 1) ||
+                gp::fixed_claims(false, groups, grid, grid) || gp::fixed_claims(true, 1, grid, grid) ||
+                gp::fixed_claims(true, groups, groups * gp::kFixedClaimBits + 1, grid)) {
+                printf("fixed_claims predicate wrong: groups=%d grid=%d\n", groups, grid);
+                return 1;
+            }
+            std::vector<char> seen((size_t)groups * gp::kFixedClaimBits, 0);
+            for (int b = 0; b < grid; ++b) {
+                int g = gp::wg_group(b, groups), j = b >> gp::log2_pow2(groups);
+                if (j >= gp::kFixedClaimBits || seen[(size_t)g * gp::kFixedClaimBits + j]) {
+                    printf("claim bit reused or out of range: groups=%d grid=%d b=%d\n", groups, grid, b);
+                    return 1;
+                }
+                seen[(size_t)g * gp::kFixedClaimBits + j] = 1;
+            }
+            ++cases;
+        }
     printf("ok %ld cases\n", cases);
     return 0;
 }
