@@ -96,7 +96,7 @@ class EmbedParams(C.Structure):
 
 # every symbol include/gpreempt_hip.h declares
 SYMBOLS = """gp_init gp_last_error gp_device_info gp_stream_create gp_stream_destroy gp_stream_sync
-gp_stream_query gp_stream_priority gp_stream_native gp_event_create gp_event_destroy gp_event_record
+gp_stream_query gp_stream_priority gp_stream_set_priority gp_stream_native gp_event_create gp_event_destroy gp_event_record
 gp_event_sync gp_event_query gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free gp_memcpy_h2d gp_memcpy_d2h
 gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_flag_relay_start
 gp_launch_gemm gp_gemm_ckpt_bytes gp_conv_ckpt_bytes gp_ckpt_reset_async gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax

@@ -12,6 +12,7 @@
 //
 // The convolution is the same main loop with a gathered A operand: row m is output pixel
 // (n, ho, wo) and column k is (r, s, ci) of an NHWC input, zero-filled outside the image.
+#include <mutex>
 #include "gemm_tile.hpp"
 #include "gemm_pipe.hpp"
 #include "plans.hpp"
@@ -62,13 +63,16 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     int grid = 0;
     auto kern = KernelOf<K>::fn;  // the launch is planned for the general form; the others need no more resources
     if (K::LDS_BYTES > 48 * 1024) {
-        static bool once = false;  // benign race: idempotent attribute
-        if (!once) {
-            GP_HIP(hipFuncSetAttribute((const void *)KernelOf<K>::fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES));
-            GP_HIP(hipFuncSetAttribute((const void *)KernelOf<K>::plain, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES));
-            GP_HIP(hipFuncSetAttribute((const void *)KernelOf<K>::fixed, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES));
-            once = true;
-        }
+        // several tenant threads launch concurrently: the attribute is set by exactly one of them
+        static std::once_flag once;
+        static hipError_t once_rc = hipSuccess;
+        std::call_once(once, [] {
+            for (const void *f : {(const void *)KernelOf<K>::fn, (const void *)KernelOf<K>::plain, (const void *)KernelOf<K>::fixed}) {
+                hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES);
+                if (e != hipSuccess) once_rc = e;
+            }
+        });
+        GP_HIP(once_rc);
     }
     int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info, 1, K::LDS_BYTES <= 64 * 1024 ? 4 : 1);
     if (rc) return rc;

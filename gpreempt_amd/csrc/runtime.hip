@@ -126,6 +126,12 @@ extern "C" int gp_stream_priority(gp_stream s, int *priority) {
     *priority = s->priority;
     return GP_SUCC;
 }
+extern "C" int gp_stream_set_priority(gp_stream s, int priority) {
+    GP_REQUIRE(s != nullptr, "null stream");
+    GP_REQUIRE(priority >= 0, "priority %d", priority);
+    s->priority = priority;
+    return GP_SUCC;
+}
 extern "C" void *gp_stream_native(gp_stream s) { return (void *)native(s); }
 
 extern "C" int gp_event_create(gp_event *out) {

@@ -5,6 +5,10 @@
 #include "gpreempt_exec_c.h"
 #include "workloads/scicomput.h"
 #include "harness.h"
+#include "gpreempt.h"
+#include <exception>
+#include <map>
+#include <mutex>
 
 using namespace foo;
 
@@ -20,6 +24,21 @@ void copy_str(char *dst, size_t n, const std::string &s) {
     std::strncpy(dst, s.c_str(), n - 1);
     dst[n - 1] = 0;
 }
+// No exception may cross the C boundary (a corrupt file can make a std::vector throw
+// bad_alloc or length_error): it becomes Status::Fail with a line on stderr.
+template <class F>
+int guarded(const char *what, F &&f) {
+    try {
+        return (int)f();
+    } catch (const std::exception &e) {
+        std::fprintf(stderr, "%s: %s\n", what, e.what());
+    } catch (...) {
+        std::fprintf(stderr, "%s: unknown exception\n", what);
+    }
+    return Status::Fail;
+}
+std::mutex g_dom_mu;
+std::map<int, std::unique_ptr<PreemptDomain>> g_domains;  // gpx_domain_create's domains by handle
 }  // namespace
 
 extern "C" {
@@ -31,11 +50,11 @@ gpx_executor gpx_create(int blp) {
     return h;
 }
 void gpx_destroy(gpx_executor e) { delete H(e); }
-int gpx_init(gpx_executor e, const char *workload) { return H(e)->ex->init(workload); }
+int gpx_init(gpx_executor e, const char *workload) { return guarded("gpx_init", [&] { return H(e)->ex->init(workload ? workload : ""); }); }
 int gpx_set_input(gpx_executor e, const char *key, void *value, size_t len, gp_stream s) { return H(e)->ex->set_input(key, value, len, s); }
 int gpx_get_output(gpx_executor e, const char *key, void *value, size_t len, gp_stream s) { return H(e)->ex->get_output(key, value, len, s); }
 size_t gpx_get_data_size(gpx_executor e, const char *key) { return H(e)->ex->get_data_size(key); }
-int gpx_execute(gpx_executor e, gp_stream s) { return H(e)->ex->execute(s); }
+int gpx_execute(gpx_executor e, gp_stream s) { return guarded("gpx_execute", [&] { return H(e)->ex->execute(s); }); }
 int gpx_launch_kernel(gpx_executor e, size_t idx, gp_stream s) { return H(e)->ex->launch_kernel(idx, s); }
 size_t gpx_get_kernel_num(gpx_executor e) { return H(e)->ex->get_kernel_num(); }
 int gpx_capture_graph(gpx_executor e, gp_stream s) {
@@ -114,7 +133,7 @@ extern "C" int gpx_set_lc_tasks(gpx_executor e, int n) { H(e)->lc_tasks.store(n)
 extern "C" int gpx_set_graph_path(gpx_executor e, const char *base) { return H(e)->ex->set_graph_path(base ? base : ""); }
 extern "C" int gpx_write_synthetic_graph(const char *base, unsigned long long vertices, unsigned degree, unsigned long long seed) {
     if (!base || vertices < 2 || vertices >= (1ULL << 28) || degree < 1 || degree > 256 || vertices * degree > (1ULL << 27)) return Status::OutOfRange;
-    return GraphCompute::write_graph(base, GraphCompute::synthetic_graph(vertices, degree, seed));
+    return guarded("gpx_write_synthetic_graph", [&] { return GraphCompute::write_graph(base, GraphCompute::synthetic_graph(vertices, degree, seed)); });
 }
 
 extern "C" int gpx_miniweather_reductions(gpx_executor e, double *mass, double *te) {
@@ -156,19 +175,28 @@ static int copy_report(Status st, const std::string &rep, char *report, size_t r
 }
 
 extern "C" int gpx_run_scenario(const char *config_json, char *report, size_t report_len) {
-    std::string rep;
-    Status st = foo::run_scenario(config_json ? config_json : "", rep);
-    return copy_report(st, rep, report, report_len);
+    return guarded("gpx_run_scenario", [&] {
+        std::string rep;
+        Status st = foo::run_scenario(config_json ? config_json : "", rep);
+        return copy_report(st, rep, report, report_len);
+    });
 }
 
 extern "C" int gpx_preempt_probe(const char *workload, int trials, int use_graph, unsigned long long seed, char *report, size_t report_len) {
-    std::string rep;
-    Status st = foo::preempt_probe(workload ? workload : "", trials, use_graph != 0, seed, rep);
-    return copy_report(st, rep, report, report_len);
+    return guarded("gpx_preempt_probe", [&] {
+        std::string rep;
+        Status st = foo::preempt_probe(workload ? workload : "", trials, use_graph != 0, seed, rep);
+        return copy_report(st, rep, report, report_len);
+    });
 }
 
 extern "C" long gpx_parse_params(const char *path, const char *key, float *out, size_t n, size_t *len) {
-    std::unique_ptr<ModelParam> params(ModelParamParser::parse_from_file(path));
+    std::unique_ptr<ModelParam> params;
+    try {
+        params.reset(ModelParamParser::parse_from_file(path));
+    } catch (const std::exception &e) {
+        std::fprintf(stderr, "gpx_parse_params: %s\n", e.what());
+    }
     if (!params) return -1;
     if (key) {
         auto it = params->find(key);
@@ -176,4 +204,59 @@ extern "C" long gpx_parse_params(const char *path, const char *key, float *out, 
         if (it != params->end() && out) std::memcpy(out, it->second.data(), sizeof(float) * std::min(n, it->second.size()));
     }
     return (long)params->size();
+}
+
+// ---- gpreempt.h through the C view ------------------------------------------------------------------
+extern "C" int gpx_set_priority(gp_stream s, int priority) {
+    NvContext ctx;
+    ctx.stream = s;
+    if (NvRmQuery(&ctx) != 0) return -1;
+    return set_priority(ctx, priority);
+}
+extern "C" int gpx_domain_create(int levels) {
+    return guarded("gpx_domain_create", [&] {
+        std::unique_ptr<PreemptDomain> d(new PreemptDomain(levels));
+        if (!d->ok()) return -1;
+        const int fd = d->fd();
+        std::lock_guard<std::mutex> g(g_dom_mu);
+        g_domains[fd] = std::move(d);
+        return fd;
+    });
+}
+extern "C" int gpx_domain_destroy(int fd) {
+    std::lock_guard<std::mutex> g(g_dom_mu);
+    return g_domains.erase(fd) ? 0 : -1;
+}
+extern "C" int gpx_get_fd(void) { return hipGetFd(); }
+extern "C" void *gpx_domain_flag(int fd, int priority) {
+    std::lock_guard<std::mutex> g(g_dom_mu);
+    auto it = g_domains.find(fd);
+    return it == g_domains.end() ? nullptr : it->second->flag_for(priority);
+}
+extern "C" int gpx_domain_flag_value(int fd, int priority) {
+    std::lock_guard<std::mutex> g(g_dom_mu);
+    auto it = g_domains.find(fd);
+    return it == g_domains.end() ? -1 : it->second->flag_value(priority);
+}
+extern "C" int gpx_domain_begin(int fd, int priority) {
+    std::lock_guard<std::mutex> g(g_dom_mu);
+    auto it = g_domains.find(fd);
+    if (it == g_domains.end()) return -1;
+    it->second->begin(priority);
+    return 0;
+}
+extern "C" int gpx_domain_end(int fd, int priority) {
+    std::lock_guard<std::mutex> g(g_dom_mu);
+    auto it = g_domains.find(fd);
+    if (it == g_domains.end()) return -1;
+    it->second->end(priority);
+    return 0;
+}
+extern "C" int gpx_suspend_streams(int fd, const int *levels, int n) {
+    std::vector<int> v(levels, levels + (n > 0 ? n : 0));
+    return hipSuspendStreams(fd, v);
+}
+extern "C" int gpx_resume_streams(int fd, const int *levels, int n) {
+    std::vector<int> v(levels, levels + (n > 0 ? n : 0));
+    return hipResumeStreams(fd, v);
 }

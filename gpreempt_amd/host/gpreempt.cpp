@@ -6,11 +6,59 @@
 
 int NvRmQuery(NvContext *ctx) { return ctx && ctx->stream ? 0 : -1; }
 
-int set_priority(NvContext &ctx, int priority) {
-    if (priority < 0 || priority >= foo::PreemptDomain::kMaxLevels) return -1;
-    ctx.priority = priority;
+int set_priority(NvContext ctx, int priority) {
+    if (priority < 0 || priority >= foo::PreemptDomain::kMaxLevels || !ctx.stream) return -1;
+    return gp_stream_set_priority(ctx.stream, priority) == 0 ? 0 : -1;
+}
+
+// ---- hipSuspendStreams / hipResumeStreams over the flag words ------------------------------------
+namespace {
+std::mutex g_fd_mu;
+std::vector<foo::PreemptDomain *> g_fds;
+foo::PreemptDomain *domain_of(int fd) {
+    std::lock_guard<std::mutex> g(g_fd_mu);
+    return fd >= 0 && (size_t)fd < g_fds.size() ? g_fds[fd] : nullptr;
+}
+
+int g_newest_fd = -1;
+int register_domain(foo::PreemptDomain *domain) {
+    std::lock_guard<std::mutex> g(g_fd_mu);
+    size_t i = 0;
+    while (i < g_fds.size() && g_fds[i] != nullptr) ++i;
+    if (i == g_fds.size()) g_fds.push_back(domain);
+    else g_fds[i] = domain;
+    g_newest_fd = (int)i;
+    return (int)i;
+}
+void unregister_domain(foo::PreemptDomain *domain) {
+    std::lock_guard<std::mutex> g(g_fd_mu);
+    for (size_t i = 0; i < g_fds.size(); ++i)
+        if (g_fds[i] == domain) {
+            g_fds[i] = nullptr;
+            if (g_newest_fd == (int)i) {
+                g_newest_fd = -1;
+                for (size_t j = 0; j < g_fds.size(); ++j) if (g_fds[j]) g_newest_fd = (int)j;
+            }
+        }
+}
+}  // namespace
+
+int hipGetFd() {
+    std::lock_guard<std::mutex> g(g_fd_mu);
+    return g_newest_fd;
+}
+
+static int each_level(int fd, std::vector<int> &ids, bool suspend) {
+    foo::PreemptDomain *d = domain_of(fd);
+    if (!d) return -1;
+    for (int p : ids)
+        if (p < 1 || p >= d->levels()) return -1;
+    for (int p : ids) suspend ? d->suspend_level(p) : d->resume_level(p);
     return 0;
 }
+int hipSuspendStreams(int fd, std::vector<int> &stream_ids) { return each_level(fd, stream_ids, true); }
+int hipResumeStreams(int fd, std::vector<int> &stream_ids) { return each_level(fd, stream_ids, false); }
+int hipResetWavefronts(int fd) { return domain_of(fd) ? 0 : -1; }
 
 namespace foo {
 
@@ -20,6 +68,7 @@ static int64_t steady_ns() {
 
 PreemptDomain::PreemptDomain(int levels, bool use_relay) : levels_(std::min(std::max(levels, 2), kMaxLevels)) {
     for (int i = 0; i < kMaxLevels; ++i) { active_[i] = 0; raised_[i] = 0; }
+    fd_ = register_domain(this);
     for (int j = 0; j + 1 < levels_; ++j)
         if (gp_flag_create(&host_[j], &dev_[j]) != 0) ok_ = false;
     if (ok_ && use_relay) {
@@ -42,6 +91,7 @@ void PreemptDomain::stop_relay() {
 }
 
 PreemptDomain::~PreemptDomain() {
+    unregister_domain(this);
     stop_relay();
     if (relay_stream_) gp_stream_destroy(relay_stream_);
     if (quit_host_) gp_flag_destroy(quit_host_);
@@ -56,12 +106,17 @@ GPUdeviceptr PreemptDomain::flag_for(int priority) const {
     return relay_on_ ? (GPUdeviceptr)(mirror_ + (p - 1)) : dev_[p - 1];
 }
 
+int PreemptDomain::flag_value(int priority) const {
+    int p = std::min(priority, levels_ - 1);
+    return p < 1 ? -1 : *host_[p - 1];
+}
+
 // word j is up while any request of a level <= j is active
 void PreemptDomain::update() {
     int run = 0;
     for (int j = 0; j + 1 < levels_; ++j) {
         run += active_[j].load();
-        int want = run > 0;
+        int want = run > 0 || forced_[j] > 0;
         if (*host_[j] != want) {
             if (want) raised_[j].store(steady_ns());
             *host_[j] = want;
@@ -87,6 +142,23 @@ void PreemptDomain::end(int priority) {
     if (p + 1 >= levels_) return;
     std::lock_guard<std::mutex> g(mu_);
     active_[p].fetch_sub(1, std::memory_order_acq_rel);
+    update();
+}
+
+void PreemptDomain::suspend_level(int priority) {
+    int p = std::min(priority, levels_ - 1);
+    if (p < 1) return;
+    std::lock_guard<std::mutex> g(mu_);
+    if (*host_[p - 1] == 0) raised_[p - 1].store(steady_ns());
+    ++forced_[p - 1];
+    update();
+}
+
+void PreemptDomain::resume_level(int priority) {
+    int p = std::min(priority, levels_ - 1);
+    if (p < 1) return;
+    std::lock_guard<std::mutex> g(mu_);
+    if (forced_[p - 1] > 0) --forced_[p - 1];
     update();
 }
 

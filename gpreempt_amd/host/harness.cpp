@@ -15,6 +15,7 @@
 #include <chrono>
 #include <cmath>
 #include <cstring>
+#include <ctime>
 #include <condition_variable>
 #include <memory>
 #include <map>
@@ -237,6 +238,8 @@ struct Shared {
         }
     }
     std::atomic<int> cores{0};
+    bool verify_outputs = false;            // hash every request's output and compare it with the tenant's stand-alone output
+    bool hp_gate = false;                   // non-preemptible tenants of level 0 submit behind a gate kernel (gpreemptclient.cpp:74-81)
     long hp_requests = 0;                   // > 0: the run ends once every priority-0 tenant served this many
     std::atomic<int> hp_unfinished{0};
     std::atomic<bool> stop{false};
@@ -266,6 +269,15 @@ struct Tenant {
     void *input = nullptr, *output = nullptr;
     size_t input_size = 0, output_size = 0;
     Stats standalone, total, infer, queueing;
+    // DISB's six phases (analyzer.cpp:90-150); prepareInput and postprocess are empty in the reference's clients
+    double phase_sum_us[4] = {0, 0, 0, 0};  // preprocess, copyInput, infer, copyOutput
+    NvContext nvctx;
+    volatile int *gate_host = nullptr;      // hp_gate: the word the gate kernels wait for
+    void *gate_dev = nullptr;
+    int *gate_timed_out = nullptr;          // device word set by a gate that gave up
+    bool have_ref_hash = false;
+    uint64_t ref_hash = 0;
+    long output_mismatches = 0;
     int64_t preemptions = 0, requests = 0;
     int64_t first_ns = 0, last_ns = 0;
     Status error = Status::Succ;
@@ -296,6 +308,18 @@ Status init_tenant(Tenant &t, Shared &sh) {
     if (t.output_size) CUDA_RETURN_STATUS(gp_host_alloc(&t.output, t.output_size));
     fill_input(t);
     CUDA_RETURN_STATUS(gp_stream_create(t.priority, &t.stream));
+    // gpreemptclient.cpp:170-177: look the tenant's context up and give it its priority
+    t.nvctx.stream = t.stream;
+    if (NvRmQuery(&t.nvctx) != 0 || set_priority(t.nvctx, t.priority) != 0) {
+        std::fprintf(stderr, "Failed to set priority %d for %s\n", t.priority, t.id.c_str());
+        return Status::Fail;
+    }
+    if (sh.hp_gate && t.priority == 0 && !preemptible) {
+        CUDA_RETURN_STATUS(gp_flag_create(&t.gate_host, &t.gate_dev));
+        CUDA_RETURN_STATUS(gp_malloc((void **)&t.gate_timed_out, sizeof(int)));
+        CUDA_RETURN_STATUS(gp_fill32_async(t.gate_timed_out, 0, 1, nullptr));
+        CUDA_RETURN_STATUS(gp_stream_sync(nullptr));
+    }
     if (t.blp) {
         t.blp->dpStop = sh.domain->flag_for(t.priority);
         if (sh.domain->relayed()) t.blp->poll_every = 1;  // the flag is a device-memory mirror
@@ -436,7 +460,17 @@ Status infer(Tenant &t, Shared &sh) {
     if (!is_async(pol)) while (sh.on_gpu_below(p) > 0) spin_pause();
     Status st = Status::Succ;
     if (!t.blp) {
-        st = t.ex->execute(t.stream);
+        if (t.gate_host) {
+            // start_blocking_stream / end_blocking_stream of the reference (gpreemptclient.cpp:74-81,
+            // 232-235): two gate kernels hold the stream while the request's kernels are queued
+            // behind them, then one host store lets everything run back to back.  The wait is
+            // bounded (about a second of polls), so a lost release cannot hang the device.
+            *t.gate_host = 0;
+            for (int i = 0; i < 2 && st == Status::Succ; ++i)
+                if (gp_launch_gate((const int *)t.gate_dev, 1ull << 22, t.gate_timed_out, t.stream) != 0) st = Status::Fail;
+        }
+        if (st == Status::Succ) st = t.ex->execute(t.stream);
+        if (t.gate_host) *t.gate_host = 1;
         if (st == Status::Succ) st = drain(t.stream);
     } else if (t.ex->graph_workload()) {
         // graph workloads drive their own loop inside execute() (graphcompute.tr.cu:142-174);
@@ -512,6 +546,13 @@ void end_request(Tenant &t, Shared &sh) {
 
 // One request: the six DISB phases (benchmark.cpp:66-135); prepareInput and postprocess are empty
 // in the reference's clients, preprocess sleeps preprocess_time (blpclient.cpp:153-155).
+static uint64_t fnv1a(const void *p, size_t n) {
+    const unsigned char *b = (const unsigned char *)p;
+    uint64_t h = 1469598103934665603ull;
+    for (size_t i = 0; i < n; ++i) { h ^= b[i]; h *= 1099511628211ull; }
+    return h;
+}
+
 Status infer_once(Tenant &t, Shared &sh, double *total_us, double *infer_us) {
     int64_t t0 = now_ns();
     std::shared_ptr<std::atomic<int>> hint;
@@ -523,6 +564,7 @@ Status infer_once(Tenant &t, Shared &sh, double *total_us, double *infer_us) {
         if (t.preprocess_us > 200) std::this_thread::sleep_for(std::chrono::microseconds(t.preprocess_us - 150));
         while (now_ns() < until) spin_pause();
     }
+    int64_t tp = now_ns();
     int expect = 0;
     if (!hint || hint->compare_exchange_strong(expect, 2)) begin_request(t, sh);  // else the daemon has begun it
     struct Retire { Tenant &t; Shared &sh; ~Retire() { end_request(t, sh); } } retire{t, sh};
@@ -543,6 +585,15 @@ Status infer_once(Tenant &t, Shared &sh, double *total_us, double *infer_us) {
     int64_t t3 = now_ns();
     *total_us = (t3 - t0) / 1e3;
     *infer_us = (t2 - t1) / 1e3;
+    t.phase_sum_us[0] += (tp - t0) / 1e3; t.phase_sum_us[1] += (t1 - tp) / 1e3;
+    t.phase_sum_us[2] += (t2 - t1) / 1e3; t.phase_sum_us[3] += (t3 - t2) / 1e3;
+    if (sh.verify_outputs && t.output_size && !t.resident_io) {
+        // same input every time, deterministic kernels: every request's output has the same bits,
+        // however often the tenant was stopped and resumed on the way
+        const uint64_t h = fnv1a(t.output, t.output_size);
+        if (!t.have_ref_hash) { t.ref_hash = h; t.have_ref_hash = true; }
+        else if (h != t.ref_hash) ++t.output_mismatches;
+    }
     return Status::Succ;
 }
 
@@ -590,6 +641,8 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     int standalone_runs = (int)cfg["standalone_runs"].number(kStandAloneRuns);
     int warmups = (int)cfg["warmups"].number(kWarmups);
     sh.hp_requests = (long)cfg["hp_requests"].number(0);
+    sh.verify_outputs = cfg["verify_outputs"].boolean(false);
+    sh.hp_gate = cfg["hp_gate"].boolean(false);
     const json::Value &tasks = cfg["tasks"];
     std::vector<std::unique_ptr<Tenant>> tenants;
     // Declared after `tenants`, so it runs first on every exit path: executors free device memory
@@ -635,6 +688,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
             if (i >= warmups) t->standalone.add(total);
         }
         t->preemptions = 0;
+        for (double &v : t->phase_sum_us) v = 0;
     }
     {
         std::lock_guard<std::mutex> g(sh.stats_mu);
@@ -711,7 +765,53 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
             be_kept += kept;
             ++n_be;
         }
+        if (sh.verify_outputs) o.set("outputMismatches") = t->output_mismatches;
         if (t->error != Status::Succ) { o.set("error") = status_name(t->error); result = t->error; }
+    }
+    // The same run in the shape DISB writes and the reference's scripts/plot/plot.py reads
+    // (third_party/disb/src/benchmark.cpp:340-354, client.cpp:74-87, analyzer.cpp:90-170): one entry
+    // per client with its analyzers' reports; latencies are whole microseconds, the throughput is
+    // requests over the whole benchmark time.
+    {
+        auto stamp = [](std::chrono::system_clock::time_point tp) {
+            char buf[25] = {0};
+            time_t tt = std::chrono::system_clock::to_time_t(tp);
+            struct tm lt;
+            localtime_r(&tt, &lt);
+            strftime(buf, sizeof(buf), "%Y-%m-%d %H:%M:%S", &lt);
+            return std::string(buf);
+        };
+        const auto wall_end = std::chrono::system_clock::now();
+        const auto wall_begin = wall_end - std::chrono::nanoseconds((int64_t)(wall_s * 1e9));
+        rep.set("beginTime") = stamp(wall_begin);
+        rep.set("endTime") = stamp(wall_end);
+        rep.set("benchmarkTime(s)") = (long)wall_s;
+        json::Value &results = rep.set("results");
+        results = json::Value::array();
+        for (auto &t : tenants) {
+            json::Value a = json::Value::object();
+            const double n = (double)std::max<int64_t>(t->requests, 1);
+            const long pre = (long)(t->phase_sum_us[0] / n), cin = (long)(t->phase_sum_us[1] / n), inf = (long)(t->phase_sum_us[2] / n),
+                       cout = (long)(t->phase_sum_us[3] / n);
+            const long total = t->requests > 0 ? pre + cin + inf + cout : 0, alone = (long)t->standalone.mean();
+            a.set("type") = "basic";
+            a.set("avgThroughput(req/s)") = t->requests > 0 && wall_s > 0 ? t->requests / wall_s : 0.0;
+            a.set("standAloneTotalLatency(us)") = alone;
+            a.set("avgPrepareInputLatency(us)") = 0L;
+            a.set("avgPreprocessLatency(us)") = t->requests > 0 ? pre : 0L;
+            a.set("avgCopyInputLatency(us)") = t->requests > 0 ? cin : 0L;
+            a.set("avgInferLatency(us)") = t->requests > 0 ? inf : 0L;
+            a.set("avgCopyOutputLatency(us)") = t->requests > 0 ? cout : 0L;
+            a.set("avgPostprocessLatency(us)") = 0L;
+            a.set("avgTotalLatency(us)") = total;
+            a.set("avgTotalLatencyIncrease(us)") = total - alone;
+            json::Value c = json::Value::object();
+            c.set("clientName") = t->name;
+            json::Value &an = c.set("analyzers");
+            an = json::Value::array();
+            an.push(a);
+            results.push(c);
+        }
     }
     rep.set("hp_busy_fraction") = busy_frac;
     rep.set("hp_p99_vs_isolated") = hp_ratio;
@@ -727,6 +827,8 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         gp_host_free(t->input);
         gp_host_free(t->output);
         for (gp_event e : t->chunk_events) if (e) gp_event_destroy(e);
+        if (t->gate_host) gp_flag_destroy(t->gate_host);
+        if (t->gate_timed_out) gp_free(t->gate_timed_out);
         gp_stream_destroy(t->stream);
     }
     tenants.clear();

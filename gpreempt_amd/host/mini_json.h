@@ -108,31 +108,38 @@ private:
     const std::string &s_;
     size_t i_ = 0;
     bool ok_ = true;
+    int depth_ = 0;
+    static constexpr int kMaxDepth = 64;  // nesting beyond this is refused instead of recursed into
     void ws() { while (i_ < s_.size() && (s_[i_] == ' ' || s_[i_] == '\n' || s_[i_] == '\t' || s_[i_] == '\r')) ++i_; }
     bool eat(char c) { ws(); if (i_ < s_.size() && s_[i_] == c) { ++i_; return true; } return false; }
     Value value() {
         ws();
         if (i_ >= s_.size()) { ok_ = false; return Value(); }
         char c = s_[i_];
+        if ((c == '{' || c == '[') && depth_ >= kMaxDepth) { ok_ = false; return Value(); }
         if (c == '{') {
             ++i_;
+            ++depth_;
             Value v = Value::object();
-            if (eat('}')) return v;
+            if (eat('}')) { --depth_; return v; }
             do {
                 ws();
                 Value k = value();
-                if (k.type != Value::String || !eat(':')) { ok_ = false; return v; }
+                if (k.type != Value::String || !eat(':')) { ok_ = false; --depth_; return v; }
                 v.set(k.str) = value();
             } while (ok_ && eat(','));
             if (!eat('}')) ok_ = false;
+            --depth_;
             return v;
         }
         if (c == '[') {
             ++i_;
+            ++depth_;
             Value v = Value::array();
-            if (eat(']')) return v;
+            if (eat(']')) { --depth_; return v; }
             do { v.arr.push_back(value()); } while (ok_ && eat(','));
             if (!eat(']')) ok_ = false;
+            --depth_;
             return v;
         }
         if (c == '"') {

@@ -26,8 +26,22 @@ struct NvContext {
 int NvRmQuery(NvContext *ctx);
 
 // priority 0 = high, 1 = low (reference include/gpreempt.h:165-173); further levels are allowed.
-// Records the level on the context and its stream; returns 0, or -1 for a bad argument.
-int set_priority(NvContext &ctx, int priority);
+// The context is passed by value as in the reference: what carries the level is the tenant's
+// stream (the priority recorded on the gp_stream handle, which selects the flag word the tenant
+// obeys).  Returns 0, or -1 for a bad argument or a context without a stream.
+int set_priority(NvContext ctx, int priority);
+
+// The HIP side of the reference's header (include/gpreempt.h:191-194) stops and restarts hardware
+// queues through a patched amdkfd.  Here "queues" are priority levels of a PreemptDomain: a
+// level is suspended by raising the flag word it obeys (its kernels leave at their next tile
+// boundary) and resumed by lowering it (the tenant then calls BLPExecutor::resume).  `fd` names a
+// PreemptDomain: hipGetFd() returns the handle of the process's newest live domain (-1: none), as
+// the reference's returns the one KFD file of the process; PreemptDomain::fd() gives a particular
+// one.  The others return 0 on success, -1 on a bad argument.
+int hipGetFd();
+int hipSuspendStreams(int fd, std::vector<int> &stream_ids);    // stream_ids: priority levels (>= 1) to stop
+int hipResumeStreams(int fd, std::vector<int> &stream_ids);
+int hipResetWavefronts(int fd);                                 // nothing to reset without the driver patch: returns 0
 
 namespace foo {
 
@@ -50,8 +64,11 @@ public:
 
     int levels() const { return levels_; }
     bool ok() const { return ok_; }
+    int fd() const { return fd_; }  // the handle hipSuspendStreams / hipResumeStreams take
     // device address of the flag a level-p (p >= 1) best-effort executor polls: BLPExecutor::dpStop
     GPUdeviceptr flag_for(int priority) const;
+    // current value of that word as the host sees it (-1: the level obeys no word)
+    int flag_value(int priority) const;
     // a request of `priority` starts / ends: raises / lowers the words of every lower level
     void begin(int priority);
     void end(int priority);
@@ -59,17 +76,22 @@ public:
     int active_above(int priority) const;
     // steady-clock nanoseconds at which the word obeyed by `priority` was last raised (0: never)
     int64_t raised_ns(int priority) const;
-    // direct control, the counterparts of hipSuspendStreams / hipResumeStreams
+    // direct control, what hipSuspendStreams / hipResumeStreams call
     void suspend_below(int priority) { begin(priority); }
     void resume_below(int priority) { end(priority); }
+    // raise / lower the one word that level `priority` (>= 1) obeys, whatever requests are active
+    void suspend_level(int priority);
+    void resume_level(int priority);
 
 private:
     void update();
     int levels_;
+    int fd_ = -1;
     bool ok_ = true;
     volatile int *host_[kMaxLevels] = {nullptr};
     void *dev_[kMaxLevels] = {nullptr};
     std::atomic<int> active_[kMaxLevels];
+    int forced_[kMaxLevels] = {0};      // suspend_level counts per word
     std::atomic<int64_t> raised_[kMaxLevels];
     std::mutex mu_;
     bool relay_on_ = false;

@@ -81,6 +81,25 @@ int gpx_preempt_probe(const char *workload, int trials, int use_graph, unsigned 
  * its values are copied to `out` and *len receives its length. */
 long gpx_parse_params(const char *path, const char *key, float *out, size_t n, size_t *len);
 
+/* include/gpreempt.h through the C view.  gpx_set_priority = NvRmQuery + set_priority on the
+ * tenant's stream (reference src/cuda-clients/gpreemptclient.cpp:170-177); 0 or -1 as the reference.
+ * A domain is a foo::PreemptDomain (one flag word per priority boundary); its handle is what
+ * hipGetFd() returns and hipSuspendStreams / hipResumeStreams take (reference
+ * include/gpreempt.h:191-194), with priority levels in the place of hardware queue ids.
+ * gpx_domain_flag returns the device-visible address of the word that level `priority` (>= 1)
+ * obeys: the value for BLPExecutor::dpStop (gpx_set_flag).  gpx_domain_begin / _end announce and
+ * retire a request of `priority`, which raises / lowers the words of every lower level. */
+int gpx_set_priority(gp_stream s, int priority);
+int gpx_domain_create(int levels);   /* handle >= 0, or -1 */
+int gpx_domain_destroy(int fd);
+int gpx_get_fd(void);                /* hipGetFd(): the newest live domain, -1 when there is none */
+void *gpx_domain_flag(int fd, int priority);
+int gpx_domain_flag_value(int fd, int priority);  /* the word's current value on the host side; -1: no such word */
+int gpx_domain_begin(int fd, int priority);
+int gpx_domain_end(int fd, int priority);
+int gpx_suspend_streams(int fd, const int *levels, int n);  /* hipSuspendStreams */
+int gpx_resume_streams(int fd, const int *levels, int n);   /* hipResumeStreams */
+
 #ifdef __cplusplus
 }
 #endif

@@ -52,6 +52,9 @@ int gp_stream_destroy(gp_stream s);
 int gp_stream_sync(gp_stream s);
 int gp_stream_query(gp_stream s, int *idle); /* *idle = 1 when all work has completed */
 int gp_stream_priority(gp_stream s, int *priority);
+/* Replaces the driver call behind set_priority (src/gpreempt.cpp:61-72: the context's timeslice):
+ * re-labels the tenant priority recorded on the handle.  The HIP stream is not touched. */
+int gp_stream_set_priority(gp_stream s, int priority);
 void *gp_stream_native(gp_stream s); /* the hipStream_t, for callers that own HIP code */
 
 int gp_event_create(gp_event *out);

@@ -1,0 +1,58 @@
+// Reader of the reference's exported model directory: TVM's graph-executor JSON (mod.json), the
+// patched TVM's host-side launch record (host.json) and, as an extension, an operator-attribute
+// sidecar (ops.json).
+//
+// parse_tvm_export follows Model::load_from_json of the reference (src/model.cpp:128-235) rule by
+// rule; what it yields is the reference's own view of a model: storages (graph nodes first, then
+// the temporary buffers) and device kernels with launch dimensions and storage indices.  The
+// exported files do not say what a kernel computes (a convolution's stride and padding, a pool's
+// window, which input of a fused add is the residual live only inside the generated device code),
+// so running an export on the native operators needs the sidecar, which the export script can
+// write from the Relay module it holds (scripts/compile/compile.py:46-57).
+#pragma once
+#include <map>
+#include <string>
+#include <vector>
+#include "model.h"
+
+namespace foo {
+
+struct TvmExport {
+    std::vector<StorageInfo> storage_infos;  // [0, global_len): graph nodes; then one "temp" per host.json temp_args entry
+    std::vector<KernelInfo> kernel_infos;    // name, launch_params, args_index as the reference fills them; "nop" for __nop nodes
+    std::vector<std::string> kernel_func;    // host function (fused operator) each kernel belongs to; "__nop" for copies
+    size_t global_len = 0;
+    size_t heads_index = 0;                  // the storage renamed to "heads"
+    std::string error;                       // what went wrong when the result is not Succ
+};
+
+// NotFound: a file cannot be opened.  Fail: malformed JSON, a missing key, a function-name mismatch
+// between the two files (src/model.cpp:208-211), or an argument index out of range.
+Status parse_tvm_export(const std::string &device_json_text, const std::string &host_json_text, TvmExport &out);
+Status load_tvm_export(const char *device_json_path, const char *host_json_path, TvmExport &out);
+
+// ---- operator-attribute sidecar (ops.json) ----------------------------------------------------------
+// { "layout": "NCHW",
+//   "funcs": [ { "name": "<host function, as in host.json>",
+//                "op": "conv2d" | "dense" | "max_pool2d" | "avg_pool2d" | "global_avg_pool2d" | "add" | "softmax" |
+//                      "layer_norm" | "batch_matmul" | "take" | "scale_shift" | "concatenate" | "reshape",
+//                "attrs": { "strides": [1,1], "padding": [1,1,1,1], "dilation": [1,1], "groups": 1, "pool_size": [3,3],
+//                           "count_include_pad": 0, "axis": 1, "epsilon_e12": 1, ... },       integers or integer lists
+//                "epilogue": ["bias", "residual", "relu"],     fused tail, in order, of "bias" "residual" "relu" "gelu"
+//                "inputs": {"data": 0, "weight": 1, "bias": 2, "residual": 3} } ] }   role -> index among the function's arguments
+struct ExportOp {
+    std::string func, op;
+    std::map<std::string, std::vector<long>> attrs;
+    std::vector<std::string> epilogue;
+    std::map<std::string, int> inputs;
+};
+struct ExportOps {
+    std::string layout = "NCHW";
+    std::vector<ExportOp> funcs;
+    std::string error;
+};
+Status parse_export_ops(const std::string &ops_json_text, ExportOps &out);
+// Every non-"__nop" host function of the export must be described exactly once, by name.
+Status check_export_ops(const TvmExport &ex, const ExportOps &ops, std::string &error);
+
+}  // namespace foo

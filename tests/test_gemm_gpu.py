@@ -414,3 +414,153 @@ def test_without_workspace_long_tiles_are_finished(gp):
     stream.sync()
     assert flag.get() == 1
     assert np.array_equal(dC.download(), want)  # all four tiles were owed and finished
+
+
+# ---- the 256 x 256 body (config 5's kernel) against the oracle ------------------------------------
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("shape", [(512, 768, 1024), (300, 520, 192), (256, 256, 64)])
+def test_gemm_256_body_matches_oracle(gp, dt, shape):
+    """Plain and preemptible launches of the 256 x 256 body, full and ragged tiles, with bias,
+    residual and ReLU, against the oracle."""
+    M, N, K = shape
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag, 32)
+
+    def preemptible(p, dC):
+        return gp.launch("gp_launch_gemm", p, st.ctx(fresh=1))
+
+    for ctx_fn in (None, preemptible):
+        st.reset()
+        got, ref, info = run_gemm(gp, dt, M, N, K, True, gp.ACT_RELU, True, True, seed=M + N + K, ctx_fn=ctx_fn, tile=256)
+        assert info.total_tiles == -(-M // 256) * -(-N // 256)
+        assert np.isfinite(got).all(), (dt, shape)
+        assert rel_err(got, ref) < TOL[dt], (dt, shape, ctx_fn is not None)
+        assert st.stop_index() == -1
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "f32"])
+def test_gemm_256_body_left_mid_k_matches_oracle(gp, dt):
+    """The checkpointing form of the 256 x 256 body: uninterrupted, and stopped between two K-steps
+    and resumed, both against the oracle (not only against another launch of the same body)."""
+    M, N, K = 768, 512, 4096 if dt != "f32" else 2048
+    rng = np.random.default_rng(11)
+    A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), dt)
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32), dt)
+    bias = O.round_to(rng.uniform(-0.1, 0.1, N).astype(np.float32), dt)
+    ref = O.gemm_bias_act(A, B, bias, act=O.ACT_RELU, b_is_nk=True)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    dA, dB, db = gp.DevBuf.from_array(A, dtype), gp.DevBuf.from_array(B, dtype), gp.DevBuf.from_array(bias, dtype)
+    dC = gp.DevBuf(M * N * gp.DTYPE_SIZE[dtype])
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N,
+                      bias=db.ptr, alpha=1.0, act=gp.ACT_RELU, batch=1, tile_m=256, tile_n=256)
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag)
+    assert st.enable_checkpoints(p) > 0
+    stream = gp.Stream(1)
+    # uninterrupted run of the checkpointing instantiation
+    dC.fill32(0)
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
+    stream.sync()
+    assert st.stop_index() == -1
+    assert rel_err(dC.download(dtype, (M, N)), ref) < TOL[dt]
+    whole = dC.download().copy()
+    # stopped by the first claim, resumed
+    dC.fill32(0)
+    st.reset(); st.clear_stop(); flag.set(0)
+    gp.check(gp.lib().gp_ckpt_reset_async(gp.vp(st.ckpt.ptr), None))
+    info = gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0, inject_at=0), stream)
+    stream.sync()
+    assert flag.get() == 1 and st.stop_index() == 0
+    assert int(st.checkpoint_headers(info.grid)[:, 0].sum()) > 0, "no tile was left half-way"
+    flag.set(0)
+    st.clear_stop()
+    gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
+    stream.sync()
+    assert st.stop_index() == -1
+    assert rel_err(dC.download(dtype, (M, N)), ref) < TOL[dt]
+    assert np.array_equal(dC.download(), whole)
+
+
+# ---- config 5 at full size: bf16 8192^3 on 256 x 256 tiles ----------------------------------------
+def gp_to_bf16(a):
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    return ((u + (((u >> 16) & 1) + 0x7FFF)) >> 16).astype(np.uint16)
+
+
+def test_config5_gemm8192_bf16_full_size(gp):
+    """Config 5's best-effort kernel at its real size: U[-1,1) bf16 operands, 1024 tiles of
+    256 x 256.  Checked on 96 seeded full output rows against the oracle, exactly on all-ones and
+    identity operands, and bit-exactly under preemption at 25 / 50 / 75 % of the tiles with the
+    executor's context (32 claim counters, checkpoint workspace: tiles are left between K-steps)."""
+    n = 8192
+    rng = np.random.default_rng(0x5EED5)
+    dA, dB, dC = gp.DevBuf(2 * n * n), gp.DevBuf(2 * n * n), gp.DevBuf(2 * n * n)
+    p = gp.GemmParams(dtype=gp.BF16, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=1, C=dC.ptr, ldc=n,
+                      alpha=1.0, act=gp.ACT_NONE, batch=1)
+    stream = gp.Stream(1)
+
+    def run_plain():
+        dC.fill32(0x7FC07FC0)  # bf16 NaN pattern: unwritten elements show up
+        info = gp.launch("gp_launch_gemm", p, None, stream)
+        stream.sync()
+        assert info.total_tiles == 1024 and info.shape[0] == 32 and info.shape[1] == 32, "config 5 must run on 256 x 256 tiles"
+        return dC.download(np_dtype=np.uint16).reshape(n, n)
+
+    # known answers: ones x ones = K (8192 is a bf16 number); identity x B^T = B^T
+    ones = np.full(n * n, 0x3F80, np.uint16)
+    dA.upload(ones); dB.upload(ones)
+    got = run_plain()
+    assert (got == gp_to_bf16(np.float32(n))).all()
+    Bf = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    Bb = gp_to_bf16(Bf)
+    eye = np.zeros((n, n), np.uint16)
+    eye[np.arange(n), np.arange(n)] = 0x3F80
+    dA.upload(eye); dB.upload(Bb)
+    del eye, ones
+    got = run_plain()
+    assert np.array_equal(got, Bb.T)
+    # seeded operands; rows spread over every tile row, checked against the oracle
+    Ab = gp_to_bf16(rng.uniform(-1, 1, (n, n)).astype(np.float32))
+    dA.upload(Ab)
+    base = run_plain().copy()
+    rows = np.sort(rng.choice(n, 96, replace=False))
+    A32 = (Ab[rows].astype(np.uint32) << 16).view(np.float32)
+    B32 = (Bb.astype(np.uint32) << 16).view(np.float32)
+    ref = O.gemm_bias_act(A32, B32, b_is_nk=True)
+    got32 = (base[rows].astype(np.uint32) << 16).view(np.float32)
+    assert np.isfinite(got32).all()
+    assert rel_err(got32, ref) < TOL["bf16"]
+    # element-wise too: |C| ~ sqrt(K)/3 = 30, bf16 rounding of the result 2^-9 relative
+    assert np.abs(got32 - ref).max() < 0.5
+    del A32, B32, Ab, Bf
+    # preemptible launch with the executor's context: same bits
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag, 32)
+    assert st.enable_checkpoints(p) > 0
+    dC.fill32(0x7FC07FC0)
+    info = gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
+    stream.sync()
+    assert info.total_tiles == 1024 and st.stop_index() == -1
+    assert np.array_equal(dC.download(np_dtype=np.uint16).reshape(n, n), base)
+    for frac in (0.25, 0.5, 0.75):
+        st.reset(); st.clear_stop(); flag.set(0)
+        gp.check(gp.lib().gp_ckpt_reset_async(gp.vp(st.ckpt.ptr), None))
+        dC.fill32(0x7FC07FC0)
+        # 256 resident workgroups, 32 counters owning 32 consecutive tiles each: the first claims of
+        # every counter are made at once, so "after frac of the tiles" is claim number frac * 32
+        # of one counter's slice (here the sixth counter's)
+        info = gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0, inject_at=5 * 32 + int(frac * 32)), stream)
+        assert info.grid == 256
+        stream.sync()
+        assert flag.get() == 1 and st.stop_index() == 0, frac
+        part = dC.download(np_dtype=np.uint16)
+        assert (part == 0x7FC0).any(), "the kernel was not interrupted"
+        relaunches = 0
+        flag.set(0)
+        while st.stop_index() != -1 or relaunches == 0:
+            st.clear_stop()
+            gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
+            stream.sync()
+            relaunches += 1
+            assert relaunches < 4
+        assert np.array_equal(dC.download(np_dtype=np.uint16).reshape(n, n), base), f"resume after {frac:.0%} differs"

@@ -93,6 +93,7 @@ def test_inception_v3_matches_oracle(gp, ex_mod, tmp_path):
 @pytest.mark.parametrize("workload,kw", [
     ("bert", dict(batch=1, seq=128, layers=12)),                       # config 3's high-priority tenant, full size
     ("bert@b=2,s=48,layers=2,dtype=f32", dict(batch=2, seq=48, layers=2)),
+    ("bert@s=384", dict(batch=1, seq=384, layers=12)),                 # config 5's high-priority tenant, full size
 ])
 def test_bert_matches_oracle(gp, ex_mod, tmp_path, workload, kw):
     dt = "f32" if "f32" in workload else "f16"

@@ -139,3 +139,99 @@ def test_vgg_and_densenet_composition_vs_torch():
     t = aff(t, "norm5").mean(dim=(2, 3))
     t = torch.softmax(t @ T(p["classifier.weight"]).T + T(p["classifier.bias"]), 1).numpy()
     assert np.abs(got - t).max() < 1e-5
+
+
+def test_inception_v3_composition_vs_torch():
+    """Inception-v3 (stem, 3 x A, B, 4 x C, D, 2 x E; TVM's relay.testing.inception_v3 layout) at an
+    eighth of the widths on a 107 x 107 image, against torch.nn.functional: branch order inside each
+    concatenation, the (kh, kw) / padding pairs of the factorised 7 x 7 and 3 x 3 filters, strides
+    of the reducing blocks and which pools count their padding."""
+    W8 = lambda c: max(c // 8, 1)
+    shapes = {}
+
+    def conv(name, cin, cout, kh=1, kw=1):
+        shapes[name + ".weight"] = (cout, cin, kh, kw)
+        shapes[name + ".bias"] = (cout,)
+        return cout
+
+    c = conv("conv", 3, W8(32), 3, 3)
+    c = conv("conv_1", c, W8(32), 3, 3)
+    c = conv("conv_2", c, W8(64), 3, 3)
+    c = conv("conv_3", c, W8(80))
+    c = conv("conv_4", c, W8(192), 3, 3)
+    i = 0
+    for proj in (32, 64, 64):
+        n = f"mixed{i}"; i += 1
+        o = conv(n + ".1x1", c, W8(64))
+        t = conv(n + ".5x5_r", c, W8(48)); o += conv(n + ".5x5", t, W8(64), 5, 5)
+        t = conv(n + ".3x3_r", c, W8(64)); t = conv(n + ".3x3_1", t, W8(96), 3, 3); o += conv(n + ".3x3_2", t, W8(96), 3, 3)
+        o += conv(n + ".proj", c, W8(proj))
+        c = o
+    n = f"mixed{i}"; i += 1
+    o = conv(n + ".3x3", c, W8(384), 3, 3)
+    t = conv(n + ".d3x3_r", c, W8(64)); t = conv(n + ".d3x3_1", t, W8(96), 3, 3); o += conv(n + ".d3x3_2", t, W8(96), 3, 3)
+    c = o + c
+    for c7 in (128, 160, 160, 192):
+        n = f"mixed{i}"; i += 1
+        o = conv(n + ".1x1", c, W8(192))
+        t = conv(n + ".7_r", c, W8(c7)); t = conv(n + ".7_1", t, W8(c7), 1, 7); o += conv(n + ".7_2", t, W8(192), 7, 1)
+        t = conv(n + ".d7_r", c, W8(c7)); t = conv(n + ".d7_1", t, W8(c7), 7, 1); t = conv(n + ".d7_2", t, W8(c7), 1, 7)
+        t = conv(n + ".d7_3", t, W8(c7), 7, 1); o += conv(n + ".d7_4", t, W8(192), 1, 7)
+        o += conv(n + ".proj", c, W8(192))
+        c = o
+    n = f"mixed{i}"; i += 1
+    t = conv(n + ".3x3_r", c, W8(192)); o = conv(n + ".3x3", t, W8(320), 3, 3)
+    t = conv(n + ".7x3_r", c, W8(192)); t = conv(n + ".7x3_1", t, W8(192), 1, 7); t = conv(n + ".7x3_2", t, W8(192), 7, 1)
+    o += conv(n + ".7x3_3", t, W8(192), 3, 3)
+    c = o + c
+    for _ in range(2):
+        n = f"mixed{i}"; i += 1
+        o = conv(n + ".1x1", c, W8(320))
+        t = conv(n + ".3_r", c, W8(384)); o += conv(n + ".3_a", t, W8(384), 1, 3) + conv(n + ".3_b", t, W8(384), 3, 1)
+        t = conv(n + ".d3_r", c, W8(448)); t = conv(n + ".d3_1", t, W8(384), 3, 3)
+        o += conv(n + ".d3_a", t, W8(384), 1, 3) + conv(n + ".d3_b", t, W8(384), 3, 1)
+        o += conv(n + ".proj", c, W8(192))
+        c = o
+    shapes["fc1.weight"] = (10, c); shapes["fc1.bias"] = (10,)
+    p = OM.random_params(shapes, 11, "cnn")
+    x = np.random.default_rng(12).normal(size=(2, 3, 107, 107)).astype(np.float32)
+    got = OM.inception_v3(p, x, "f32")
+
+    def cv(name, t, stride=1, pad=0):
+        return F.relu(F.conv2d(t, T(p[name + ".weight"]), T(p[name + ".bias"]), stride, pad))
+
+    avg = lambda t: F.avg_pool2d(t, 3, 1, 1, count_include_pad=True)
+    t = cv("conv", T(x), 2)
+    t = cv("conv_1", t)
+    t = cv("conv_2", t, 1, 1)
+    t = F.max_pool2d(t, 3, 2)
+    t = cv("conv_3", t)
+    t = cv("conv_4", t)
+    t = F.max_pool2d(t, 3, 2)
+    assert t.shape[2] == 11
+    for k in range(3):  # A blocks: 1x1 | 1x1-5x5 | 1x1-3x3-3x3 | avgpool-1x1
+        n = f"mixed{k}"
+        t = torch.cat([cv(n + ".1x1", t), cv(n + ".5x5", cv(n + ".5x5_r", t), 1, 2),
+                       cv(n + ".3x3_2", cv(n + ".3x3_1", cv(n + ".3x3_r", t), 1, 1), 1, 1), cv(n + ".proj", avg(t))], 1)
+    n = "mixed3"  # B: 3x3/2 | 1x1-3x3-3x3/2 | maxpool/2
+    t = torch.cat([cv(n + ".3x3", t, 2), cv(n + ".d3x3_2", cv(n + ".d3x3_1", cv(n + ".d3x3_r", t), 1, 1), 2), F.max_pool2d(t, 3, 2)], 1)
+    assert t.shape[2] == 5
+    for k in range(4, 8):  # C blocks: 1x1 | 1x1-1x7-7x1 | 1x1-7x1-1x7-7x1-1x7 | avgpool-1x1
+        n = f"mixed{k}"
+        b1 = cv(n + ".7_2", cv(n + ".7_1", cv(n + ".7_r", t), 1, (0, 3)), 1, (3, 0))
+        b2 = cv(n + ".d7_r", t)
+        b2 = cv(n + ".d7_1", b2, 1, (3, 0)); b2 = cv(n + ".d7_2", b2, 1, (0, 3)); b2 = cv(n + ".d7_3", b2, 1, (3, 0)); b2 = cv(n + ".d7_4", b2, 1, (0, 3))
+        t = torch.cat([cv(n + ".1x1", t), b1, b2, cv(n + ".proj", avg(t))], 1)
+    n = "mixed8"  # D: 1x1-3x3/2 | 1x1-1x7-7x1-3x3/2 | maxpool/2
+    b1 = cv(n + ".7x3_3", cv(n + ".7x3_2", cv(n + ".7x3_1", cv(n + ".7x3_r", t), 1, (0, 3)), 1, (3, 0)), 2)
+    t = torch.cat([cv(n + ".3x3", cv(n + ".3x3_r", t), 2), b1, F.max_pool2d(t, 3, 2)], 1)
+    assert t.shape[2] == 2
+    for k, pool in ((9, avg), (10, lambda u: F.max_pool2d(u, 3, 1, 1))):  # E blocks
+        n = f"mixed{k}"
+        u = cv(n + ".3_r", t)
+        v = cv(n + ".d3_1", cv(n + ".d3_r", t), 1, 1)
+        t = torch.cat([cv(n + ".1x1", t), cv(n + ".3_a", u, 1, (0, 1)), cv(n + ".3_b", u, 1, (1, 0)),
+                       cv(n + ".d3_a", v, 1, (0, 1)), cv(n + ".d3_b", v, 1, (1, 0)), cv(n + ".proj", pool(t))], 1)
+    t = t.mean(dim=(2, 3))
+    want = torch.softmax(t @ T(p["fc1.weight"]).T + T(p["fc1.bias"]), 1).numpy()
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-4
