@@ -6,7 +6,11 @@
 #include "workloads/scicomput.h"
 #include "harness.h"
 #include "gpreempt.h"
+#include "mini_json.h"
+#include "tvm_export.h"
 #include <exception>
+#include <fstream>
+#include <iterator>
 #include <map>
 #include <mutex>
 
@@ -259,4 +263,66 @@ extern "C" int gpx_suspend_streams(int fd, const int *levels, int n) {
 extern "C" int gpx_resume_streams(int fd, const int *levels, int n) {
     std::vector<int> v(levels, levels + (n > 0 ? n : 0));
     return hipResumeStreams(fd, v);
+}
+
+// ---- exported-model reader ---------------------------------------------------------------------------
+extern "C" int gpx_parse_tvm_export(const char *device_json, const char *host_json, const char *ops_json, char *report, size_t report_len) {
+    return guarded("gpx_parse_tvm_export", [&] {
+        TvmExport ex;
+        Status st = load_tvm_export(device_json ? device_json : "", host_json ? host_json : "", ex);
+        json::Value rep = json::Value::object();
+        if (st == Status::Succ && ops_json && *ops_json) {
+            std::ifstream f(ops_json, std::ios::binary);
+            if (!f.is_open()) { st = Status::NotFound; ex.error = std::string("Cannot open the json file: ") + ops_json; }
+            else {
+                std::string text((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+                ExportOps ops;
+                st = parse_export_ops(text, ops);
+                if (st != Status::Succ) ex.error = ops.error;
+                else st = check_export_ops(ex, ops, ex.error);
+                json::Value &jo = rep.set("ops");
+                jo = json::Value::array();
+                for (const ExportOp &o : ops.funcs) {
+                    json::Value e = json::Value::object();
+                    e.set("name") = o.func; e.set("op") = o.op;
+                    json::Value &a = e.set("attrs");
+                    a = json::Value::object();
+                    for (const auto &kv : o.attrs) { json::Value &l = a.set(kv.first); l = json::Value::array(); for (long v : kv.second) l.push(json::Value(v)); }
+                    json::Value &ep = e.set("epilogue");
+                    ep = json::Value::array();
+                    for (const std::string &t : o.epilogue) ep.push(json::Value(t));
+                    json::Value &in = e.set("inputs");
+                    in = json::Value::object();
+                    for (const auto &kv : o.inputs) in.set(kv.first) = kv.second;
+                    jo.push(e);
+                }
+                rep.set("layout") = ops.layout;
+            }
+        }
+        rep.set("error") = ex.error;
+        rep.set("global_len") = ex.global_len;
+        rep.set("heads_index") = ex.heads_index;
+        json::Value &js = rep.set("storages");
+        js = json::Value::array();
+        for (const StorageInfo &s : ex.storage_infos) {
+            json::Value e = json::Value::object();
+            e.set("name") = s.name; e.set("stype") = s.stype; e.set("size") = s.size;
+            js.push(e);
+        }
+        json::Value &jk = rep.set("kernels");
+        jk = json::Value::array();
+        for (size_t i = 0; i < ex.kernel_infos.size(); ++i) {
+            const KernelInfo &k = ex.kernel_infos[i];
+            json::Value e = json::Value::object();
+            e.set("name") = k.name; e.set("func") = ex.kernel_func[i];
+            json::Value &lp = e.set("launch_params");
+            lp = json::Value::array();
+            for (int j = 0; j < 6; ++j) lp.push(json::Value((long)k.launch_params[j]));
+            json::Value &ai = e.set("args_index");
+            ai = json::Value::array();
+            for (size_t a : k.args_index) ai.push(json::Value(a));
+            jk.push(e);
+        }
+        return copy_report(st, rep.dump(), report, report_len);
+    });
 }

@@ -9,7 +9,9 @@
 #include <fstream>
 
 #include "numeric.h"
+#include "tvm_export.h"
 #include "zoo.h"
+#include <sys/stat.h>
 
 namespace foo {
 
@@ -19,17 +21,23 @@ static const char kParamMagic[] = "TVM_MODEL_PARAMS";  // 16 chars + NUL = 17 by
 ModelParam *ModelParamParser::parse_from_file(const char *param_file) {
     FILE *fp = std::fopen(param_file, "rb");
     if (!fp) return nullptr;
+    // every count read from the file is checked against what the file can still hold before
+    // anything is allocated for it: a corrupt header must not ask for 64 GiB
+    struct stat sb;
+    const uint64_t file_size = fstat(fileno(fp), &sb) == 0 && sb.st_size > 0 ? (uint64_t)sb.st_size : 0;
     std::unique_ptr<ModelParam> params(new ModelParam());
     char magic[sizeof(kParamMagic)];
     uint64_t count = 0;
     bool ok = std::fread(magic, 1, sizeof(magic), fp) == sizeof(magic) && std::memcmp(magic, kParamMagic, sizeof(magic)) == 0 &&
-              std::fread(&count, sizeof(count), 1, fp) == 1 && count != 0;
+              std::fread(&count, sizeof(count), 1, fp) == 1 && count != 0 && count <= file_size / 10;  // a tensor takes >= 10 bytes
     for (uint64_t i = 0; ok && i < count; ++i) {
         std::string key;
         int c;
         while ((c = std::fgetc(fp)) != EOF && c != 0 && key.size() < 255) key.push_back((char)c);
         uint64_t n = 0;
         ok = c == 0 && std::fread(&n, sizeof(n), 1, fp) == 1 && n != 0 && n < (1ull << 34);
+        const long at = ok ? std::ftell(fp) : -1;
+        ok = ok && at >= 0 && (uint64_t)at <= file_size && n <= (file_size - (uint64_t)at) / sizeof(float);
         if (!ok) break;
         std::vector<float> values(n);
         ok = std::fread(values.data(), sizeof(float), n, fp) == n;
@@ -71,14 +79,49 @@ static std::string parent_dir_name(const std::string &path) {
     return b == std::string::npos ? dir : dir.substr(b + 1);
 }
 
-Status Model::load_model(const std::string &device_json, const std::string & /*host_json*/, const std::string & /*module*/) {
+Status Model::load_model(const std::string &device_json, const std::string &host_json, const std::string & /*module*/) {
     if (is_loaded()) {
         std::fprintf(stderr, "The model is already loaded\n");  // reference model.cpp:81-84
         return Status::Fail;
     }
     std::string name = parent_dir_name(device_json);
     if (name.empty()) return Status::NotFound;
-    return build(name);
+    // an exported graph next to the parameters is read the reference's way and checked below
+    std::ifstream dj(device_json), hj(host_json);
+    const bool have_export = dj.is_open() && hj.is_open();
+    dj.close(); hj.close();
+    if (have_export) {
+        Status s = load_from_json(device_json.c_str(), host_json.c_str());
+        if (s != Status::Succ) {
+            std::fprintf(stderr, "load_model: %s\n", export_ ? export_->error.c_str() : "cannot read the exported graph");
+            return s;
+        }
+    }
+    RETURN_STATUS(build(name));
+    if (have_export) {
+        // the native graph runs; the export must at least agree with it on what goes in and comes out
+        auto size_of = [](const std::vector<StorageInfo> &v, const std::string &key) -> long {
+            for (const StorageInfo &s : v) if (s.name == key) return (long)s.size;
+            return -1;
+        };
+        for (const char *key : {"data", "heads"}) {
+            const long a = size_of(export_->storage_infos, key), b = size_of(storage_infos, key);
+            if (a != b) {
+                std::fprintf(stderr, "load_model: %s describes a model whose \"%s\" is %ld bytes; the native graph of workload '%s' has %ld: refusing to run a different model under this name\n",
+                             device_json.c_str(), key, a, name.c_str(), b);
+                clear();
+                return Status::Fail;
+            }
+        }
+        std::fprintf(stderr, "load_model: %s and %s read (%zu storages, %zu kernels); the kernels that run are the native ones of workload '%s'\n",
+                     device_json.c_str(), host_json.c_str(), export_->storage_infos.size(), export_->kernel_infos.size(), name.c_str());
+    }
+    return Status::Succ;
+}
+
+Status Model::load_from_json(const char *device_json, const char *host_json) {
+    export_ = std::make_shared<TvmExport>();
+    return load_tvm_export(device_json, host_json, *export_);
 }
 
 Status Model::build(const std::string &workload) {

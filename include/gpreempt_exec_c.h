@@ -81,6 +81,13 @@ int gpx_preempt_probe(const char *workload, int trials, int use_graph, unsigned 
  * its values are copied to `out` and *len receives its length. */
 long gpx_parse_params(const char *path, const char *key, float *out, size_t n, size_t *len);
 
+/* Reads an exported model directory's mod.json + host.json as Model::load_from_json of the
+ * reference does (src/model.cpp:128-235) and, when ops_json is given, the operator-attribute
+ * sidecar (include/tvm_export.h), checked against the export.  The JSON report holds "storages"
+ * (name, stype, size), "kernels" (name, func, launch_params, args_index), "global_len",
+ * "heads_index", "ops" and "error".  Needs no GPU. */
+int gpx_parse_tvm_export(const char *device_json, const char *host_json, const char *ops_json, char *report, size_t report_len);
+
 /* include/gpreempt.h through the C view.  gpx_set_priority = NvRmQuery + set_priority on the
  * tenant's stream (reference src/cuda-clients/gpreemptclient.cpp:170-177); 0 or -1 as the reference.
  * A domain is a foo::PreemptDomain (one flag word per priority boundary); its handle is what

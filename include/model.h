@@ -16,6 +16,7 @@
 namespace foo {
 
 using namespace foo::util;
+struct TvmExport;
 
 class StorageInfo {
 public:
@@ -85,7 +86,17 @@ public:
     // The three paths name files inside MODEL_PATH/<workload>/ as in the reference
     // (src/executor.cpp:110-113); the workload is the name of that directory and the graph is
     // built natively from it.  `workload` may carry options: "resnet152@b=8,dtype=f16".
+    // When mod.json and host.json exist they are read as the reference reads them (load_from_json)
+    // and must describe a model with the same input ("data") and output ("heads") sizes as the
+    // native graph of that workload name; a mismatch, or files that do not parse, is Status::Fail
+    // (a caller that brings a different graph under a known name must not silently get the built-in
+    // one).  The kernels that run are always the native ones.
     Status load_model(const std::string &device_json, const std::string &host_json, const std::string &cuda_module);
+    // Model::load_from_json of the reference (src/model.cpp:128-235): storages and device kernels
+    // of an exported model.  The result is kept for inspection (tvm_export()); it does not replace
+    // the native graph.
+    Status load_from_json(const char *device_json, const char *host_json);
+    const struct TvmExport *tvm_export() const { return export_.get(); }
     Status build(const std::string &workload);
 
     // Reads a "TVM_MODEL_PARAMS" file (format of reference src/model.cpp:15-55) and uploads every
@@ -163,6 +174,7 @@ private:
     size_t ckpt_bytes_ = 0;
     int last_launch_tag_ = 0;
     std::string workload_, dtype_;
+    std::shared_ptr<struct TvmExport> export_;
     std::vector<StorageInfo> storage_infos;
     std::vector<ParamLayout> layouts;
     std::vector<KernelInfo> kernel_infos;

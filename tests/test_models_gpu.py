@@ -276,3 +276,35 @@ def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path, program):
     assert any(s != -1 for s in stops), stops  # at least one run was really interrupted
     ex.set_running(False)
     ex.resume(stream)  # running == false: no-op (executor.cpp:281)
+
+
+def test_exported_graph_next_to_the_model_is_read_and_checked(gp, ex_mod, tmp_path):
+    """mod.json + host.json in the model directory are read as the reference reads them; an export
+    that describes another model than the native graph of that name is refused, not ignored."""
+    import json
+
+    def export(n_elems):
+        mod = {"nodes": [{"op": "null", "name": "data", "inputs": []},
+                         {"op": "tvm_op", "name": "fused_add", "attrs": {"func_name": "fused_add"}, "inputs": [[0, 0, 0]]}],
+               "heads": [[1, 0, 0]],
+               "attrs": {"dltype": ["list_str", ["float32", "float32"]], "shape": ["list_shape", [[n_elems], [n_elems]]]}}
+        host = {"temp_args": [], "funcs": [{"name": "fused_add", "kernels": [{"name": "fused_add_kernel0", "launch_params": [16, 1, 1, 256, 1, 1], "args": [0, 1]}]}]}
+        return mod, host
+
+    root = tmp_path / "models"
+    d = root / "toy"
+    d.mkdir(parents=True)
+    mod, host = export(64 * 64)
+    (d / "mod.json").write_text(json.dumps(mod)); (d / "host.json").write_text(json.dumps(host))
+    ex = ex_mod.Executor("toy", model_root=str(root))  # agrees with the native toy graph (64 x 64 fp32 in and out)
+    x = np.arange(64 * 64, dtype=np.float32)
+    assert np.array_equal(run(gp, ex, x, gp.F32, (64 * 64,)), 8 * x)
+    mod, host = export(100)
+    (d / "mod.json").write_text(json.dumps(mod))
+    with pytest.raises(ex_mod.StatusError) as e:
+        ex_mod.Executor("toy", model_root=str(root))
+    assert e.value.status == 1  # Fail
+    (d / "mod.json").write_text("{ not json")
+    with pytest.raises(ex_mod.StatusError) as e:
+        ex_mod.Executor("toy", model_root=str(root))
+    assert e.value.status == 1
