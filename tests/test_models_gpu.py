@@ -308,3 +308,6 @@ def test_exported_graph_next_to_the_model_is_read_and_checked(gp, ex_mod, tmp_pa
     with pytest.raises(ex_mod.StatusError) as e:
         ex_mod.Executor("toy", model_root=str(root))
     assert e.value.status == 1
+    # the model root is process-wide (an environment variable): leave one without exported files behind
+    (d / "mod.json").unlink(); (d / "host.json").unlink()
+    os.environ["GPREEMPT_MODEL_PATH"] = str(tmp_path)
