@@ -328,3 +328,81 @@ extern "C" int gp_ckpt_reset_async(void *ckpt, gp_stream s) {
     GP_REQUIRE(ckpt != nullptr, "null checkpoint workspace");
     return gp_fill32_async(ckpt, 0, (size_t)CKPT_MAX_WGS * CKPT_HEADER_INTS, s);
 }
+
+// ---- a preemptible GEMM launch that allocates nothing -----------------------------------------------
+// gp_launch_gemm takes its claim counters and stop index from the caller's context, which somebody
+// had to allocate.  Callers that cannot allocate (code under HIP graph capture, tight serving loops,
+// harnesses that forbid it) get the same launch with that state in a file-scope device array: 64
+// kernel slots of 32 counters (one per 64-byte line), then one line that holds the stop index.
+// The array exists once per GPU for the life of the process; every call on a GPU shares it and it
+// keeps the last call's contents, so calls that overlap on one GPU race.
+namespace gp {
+constexpr int kStaticSlots = 64;      // kernels whose counters the array can hold at once
+constexpr int kStaticGroups = 32;     // claim counters per kernel, as BLPExecutor uses
+constexpr int kStaticSlotInts = kStaticGroups * COUNTER_STRIDE;
+constexpr int kStaticInts = kStaticSlots * kStaticSlotInts + COUNTER_STRIDE;   // 131 136 bytes
+constexpr int kStaticMaxDevices = 16;
+static __device__ __align__(256) int scratch[kStaticInts];
+
+// `scratch` is only a host-side stand-in here: the array's address on each device comes from
+// hipGetSymbolAddress, once per device, with that device current.
+static std::mutex g_scratch_mu;
+static int *g_scratch_ptr[kStaticMaxDevices] = {nullptr};
+
+int static_scratch_setup(int **out) {
+    int dev = -1;
+    GP_HIP(hipGetDevice(&dev));
+    GP_REQUIRE(dev >= 0 && dev < kStaticMaxDevices, "device %d is beyond the %d the static scratch serves", dev, kStaticMaxDevices);
+    std::lock_guard<std::mutex> g(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        GP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        GP_REQUIRE(p != nullptr, "hipGetSymbolAddress returned no address for the static scratch");
+        g_scratch_ptr[dev] = (int *)p;
+    }
+    if (out) *out = g_scratch_ptr[dev];
+    return GP_SUCC;
+}
+
+// Clears one slot's counter lines and re-arms the stop index (a kernel, not a memset: the call may
+// be recorded into a graph).
+__global__ void static_reset_kernel(int *counters, int n, int *stop) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (counters && i < n) counters[i] = 0;
+    if (stop && i == 0) *stop = -1;
+}
+__global__ void static_report_kernel(const int *stop, int *out) {
+    if (threadIdx.x == 0) __hip_atomic_store(out, *stop, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+}  // namespace gp
+
+extern "C" int gp_launch_gemm_noalloc(const gp_gemm_params *p, int *flag, int slot, int mode, int inject_at, int *stop_index_out,
+                                      gp_stream s, gp_launch_info *info) {
+    GP_REQUIRE(mode >= 0 && mode <= (GP_NOALLOC_CLEAR | GP_NOALLOC_REARM), "mode %d", mode);
+    GP_REQUIRE(slot >= 0 && slot < kStaticSlots, "slot %d: the static scratch holds the counters of %d kernels (slots 0..%d)", slot, kStaticSlots, kStaticSlots - 1);
+    MatPlan pl;
+    int rc = plan_gemm(p, &pl);
+    if (rc) return rc;
+    // every claim must be countable in the slot: the tile grid is bounded like a launch's
+    GP_REQUIRE((long)pl.sx * pl.sy * pl.batch <= (1L << 24), "gemm of %ld tiles: the static scratch serves at most %ld per launch", (long)pl.sx * pl.sy * pl.batch, 1L << 24);
+    int *base = nullptr;
+    rc = static_scratch_setup(&base);
+    if (rc) return rc;
+    int *counters = base + (size_t)slot * kStaticSlotInts, *stop = base + (size_t)kStaticSlots * kStaticSlotInts;
+    if (mode) {
+        hipLaunchKernelGGL(static_reset_kernel, dim3((kStaticSlotInts + 255) / 256), dim3(256), 0, native(s),
+                           (mode & GP_NOALLOC_CLEAR) ? counters : (int *)nullptr, kStaticSlotInts, (mode & GP_NOALLOC_REARM) ? stop : (int *)nullptr);
+        GP_HIP(hipGetLastError());
+    }
+    gp_preempt_ctx ctx{};
+    ctx.flag = flag; ctx.stop_index = stop; ctx.executed = counters; ctx.kernel_id = slot; ctx.inject_at = inject_at;
+    ctx.counter_groups = kStaticGroups;
+    ctx.fresh = (mode & GP_NOALLOC_CLEAR) != 0;
+    rc = launch_mat_plan(pl, &ctx, s, info);
+    if (rc) return rc;
+    if (stop_index_out) {
+        hipLaunchKernelGGL(static_report_kernel, dim3(1), dim3(64), 0, native(s), (const int *)stop, stop_index_out);
+        GP_HIP(hipGetLastError());
+    }
+    return GP_SUCC;
+}

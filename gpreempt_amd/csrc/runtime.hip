@@ -13,6 +13,7 @@ void set_error(const char *fmt, ...) {
     va_end(ap);
 }
 
+int static_scratch_setup(int **out);  // gemm.hip
 static std::atomic<int> g_cus{0};
 static std::atomic<int> g_device{-1};
 int device_cus() {
@@ -79,6 +80,8 @@ extern "C" int gp_init(int device) {
     GP_HIP(hipGetDeviceCount(&n));
     GP_REQUIRE(device >= 0 && device < n, "device %d not present (%d visible)", device, n);
     GP_HIP(hipSetDevice(device));
+    // address of the library's static scratch on this device (gp_launch_gemm_noalloc)
+    if (int rc = static_scratch_setup(nullptr)) return rc;
     if (g_device.load() != device) {
         hipDeviceProp_t prop;
         GP_HIP(hipGetDeviceProperties(&prop, device));

@@ -175,6 +175,24 @@ typedef struct gp_gemm_params {
     int variant;        /* enum gp_mat_variant; 0 = chosen by the launcher */
 } gp_gemm_params;
 int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+/* No counterpart in the reference: gp_launch_gemm for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The
+ * preemption state that gp_preempt_ctx otherwise brings in (32 claim counters per kernel, the stop
+ * index) lives in a device array inside the library: 64 kernel slots, 131 136 bytes per GPU, held
+ * until the process ends.  This call allocates and frees nothing.
+ *   flag            device-visible address of the preempt flag (gp_flag_create), may be NULL
+ *   slot            0..63: which kernel's counters to use; also the kernel id written to the stop index
+ *   mode            GP_NOALLOC_CLEAR: zero the slot's counters first (a fresh run of this kernel);
+ *                   GP_NOALLOC_REARM: set the stop index to -1 first (the first kernel of a submission
+ *                   or of a resume); 0 continues from the counters as they are (BLPExecutor::resume)
+ *   inject_at       test hook as gp_preempt_ctx::inject_at; -1 = off
+ *   stop_index_out  may be NULL: device-visible int that receives the stop index after the launch
+ * Every call on a GPU shares that GPU's array, which keeps the last call's contents: calls that
+ * overlap on one GPU (two streams, two threads) race.  Long tiles are finished, not left half-way
+ * (there is no checkpoint workspace).  Slots beyond 63 and GEMMs of more than 2^24 tiles are refused. */
+enum { GP_NOALLOC_CLEAR = 1, GP_NOALLOC_REARM = 2 };
+int gp_launch_gemm_noalloc(const gp_gemm_params *p, int *flag, int slot, int mode, int inject_at, int *stop_index_out,
+                           gp_stream s, gp_launch_info *info);
 /* Bytes of gp_preempt_ctx::ckpt workspace this GEMM can use (0: it runs on a body whose tiles are
  * short and always finished), and the reset of such a workspace.  Extension of the dispatcher that
  * scripts/compile/convert_to_blp.py:40-69 generates (which can only stop between tiles). */
