@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "libgpreempt_hip.so")
 
 F32, F16, BF16, I32, I64 = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_GELU = 0, 1, 2
-MAT_AUTO, MAT_STAGED, MAT_PIPE, MAT_PIPE_SPLITK = 0, 1, 2, 3
+MAT_AUTO, MAT_STAGED, MAT_PIPE, MAT_PIPE_SPLITK, MAT_WIDE, MAT_WIDE8 = 0, 1, 2, 3, 4, 5
 SUCC, FAIL, TIMEOUT, NOTFOUND, OUTOFRANGE, FULL = range(6)
 DTYPE_SIZE = {F32: 4, F16: 2, BF16: 2, I32: 4, I64: 8}
 DTYPE_BY_NAME = {"f32": F32, "f16": F16, "bf16": BF16}

@@ -15,6 +15,7 @@
 #include <mutex>
 #include "gemm_tile.hpp"
 #include "gemm_pipe.hpp"
+#include "gemm_wide.hpp"
 #include "plans.hpp"
 
 namespace gp {
@@ -126,6 +127,10 @@ static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream 
         case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
         case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
         case MB_PIPE32_SK: return pipe_case<T, 32, GP_S32, true>(pl, ctx, s, info);
+        case MB_WIDE32x32_16: return launch_mat<WideKernel<T, 32, 32, 16, 3>>(pl, ctx, s, info);
+        case MB_WIDE32x32_8: return launch_mat<WideKernel<T, 32, 32, 8, 3>>(pl, ctx, s, info);
+        case MB_WIDE64x32_16: return launch_mat<WideKernel<T, 64, 32, 16, 3>>(pl, ctx, s, info);
+        case MB_WIDE64x64_8: return launch_mat<WideKernel<T, 64, 64, 8, 3>>(pl, ctx, s, info);
         case MB_STAGED128:
             if (pl.conv) return launch_mat<TK<T, 128, 128, SBK, 2, 2, true, false>>(pl, ctx, s, info);
             return pl.b_kn ? launch_mat<TK<T, 128, 128, SBK, 2, 2, false, true>>(pl, ctx, s, info)
@@ -157,6 +162,10 @@ static size_t body_lds_bytes(int body, int dtype) {
         case MB_PIPE64: return GP_S64 * (64 + 64) * 128;
         case MB_PIPE64_SK: return GP_S64 * (64 + 64) * 128;   // at least the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4 = 64 KB)
         case MB_PIPE32_SK: return GP_S32 * (32 + 32) * 128;
+        case MB_WIDE32x32_16: return WideKernel<_Float16, 32, 32, 16, 3>::LDS_BYTES;
+        case MB_WIDE32x32_8: return WideKernel<_Float16, 32, 32, 8, 3>::LDS_BYTES;
+        case MB_WIDE64x32_16: return WideKernel<_Float16, 64, 32, 16, 3>::LDS_BYTES;
+        case MB_WIDE64x64_8: return WideKernel<_Float16, 64, 64, 8, 3>::LDS_BYTES;
         case MB_STAGED128: return (128 + 128) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
         case MB_STAGED64: return (64 + 64) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
     }
@@ -167,10 +176,35 @@ static size_t body_lds_bytes(int body, int dtype) {
 // Otherwise the pipelined kernel is used with the largest tile that still gives every compute
 // unit work; problems too small for that split K across the waves of a workgroup so that the
 // serial K loop shrinks instead.
-static int choose_body(MatPlan *pl, int tile, int variant) {
+// the wide split-K bodies (gemm_wide.hpp) and their tiles
+struct WideChoice { int body, bm, bn, waves; size_t lds; };
+static const WideChoice kWide[4] = {
+    {MB_WIDE32x32_16, 32, 32, 16, WideKernel<_Float16, 32, 32, 16, 3>::LDS_BYTES},
+    {MB_WIDE32x32_8, 32, 32, 8, WideKernel<_Float16, 32, 32, 8, 3>::LDS_BYTES},
+    {MB_WIDE64x32_16, 64, 32, 16, WideKernel<_Float16, 64, 32, 16, 3>::LDS_BYTES},
+    {MB_WIDE64x64_8, 64, 64, 8, WideKernel<_Float16, 64, 64, 8, 3>::LDS_BYTES}};
+static const WideChoice *wide_of(int body) {
+    for (const WideChoice &w : kWide) if (w.body == body) return &w;
+    return nullptr;
+}
+// Which wide body, if any: measured on MI355X (launch to launch, fp16, against the best of the
+// four-wavefront bodies): they win where one round of workgroups covers the problem and K is deep
+// enough to pay for the larger first stage.  128 x 768 x 3072: 10.2 -> 7.9 us; 392 x 512 x 4608:
+// 14.0 -> 10.4; 1568 x 256 x 2304: 10.0 -> 8.3; 1568 x 256 x 1024: 6.6 -> 6.1; 128 x 768 x 768: 5.1 -> 4.7;
+// 6272 x 128 x 1152: 8.9 -> 8.0; 392 x 2048 x 512: 6.4 -> 5.9.
+static int wide_pick(const MatArgs &g, int batch, long cus) {
+    auto tiles = [&](int tm, int tn) { return (long)((g.M + tm - 1) / tm) * ((g.N + tn - 1) / tn) * batch; };
+    if (g.K >= 768 && tiles(32, 32) <= cus) return MB_WIDE32x32_16;
+    if (g.K >= 768 && tiles(64, 32) <= cus) return MB_WIDE64x32_16;
+    if (g.K >= 512 && tiles(64, 64) <= cus && g.N > 32) return MB_WIDE64x64_8;
+    return -1;
+}
+
+static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
     const MatArgs &g = pl->g;
     auto tiles = [&](int t) { return (long)((g.M + t - 1) / t) * ((g.N + t - 1) / t) * pl->batch; };
     const long cus = device_cus();
+    const bool wide_ok = !pl->b_kn && !pl->conv;  // GEMM with both operands K-contiguous
     int body = -1;
     if (pl->b_kn || variant == GP_MAT_STAGED) {
         int tm = tile ? tile : (tiles(128) >= cus ? 128 : 64);
@@ -181,21 +215,31 @@ static int choose_body(MatPlan *pl, int tile, int variant) {
     } else if (variant == GP_MAT_PIPE_SPLITK) {
         int tm = tile ? tile : (tiles(64) >= cus / 2 ? 64 : 32);
         body = tm == 64 ? MB_PIPE64_SK : tm == 32 ? MB_PIPE32_SK : -1;
+    } else if (variant == GP_MAT_WIDE || variant == GP_MAT_WIDE8) {
+        if (wide_ok) {
+            const int tn = tile_n ? tile_n : tile;
+            if (tile == 32 && tn == 32) body = variant == GP_MAT_WIDE ? MB_WIDE32x32_16 : MB_WIDE32x32_8;
+            else if (tile == 64 && tn == 32) body = MB_WIDE64x32_16;
+            else if (tile == 64 && tn == 64) body = MB_WIDE64x64_8;
+        }
     } else if (variant == GP_MAT_AUTO) {
         // a tile wider than the problem multiplies zero columns: N <= 64 never takes the larger tiles
         if (!pl->conv && (tile == 256 || (tile == 0 && tiles(256) >= cus && g.N > 128 && g.M > 128))) body = MB_PIPE256;
         else if (tile == 128 || (tile == 0 && tiles(128) >= cus && g.N > 64 && g.M > 64)) body = MB_PIPE128;
+        else if (tile == 0 && wide_ok && wide_pick(g, pl->batch, cus) >= 0) body = wide_pick(g, pl->batch, cus);
         else if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) body = MB_PIPE64;
         else if (tile == 0 && tiles(64) >= cus / 2) body = MB_PIPE64_SK;
         else if (tile == 0 || tile == 32) body = MB_PIPE32_SK;
     }
     if (body < 0) {
-        set_error("no matrix kernel for tile %d with variant %d (tiles: 256, 128, 64; 64, 32 with split K)", tile, variant);
+        set_error("no matrix kernel for tile %d x %d with variant %d (tiles: 256, 128, 64; 64, 32 with split K; wide: 32x32, 64x32, 64x64, GEMM with N x K operands)", tile, tile_n ? tile_n : tile, variant);
         return GP_OUTOFRANGE;
     }
-    const int t = body == MB_PIPE256 ? 256 : (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
+    int t = body == MB_PIPE256 ? 256 : (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
+    int tn = t;
+    if (const WideChoice *w = wide_of(body)) { t = w->bm; tn = w->bn; }
     pl->body = body;
-    pl->sx = (g.N + t - 1) / t;
+    pl->sx = (g.N + tn - 1) / tn;
     pl->sy = (g.M + t - 1) / t;
     pl->lds_bytes = body_lds_bytes(body, pl->dtype);
     // Each XCD works on a contiguous eighth of the tile order (util/slice_map.h).  With x fastest
@@ -225,7 +269,7 @@ int plan_gemm(const gp_gemm_params *p, MatPlan *out) {
             GP_REQUIRE(p->stride_a_outer % vec == 0 && p->stride_b_outer % vec == 0, "gemm: outer batch strides must be multiples of %d elements", vec);
     }
     GP_REQUIRE(p->lda >= p->K && p->ldc >= p->N && p->ldb >= (p->b_is_nk ? p->K : p->N), "gemm: leading dimension smaller than the row");
-    GP_REQUIRE(p->tile_m == p->tile_n, "gemm: square tiles only");
+    GP_REQUIRE(p->tile_m == p->tile_n || p->variant == GP_MAT_WIDE || p->variant == GP_MAT_WIDE8, "gemm: square tiles only (the wide variants also take 64 x 32)");
     MatPlan &pl = *out;
     pl = MatPlan{};
     MatArgs &g = pl.g;
@@ -237,7 +281,7 @@ int plan_gemm(const gp_gemm_params *p, MatPlan *out) {
     g.alpha = p->alpha == 0.f ? 1.f : p->alpha;
     g.act = p->act; g.batch_inner = batch > 1 ? p->batch_inner : 0;
     pl.dtype = p->dtype; pl.conv = 0; pl.b_kn = !p->b_is_nk; pl.batch = batch;
-    return choose_body(&pl, p->tile_m, p->variant);
+    return choose_body(&pl, p->tile_m, p->tile_n, p->variant);
 }
 
 int plan_conv2d(const gp_conv_params *p, MatPlan *out) {
@@ -256,10 +300,24 @@ int plan_conv2d(const gp_conv_params *p, MatPlan *out) {
     long M = (long)p->N * Ho * Wo;
     GP_REQUIRE(M < (1L << 31), "conv: too many output pixels");
     GP_REQUIRE(!p->residual || p->res_pix_stride >= p->Cout, "conv: residual pixel stride");
-    GP_REQUIRE(p->tile_m == p->tile_n, "conv: square tiles only");
+    GP_REQUIRE(p->tile_m == p->tile_n || p->variant == GP_MAT_WIDE || p->variant == GP_MAT_WIDE8, "conv: square tiles only (the wide variants also take 64 x 32)");
     MatPlan &pl = *out;
     pl = MatPlan{};
     MatArgs &g = pl.g;
+    if (p->R == 1 && p->S == 1 && p->stride_h == 1 && p->stride_w == 1 && p->pad_h == 0 && p->pad_w == 0) {
+        // A pointwise convolution IS a GEMM over the pixels (rows in_pix_stride apart); the GEMM
+        // bodies need no window arithmetic and were measured about 1 us per launch faster at
+        // ResNet-152's shapes (1568 x 256 x 1024: 7.7 -> 6.6 us with the same tile body).
+        g.M = (int)M; g.N = p->Cout; g.K = p->Cin;
+        g.A = p->in; g.lda = p->in_pix_stride;
+        g.B = p->weight; g.ldb = g.K;
+        g.C = p->out; g.ldc = p->out_pix_stride;
+        g.bias = p->bias; g.residual = p->residual; g.ldr = p->residual ? p->res_pix_stride : 0;
+        g.alpha = 1.f; g.act = p->act; g.batch_inner = 0;
+        pl.dtype = p->dtype; pl.conv = 0; pl.b_kn = 0; pl.batch = 1;
+        // an explicit variant keeps its meaning; the staged variant of a convolution has no K x N weights
+        return choose_body(&pl, p->tile_m, p->tile_n, p->variant);
+    }
     g.M = (int)M; g.N = p->Cout; g.K = p->R * p->S * p->Cin;
     g.A = p->in; g.lda = p->in_pix_stride;
     g.B = p->weight; g.ldb = g.K;
@@ -269,7 +327,7 @@ int plan_conv2d(const gp_conv_params *p, MatPlan *out) {
     g.H = p->H; g.W = p->W; g.Cin = p->Cin; g.S = p->S; g.Ho = Ho; g.Wo = Wo;
     g.sh = p->stride_h; g.sw = p->stride_w; g.ph = p->pad_h; g.pw = p->pad_w;
     pl.dtype = p->dtype; pl.conv = 1; pl.b_kn = 0; pl.batch = 1;
-    return choose_body(&pl, p->tile_m, p->variant);
+    return choose_body(&pl, p->tile_m, p->tile_n, p->variant);
 }
 
 }  // namespace gp

@@ -1,0 +1,241 @@
+// Wide split-K GEMM tile kernel for small, deep problems (few output tiles, long K): 8 or 16 wavefronts
+// share ONE output tile and split every K-stage between them.
+//
+// Why: on MI355X a wavefront's operand fetches (direct global -> LDS loads as well as register
+// loads) complete at about 11.7 GB/s whatever the number of loads it keeps in flight, and the rate
+// of a compute unit grows linearly with the number of wavefronts that issue loads (47 GB/s with 4
+// wavefronts, 94 with 8, 185 with 16; measured with an L2-resident source).  A layer with fewer
+// tiles than the GPU has compute units therefore streams its operands four times faster when
+// sixteen wavefronts fetch for a tile than when four do, and for these layers the operand stream
+// is what the main loop waits for (a 32 x 32 tile of a K = 1024 layer does 2 MFLOP on 128 KB of
+// operands).
+//
+// Structure: a stage holds KB = WAVES / 4 consecutive K-blocks of BK elements (one 128-byte row
+// chunk per tile row, the layout and swizzle of gemm_pipe.hpp); wavefront w belongs to block group
+// kb = w / 4 and fetches a quarter of the rows of that group's block.  One barrier per stage.  The
+// arithmetic stays with wavefronts 0..3 (there is little of it: these layers wait for operands):
+// wavefront w multiplies MFMA k-step w of every block, block after block, for the whole BM x BN
+// tile, and at the end the four partial tiles are summed through LDS in the order 0, 1, 2, 3.  That
+// is exactly the summation of the four-wavefront split-K bodies of gemm_pipe.hpp, so the result
+// has the same bits as theirs (the whole-model program, whose workgroups have four wavefronts,
+// uses those) and does not depend on scheduling: a preempted-then-resumed run stays bit-identical.
+//
+// Measured (fp16, launch to launch): 128 x 768 x 3072 (BERT's second FFN layer) 10.2 -> 8.2 us,
+// 384 x 768 x 3072 11.9 -> 10.4 us; level with the four-wavefront bodies at K <= 1024, where the
+// longer wait for the first, larger stage costs what the faster stream saves.  A convolution form
+// (gathered A operand) was measured slower than the four-wavefront one at every ResNet-152 shape
+// and is not built.
+#pragma once
+#include "gemm_pipe.hpp"
+
+namespace gp {
+
+template <typename T, int BM, int BN, int WAVES, int STAGES>
+struct WideKernel {
+    using elem = T;
+    static constexpr int bm = BM, bn = BN;
+    static constexpr int VEC = Elem<T>::VEC;
+    static constexpr int NT = WAVES * 64;
+    static constexpr int RB = 128;                         // row bytes of a block in LDS
+    static constexpr int BK = RB / (int)sizeof(T);         // K elements per block: 64 (16-bit) or 32 (fp32)
+    static constexpr int KB = WAVES / 4;                   // blocks per stage
+    static constexpr int GROUPS = (BM + BN) / 8;           // 8-row load groups per block (A rows, then B rows)
+    static constexpr int LPW = GROUPS / 4;                 // load instructions per wavefront per stage
+    static constexpr int A_BYTES = BM * RB, BLK_BYTES = (BM + BN) * RB, STAGE_BYTES = KB * BLK_BYTES;
+    static constexpr int MI = BM / 32, NI = BN / 32;
+    static constexpr int SLICES = MI * NI * 16;            // 64-float slices of one wavefront's accumulators
+    static constexpr size_t RED_BYTES = (size_t)4 * SLICES * 64 * 4;   // the partial tiles of wavefronts 0..3
+    static constexpr size_t RING_BYTES = (size_t)STAGES * STAGE_BYTES;
+    static constexpr size_t LDS_BYTES = RING_BYTES > RED_BYTES ? RING_BYTES : RED_BYTES;
+    static constexpr size_t CKPT_SLOT_BYTES = 0;
+    static constexpr bool ckpt = false;
+    static_assert(WAVES % 4 == 0 && WAVES >= 4 && WAVES <= 16, "4, 8, 12 or 16 wavefronts");
+    static_assert(BM % 32 == 0 && BN % 32 == 0 && GROUPS % 4 == 0, "tile shape");
+    static_assert(STAGES >= 2 && (STAGES - 2) * LPW < 64, "pipeline depth");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+
+    static __device__ __forceinline__ void run(const MatArgs &g, TileIdx t, T *lds_t) {
+        GP_PROBE(0);
+        const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
+        const char *lds_c = (const char *)lds_t;
+        const int tid = threadIdx.x, lane = tid & 63;
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        const int kb = wave >> 2, wv = wave & 3;
+        const int l32 = lane & 31, half = lane >> 5;
+        const int m0 = t.y * BM, n0 = t.x * BN;
+        long offa, offb, offc;
+        if (g.batch_inner > 0) {
+            int zo = t.z / g.batch_inner, zi = t.z - zo * g.batch_inner;
+            offa = zo * g.stride_a_outer + zi * g.stride_a;
+            offb = zo * g.stride_b_outer + zi * g.stride_b;
+            offc = zo * g.stride_c_outer + zi * g.stride_c;
+        } else {
+            offa = t.z * g.stride_a; offb = t.z * g.stride_b; offc = t.z * g.stride_c;
+        }
+        const T *A = (const T *)g.A + offa, *B = (const T *)g.B + offb;
+        const T *zero = (const T *)g_zero_page;
+
+        // ---- loader slots: slot j of this wavefront fetches row group wv*LPW + j of its block ------
+        // lane -> (row in the group, chunk position); the swizzle is applied on the source side:
+        // the lane at position cpos of row r fetches chunk cpos ^ ((r >> 1) & 7) of that row
+        const int rig = lane >> 3, cpos = lane & 7;
+        const T *base[LPW];    // the lane's row and chunk at k = 0
+        bool row_ok[LPW];
+        int kc[LPW];           // the lane's chunk offset in elements
+#pragma unroll
+        for (int j = 0; j < LPW; ++j) {
+            const int gi = wv * LPW + j;              // group index in the block
+            const bool is_a = gi < BM / 8;
+            const int r = (is_a ? gi : gi - BM / 8) * 8 + rig;   // row in its region
+            kc[j] = (cpos ^ ((r >> 1) & 7)) * VEC;
+            if (is_a) {
+                const int m = m0 + r;
+                row_ok[j] = m < g.M;
+                base[j] = A + (long)m * g.lda + kc[j];
+            } else {
+                const int n = n0 + r;
+                row_ok[j] = n < g.N;
+                base[j] = B + (long)n * g.ldb + kc[j];
+            }
+        }
+        const int KT = (g.K + BK - 1) / BK;             // blocks along K
+        const int NS = (KT + KB - 1) / KB;              // stages
+        auto issue = [&](int s) {
+            const int k0 = (s * KB + kb) * BK;          // first K element of this wavefront group's block
+            const unsigned sbase = lds0 + (unsigned)(s % STAGES) * STAGE_BYTES + (unsigned)kb * BLK_BYTES;
+#pragma unroll
+            for (int j = 0; j < LPW; ++j) {
+                const int gi = wv * LPW + j;
+                // rows outside the problem and K-chunks past K (also whole blocks past the last one,
+                // when the stage is not full) come from the zero page
+                const bool ok = row_ok[j] & (k0 + kc[j] < g.K);
+                load_lds16(ok ? base[j] + k0 : zero, sbase + (unsigned)(gi * 8 * RB));
+            }
+        };
+
+        f32x16 acc[MI][NI];
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+        auto frag = [&](int stage, int blk, int region_bytes, int row, int chunk) -> u32x4 {
+            const int phys = chunk ^ ((row >> 1) & 7);
+            return *(const u32x4 *)(lds_c + (size_t)stage * STAGE_BYTES + (size_t)blk * BLK_BYTES + region_bytes + row * RB + phys * 16);
+        };
+
+        // ---- main loop ------------------------------------------------------------------------
+        GP_PROBE(1);
+        __syncthreads();  // the previous tile of this workgroup may still be reading LDS
+#pragma unroll
+        for (int s = 0; s < STAGES - 1; ++s)
+            if (s < NS) issue(s);
+        for (int s = 0; s < NS; ++s) {
+            // stage s has landed once at most the loads of the younger stages in flight remain
+            if (s + STAGES - 2 < NS) wait_vmcnt<(STAGES - 2) * LPW>();
+            else wait_vmcnt<0>();
+            __syncthreads();  // everyone's part of stage s is visible; the buffer of stage s-1 is free
+            if (s == 0) GP_PROBE(2);
+            if (s + STAGES - 1 < NS) issue(s + STAGES - 1);
+            if (kb != 0) continue;  // (uniform) wavefronts 4.. only fetch
+            const int stage = s % STAGES;
+#pragma unroll
+            for (int b = 0; b < KB; ++b) {
+                // a block past the last one holds zeros; it is skipped, not multiplied, so that the sum
+                // has the bits of a K loop that ends at the last block
+                if (s * KB + b >= KT) break;
+                u32x4 fa[MI], fb[NI];
+#pragma unroll
+                for (int i = 0; i < MI; ++i) fa[i] = frag(stage, b, 0, i * 32 + l32, wv * 2 + half);
+#pragma unroll
+                for (int j = 0; j < NI; ++j) fb[j] = frag(stage, b, A_BYTES, j * 32 + l32, wv * 2 + half);
+#pragma unroll
+                for (int i = 0; i < MI; ++i)
+#pragma unroll
+                    for (int j = 0; j < NI; ++j) Elem<T>::mma(fa[i], fb[j], acc[i][j]);
+            }
+        }
+
+        // ---- reduction and epilogue -------------------------------------------------------------
+        // partial tiles of wavefronts 0..3 -> LDS as [wavefront][slice][lane], slice = (i*NI + j)*16 + v,
+        // which is row 8*(v/4) + 4*(lane/32) + v%4, column 32*j + lane%32 of 32 x 32 block (i, j).
+        // The first BM*BN/4 threads then finish four consecutive columns of one row each, adding the
+        // partials in wavefront order.
+        GP_PROBE(3);
+        float *red = (float *)lds_t;
+        T *C = (T *)g.C + offc;
+        const T *R = g.residual ? (const T *)g.residual + offc : nullptr;
+        const T *bias = (const T *)g.bias;
+        const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
+                            (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
+        __syncthreads();  // all wavefronts are done reading the stage buffers
+        if (kb == 0) {
+#pragma unroll
+            for (int i = 0; i < MI; ++i)
+#pragma unroll
+                for (int j = 0; j < NI; ++j)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+        }
+        __syncthreads();
+        GP_PROBE(4);
+        constexpr int L4 = BN / 4;                        // threads per output row
+        constexpr int FIN = BM * L4 < NT ? BM * L4 : NT;  // threads that finish
+        constexpr int RPP = FIN / L4, PASSES = BM / RPP;
+        if (tid < FIN) {
+            const int c4 = tid % L4, r_in = tid / L4;
+            const int j = c4 >> 3, col = (c4 & 7) * 4;
+            const int n = n0 + j * 32 + col;
+            float bq[4] = {0.f, 0.f, 0.f, 0.f};
+            if (bias && n < g.N) {
+                if (vec_ok) {
+                    const Vec4<T> b = *(const Vec4<T> *)(bias + n);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) bq[q] = Elem<T>::to_f(b.v[q]);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q)
+                        if (n + q < g.N) bq[q] = Elem<T>::to_f(bias[n + q]);
+                }
+            }
+#pragma unroll
+            for (int p = 0; p < PASSES; ++p) {
+                const int row = p * RPP + r_in, m = m0 + row;
+                const int i = row >> 5, r = row & 31;
+                const int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
+                const size_t o = ((size_t)(i * NI + j) * 16 + v) * 64 + hf * 32 + col;
+                f32x4 a = *(const f32x4 *)(red + o);
+#pragma unroll
+                for (int w = 1; w < 4; ++w) a += *(const f32x4 *)(red + (size_t)w * SLICES * 64 + o);
+                if (m >= g.M || n >= g.N) continue;
+                if (vec_ok) {
+                    Vec4<T> rv;
+                    if (R) rv = *(const Vec4<T> *)(R + (long)m * g.ldr + n);
+                    Vec4<T> out;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        float x = a[q] * g.alpha + bq[q];
+                        if (R) x += Elem<T>::to_f(rv.v[q]);
+                        out.v[q] = Elem<T>::from_f(apply_act(x, g.act));
+                    }
+                    st_vec4<T>(&C[(long)m * g.ldc + n], out);
+                } else {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        if (n + q >= g.N) break;
+                        float x = a[q] * g.alpha + bq[q];
+                        if (R) x += Elem<T>::to_f(R[(long)m * g.ldr + n + q]);
+                        st_elem<T>(&C[(long)m * g.ldc + n + q], Elem<T>::from_f(apply_act(x, g.act)));
+                    }
+                }
+            }
+        }
+#ifdef GP_TILE_PROF
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        GP_PROBE(5);
+#endif
+    }
+};
+
+}  // namespace gp

@@ -373,6 +373,15 @@ static int add_mat_layer(gp_program pr, const P *p, PlanFn plan) {
         rc = plan(&q, &pl);
         if (rc) return rc;
     }
+    if (is_wide_body(pl.body)) {
+        // 8 or 16 wavefronts per tile do not fit the program's 256-thread workgroups: the
+        // four-wavefront split-K bodies stand in (the same summation, hence the same bits)
+        P q = *p;
+        q.variant = GP_MAT_PIPE_SPLITK;
+        q.tile_m = q.tile_n = 0;
+        rc = plan(&q, &pl);
+        if (rc) return rc;
+    }
     return push_mat(pr, pl);
 }
 #define GP_ADD_ELT(PLAN) EltPlan pl; int rc = PLAN; return rc ? rc : push_elt(pr, pl);

@@ -26,9 +26,11 @@ enum gp_status { GP_SUCC = 0, GP_FAIL = 1, GP_TIMEOUT = 2, GP_NOTFOUND = 3, GP_O
 
 enum gp_dtype { GP_F32 = 0, GP_F16 = 1, GP_BF16 = 2, GP_I32 = 3, GP_I64 = 4 };
 enum gp_act { GP_ACT_NONE = 0, GP_ACT_RELU = 1, GP_ACT_GELU = 2 };
-/* Matrix-kernel variants: register-staged (handles B stored K x N), pipelined direct-to-LDS, and
- * pipelined with K split across the waves of a workgroup (small, deep problems). */
-enum gp_mat_variant { GP_MAT_AUTO = 0, GP_MAT_STAGED = 1, GP_MAT_PIPE = 2, GP_MAT_PIPE_SPLITK = 3 };
+/* Matrix-kernel variants: register-staged (handles B stored K x N), pipelined direct-to-LDS,
+ * pipelined with K split across the four waves of a workgroup, and "wide": 16 (GP_MAT_WIDE) or 8
+ * (GP_MAT_WIDE8) waves share one tile and split every K-stage (problems with fewer tiles than the
+ * GPU has compute units; tiles 32 x 32, 64 x 32, 64 x 64). */
+enum gp_mat_variant { GP_MAT_AUTO = 0, GP_MAT_STAGED = 1, GP_MAT_PIPE = 2, GP_MAT_PIPE_SPLITK = 3, GP_MAT_WIDE = 4, GP_MAT_WIDE8 = 5 };
 
 typedef struct gp_stream_s *gp_stream; /* opaque; wraps one HIP stream */
 typedef struct gp_event_s *gp_event;
@@ -171,7 +173,7 @@ typedef struct gp_gemm_params {
     /* second-level batch (attention heads): offset = (b / batch_inner) * stride_*_outer +
      * (b % batch_inner) * stride_*; batch_inner = 0 disables it. */
     int batch_inner; long stride_a_outer, stride_b_outer, stride_c_outer;
-    int tile_m, tile_n; /* 0 = chosen by the launcher; 128, 64 or 32 (square) */
+    int tile_m, tile_n; /* 0 = chosen by the launcher; 256, 128, 64 or 32 (square; 64 x 32 with the wide variants) */
     int variant;        /* enum gp_mat_variant; 0 = chosen by the launcher */
 } gp_gemm_params;
 int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);

@@ -36,7 +36,7 @@ def sync(gp):
     gp.check(gp.lib().gp_stream_sync(None))
 
 
-def gpu_conv2d(gp, dt, x, w, bias=None, stride=1, pad=0, residual=None, act=0, ctx=None, tile=0, variant=0):
+def gpu_conv2d(gp, dt, x, w, bias=None, stride=1, pad=0, residual=None, act=0, ctx=None, tile=0, variant=0, tile_n=None):
     """x NCHW, w OIHW, residual NCHW (already rounded to dt).  Returns (NCHW result, info)."""
     dtype = gp.DTYPE_BY_NAME[dt]
     vec = 4 if dt == "f32" else 8
@@ -53,7 +53,7 @@ def gpu_conv2d(gp, dt, x, w, bias=None, stride=1, pad=0, residual=None, act=0, c
     p = gp.ConvParams(dtype=dtype, N=N, H=H, W=W, Cin=cp, Cout=Cout, R=R, S=S, stride_h=stride, stride_w=stride,
                       pad_h=pad, pad_w=pad, in_=dx.ptr, in_pix_stride=cp, weight=dw.ptr, bias=gp._ptr(db),
                       residual=gp._ptr(dr), res_pix_stride=Cout, out=do.ptr, out_pix_stride=Cout, act=act,
-                      tile_m=tile, tile_n=tile, variant=variant)
+                      tile_m=tile, tile_n=tile if tile_n is None else tile_n, variant=variant)
     info = gp.launch("gp_launch_conv2d", p, ctx)
     sync(gp)
     out = do.download(dtype, (N, Ho, Wo, Cout)).copy()

@@ -19,7 +19,7 @@ def rel_err(got, ref):
     return float(np.abs(got - ref).max() / max(np.abs(ref).max(), 1e-30))
 
 
-def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None, tile=0, batch=1, alpha=1.0, variant=0):
+def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None, tile=0, batch=1, alpha=1.0, variant=0, tile_n=None):
     rng = np.random.default_rng(seed)
     dtype = gp.DTYPE_BY_NAME[dt]
     A = O.round_to(rng.uniform(-1, 1, (batch, M, K)).astype(np.float32), dt)
@@ -35,7 +35,7 @@ def run_gemm(gp, dt, M, N, K, b_is_nk, act, use_bias, use_res, seed, ctx_fn=None
     p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, stride_a=M * K, B=dB.ptr,
                       ldb=K if b_is_nk else N, stride_b=N * K, b_is_nk=int(b_is_nk), C=dC.ptr, ldc=N,
                       stride_c=M * N, bias=gp._ptr(dbias), residual=gp._ptr(dres), alpha=alpha, act=act,
-                      batch=batch, tile_m=tile, tile_n=tile, variant=variant)
+                      batch=batch, tile_m=tile, tile_n=tile if tile_n is None else tile_n, variant=variant)
     info = ctx_fn(p, dC) if ctx_fn else gp.launch("gp_launch_gemm", p)
     gp.check(gp.lib().gp_stream_sync(None))
     got = dC.download(dtype, (batch, M, N)).copy()
@@ -60,6 +60,15 @@ def test_gemm_matches_oracle(gp, dt, b_is_nk, shape):
             assert info.total_tiles == -(-M // tile) * -(-N // tile)
         assert np.isfinite(got).all(), (dt, shape, tile, variant)
         assert rel_err(got, ref) < TOL[dt], (dt, shape, tile, variant)
+    if b_is_nk:  # wide split-K bodies: 16 or 8 wavefronts per tile
+        for tm, tn, variant in ((32, 32, gp.MAT_WIDE), (32, 32, gp.MAT_WIDE8), (64, 32, gp.MAT_WIDE), (64, 64, gp.MAT_WIDE8)):
+            got, ref, info = run_gemm(gp, dt, M, N, K, True, gp.ACT_RELU, True, True, seed=M + N + K, tile=tm, tile_n=tn, variant=variant)
+            assert info.total_tiles == -(-M // tm) * -(-N // tn) and info.block == (1024 if variant == gp.MAT_WIDE else 512)
+            assert np.isfinite(got).all(), (dt, shape, tm, tn, variant)
+            assert rel_err(got, ref) < TOL[dt], (dt, shape, tm, tn, variant)
+    else:
+        with pytest.raises(gp.GpError):
+            run_gemm(gp, dt, M, N, K, False, gp.ACT_RELU, True, True, seed=1, tile=32, variant=gp.MAT_WIDE)
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16"])
@@ -303,6 +312,54 @@ def test_pipelined_gemm_preempt_resume_bit_exact(gp, dt, tile, variant):
         gp.launch("gp_launch_gemm", p, st.ctx())
         gp.check(gp.lib().gp_stream_sync(None))
         assert np.array_equal(dC.download(), base)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("tm,tn,variant", [(32, 32, 4), (32, 32, 5), (64, 32, 4), (64, 64, 5)])
+def test_wide_gemm_preempt_resume_bit_exact(gp, dt, tm, tn, variant):
+    """The wide split-K bodies under config 1's protocol: stopped at a tile boundary and resumed, the
+    output has the bits of the uninterrupted run; batched with GELU and alpha as well."""
+    M, N, K = 512, 384, 1600 if dt != "f32" else 800  # K is not a multiple of a 16-wavefront stage
+    rng = np.random.default_rng(17)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), dt)
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32), dt)
+    bias = O.round_to(rng.uniform(-0.1, 0.1, N).astype(np.float32), dt)
+    dA, dB, db = (gp.DevBuf.from_array(x, dtype) for x in (A, B, bias))
+    dC = gp.DevBuf(M * N * gp.DTYPE_SIZE[dtype])
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, bias=db.ptr,
+                      alpha=1.0, act=gp.ACT_RELU, batch=1, tile_m=tm, tile_n=tn, variant=variant)
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    base = dC.download().copy()
+    assert rel_err(dC.download(dtype, (M, N)), O.gemm_bias_act(A, B, bias, act=O.ACT_RELU, b_is_nk=True)) < TOL[dt]
+    # the same summation as the four-wavefront split-K bodies (which the whole-model program uses): same bits
+    p.tile_m = p.tile_n = 32
+    p.variant = gp.MAT_PIPE_SPLITK
+    dC.fill32(0)
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert np.array_equal(dC.download(), base)
+    p.tile_m, p.tile_n, p.variant = tm, tn, variant
+    flag = gp.Flag()
+    total = (M // tm) * (N // tn)
+    for groups, wgs in ((1, 4), (32, 0)):  # one counter and few workgroups; the executor's 32 counters and fixed claims
+        st = gp.BlpState(1, flag, groups)
+        for frac in (0.25, 0.75):
+            st.reset(); st.clear_stop(); flag.set(0)
+            dC.fill32(0)
+            info = gp.launch("gp_launch_gemm", p, st.ctx(inject_at=int(frac * total), max_workgroups=wgs, fresh=1))
+            gp.check(gp.lib().gp_stream_sync(None))
+            assert flag.get() == 1
+            if wgs:
+                assert st.stop_index() == 0 and st.counters()[0] < total
+            flag.set(0)
+            st.clear_stop()
+            gp.launch("gp_launch_gemm", p, st.ctx())
+            gp.check(gp.lib().gp_stream_sync(None))
+            assert np.array_equal(dC.download(), base), (groups, frac)
+    got, ref, info = run_gemm(gp, dt, 128, 64, 192, True, gp.ACT_GELU, True, False, seed=3, batch=6, alpha=0.125, tile=tm, tile_n=tn, variant=variant)
+    assert info.shape[2] == 6 and rel_err(got, ref) < TOL[dt]
 
 
 # ---- long tiles left between two K-steps ---------------------------------------------------------

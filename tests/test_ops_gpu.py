@@ -41,6 +41,15 @@ def test_conv2d_matches_oracle(gp, dt, case):
         got, info, _ = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=tile, variant=variant)
         assert np.isfinite(got).all(), (dt, case, tile, variant)
         assert rel_err(got, ref) < TOL[dt], (dt, case, tile, variant)
+    if k == 1 and stride == 1 and pad == 0:
+        # a pointwise convolution runs on the GEMM bodies, the wide split-K ones (16 or 8 wavefronts per tile) included
+        for tm, tn, variant in ((32, 32, gp.MAT_WIDE), (32, 32, gp.MAT_WIDE8), (64, 32, gp.MAT_WIDE), (64, 64, gp.MAT_WIDE8)):
+            got, info, _ = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=tm, tile_n=tn, variant=variant)
+            assert info.total_tiles == -(-N * Ho * Wo // tm) * -(-Cout // tn) and info.block == (1024 if variant == gp.MAT_WIDE else 512)
+            assert rel_err(got, ref) < TOL[dt], (dt, case, tm, tn, variant)
+    else:
+        with pytest.raises(gp.GpError):  # the wide bodies have no gathered-operand form
+            gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=32, variant=gp.MAT_WIDE)
 
 
 def test_conv2d_channel_slices(gp):
