@@ -189,10 +189,11 @@ def config1_gemm1024(iters=20):
             "note": "a 1024^3 launch is 14 us of MFMA work at the fp32 peak; both forms are launch- and latency-bound"}
 
 
-def gemm_roofline(iters=10):
+def gemm_roofline(iters=10, operands="random"):
     """BASELINE config 5's best-effort tenant alone: bf16 8192^3 GEMM (fp32 accumulate): launched
     plainly, preemptibly (tiles are finished), and preemptibly with the checkpoint workspace that
-    lets a 256 x 256 tile be left between two K-steps."""
+    lets a 256 x 256 tile be left between two K-steps.  operands = "const" fills both matrices with
+    1.0 instead (fewer bits toggle in the matrix cores: the same instruction stream at lower power)."""
     from gpreempt_amd import capi as gp
     import numpy as np
     n = 8192
@@ -200,6 +201,9 @@ def gemm_roofline(iters=10):
     rng = np.random.default_rng(5)
     dA, dB, dC = gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2), gp.DevBuf(n * n * 2)
     for d in (dA, dB):
+        if operands == "const":
+            d.fill32(0x3F803F80)
+            continue
         f = rng.random(n * n, dtype=np.float32) * 2.0 - 1.0
         d.upload((f.view(np.uint32) >> 16).astype(np.uint16))  # bf16 by truncation: the values only need to be random
     p = gp.GemmParams(dtype=gp.BF16, M=n, N=n, K=n, A=dA.ptr, lda=n, B=dB.ptr, ldb=n, b_is_nk=1, C=dC.ptr, ldc=n, alpha=1.0, batch=1)
@@ -213,7 +217,7 @@ def gemm_roofline(iters=10):
     t_ck, _ = _time_gemm(gp, p, stream, st_ck, iters)
     flop = 2.0 * n ** 3
     ach = flop / t / 1e12
-    return {"bound": "mfma", "achieved": ach, "peak": PEAK["bf16"], "unit": "TFLOP/s", "frac": ach / PEAK["bf16"], "ms": t * 1e3,
+    return {"bound": "mfma", "operands": operands, "achieved": ach, "peak": PEAK["bf16"], "unit": "TFLOP/s", "frac": ach / PEAK["bf16"], "ms": t * 1e3,
             "tiles": info.total_tiles, "grid": info.grid,
             "plain_launch": {"ms": t_plain * 1e3, "achieved": flop / t_plain / 1e12, "frac": flop / t_plain / 1e12 / PEAK["bf16"]},
             "with_checkpoint_workspace": {"ms": t_ck * 1e3, "achieved": flop / t_ck / 1e12, "frac": flop / t_ck / 1e12 / PEAK["bf16"]}}
@@ -393,6 +397,7 @@ def main():
     ap.add_argument("--be-model", default="resnet152")
     ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal")
     ap.add_argument("--cpu-requests", type=int, default=4)
+    ap.add_argument("--gemm-operands", default="random", choices=("random", "const"), help="operands of the 8192^3 GEMM leg (--only gemm)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the executor is a single-device path); run with --gpus 1")
@@ -408,6 +413,13 @@ def main():
         rep = summarize(scenario(args.steps, args.warmup, args.policy, args.hp_rate, args.be_model, args.hp_model))
         out.update({"value": rep["hp_p99_vs_isolated"], "steps": rep["hp_requests"], "ms_per_step": rep["hp_corun_ms"]["mean"]})
         out.update({k: v for k, v in rep.items() if k not in ("hp_p99_vs_isolated", "hp_requests")})
+        # `value` is a p99 over `steps` requests; with few steps that is the maximum of a handful of
+        # samples.  The same scenario over 600 requests rides along whatever --steps says.
+        if rep["hp_requests"] >= 600:
+            out["headline_600"] = {"value": rep["hp_p99_vs_isolated"], **{k: rep[k] for k in ("hp_requests", "hp_isolated_ms", "hp_corun_ms", "preemption_latency_us", "be_throughput_kept", "be_throughput_req_s", "be_isolated_req_s")}}
+        elif not args.only:
+            r6 = summarize(scenario(600, args.warmup, args.policy, args.hp_rate, args.be_model, args.hp_model))
+            out["headline_600"] = {"value": r6["hp_p99_vs_isolated"], **{k: r6[k] for k in ("hp_requests", "hp_isolated_ms", "hp_corun_ms", "preemption_latency_us", "be_throughput_kept", "be_throughput_req_s", "be_isolated_req_s")}}
         if not args.only:
             # the other policies and the single-tenant probe ride along as context
             out["other_policies"] = {}
@@ -424,7 +436,7 @@ def main():
     if args.only in ("", "roofline"):
         out["roofline"] = roofline(args.be_model, 10, "f16")
     if args.only in ("", "gemm"):
-        out["config5_gemm8192_bf16"] = gemm_roofline()
+        out["config5_gemm8192_bf16"] = gemm_roofline(operands=args.gemm_operands)
         out["config1_gemm1024_f32"] = config1_gemm1024()
     if args.only in ("", "hbm"):
         out["hbm_bound_ops"] = hbm_ops()

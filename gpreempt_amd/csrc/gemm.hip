@@ -12,6 +12,7 @@
 //
 // The convolution is the same main loop with a gathered A operand: row m is output pixel
 // (n, ho, wo) and column k is (r, s, ci) of an NHWC input, zero-filled outside the image.
+#include <cstdlib>
 #include <mutex>
 #include "gemm_tile.hpp"
 #include "gemm_pipe.hpp"
@@ -41,14 +42,14 @@ template <typename T, int BM, int BN, int BK, int WGM, int WGN, bool CONV, bool 
 using TK = TileKernel<T, BM, BN, BK, WGM, WGN, CONV, B_KN>;
 
 template <class K> struct K_is_ckpt { static constexpr bool value = false; };
-template <typename T, int BM, int BN, int ST, bool CV> struct K_is_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true>> { static constexpr bool value = true; };
+template <typename T, int BM, int BN, int ST, bool CV, int W> struct K_is_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true, W>> { static constexpr bool value = true; };
 template <class K> struct KernelOf {
     static constexpr auto fn = mat_kernel<K, LOOP_ANY>;
     static constexpr auto plain = mat_kernel<K, LOOP_PLAIN>;
     static constexpr auto fixed = mat_kernel<K, LOOP_FIXED>;
 };
-template <typename T, int BM, int BN, int ST, bool CV> struct KernelOf<PipeKernel<T, BM, BN, ST, CV, false, true>> {
-    static constexpr auto fn = mat_kernel_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true>>;
+template <typename T, int BM, int BN, int ST, bool CV, int W> struct KernelOf<PipeKernel<T, BM, BN, ST, CV, false, true, W>> {
+    static constexpr auto fn = mat_kernel_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true, W>>;
     static constexpr auto plain = fn;
     static constexpr auto fixed = fn;
 };
@@ -96,6 +97,9 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
 #ifndef GP_S128
 #define GP_S128 3
 #endif
+#ifndef GP_W256
+#define GP_W256 8  // wavefronts of the 256 x 256 body
+#endif
 #ifndef GP_S64
 #define GP_S64 4
 #endif
@@ -121,8 +125,8 @@ static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream 
     constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
     switch (pl.body) {
         case MB_PIPE256:  // GEMM only: the gathered A operand of a convolution does not fit its register budget
-            if (ctx && ctx->ckpt) return launch_mat<PipeKernel<T, 256, 256, 2, false, false, true>>(pl, ctx, s, info);
-            return launch_mat<PipeKernel<T, 256, 256, 2, false, false, false>>(pl, ctx, s, info);
+            if (ctx && ctx->ckpt) return launch_mat<PipeKernel<T, 256, 256, 2, false, false, true, GP_W256>>(pl, ctx, s, info);
+            return launch_mat<PipeKernel<T, 256, 256, 2, false, false, false, GP_W256>>(pl, ctx, s, info);
         case MB_PIPE128: return pipe_case_ckpt<T, 128, GP_S128>(pl, ctx, s, info);
         case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
         case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
@@ -248,6 +252,12 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
     const double a_elems = pl->conv ? (double)(g.M / (g.Ho * g.Wo > 0 ? g.Ho * g.Wo : 1)) * g.H * g.W * g.Cin : (double)g.M * g.K;
     const double b_elems = (double)g.N * g.K;
     pl->order = b_elems > a_elems ? 1 : 0;
+    // Large GEMMs on the 256 x 256 tiles: an XCD runs 32 of them side by side, and a single tile row
+    // with 32 column panels means 33 distinct operand panels streaming through its 4 MB L2; taken
+    // as bands of two tile rows it is 18.  Measured at 8192^3 bf16, plain launches: constant
+    // operands 889 -> 718 us, U[-1,1) operands 956 -> 928 us (those are bounded by power, see the
+    // profile of this kernel); bands of 4, 8 and 16 rows were level or worse.
+    if (!pl->conv && body == MB_PIPE256 && pl->sx >= 16 && pl->sy >= 16) pl->order = 2;
     return GP_SUCC;
 }
 
@@ -360,7 +370,7 @@ extern "C" int gp_debug_tile_prof(unsigned long long *out, int n) {
 // bodies): headers plus one accumulator slot per resident workgroup.
 namespace gp {
 static size_t plan_ckpt_bytes(const MatPlan &pl) {
-    if (pl.body == MB_PIPE256) return ckpt_workspace_bytes(PipeKernel<float, 256, 256, 2, false, false, true>::CKPT_SLOT_BYTES, (int)device_cus());
+    if (pl.body == MB_PIPE256) return ckpt_workspace_bytes(PipeKernel<float, 256, 256, 2, false, false, true, GP_W256>::CKPT_SLOT_BYTES, (int)device_cus());
     if (pl.body == MB_PIPE128) return ckpt_workspace_bytes(PipeKernel<float, 128, 128, GP_S128, false, false, true>::CKPT_SLOT_BYTES, 2 * (int)device_cus());
     return 0;
 }

@@ -87,12 +87,17 @@ struct CkptCtx {       // what a checkpointing body needs from the dispatcher, p
     int kernel_id;
 };
 
-template <typename T, int BM, int BN, int STAGES, bool CONV, bool SPLITK, bool CKPT = false>
+// NWAVES: wavefronts per workgroup.  A wavefront's operand loads complete at about 11.7 GB/s however
+// many it keeps in flight, so four wavefronts fetch 47 GB/s per compute unit: a 256 x 256 tile
+// needs 64 KB per K-step, which then takes longer (1.4 us) than the step's MFMAs (0.85 us at
+// 2.4 GHz).  With eight wavefronts (two per SIMD, 128 accumulator registers each) the stream keeps
+// up and the second wavefront of a SIMD covers the first one's barrier and LDS waits.
+template <typename T, int BM, int BN, int STAGES, bool CONV, bool SPLITK, bool CKPT = false, int NWAVES = 4>
 struct PipeKernel {
     using elem = T;
     static constexpr int bm = BM, bn = BN;
     static constexpr int VEC = Elem<T>::VEC;
-    static constexpr int NT = 256, WAVES = 4;
+    static constexpr int WAVES = NWAVES, NT = WAVES * 64;
     static constexpr int RB = 128;                        // row bytes in LDS
     static constexpr int BK = RB / (int)sizeof(T);        // 64 (16-bit) or 32 (fp32) elements
     static constexpr int KSTEPS = 4;                      // mma() calls per stage along K (2 chunks each)
@@ -100,7 +105,7 @@ struct PipeKernel {
     static constexpr int A_PW = BM / 8 / WAVES, B_PW = BN / 8 / WAVES;  // load instructions per wave per stage
     static constexpr int LPS = A_PW + B_PW;
     static constexpr int NLOADS = LPS + (CKPT ? 1 : 0);   // + the stop-word load of a checkpointing body
-    static constexpr int WGM = SPLITK ? 1 : 2, WGN = SPLITK ? 1 : 2;
+    static constexpr int WGM = SPLITK ? 1 : 2, WGN = SPLITK ? 1 : WAVES / 2;  // 2 x 2 or 2 x 4 wavefronts over the tile
     static constexpr int WM = BM / WGM, WN = BN / WGN, MI = WM / 32, NI = WN / 32;
     static constexpr size_t RED_BYTES = (size_t)WAVES * (SPLITK ? MI : 1) * NI * 16 * 64 * 4;  // epilogue staging
     static constexpr size_t RING_BYTES = (size_t)STAGES * STAGE_BYTES > RED_BYTES ? (size_t)STAGES * STAGE_BYTES : RED_BYTES;
@@ -112,6 +117,7 @@ struct PipeKernel {
     // loads) but looked at every POLL_EVERY-th K-step: about every 2.5 us for either tile size.
     static constexpr int POLL_EVERY = BM >= 256 ? 2 : 4;
     static_assert(!CKPT || !SPLITK, "checkpointing is built for the bodies without split K");
+    static_assert(WAVES == 4 || (WAVES == 8 && !SPLITK), "4 wavefronts, or 8 without split K");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && A_PW >= 1 && B_PW >= 1, "tile shape");
     static_assert(STAGES >= 2 && (STAGES - 2) * NLOADS < 64, "pipeline depth");
 

@@ -17,7 +17,7 @@ struct MatPlan {
     MatArgs g;
     int dtype, body, conv, b_kn, batch;
     int sx, sy;        // tile grid (x over N, y over M, z = batch)
-    int order;         // tile order handed to the dispatcher: 0 = x fastest, 1 = y fastest
+    int order;         // tile order handed to the dispatcher: 0 = x fastest, 1 = y fastest, G >= 2 = bands of G tile rows
     size_t lds_bytes;
 };
 

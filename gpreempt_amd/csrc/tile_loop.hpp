@@ -49,7 +49,7 @@ struct BlpArgs {
     int inject_at;    // -1 = off
     int poll_mask;    // the claim numbered c reads the host flag when (c & poll_mask) == 0
     int groups;       // claim counters per kernel (>= 1); counter g sits at executed + g * COUNTER_STRIDE
-    int order;        // tile order: 0 = x fastest (the reference's), 1 = y fastest
+    int order;        // tile order: 0 = x fastest (the reference's), 1 = y fastest, G >= 2 = bands of G tile rows (decode_tile)
     void *ckpt;       // checkpoint workspace of kernels that can leave a tile half-way, or nullptr
     int batch;        // tiles per claim (>= 1): a claim of index u stands for tiles [u*batch, (u+1)*batch)
     int tiles;        // number of tiles (total = ceil(tiles / batch) claims)
@@ -69,8 +69,21 @@ struct TileIdx { int x, y, z; };
 __device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy, int order = 0) {
     // x = idx % sx; y = (idx / sx) % sy; z = idx / (sx*sy)   (convert_to_blp.py:52-54);
     // order 1 swaps the roles of x and y, so that consecutive indices share a tile column
+    // order G >= 2: bands of G tile rows, y fastest inside a band, so that consecutive indices
+    // form G-row blocks: the workgroups an XCD runs side by side then share G row panels and a few
+    // column panels instead of one row panel and every column panel (large GEMMs, whose panels
+    // do not fit the XCD's L2)
     TileIdx t;
-    if (order == 0) {
+    if (order >= 2) {
+        const int per = sx * sy;
+        t.z = idx / per;
+        const int i = idx - t.z * per;
+        const int band = i / (order * sx), first_y = band * order;
+        const int rows = sy - first_y < order ? sy - first_y : order;
+        const int local = i - band * order * sx;
+        t.x = local / rows;
+        t.y = first_y + (local - t.x * rows);
+    } else if (order == 0) {
         int q = idx / sx;
         t.x = idx - q * sx;
         t.z = q / sy;
