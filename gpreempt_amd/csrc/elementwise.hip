@@ -76,12 +76,14 @@ int plan_pool2d(const gp_pool_params *p, EltPlan *out) {
         Wo = (p->W + 2 * p->pad - p->S) / p->stride + 1;
         GP_REQUIRE(Ho > 0 && Wo > 0, "pool: empty output");
     }
-    long items = (long)p->N * Ho * Wo * (p->C / vec);
+    // a 3 x 3 maximum window moving by 2: four neighbouring outputs per item (pool_tile_block2)
+    const int block2 = p->mode == 0 && p->R == 3 && p->S == 3 && p->stride == 2 && p->pad <= 1 && Ho >= 2 && Wo >= 2;
+    long items = block2 ? (long)p->N * ((Ho + 1) / 2) * ((Wo + 1) / 2) * (p->C / vec) : (long)p->N * Ho * Wo * (p->C / vec);
     GP_REQUIRE(items < (1L << 31), "pool: too large (2^31 16-byte items at most)");
     *out = EltPlan{};
     out->op = OP_POOL; out->dtype = p->dtype;
     out->sx = (int)((items + NT - 1) / NT); out->sy = 1;
-    out->u.pool = PoolArgs{*p, Ho, Wo, items};
+    out->u.pool = PoolArgs{*p, Ho, Wo, items, block2};
     return GP_SUCC;
 }
 

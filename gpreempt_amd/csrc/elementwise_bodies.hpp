@@ -120,9 +120,82 @@ __global__ __launch_bounds__(NT) void nchw_to_nhwc_kernel(LayoutArgs a, BlpArgs 
 
 // ---- pooling, NHWC -------------------------------------------------------------------------
 // item = (output pixel, 16-byte channel chunk); tile = 256 items.
-struct PoolArgs { gp_pool_params p; int Ho, Wo; long items; };
+// block2: a 3 x 3 / stride 2 max pool, an item is a 2 x 2 block of output pixels (one 16-byte channel
+// chunk): its four windows overlap in a 5 x 5 input patch, 25 loads instead of 36.  The kernel is
+// bound by the number of load requests (every input element is wanted by up to four windows), so
+// fewer requests per output is what makes it faster: 2.7 -> 3.5 TB/s from issuing all taps without
+// branches between them, and on to the figure in the profile with the shared patch.
+struct PoolArgs { gp_pool_params p; int Ho, Wo; long items; int block2; };
+
+// element-wise maximum of two 16-byte chunks, in the storage type (a maximum needs no wider arithmetic)
+template <typename T> __device__ __forceinline__ u32x4 chunk_max(u32x4 a, u32x4 b);
+template <> __device__ __forceinline__ u32x4 chunk_max<float>(u32x4 a, u32x4 b) {
+    return __builtin_bit_cast(u32x4, __builtin_elementwise_max(__builtin_bit_cast(f32x4, a), __builtin_bit_cast(f32x4, b)));
+}
+template <> __device__ __forceinline__ u32x4 chunk_max<_Float16>(u32x4 a, u32x4 b) {
+    return __builtin_bit_cast(u32x4, __builtin_elementwise_max(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b)));
+}
+template <> __device__ __forceinline__ u32x4 chunk_max<__bf16>(u32x4 a, u32x4 b) {
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // a bf16 is the upper half of a float
+        const float al = __builtin_bit_cast(float, a[i] << 16), bl = __builtin_bit_cast(float, b[i] << 16);
+        const float ah = __builtin_bit_cast(float, a[i] & 0xFFFF0000u), bh = __builtin_bit_cast(float, b[i] & 0xFFFF0000u);
+        o[i] = (__builtin_bit_cast(unsigned, fmaxf(al, bl)) >> 16) | (__builtin_bit_cast(unsigned, fmaxf(ah, bh)) & 0xFFFF0000u);
+    }
+    return o;
+}
+
+// (max pooling only.  A tap outside the image is fetched from the clamped coordinate instead: that
+// element lies inside the same window, so the maximum is unchanged and nothing has to be masked.)
+template <typename T>
+__device__ __forceinline__ void pool_tile_block2(const PoolArgs &a, TileIdx t) {
+    const gp_pool_params &p = a.p;
+    constexpr int VEC = VecIO<T>::VEC;
+    const int chunks = p.C / VEC;
+    const int Hb = (a.Ho + 1) / 2, Wb = (a.Wo + 1) / 2;
+    const unsigned item = (unsigned)t.x * NT + threadIdx.x;
+    if (item >= (unsigned)a.items) return;
+    const unsigned ublk = item / (unsigned)chunks;
+    const int ch = (int)(item - ublk * (unsigned)chunks);
+    const unsigned q = ublk / (unsigned)Wb;
+    const int wb = (int)(ublk - q * (unsigned)Wb);
+    const long n = q / (unsigned)Hb;
+    const int hb = (int)(q - (unsigned)n * (unsigned)Hb);
+    const T *in = (const T *)p.in;
+    T *out = (T *)p.out;
+    const int h_first = hb * 4 - p.pad, w_first = wb * 4 - p.pad;  // input coordinate of the patch's corner
+    u32x4 f[25];
+#pragma unroll
+    for (int r = 0; r < 5; ++r) {
+#pragma unroll
+        for (int s = 0; s < 5; ++s) {
+            const int hi = h_first + r, wi = w_first + s;
+            const int hc = hi < 0 ? 0 : (hi >= p.H ? p.H - 1 : hi), wc = wi < 0 ? 0 : (wi >= p.W ? p.W - 1 : wi);
+            f[r * 5 + s] = *(const u32x4 *)(in + ((n * p.H + hc) * p.W + wc) * p.in_pix_stride + ch * VEC);
+        }
+    }
+    // column maxima of the three row triples a window can take, then the windows
+#pragma unroll
+    for (int dy = 0; dy < 2; ++dy) {
+        const int ho = hb * 2 + dy;
+        if (ho >= a.Ho) continue;
+        u32x4 col[5];
+#pragma unroll
+        for (int s = 0; s < 5; ++s) col[s] = chunk_max<T>(chunk_max<T>(f[(dy * 2) * 5 + s], f[(dy * 2 + 1) * 5 + s]), f[(dy * 2 + 2) * 5 + s]);
+#pragma unroll
+        for (int dx = 0; dx < 2; ++dx) {
+            const int wo = wb * 2 + dx;
+            if (wo >= a.Wo) continue;
+            const u32x4 m = chunk_max<T>(chunk_max<T>(col[dx * 2], col[dx * 2 + 1]), col[dx * 2 + 2]);
+            st_out128(out + ((n * a.Ho + ho) * a.Wo + wo) * p.out_pix_stride + ch * VEC, __builtin_bit_cast(out_u32x4, m));
+        }
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ void pool_tile(const PoolArgs &a, TileIdx t) {
+    if (a.block2) { pool_tile_block2<T>(a, t); return; }
     const gp_pool_params &p = a.p;
     const int Ho = a.Ho, Wo = a.Wo;
     const long items = a.items;
@@ -168,21 +241,26 @@ __device__ __forceinline__ void pool_tile(const PoolArgs &a, TileIdx t) {
             constexpr int R = decltype(RC)::value, S = decltype(SC)::value;
             float f[R * S][VEC];
             bool in_range[R * S];
+            // every tap is loaded, from a clamped coordinate when it lies outside the image, and
+            // dropped afterwards: no branch sits between the loads, so all R*S are in flight at once
 #pragma unroll
             for (int r = 0; r < R; ++r) {
 #pragma unroll
                 for (int s = 0; s < S; ++s) {
                     const int hi = ho * p.stride - p.pad + r, wi = wo * p.stride - p.pad + s;
                     in_range[r * S + s] = (unsigned)hi < (unsigned)p.H && (unsigned)wi < (unsigned)p.W;
-                    if (in_range[r * S + s]) VecIO<T>::load(in + ((n * p.H + hi) * p.W + wi) * p.in_pix_stride + ch * VEC, f[r * S + s]);
+                    const int hc = hi < 0 ? 0 : (hi >= p.H ? p.H - 1 : hi), wc = wi < 0 ? 0 : (wi >= p.W ? p.W - 1 : wi);
+                    VecIO<T>::load(in + ((n * p.H + hc) * p.W + wc) * p.in_pix_stride + ch * VEC, f[r * S + s]);
                 }
             }
 #pragma unroll
             for (int i = 0; i < R * S; ++i) {
-                if (!in_range[i]) continue;
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) acc[j] = p.mode == 0 ? fmaxf(acc[j], f[i][j]) : acc[j] + f[i][j];
-                ++cnt;
+                for (int j = 0; j < VEC; ++j) {
+                    const float v = in_range[i] ? f[i][j] : (p.mode == 0 ? -INFINITY : 0.f);
+                    acc[j] = p.mode == 0 ? fmaxf(acc[j], v) : acc[j] + v;
+                }
+                cnt += in_range[i];
             }
         };
         if (p.R == 3 && p.S == 3) window(IntC<3>{}, IntC<3>{});

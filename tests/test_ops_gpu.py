@@ -88,13 +88,17 @@ def test_nchw_to_nhwc(gp, dt_in, dt_out):
 
 
 @pytest.mark.parametrize("dt", DTS)
-@pytest.mark.parametrize("cfg", [(3, 2, 1, "max"), (2, 2, 0, "max"), (2, 2, 0, "avg"), (3, 1, 1, "avg"), (3, 1, 1, "avg_pad"), (7, 1, 0, "gap")])
+@pytest.mark.parametrize("cfg", [(3, 2, 1, "max"), (2, 2, 0, "max"), (2, 2, 0, "avg"), (3, 1, 1, "avg"), (3, 1, 1, "avg_pad"), (7, 1, 0, "gap"),
+                                 # 3 x 3 windows moving by 2 take the path with four outputs per item: odd and even output sizes, every mode
+                                 (3, 2, 0, "max", 15, 13), (3, 2, 1, "avg", 15, 13), (3, 2, 1, "avg_pad", 16, 9), (3, 2, 1, "max", 9, 16), (3, 2, 0, "avg", 5, 5)])
 def test_pool2d(gp, dt, cfg):
-    k, stride, pad, mode = cfg
+    k, stride, pad, mode = cfg[:4]
     rng = np.random.default_rng(k * 10 + stride)
     N, Cc, H, W = 2, 24, 14, 14 if mode != "gap" else 7
     if mode == "gap":
         H = 7
+    if len(cfg) > 4:
+        H, W = cfg[4:]
     x = rnd(rng, (N, Cc, H, W), dt)
     dtype = gp.DTYPE_BY_NAME[dt]
     di = gp.DevBuf.from_array(nchw_to_nhwc(x), dtype)
