@@ -26,7 +26,10 @@ template <class TK, int LOOP>
 __global__ __launch_bounds__(TK::NT) void mat_kernel(MatArgs g, BlpArgs blp) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     auto *lds = reinterpret_cast<typename TK::elem *>(lds_raw);
-    tiles<LOOP>(blp, [&](TileIdx t) { TK::run(g, t, lds); });
+    if constexpr (LOOP == LOOP_FIXED && TK::early_stop)
+        tile_fixed_early(blp, [&](TileIdx t, int *stop) { return TK::run(g, t, lds, CkptCtx{stop, nullptr, nullptr, 0}); });
+    else
+        tiles<LOOP>(blp, [&](TileIdx t) { TK::run(g, t, lds); });
 }
 
 // bodies that can leave a tile between two K-steps (tile_loop_ckpt)

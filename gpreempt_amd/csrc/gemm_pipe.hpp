@@ -113,6 +113,7 @@ struct PipeKernel {
     static constexpr size_t LDS_BYTES = RING_BYTES + POLL_BYTES;
     static constexpr size_t CKPT_SLOT_BYTES = (size_t)WAVES * MI * NI * 16 * 64 * 4;  // one workgroup's accumulators
     static constexpr bool ckpt = CKPT;
+    static constexpr bool early_stop = !CKPT;  // run() takes an early-stop word (see there)
     // The stop words are fetched with every stage (so that every wave issues the same number of
     // loads) but looked at every POLL_EVERY-th K-step: about every 2.5 us for either tile size.
     static constexpr int POLL_EVERY = BM >= 256 ? 2 : 4;
@@ -122,9 +123,19 @@ struct PipeKernel {
     static_assert(STAGES >= 2 && (STAGES - 2) * NLOADS < 64, "pipeline depth");
 
     // Returns true when the tile was left half-way (CKPT only); kt0 > 0 continues such a tile.
+    //
+    // Bodies without checkpoints take cc.stop_index as an "early stop" word (nullptr: none): it is
+    // fetched once, with the first stage's operands, and looked at when that stage has landed,
+    // about 2 us into the tile.  If a stop has been recorded by then the tile is not run and the
+    // function returns true: the caller withdraws the claim.  This is for launches whose workgroups
+    // all claim at once while a few spare workgroups read the host flag (tile_loop.hpp): the flag
+    // read takes 1-2 us, so without the second look a kernel launched just after the flag went up
+    // would still run to its end.
     static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0},
                                                int tile_index = 0, int kt0 = 0) {
         GP_PROBE(0);
+        __shared__ int early_slot[64];  // landing place of the early-stop word (lane 0's dword)
+        const bool early = !CKPT && cc.stop_index != nullptr;
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
         const int tid = threadIdx.x, lane = tid & 63;
@@ -414,6 +425,9 @@ struct PipeKernel {
                 __builtin_amdgcn_sched_barrier(0);
             }
             int stop_now = 0;
+            if constexpr (!CKPT) {
+                if (early && kt == kt0) stop_now = __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1;
+            }
             if constexpr (CKPT) {
                 const int sw = __builtin_amdgcn_readfirstlane(stop_word), fw = __builtin_amdgcn_readfirstlane(flag_word);
                 if (fw != 0 && tid == 0) atomicCAS(cc.stop_index, -1, cc.kernel_id);  // pass the host flag on
@@ -443,15 +457,27 @@ struct PipeKernel {
         GP_PROBE(1);
         __syncthreads();  // the previous tile of this workgroup may still be reading LDS
 #pragma unroll
-        for (int s = 0; s < STAGES - 1; ++s)
+        for (int s = 0; s < STAGES - 1; ++s) {
             if (kt0 + s < KT) issue(kt0 + s);
+            // (older than every later stage's loads, so the wait for the first stage covers it; the
+            // other waves issue nothing extra: each wave counts its own loads)
+            if (!CKPT && s == 0 && early && wave == 0)
+                load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
+        }
         int kt = kt0, stopped = 0;
         for (; kt + STAGES - 1 < KT; ++kt) {
             stopped = ktile(kt, false, IntC<1>{});
-            if (CKPT && stopped) break;
+            if (stopped) break;  // (CKPT: leave the tile here; otherwise only the early look at the first step can say so)
         }
-        if (!(CKPT && stopped))
-            for (; kt < KT; ++kt) ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
+        if (!stopped)
+            for (; kt < KT; ++kt) {
+                const int st = ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
+                if (!CKPT && st) { stopped = 1; break; }  // (a checkpointing body finishes a tile whose last stages are in flight)
+            }
+        if (!CKPT && stopped) {
+            wait_vmcnt<0>();  // operand loads still landing in LDS must not outlive the workgroup
+            return true;
+        }
         if (!SPLITK && KT > kt0) mma_all((KSTEPS - 1) & 1);
         GP_PROBE(3);
         // When `stopped` (CKPT only), K-steps kt0..kt are in the accumulators and the "epilogue" below

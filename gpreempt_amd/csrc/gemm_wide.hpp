@@ -49,13 +49,17 @@ struct WideKernel {
     static constexpr size_t LDS_BYTES = RING_BYTES > RED_BYTES ? RING_BYTES : RED_BYTES;
     static constexpr size_t CKPT_SLOT_BYTES = 0;
     static constexpr bool ckpt = false;
+    static constexpr bool early_stop = true;  // as PipeKernel::run: a second look at the stop index when the first stage has landed
     static_assert(WAVES % 4 == 0 && WAVES >= 4 && WAVES <= 16, "4, 8, 12 or 16 wavefronts");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && GROUPS % 4 == 0, "tile shape");
     static_assert(STAGES >= 2 && (STAGES - 2) * LPW < 64, "pipeline depth");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 
-    static __device__ __forceinline__ void run(const MatArgs &g, TileIdx t, T *lds_t) {
+    // Returns true when the early look found a stop recorded: the tile was not run.
+    static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0}) {
         GP_PROBE(0);
+        __shared__ int early_slot[64];
+        const bool early = cc.stop_index != nullptr;
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
         const int tid = threadIdx.x, lane = tid & 63;
@@ -129,14 +133,20 @@ struct WideKernel {
         GP_PROBE(1);
         __syncthreads();  // the previous tile of this workgroup may still be reading LDS
 #pragma unroll
-        for (int s = 0; s < STAGES - 1; ++s)
+        for (int s = 0; s < STAGES - 1; ++s) {
             if (s < NS) issue(s);
+            if (s == 0 && early && wave == 0) load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
+        }
         for (int s = 0; s < NS; ++s) {
             // stage s has landed once at most the loads of the younger stages in flight remain
             if (s + STAGES - 2 < NS) wait_vmcnt<(STAGES - 2) * LPW>();
             else wait_vmcnt<0>();
             __syncthreads();  // everyone's part of stage s is visible; the buffer of stage s-1 is free
             if (s == 0) GP_PROBE(2);
+            if (s == 0 && early && __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1) {
+                wait_vmcnt<0>();  // loads still landing in LDS must not outlive the workgroup
+                return true;
+            }
             if (s + STAGES - 1 < NS) issue(s + STAGES - 1);
             if (kb != 0) continue;  // (uniform) wavefronts 4.. only fetch
             const int stage = s % STAGES;
@@ -235,6 +245,7 @@ struct WideKernel {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         GP_PROBE(5);
 #endif
+        return false;
     }
 };
 

@@ -251,6 +251,25 @@ __device__ __forceinline__ int fixed_claim_of_workgroup(const BlpArgs &b) {
     return __builtin_amdgcn_readfirstlane(mailbox);
 }
 
+// Fixed claims with a second look: body(TileIdx, stop word or nullptr) returns true when it found a
+// stop recorded shortly after the claim and did not run the tile; the claim is then withdrawn
+// (bit cleared, count lowered), so that the relaunch runs it.  The word is handed over only when
+// the launch has spare workgroups reading the flag: that read is what the second look waits for.
+__device__ __forceinline__ void unclaim_fixed(const BlpArgs &b) {
+    const int grp = wg_group((int)blockIdx.x, b.groups);
+    const int j = (int)blockIdx.x >> log2_pow2(b.groups);
+    int *line = b.executed + grp * COUNTER_STRIDE;
+    __hip_atomic_fetch_and(line + 1 + (j >> 5), ~(1 << (j & 31)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_fetch_add(line, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <class Body>
+__device__ __forceinline__ void tile_fixed_early(const BlpArgs &b, Body &&body) {
+    const int idx = fixed_claim_of_workgroup(b);
+    if (idx < 0) return;
+    const bool left = body(decode_tile(idx, b.sx, b.sy, b.order), b.spare ? b.stop_index : nullptr);
+    if (left && threadIdx.x == 0) unclaim_fixed(b);
+}
+
 template <class Body>
 __device__ __forceinline__ void tile_fixed(const BlpArgs &b, Body &&body) {
     const int idx = fixed_claim_of_workgroup(b);

@@ -275,6 +275,9 @@ struct Tenant {
     volatile int *gate_host = nullptr;      // hp_gate: the word the gate kernels wait for
     void *gate_dev = nullptr;
     int *gate_timed_out = nullptr;          // device word set by a gate that gave up
+    // the slowest drains of this tenant: how long, and which kernel the stop index named afterwards
+    struct Drain { double us; int stop_kernel; int queued; };
+    std::vector<Drain> drains;
     bool have_ref_hash = false;
     uint64_t ref_hash = 0;
     long output_mismatches = 0;
@@ -389,18 +392,28 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             st = drain(t.stream);
             if (st != Status::Succ) break;
             int64_t drained = now_ns();
+            const int queued = inflight;
             inflight = 0; head = tail;
             sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
-            int64_t raised = sh.domain->raised_ns(p);
-            if (raised > 0 && drained >= raised) {
-                std::lock_guard<std::mutex> g(sh.stats_mu);
-                sh.preempt_latency.add((drained - raised) / 1e3);
+            // read the stop index back (and re-arm it) while the higher level has the GPU: nothing of
+            // this tenant is in flight, and the blocking read-back (10-20 us) then costs nobody anything
+            st = ex->getStopPoint(t.stream);
+            if (st != Status::Succ) { sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel); break; }
+            const int stop = ex->last_stop_index();
+            const int64_t raised = sh.domain->raised_ns(p);
+            // a preemption-latency sample needs something to have been preempted: kernels in flight
+            // when the request was noticed, or a kernel recorded as stopped.  (A request that finds
+            // this tenant between two submissions waits for nothing.)
+            if ((queued > 0 || stop >= 0) && raised > 0 && drained >= raised) {
+                const double drain_us = (drained - raised) / 1e3;
+                {
+                    std::lock_guard<std::mutex> g(sh.stats_mu);
+                    sh.preempt_latency.add(drain_us);
+                }
+                t.drains.push_back({drain_us, stop, queued});
             }
             while (sh.active_above(p) > 0) spin_pause();
             sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
-            st = ex->getStopPoint(t.stream);  // re-arms the stop index
-            if (st != Status::Succ) break;
-            int stop = ex->last_stop_index();
             if (stop >= 0) { next = (size_t)stop; ++t.preemptions; }  // kernels from the stopped one on are submitted again
             continue;
         }
@@ -764,6 +777,25 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
             o.set("throughput_kept") = kept;
             be_kept += kept;
             ++n_be;
+        }
+        if (!t->drains.empty()) {
+            std::sort(t->drains.begin(), t->drains.end(), [](const Tenant::Drain &a, const Tenant::Drain &b) { return a.us > b.us; });
+            json::Value &sd = o.set("slowestDrains");
+            sd = json::Value::array();
+            auto model = t->ex->get_model();
+            for (size_t i = 0; i < t->drains.size() && i < 12; ++i) {
+                json::Value e = json::Value::object();
+                e.set("us") = t->drains[i].us;
+                e.set("stopKernel") = t->drains[i].stop_kernel;
+                e.set("chunksInFlight") = t->drains[i].queued;
+                if (model && t->drains[i].stop_kernel >= 0 && (size_t)t->drains[i].stop_kernel < model->get_kernel_num()) {
+                    KernelInfo &k = model->get_kernel_info(t->drains[i].stop_kernel);
+                    e.set("name") = k.name;
+                    e.set("tiles") = k.total_blocks;
+                    e.set("gflop") = k.flops / 1e9;
+                }
+                sd.push(e);
+            }
         }
         if (sh.verify_outputs) o.set("outputMismatches") = t->output_mismatches;
         if (t->error != Status::Succ) { o.set("error") = status_name(t->error); result = t->error; }
