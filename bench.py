@@ -11,7 +11,7 @@ p99 (the first figure of BASELINE.json's metric); the other two (preemption late
 throughput kept) and the absolute latencies ride along in the same line, together with
   roofline      the dominant kernel (MFMA implicit-GEMM convolution of the best-effort model),
                 timed live with HIP events on the stream it is launched on
-  cpu_baseline  the same high-priority graph on the host cores (CPU oracle), bounded sample
+  cpu_baseline  the same kernel lists on the host cores (C tile-loop executor under oracle/), bounded sample
 """
 import argparse
 import ctypes as C
@@ -361,11 +361,7 @@ def copy_calibration(mib=256, iters=10):
     return {"bytes_per_copy": n, "copies": iters}
 
 
-def cpu_baseline(requests):
-    """The high-priority graph (BERT-base, seq 128, fp16 storage) on the host cores through the
-    CPU oracle.  Bounded sample: `requests` whole requests."""
-    import numpy as np
-    from oracle import models as OM
+def bert_base_shapes():
     H, F, L = 768, 3072, 12
     shapes = {"embeddings.word": (30522, H), "embeddings.position": (512, H), "embeddings.token_type": (1, H),
               "embeddings.ln.gamma": (H,), "embeddings.ln.beta": (H,)}
@@ -374,16 +370,57 @@ def cpu_baseline(requests):
         shapes.update({n + ".attn.qkv.weight": (3 * H, H), n + ".attn.qkv.bias": (3 * H,), n + ".attn.proj.weight": (H, H),
                        n + ".attn.proj.bias": (H,), n + ".ln1.gamma": (H,), n + ".ln1.beta": (H,), n + ".ffn1.weight": (F, H),
                        n + ".ffn1.bias": (F,), n + ".ffn2.weight": (H, F), n + ".ffn2.bias": (H,), n + ".ln2.gamma": (H,), n + ".ln2.beta": (H,)})
-    params = OM.random_params(shapes, 0, "bert")
-    ids = np.random.default_rng(0).integers(0, 30522, 128)
-    OM.bert(params, ids, "f16", 1, 128, 1)  # touch the library
-    t0 = time.perf_counter()
-    for _ in range(requests):
-        OM.bert(params, ids, "f16", 1, 128, L)
-    dt = (time.perf_counter() - t0) / requests
-    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": dt * 1e3, "unit": "ms per high-priority request (isolated)", "cores": cores, "kind": "port",
-            "sample": f"{requests} BERT-base b1 s128 requests through oracle/models.py (double accumulation, fp16 storage rounding, OpenMP)"}
+    return shapes
+
+
+def resnet_shapes(blocks, width=64, classes=1000):
+    s = {"conv1.weight": (width, 3, 7, 7), "conv1.bias": (width,)}
+    cin = width
+    for st in range(4):
+        w = width << st
+        for b in range(blocks[st]):
+            n = f"layer{st + 1}.{b}"
+            if b == 0:
+                s[n + ".downsample.weight"] = (4 * w, cin, 1, 1); s[n + ".downsample.bias"] = (4 * w,)
+            s[n + ".conv1.weight"] = (w, cin, 1, 1); s[n + ".conv1.bias"] = (w,)
+            s[n + ".conv2.weight"] = (w, w, 3, 3); s[n + ".conv2.bias"] = (w,)
+            s[n + ".conv3.weight"] = (4 * w, w, 1, 1); s[n + ".conv3.bias"] = (4 * w,)
+            cin = 4 * w
+    s["fc.weight"] = (classes, cin); s["fc.bias"] = (classes,)
+    return s
+
+
+def cpu_baseline(runs):
+    """The same kernel lists on the host cores: the C tile-loop executor of oracle/oracle_exec.c
+    (persistent pinned workers that claim tiles and poll the preempt flag as the block-level-
+    preemption loop does; fp32), one worker per core.  Bounded: `runs` timed submissions of each
+    graph after warm-ups.  The headline entry is the high-priority request (BERT-base, b1, s128);
+    the 1024^3 GEMM and one ResNet-152 image are listed beside it."""
+    import numpy as np
+    from oracle import cpu_executor as X
+    from oracle import models as OM
+    threads = X.default_threads()
+    rng = np.random.default_rng(0)
+    legs = {}
+    A, B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32), rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    g, _ = X.gemm_graph(A, B, np.zeros(1024, np.float32))
+    mean, p50, p99 = X.timed(g, 3, max(runs, 30), threads)
+    legs["gemm_1024"] = {"ms_mean": mean, "ms_p50": p50, "ms_p99": p99, "gflops": g.flops / mean / 1e6, "runs": max(runs, 30)}
+    params = OM.random_params(bert_base_shapes(), 0, "bert")
+    g, _ = X.bert_graph(params, rng.integers(0, 30522, 128))
+    mean, p50, p99 = X.timed(g, 2, runs, threads)
+    legs["bert_b1_s128"] = {"ms_mean": mean, "ms_p50": p50, "ms_p99": p99, "gflops": g.flops / mean / 1e6, "runs": runs, "kernels": len(g.layers)}
+    hp_ms = mean
+    del g, params
+    blocks = OM.RESNET_BLOCKS["resnet152"]
+    params = OM.random_params(resnet_shapes(blocks), 0, "cnn")
+    g, _ = X.resnet_graph(params, rng.normal(size=(1, 3, 224, 224)).astype(np.float32), blocks)
+    mean, p50, p99 = X.timed(g, 1, runs, threads)
+    legs["resnet152_b1"] = {"ms_mean": mean, "ms_p50": p50, "ms_p99": p99, "gflops": g.flops / mean / 1e6, "runs": runs, "kernels": len(g.layers)}
+    return {"value": hp_ms, "unit": "ms per high-priority request (isolated)", "cores": threads, "kind": "port",
+            "sample": f"{runs} timed submissions each of BERT-base b1 s128 (the high-priority request), ResNet-152 b1 and (x{max(runs, 30)}) the 1024^3 GEMM "
+                      "through oracle/oracle_exec.c: C tile-loop executor, fp32, one pinned worker per core",
+            "legs": legs}
 
 
 def main():
@@ -396,7 +433,7 @@ def main():
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
     ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal")
-    ap.add_argument("--cpu-requests", type=int, default=4)
+    ap.add_argument("--cpu-requests", type=int, default=10, help="timed submissions per graph in the cpu_baseline leg")
     ap.add_argument("--gemm-operands", default="random", choices=("random", "const"), help="operands of the 8192^3 GEMM leg (--only gemm)")
     args = ap.parse_args()
     if args.gpus != 1:
