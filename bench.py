@@ -266,7 +266,7 @@ def hbm_ops(iters=20):
         x, r, g, be, o = buf(rows * cols * 2), buf(rows * cols * 2), buf(cols * 2), buf(cols * 2), buf(rows * cols * 2)
         p = gp.LayernormParams(dtype=gp.F16, rows=rows, cols=cols, x=x.ptr, residual=r.ptr, gamma=g.ptr, beta=be.ptr, out=o.ptr, eps=1e-12)
         out["residual_layernorm_f16_" + tag] = timed("gp_launch_layernorm", p, 3 * rows * cols * 2)
-    for tag, rows, cols in (("bert_s128_12heads", 12 * 128, 128), ("large", 1 << 19, 128)):
+    for tag, rows, cols in (("bert_s128_12heads", 12 * 128, 128), ("large", 1 << 21, 128)):
         x, o = buf(rows * cols * 2), buf(rows * cols * 2)
         p = gp.SoftmaxParams(dtype=gp.F16, rows=rows, cols=cols, x=x.ptr, out=o.ptr, scale=0.125)
         out["softmax_f16_" + tag] = timed("gp_launch_softmax", p, 2 * rows * cols * 2)

@@ -99,7 +99,8 @@ int plan_eltwise(const gp_eltwise_params *p, EltPlan *out) {
     GP_REQUIRE(items < (1L << 31), "eltwise: too large (2^31 16-byte items at most)");
     *out = EltPlan{};
     out->op = OP_ELTWISE; out->dtype = p->dtype; out->sx = (int)tiles; out->sy = 1;
-    out->u.elt = EltwiseArgs{*p, items};
+    const long bytes = p->rows * p->cols * (long)dtype_size(p->dtype) * (p->b ? 3 : 2);
+    out->u.elt = EltwiseArgs{*p, items, bytes > kStreamBytes};
     return GP_SUCC;
 }
 
@@ -126,12 +127,14 @@ int plan_layernorm(const gp_layernorm_params *p, EltPlan *out) {
     GP_REQUIRE(p->rows > 0 && p->cols > 0 && p->cols % vec == 0, "layernorm: cols must be a positive multiple of %d", vec);
     GP_REQUIRE(p->cols <= 64 * vec * 16, "layernorm: at most %d columns", 64 * vec * 16);
     GP_REQUIRE(al16(p->x) && al16(p->out) && al16(p->residual) && al16(p->gamma) && al16(p->beta), "layernorm: 16-byte alignment");
-    long tiles = (p->rows + 3) / 4;
-    GP_REQUIRE(tiles < (1L << 31), "layernorm: too many rows");
     int chunks_per_lane = (p->cols / vec + 63) / 64;
+    // short rows of a large problem: a wavefront takes two rows at a time, so that twice the bytes are in flight
+    const int rpw = (chunks_per_lane <= 2 && p->rows >= 16384) ? 2 : 1;
+    long tiles = (p->rows + 4 * rpw - 1) / (4 * rpw);
+    GP_REQUIRE(tiles < (1L << 31), "layernorm: too many rows");
     *out = EltPlan{};
     out->op = OP_LAYERNORM; out->dtype = p->dtype; out->sx = (int)tiles; out->sy = 1;
-    out->sub = chunks_per_lane <= 2 ? 2 : chunks_per_lane <= 8 ? 8 : 16;
+    out->sub = (chunks_per_lane <= 2 ? 2 : chunks_per_lane <= 8 ? 8 : 16) | (rpw == 2 ? kLnTwoRows : 0);
     out->u.ln = *p;
     return GP_SUCC;
 }
@@ -195,9 +198,10 @@ int launch_elt_plan(const EltPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
         case OP_ELTWISE: GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(eltwise_kernel<T), pl.sx, pl.sy, ctx, s, info, pl.u.elt)); break;
         case OP_SOFTMAX: GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(softmax_kernel<T), pl.sx, pl.sy, ctx, s, info, pl.u.softmax)); break;
         case OP_LAYERNORM:
-            if (pl.sub == 2) { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 2), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
-            else if (pl.sub == 8) { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 8), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
-            else { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 16), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
+            if (pl.sub == (2 | kLnTwoRows)) { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 2, 2), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
+            else if (pl.sub == 2) { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 2, 1), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
+            else if (pl.sub == 8) { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 8, 1), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
+            else { GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(layernorm_kernel<T, 16, 1), pl.sx, pl.sy, ctx, s, info, pl.u.ln)); }
             break;
         case OP_EMBED: GP_BY_DTYPE(pl.dtype, launch_tiles(GP_KSET(embed_kernel<T), pl.sx, pl.sy, ctx, s, info, pl.u.embed)); break;
         case OP_COPY: return launch_tiles(GP_KSET(copy_kernel<0), pl.sx, pl.sy, ctx, s, info, pl.u.copy);

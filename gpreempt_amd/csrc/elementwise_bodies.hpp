@@ -17,6 +17,15 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// A float that the compiler must materialise as such.  Conversions to fp16 go through it: otherwise
+// the compiler may fold "multiply-add, then convert" into one v_fma_mixlo_f16, which rounds once
+// where the two instructions round twice, and it decides that per instantiation: the same row
+// would get different bits from two forms of one kernel.
+__device__ __forceinline__ float pin_f32(float v) {
+    asm("" : "+v"(v));
+    return v;
+}
+
 template <typename T> struct VecIO;
 template <> struct VecIO<float> {
     static constexpr int VEC = 4;
@@ -31,6 +40,17 @@ template <> struct VecIO<float> {
         for (int i = 0; i < 4; ++i) v[i] = f[i];
         st_out128(p, __builtin_bit_cast(out_u32x4, v));
     }
+    static __device__ __forceinline__ void unpack(out_u32x4 r, float (&f)[4]) {
+        f32x4 v = __builtin_bit_cast(f32x4, r);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = v[i];
+    }
+    static __device__ __forceinline__ out_u32x4 pack(const float (&f)[4]) {
+        f32x4 v;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = f[i];
+        return __builtin_bit_cast(out_u32x4, v);
+    }
     static __device__ __forceinline__ float ld1(const float *p) { return *p; }
     static __device__ __forceinline__ void st1(float *p, float v) { st_elem<float>(p, v); }
 };
@@ -44,11 +64,22 @@ template <> struct VecIO<_Float16> {
     static __device__ __forceinline__ void store(_Float16 *p, const float (&f)[8]) {
         f16x8 v;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = (_Float16)f[i];
+        for (int i = 0; i < 8; ++i) v[i] = (_Float16)pin_f32(f[i]);
         st_out128(p, __builtin_bit_cast(out_u32x4, v));
     }
+    static __device__ __forceinline__ void unpack(out_u32x4 r, float (&f)[8]) {
+        f16x8 v = __builtin_bit_cast(f16x8, r);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+    }
+    static __device__ __forceinline__ out_u32x4 pack(const float (&f)[8]) {
+        f16x8 v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (_Float16)pin_f32(f[i]);
+        return __builtin_bit_cast(out_u32x4, v);
+    }
     static __device__ __forceinline__ float ld1(const _Float16 *p) { return (float)*p; }
-    static __device__ __forceinline__ void st1(_Float16 *p, float v) { st_elem<_Float16>(p, (_Float16)v); }
+    static __device__ __forceinline__ void st1(_Float16 *p, float v) { st_elem<_Float16>(p, (_Float16)pin_f32(v)); }
 };
 template <> struct VecIO<__bf16> {
     static constexpr int VEC = 8;
@@ -63,9 +94,33 @@ template <> struct VecIO<__bf16> {
         for (int i = 0; i < 8; ++i) v[i] = (__bf16)f[i];
         st_out128(p, __builtin_bit_cast(out_u32x4, v));
     }
+    static __device__ __forceinline__ void unpack(out_u32x4 r, float (&f)[8]) {
+        bf16x8 v = __builtin_bit_cast(bf16x8, r);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)v[i];
+    }
+    static __device__ __forceinline__ out_u32x4 pack(const float (&f)[8]) {
+        bf16x8 v;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = (__bf16)f[i];
+        return __builtin_bit_cast(out_u32x4, v);
+    }
     static __device__ __forceinline__ float ld1(const __bf16 *p) { return (float)*p; }
     static __device__ __forceinline__ void st1(__bf16 *p, float v) { st_elem<__bf16>(p, (__bf16)v); }
 };
+
+// A tensor that cannot stay in the 256 MiB last-level cache is streamed: its loads and stores carry
+// the nontemporal hint, so that lines nobody will read again do not push out ones that somebody will.
+// Measured on 384 MiB buffers: copy 5.6 -> 6.2 TB/s, add (two reads, one write) 5.5 -> 6.3 TB/s.
+constexpr long kStreamBytes = 256L << 20;
+template <bool NTH> __device__ __forceinline__ out_u32x4 ld_raw128(const void *p) {
+    if (NTH) return __builtin_nontemporal_load((const out_u32x4 *)p);
+    return *(const out_u32x4 *)p;
+}
+template <bool NTH> __device__ __forceinline__ void st_raw128(void *p, out_u32x4 v) {
+    if (NTH && !kCoherentStores) __builtin_nontemporal_store(v, (out_u32x4 *)p);
+    else st_out128(p, v);
+}
 
 __device__ __forceinline__ float act_f(float v, int act) {
     if (act == GP_ACT_RELU) return v > 0.f ? v : 0.f;
@@ -295,45 +350,91 @@ __global__ __launch_bounds__(NT) void pool_kernel(PoolArgs a, BlpArgs blp) {
 // ---- elementwise ---------------------------------------------------------------------------
 // item = (row, 16-byte chunk); tile = 1024 items (4 per thread, strided by 256 for coalescing).
 constexpr int ELT_PER = 4;
-struct EltwiseArgs { gp_eltwise_params p; long items; };
+struct EltwiseArgs { gp_eltwise_params p; long items; int stream; };
+template <typename T>
+__device__ __forceinline__ void eltwise_finish(const gp_eltwise_params &p, int ch, float (&a)[VecIO<T>::VEC]) {
+    constexpr int VEC = VecIO<T>::VEC;
+    if (p.scale) {
+        float sc[VEC];
+        VecIO<T>::load((const T *)p.scale + ch * VEC, sc);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) a[j] *= sc[j];
+    }
+    if (p.shift) {
+        float sh[VEC];
+        VecIO<T>::load((const T *)p.shift + ch * VEC, sh);
+#pragma unroll
+        for (int j = 0; j < VEC; ++j) a[j] += sh[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; ++j) a[j] = act_f(a[j], p.act);
+}
+// A tile whose 1024 items all exist: no bounds checks, so every load of the tile is in flight
+// before the first value is needed (with the checks the compiler serialises the four items).
+template <typename T, bool NTH>
+__device__ __forceinline__ void eltwise_full_tile(const EltwiseArgs &a, unsigned base) {
+    const gp_eltwise_params &p = a.p;
+    constexpr int VEC = VecIO<T>::VEC;
+    const unsigned chunks = (unsigned)(p.cols / VEC);
+    long row[ELT_PER];
+    int ch[ELT_PER];
+    out_u32x4 ra[ELT_PER], rb[ELT_PER];
+#pragma unroll
+    for (int u = 0; u < ELT_PER; ++u) {
+        const unsigned item = base + u * NT + threadIdx.x;
+        const unsigned urow = item / chunks;
+        ch[u] = (int)(item - urow * chunks);
+        row[u] = urow;
+        ra[u] = ld_raw128<NTH>((const T *)p.a + row[u] * p.a_stride + ch[u] * VEC);
+    }
+    if (p.b) {
+#pragma unroll
+        for (int u = 0; u < ELT_PER; ++u) rb[u] = ld_raw128<NTH>((const T *)p.b + row[u] * p.b_stride + ch[u] * VEC);
+    }
+#pragma unroll
+    for (int u = 0; u < ELT_PER; ++u) {
+        float x[VEC];
+        VecIO<T>::unpack(ra[u], x);
+        if (p.b) {
+            float y[VEC];
+            VecIO<T>::unpack(rb[u], y);
+#pragma unroll
+            for (int j = 0; j < VEC; ++j) x[j] += y[j];
+        }
+        eltwise_finish<T>(p, ch[u], x);
+        st_raw128<NTH>((T *)p.out + row[u] * p.out_stride + ch[u] * VEC, VecIO<T>::pack(x));
+    }
+}
 template <typename T>
 __device__ __forceinline__ void eltwise_tile(const EltwiseArgs &a, TileIdx t) {
     const gp_eltwise_params &p = a.p;
     const long items = a.items;
     constexpr int VEC = VecIO<T>::VEC;
     const int chunks = p.cols / VEC;
-    
+    const unsigned base = (unsigned)t.x * ELT_PER * NT;  // 32-bit: see pool_tile
+    if ((long)base + ELT_PER * NT <= items) {
+        if (a.stream) eltwise_full_tile<T, true>(a, base);
+        else eltwise_full_tile<T, false>(a, base);
+        return;
+    }
 #pragma unroll
-        for (int u = 0; u < ELT_PER; ++u) {
-            const unsigned item = ((unsigned)t.x * ELT_PER + u) * NT + threadIdx.x;  // 32-bit: see pool_tile
-            if (item >= (unsigned)items) continue;
-            const unsigned urow = item / (unsigned)chunks;
-            const int ch = (int)(item - urow * (unsigned)chunks);
-            const long row = urow;
-            float a[VEC];
-            VecIO<T>::load((const T *)p.a + row * p.a_stride + ch * VEC, a);
-            if (p.b) {
-                float b[VEC];
-                VecIO<T>::load((const T *)p.b + row * p.b_stride + ch * VEC, b);
+    for (int u = 0; u < ELT_PER; ++u) {
+        const unsigned item = base + u * NT + threadIdx.x;
+        if (item >= (unsigned)items) continue;
+        const unsigned urow = item / (unsigned)chunks;
+        const int ch = (int)(item - urow * (unsigned)chunks);
+        const long row = urow;
+        float x[VEC];
+        VecIO<T>::load((const T *)p.a + row * p.a_stride + ch * VEC, x);
+        if (p.b) {
+            float y[VEC];
+            VecIO<T>::load((const T *)p.b + row * p.b_stride + ch * VEC, y);
 #pragma unroll
-                for (int j = 0; j < VEC; ++j) a[j] += b[j];
-            }
-            if (p.scale) {
-                float sc[VEC];
-                VecIO<T>::load((const T *)p.scale + ch * VEC, sc);
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) a[j] *= sc[j];
-            }
-            if (p.shift) {
-                float sh[VEC];
-                VecIO<T>::load((const T *)p.shift + ch * VEC, sh);
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) a[j] += sh[j];
-            }
-#pragma unroll
-            for (int j = 0; j < VEC; ++j) a[j] = act_f(a[j], p.act);
-            VecIO<T>::store((T *)p.out + row * p.out_stride + ch * VEC, a);
+            for (int j = 0; j < VEC; ++j) x[j] += y[j];
         }
+        eltwise_finish<T>(p, ch, x);
+        VecIO<T>::store((T *)p.out + row * p.out_stride + ch * VEC, x);
+    }
 }
 template <typename T, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void eltwise_kernel(EltwiseArgs a, BlpArgs blp) {
@@ -355,7 +456,7 @@ __host__ __device__ inline int softmax_rows_per_tile(int cols, int vec) {
     return g ? 4 * (64 / g) : 4;
 }
 
-template <typename T, int G, int C>
+template <typename T, int G, int C, bool NTH>
 __device__ __forceinline__ void softmax_rows_grouped(const gp_softmax_params &p, TileIdx t) {
     constexpr int VEC = VecIO<T>::VEC;
     const int lane = threadIdx.x & 63, sub = lane % G;
@@ -369,7 +470,7 @@ __device__ __forceinline__ void softmax_rows_grouped(const gp_softmax_params &p,
     for (int i = 0; i < C; ++i) {
         const int ch = sub + i * G;
         if (live && ch < chunks) {
-            VecIO<T>::load(x + ch * VEC, v[i]);
+            VecIO<T>::unpack(ld_raw128<NTH>(x + ch * VEC), v[i]);
 #pragma unroll
             for (int j = 0; j < VEC; ++j) { v[i][j] *= p.scale; mx = fmaxf(mx, v[i][j]); }
         }
@@ -395,7 +496,7 @@ __device__ __forceinline__ void softmax_rows_grouped(const gp_softmax_params &p,
         if (live && ch < chunks) {
 #pragma unroll
             for (int j = 0; j < VEC; ++j) v[i][j] *= inv;
-            VecIO<T>::store(out + ch * VEC, v[i]);
+            st_raw128<NTH>(out + ch * VEC, VecIO<T>::pack(v[i]));
         }
     }
 }
@@ -404,10 +505,15 @@ template <typename T>
 __device__ __forceinline__ void softmax_tile(const gp_softmax_params &p, TileIdx t) {
     constexpr int VEC = VecIO<T>::VEC;
     const int g = softmax_group(p.cols, VEC);  // uniform
-    if (g == 16) { softmax_rows_grouped<T, 16, 1>(p, t); return; }
+    const bool stream = p.rows * (long)p.cols * (long)sizeof(T) * 2 > kStreamBytes;  // uniform
+    if (g == 16) {
+        if (stream) softmax_rows_grouped<T, 16, 1, true>(p, t);
+        else softmax_rows_grouped<T, 16, 1, false>(p, t);
+        return;
+    }
     if (g == 64) {
-        if (p.cols / VEC <= 64) softmax_rows_grouped<T, 64, 1>(p, t);
-        else softmax_rows_grouped<T, 64, 4>(p, t);
+        if (p.cols / VEC <= 64) softmax_rows_grouped<T, 64, 1, false>(p, t);
+        else softmax_rows_grouped<T, 64, 4, false>(p, t);
         return;
     }
     // scalar path: one wavefront per row, 4 rows per tile; lane i reads elements i, i+64, ...
@@ -431,63 +537,91 @@ __global__ __launch_bounds__(NT) void softmax_kernel(gp_softmax_params p, BlpArg
 }
 
 // ---- layer norm ----------------------------------------------------------------------------
-// one wavefront per row, 4 rows per tile; the row (plus residual) is kept in registers
-// (up to MAXC 16-byte chunks per lane), so HBM sees one read and one write per element.
-template <typename T, int MAXC>
-__device__ __forceinline__ void layernorm_tile(const gp_layernorm_params &p, TileIdx t) {
+// one wavefront per RPW rows, 4 * RPW rows per tile; the rows (plus residual) are kept in registers
+// (up to MAXC 16-byte chunks per lane and row), so HBM sees one read and one write per element.
+// All loads of the wavefront's rows are issued before the first reduction.
+constexpr int kLnTwoRows = 0x100;  // flag in the plan's `sub`: RPW = 2
+template <typename T, int MAXC, int RPW, bool NTH>
+__device__ __forceinline__ void layernorm_rows(const gp_layernorm_params &p, TileIdx t) {
     constexpr int VEC = VecIO<T>::VEC;
     const int chunks = p.cols / VEC;
-    
-        long row = (long)t.x * 4 + (threadIdx.x >> 6);
-        if (row >= p.rows) return;
-        const int lane = threadIdx.x & 63;
+    const int lane = threadIdx.x & 63;
+    const long row0 = ((long)t.x * 4 + (threadIdx.x >> 6)) * RPW;
+    if (row0 >= p.rows) return;
+    out_u32x4 rx[RPW][MAXC], rr[RPW][MAXC];
+#pragma unroll
+    for (int q = 0; q < RPW; ++q) {
+        const long row = row0 + q < p.rows ? row0 + q : row0;  // a missing second row re-reads the first and is not stored
         const T *x = (const T *)p.x + row * p.cols;
-        const T *r = p.residual ? (const T *)p.residual + row * p.cols : nullptr;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            const int ch = lane + i * 64;
+            if (ch < chunks) rx[q][i] = ld_raw128<NTH>(x + ch * VEC);
+        }
+        if (p.residual) {
+            const T *r = (const T *)p.residual + row * p.cols;
+#pragma unroll
+            for (int i = 0; i < MAXC; ++i) {
+                const int ch = lane + i * 64;
+                if (ch < chunks) rr[q][i] = ld_raw128<NTH>(r + ch * VEC);
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < RPW; ++q) {
         float v[MAXC][VEC];
         float sum = 0.f;
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
-            int ch = lane + i * 64;
+            const int ch = lane + i * 64;
             if (ch < chunks) {
-                VecIO<T>::load(x + ch * VEC, v[i]);
-                if (r) {
-                    float rr[VEC];
-                    VecIO<T>::load(r + ch * VEC, rr);
+                VecIO<T>::unpack(rx[q][i], v[i]);
+                if (p.residual) {
+                    float r[VEC];
+                    VecIO<T>::unpack(rr[q][i], r);
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) v[i][j] += rr[j];
+                    for (int j = 0; j < VEC; ++j) v[i][j] += r[j];
                 }
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) sum += v[i][j];
             }
         }
-        float mean = wave_sum(sum) / (float)p.cols;
+        const float mean = wave_sum(sum) / (float)p.cols;
         float sq = 0.f;
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
-            int ch = lane + i * 64;
+            const int ch = lane + i * 64;
             if (ch < chunks) {
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) { float d = v[i][j] - mean; sq += d * d; }
             }
         }
-        float inv = rsqrtf(wave_sum(sq) / (float)p.cols + p.eps);
-        T *o = (T *)p.out + row * p.cols;
+        const float inv = rsqrtf(wave_sum(sq) / (float)p.cols + p.eps);
+        if (row0 + q >= p.rows) break;
+        T *o = (T *)p.out + (row0 + q) * p.cols;
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
-            int ch = lane + i * 64;
+            const int ch = lane + i * 64;
             if (ch < chunks) {
                 float ga[VEC], be[VEC], y[VEC];
                 VecIO<T>::load((const T *)p.gamma + ch * VEC, ga);
                 VecIO<T>::load((const T *)p.beta + ch * VEC, be);
 #pragma unroll
                 for (int j = 0; j < VEC; ++j) y[j] = (v[i][j] - mean) * inv * ga[j] + be[j];
-                VecIO<T>::store(o + ch * VEC, y);
+                st_raw128<NTH>(o + ch * VEC, VecIO<T>::pack(y));
             }
         }
+    }
 }
-template <typename T, int MAXC, int LOOP = LOOP_ANY>
+template <typename T, int MAXC, int RPW = 1>
+__device__ __forceinline__ void layernorm_tile(const gp_layernorm_params &p, TileIdx t) {
+    const bool stream = p.rows * (long)p.cols * (long)sizeof(T) * (p.residual ? 3 : 2) > kStreamBytes;  // uniform
+    if (stream) layernorm_rows<T, MAXC, RPW, true>(p, t);
+    else layernorm_rows<T, MAXC, RPW, false>(p, t);
+}
+template <typename T, int MAXC, int RPW = 1, int LOOP = LOOP_ANY>
 __global__ __launch_bounds__(NT) void layernorm_kernel(gp_layernorm_params p, BlpArgs blp) {
-    tiles<LOOP>(blp, [&](TileIdx t) { layernorm_tile<T, MAXC>(p, t); });
+    tiles<LOOP>(blp, [&](TileIdx t) { layernorm_tile<T, MAXC, RPW>(p, t); });
 }
 
 // ---- embedding -----------------------------------------------------------------------------

@@ -117,7 +117,8 @@ __device__ __forceinline__ void run_layer(const LayerDesc &d, TileIdx t, T *lds)
         case OP_SOFTMAX: { const gp_softmax_params a = d.u.softmax; softmax_tile<T>(a, t); break; }
         case OP_LAYERNORM: {
             const gp_layernorm_params a = d.u.ln;
-            if (d.sub == 2) layernorm_tile<T, 2>(a, t);
+            if (d.sub == (2 | kLnTwoRows)) layernorm_tile<T, 2, 2>(a, t);
+            else if (d.sub == 2) layernorm_tile<T, 2>(a, t);
             else if (d.sub == 8) layernorm_tile<T, 8>(a, t);
             else layernorm_tile<T, 16>(a, t);
             break;

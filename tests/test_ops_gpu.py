@@ -178,6 +178,46 @@ def test_layernorm(gp, dt, shape):
         assert rel_err(do.download(dtype, shape), ref) < TOL[dt]
 
 
+def _sample_rows(rng, rows):
+    return np.unique(np.concatenate([np.arange(512), np.arange(rows - 512, rows), rng.integers(0, rows, 1024)]))
+
+
+@pytest.mark.parametrize("op,dt,rows,cols", [("add", "f16", 65539, 1024), ("layernorm", "f16", 65537, 768), ("layernorm", "f32", 16385, 256),
+                                             ("layernorm", "bf16", 16386, 1024), ("softmax", "f16", (1 << 19) + 5, 128)])
+def test_large_tensors_streamed_and_paired_rows(gp, op, dt, rows, cols):
+    """Tensors past the last-level cache take nontemporal loads and stores, full eltwise tiles skip
+    their bounds checks, and layer-norm gives a wavefront two rows: sampled rows against the oracle,
+    and bit for bit against the same rows sent through a small launch (the default forms)."""
+    rng = np.random.default_rng(rows)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    x, r = rnd(rng, (rows, cols), dt, -2, 2), rnd(rng, (rows, cols), dt, -2, 2)
+    g, b = rnd(rng, (cols,), dt, 0.5, 1.5), rnd(rng, (cols,), dt)
+    idx = _sample_rows(rng, rows)
+
+    def run(xa, ra):
+        n = xa.shape[0]
+        dx, dr, dg, db = (gp.DevBuf.from_array(v, dtype) for v in (xa, ra, g, b))
+        do = gp.DevBuf(xa.size * gp.DTYPE_SIZE[dtype])
+        if op == "add":
+            gp.launch("gp_launch_eltwise", gp.EltwiseParams(dtype, n, cols, dx.ptr, cols, dr.ptr, cols, None, None, do.ptr, cols, gp.ACT_RELU))
+        elif op == "layernorm":
+            gp.launch("gp_launch_layernorm", gp.LayernormParams(dtype, n, cols, dx.ptr, dr.ptr, dg.ptr, db.ptr, do.ptr, 1e-12))
+        else:
+            gp.launch("gp_launch_softmax", gp.SoftmaxParams(dtype, n, cols, dx.ptr, do.ptr, 0.125))
+        sync(gp)
+        return do.download(dtype, (n, cols))
+
+    big = run(x, r)
+    xs, rs = np.ascontiguousarray(x[idx]), np.ascontiguousarray(r[idx])
+    small = run(xs, rs)
+    bad = np.nonzero((big[idx] != small).any(axis=1))[0]
+    assert bad.size == 0, f"{bad.size} of {idx.size} sampled rows differ from the small launch, first rows {idx[bad[:8]]}, max diff {np.abs(big[idx] - small).max()}"
+    ref = O.add_act(xs, rs, O.ACT_RELU) if op == "add" else O.layernorm(xs, g, b, 1e-12, rs) if op == "layernorm" else O.softmax(xs * np.float32(0.125))
+    assert rel_err(big[idx], ref) < TOL[dt]
+    if op == "add":  # cheap enough to check everywhere
+        assert big.tobytes() == O.round_to(np.maximum(x + r, 0), dt).astype(big.dtype).tobytes()
+
+
 @pytest.mark.parametrize("dt", DTS)
 def test_embed(gp, dt):
     rng = np.random.default_rng(9)
