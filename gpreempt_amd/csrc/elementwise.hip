@@ -110,7 +110,7 @@ int plan_softmax(const gp_softmax_params *p, EltPlan *out) {
     GP_REQUIRE(p->rows > 0 && p->cols > 0, "softmax shape");
     // rows made of whole 16-byte chunks are read as vectors
     GP_REQUIRE(softmax_group(p->cols, vec_of(p->dtype)) == 0 || (al16(p->x) && al16(p->out)), "softmax: 16-byte alignment");
-    const int rpt = softmax_rows_per_tile(p->cols, vec_of(p->dtype));
+    const int rpt = softmax_rows_per_tile(p->cols, vec_of(p->dtype), p->rows);
     long tiles = (p->rows + rpt - 1) / rpt;
     GP_REQUIRE(tiles < (1L << 31), "softmax: too many rows");
     *out = EltPlan{};

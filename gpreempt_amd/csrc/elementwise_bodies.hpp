@@ -451,52 +451,70 @@ __host__ __device__ inline int softmax_group(int cols, int vec) {  // lanes per 
     const int chunks = cols / vec;
     return chunks <= 16 ? 16 : chunks <= 256 ? 64 : 0;
 }
-__host__ __device__ inline int softmax_rows_per_tile(int cols, int vec) {
+// lane groups of a large problem take RPW rows each at a time: with one 16-byte load per lane and row
+// a wavefront has 1 KB in flight, too little to keep HBM busy
+__host__ __device__ inline int softmax_rows_per_group(int cols, int vec, long rows) {
+    return softmax_group(cols, vec) == 16 && rows >= 65536 ? 4 : 1;
+}
+__host__ __device__ inline int softmax_rows_per_tile(int cols, int vec, long rows) {
     const int g = softmax_group(cols, vec);
-    return g ? 4 * (64 / g) : 4;
+    return g ? 4 * (64 / g) * softmax_rows_per_group(cols, vec, rows) : 4;
 }
 
-template <typename T, int G, int C, bool NTH>
+template <typename T, int G, int C, bool NTH, int RPW = 1>
 __device__ __forceinline__ void softmax_rows_grouped(const gp_softmax_params &p, TileIdx t) {
     constexpr int VEC = VecIO<T>::VEC;
     const int lane = threadIdx.x & 63, sub = lane % G;
-    const long row = ((long)t.x * 4 + (threadIdx.x >> 6)) * (64 / G) + lane / G;
     const int chunks = p.cols / VEC;
-    const bool live = row < p.rows;
-    const T *x = (const T *)p.x + (live ? row : 0) * p.cols;
-    float v[C][VEC];
-    float mx = -INFINITY;
+    out_u32x4 raw[RPW][C];
+    long rowq[RPW];
 #pragma unroll
-    for (int i = 0; i < C; ++i) {
-        const int ch = sub + i * G;
-        if (live && ch < chunks) {
-            VecIO<T>::unpack(ld_raw128<NTH>(x + ch * VEC), v[i]);
+    for (int q = 0; q < RPW; ++q) {
+        rowq[q] = (((long)t.x * 4 + (threadIdx.x >> 6)) * RPW + q) * (64 / G) + lane / G;
+        const T *x = (const T *)p.x + (rowq[q] < p.rows ? rowq[q] : 0) * p.cols;
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) { v[i][j] *= p.scale; mx = fmaxf(mx, v[i][j]); }
+        for (int i = 0; i < C; ++i) {
+            const int ch = sub + i * G;
+            if (rowq[q] < p.rows && ch < chunks) raw[q][i] = ld_raw128<NTH>(x + ch * VEC);
         }
     }
 #pragma unroll
-    for (int o = G / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-    float sum = 0.f;
+    for (int q = 0; q < RPW; ++q) {
+        const bool live = rowq[q] < p.rows;
+        float v[C][VEC];
+        float mx = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < C; ++i) {
-        const int ch = sub + i * G;
-        if (live && ch < chunks) {
+        for (int i = 0; i < C; ++i) {
+            const int ch = sub + i * G;
+            if (live && ch < chunks) {
+                VecIO<T>::unpack(raw[q][i], v[i]);
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) { v[i][j] = __expf(v[i][j] - mx); sum += v[i][j]; }
+                for (int j = 0; j < VEC; ++j) { v[i][j] *= p.scale; mx = fmaxf(mx, v[i][j]); }
+            }
         }
-    }
 #pragma unroll
-    for (int o = G / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
-    const float inv = 1.f / sum;
-    T *out = (T *)p.out + (live ? row : 0) * p.cols;
+        for (int o = G / 2; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < C; ++i) {
-        const int ch = sub + i * G;
-        if (live && ch < chunks) {
+        for (int i = 0; i < C; ++i) {
+            const int ch = sub + i * G;
+            if (live && ch < chunks) {
 #pragma unroll
-            for (int j = 0; j < VEC; ++j) v[i][j] *= inv;
-            st_raw128<NTH>(out + ch * VEC, VecIO<T>::pack(v[i]));
+                for (int j = 0; j < VEC; ++j) { v[i][j] = __expf(v[i][j] - mx); sum += v[i][j]; }
+            }
+        }
+#pragma unroll
+        for (int o = G / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+        const float inv = 1.f / sum;
+        T *out = (T *)p.out + (live ? rowq[q] : 0) * p.cols;
+#pragma unroll
+        for (int i = 0; i < C; ++i) {
+            const int ch = sub + i * G;
+            if (live && ch < chunks) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) v[i][j] *= inv;
+                st_raw128<NTH>(out + ch * VEC, VecIO<T>::pack(v[i]));
+            }
         }
     }
 }
@@ -507,8 +525,12 @@ __device__ __forceinline__ void softmax_tile(const gp_softmax_params &p, TileIdx
     const int g = softmax_group(p.cols, VEC);  // uniform
     const bool stream = p.rows * (long)p.cols * (long)sizeof(T) * 2 > kStreamBytes;  // uniform
     if (g == 16) {
-        if (stream) softmax_rows_grouped<T, 16, 1, true>(p, t);
-        else softmax_rows_grouped<T, 16, 1, false>(p, t);
+        if (softmax_rows_per_group(p.cols, VEC, p.rows) == 4) {
+            if (stream) softmax_rows_grouped<T, 16, 1, true, 4>(p, t);
+            else softmax_rows_grouped<T, 16, 1, false, 4>(p, t);
+        } else {
+            softmax_rows_grouped<T, 16, 1, false>(p, t);
+        }
         return;
     }
     if (g == 64) {

@@ -87,11 +87,9 @@ struct CkptCtx {       // what a checkpointing body needs from the dispatcher, p
     int kernel_id;
 };
 
-// NWAVES: wavefronts per workgroup.  A wavefront's operand loads complete at about 11.7 GB/s however
-// many it keeps in flight, so four wavefronts fetch 47 GB/s per compute unit: a 256 x 256 tile
-// needs 64 KB per K-step, which then takes longer (1.4 us) than the step's MFMAs (0.85 us at
-// 2.4 GHz).  With eight wavefronts (two per SIMD, 128 accumulator registers each) the stream keeps
-// up and the second wavefront of a SIMD covers the first one's barrier and LDS waits.
+// NWAVES: wavefronts per workgroup.  With eight (two per SIMD, 128 accumulator registers each) the
+// second wavefront of a SIMD covers the first one's barrier, vmcnt and LDS waits, and each wavefront
+// issues half of a stage's loads: measured 5-8 % faster than four on the 256 x 256 tile.
 template <typename T, int BM, int BN, int STAGES, bool CONV, bool SPLITK, bool CKPT = false, int NWAVES = 4>
 struct PipeKernel {
     using elem = T;
@@ -365,7 +363,10 @@ struct PipeKernel {
         // instead of in front of it, and the requests reach the memory system as a steady stream.
         constexpr int NM = MI * NI;
         constexpr int EVEN = KSTEPS * NM / NLOADS > 0 ? KSTEPS * NM / NLOADS : 1;
-        constexpr int SPREAD = GP_LOAD_SPREAD > 0 ? GP_LOAD_SPREAD : (EVEN >= 4 ? EVEN - 1 : EVEN);  // measured: slightly front-loaded beats even for the 256x256 tile
+        // measured: slightly front-loaded beats even for the 256x256 tile; with eight wavefronts (each issues
+        // half the loads) every second slot is better still: the last load of a stage then leaves 40 % into
+        // the stage instead of 70 %, and the stage's end waits less for it (8192^3: 3-7 % of the launch)
+        constexpr int SPREAD = GP_LOAD_SPREAD > 0 ? GP_LOAD_SPREAD : (BM == 256 && WAVES == 8 && EVEN >= 4) ? 2 : (EVEN >= 4 ? EVEN - 1 : EVEN);
         static_assert(SPLITK || NLOADS <= KSTEPS * NM, "every load of a stage needs an MFMA slot");
         auto phase = [&](int buf, auto issue_c, const StageAddr &sa, auto p_c) {
             constexpr bool ISSUE = decltype(issue_c)::value != 0;
