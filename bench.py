@@ -376,6 +376,31 @@ def graph_workloads(runs=5):
     return out
 
 
+def vendor_gemm(operands="random", iters=20):
+    """For scale only (never part of the default run or of `value`): the vendor library's GEMM through
+    torch.matmul at config 5's size and operand layout (A [M,K] times the transpose of B [N,K])."""
+    import torch
+    n = 8192
+    if operands == "random":
+        a = (torch.rand(n, n, device="cuda") * 2 - 1).bfloat16()
+        b = (torch.rand(n, n, device="cuda") * 2 - 1).bfloat16()
+    else:
+        a = torch.full((n, n), 0.5, device="cuda").bfloat16()
+        b = torch.full((n, n), 0.25, device="cuda").bfloat16()
+    for _ in range(5):
+        c = a @ b.t()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        c = a @ b.t()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / iters
+    del c
+    return {"operands": operands, "ms": ms, "achieved": 2.0 * n ** 3 / ms / 1e9, "peak": PEAK["bf16"], "unit": "TFLOP/s", "frac": 2.0 * n ** 3 / ms / 1e9 / PEAK["bf16"]}
+
+
 def copy_calibration(mib=256, iters=10):
     """A plain device-to-device copy of known size (the runtime's copy kernel), used to scale
     the FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc runs."""
@@ -461,13 +486,17 @@ def main():
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
-    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal | vendor")
     ap.add_argument("--cpu-requests", type=int, default=10, help="timed submissions per graph in the cpu_baseline leg")
     ap.add_argument("--gemm-operands", default="random", choices=("random", "const"), help="operands of the 8192^3 GEMM leg (--only gemm)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the executor is a single-device path); run with --gpus 1")
 
+    if args.only == "vendor":
+        # torch brings its own HIP runtime: this leg runs without loading the library under test
+        print(json.dumps({"vendor_gemm8192_bf16": vendor_gemm(args.gemm_operands)}))
+        return
     from gpreempt_amd import capi as gp
     gp.init(0)
     out = {"metric": "HP p99 latency vs isolated (co-run p99 / isolated p99); preemption latency (us); BE throughput kept",
