@@ -81,10 +81,10 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         if (*grid < blp->groups) *grid = blp->groups;  // every counter needs a workgroup to serve its slice
         // a launch with fixed claims gets four workgroups more, which only read the flag (tile_loop.hpp)
         blp->spare = 0;
-        // (only when the whole grid starts at once: the last workgroups of a longer grid start last,
+        // (only when the whole grid, the four included, starts at once: the last workgroups of a longer grid start last,
         // and a flag read at the end of a kernel stops nothing; there every eighth workgroup of the
         // first four groups reads it after its claim, as in the general loop)
-        if (ctx->flag && blp->poll_mask != 0 && *grid <= resident && fixed_claims(true, ng, *grid, (int)total) && fixed_claims(true, ng, *grid + 4, (int)total)) {
+        if (ctx->flag && blp->poll_mask != 0 && *grid + 4 <= resident && fixed_claims(true, ng, *grid, (int)total) && fixed_claims(true, ng, *grid + 4, (int)total)) {
             blp->spare = 4;
             *grid += 4;
         }

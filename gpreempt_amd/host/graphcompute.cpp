@@ -22,6 +22,12 @@ bool read_array(const std::string &path, std::vector<T> &out) {
     if (!fp) return false;
     uint64_t count = 0, tag = 0;
     bool ok = std::fread(&count, sizeof(count), 1, fp) == 1 && std::fread(&tag, sizeof(tag), 1, fp) == 1 && count < (1ULL << 36);
+    if (ok) {  // the header's count must fit what is left of the file, before anything is allocated for it
+        const long here = std::ftell(fp);
+        ok = here >= 0 && std::fseek(fp, 0, SEEK_END) == 0;
+        const long end = ok ? std::ftell(fp) : -1;
+        ok = ok && end >= here && (uint64_t)(end - here) / sizeof(T) >= count && std::fseek(fp, here, SEEK_SET) == 0;
+    }
     if (ok) {
         out.resize(count);
         ok = std::fread(out.data(), sizeof(T), count, fp) == count;

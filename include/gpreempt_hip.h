@@ -119,8 +119,10 @@ typedef struct gp_preempt_ctx {
                      /* four workgroups more that own no claim and read the flag at launch         */
     int counter_groups; /* 0 or 1: *executed is one int (the reference's layout).  A power of two */
                      /* n > 1: executed points at n counters spaced 16 ints (64 bytes) apart;     */
-                     /* workgroup w claims from counter w % n, which owns a contiguous slice of   */
-                     /* the tiles.  Spreads the claim atomics, which serialise on one address.   */
+                     /* every counter owns a contiguous slice of the tiles and is served by the    */
+                     /* workgroups of one XCD (workgroup w runs on XCD w % 8; counter              */
+                     /* (w % 8) * (n / 8) + (w / 8) % (n / 8) for n >= 8, see util/slice_map.h).   */
+                     /* Spreads the claim atomics, which serialise on one address.                 */
     int fresh;       /* nonzero: the caller vouches that this kernel has not been launched since its    */
                      /* counters were last cleared.  With counter_groups > 1 a launch of at least as   */
                      /* many workgroups as claims then records its claims (a bit per workgroup in      */
