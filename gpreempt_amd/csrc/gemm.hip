@@ -123,6 +123,12 @@ static int pipe_case_ckpt(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_strea
     return launch_mat<PipeKernel<T, TILE, TILE, STAGES, false, false, true>>(pl, ctx, s, info);
 }
 
+template <typename T, int BM, int BN, int WAVES>
+static int wide_case(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
+    if (pl.conv) return launch_mat<WideKernel<T, BM, BN, WAVES, 3, true>>(pl, ctx, s, info);
+    return launch_mat<WideKernel<T, BM, BN, WAVES, 3, false>>(pl, ctx, s, info);
+}
+
 template <typename T>
 static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
@@ -134,10 +140,10 @@ static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream 
         case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
         case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
         case MB_PIPE32_SK: return pipe_case<T, 32, GP_S32, true>(pl, ctx, s, info);
-        case MB_WIDE32x32_16: return launch_mat<WideKernel<T, 32, 32, 16, 3>>(pl, ctx, s, info);
-        case MB_WIDE32x32_8: return launch_mat<WideKernel<T, 32, 32, 8, 3>>(pl, ctx, s, info);
-        case MB_WIDE64x32_16: return launch_mat<WideKernel<T, 64, 32, 16, 3>>(pl, ctx, s, info);
-        case MB_WIDE64x64_8: return launch_mat<WideKernel<T, 64, 64, 8, 3>>(pl, ctx, s, info);
+        case MB_WIDE32x32_16: return wide_case<T, 32, 32, 16>(pl, ctx, s, info);
+        case MB_WIDE32x32_8: return wide_case<T, 32, 32, 8>(pl, ctx, s, info);
+        case MB_WIDE64x32_16: return wide_case<T, 64, 32, 16>(pl, ctx, s, info);
+        case MB_WIDE64x64_8: return wide_case<T, 64, 64, 8>(pl, ctx, s, info);
         case MB_STAGED128:
             if (pl.conv) return launch_mat<TK<T, 128, 128, SBK, 2, 2, true, false>>(pl, ctx, s, info);
             return pl.b_kn ? launch_mat<TK<T, 128, 128, SBK, 2, 2, false, true>>(pl, ctx, s, info)
@@ -211,7 +217,10 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
     const MatArgs &g = pl->g;
     auto tiles = [&](int t) { return (long)((g.M + t - 1) / t) * ((g.N + t - 1) / t) * pl->batch; };
     const long cus = device_cus();
-    const bool wide_ok = !pl->b_kn && !pl->conv;  // GEMM with both operands K-contiguous
+    // both operands K-contiguous; a convolution, whose A operand is gathered, when a K-block never straddles
+    // two filter taps and a bit per tap fits a word
+    const int wide_bk = pl->dtype == GP_F32 ? 32 : 64;
+    const bool wide_ok = !pl->b_kn && (!pl->conv || (g.Cin % wide_bk == 0 && g.K / g.Cin <= 32 && g.S < 32));
     int body = -1;
     if (pl->b_kn || variant == GP_MAT_STAGED) {
         int tm = tile ? tile : (tiles(128) >= cus ? 128 : 64);
@@ -239,7 +248,7 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
         else if (tile == 0 || tile == 32) body = MB_PIPE32_SK;
     }
     if (body < 0) {
-        set_error("no matrix kernel for tile %d x %d with variant %d (tiles: 256, 128, 64; 64, 32 with split K; wide: 32x32, 64x32, 64x64, GEMM with N x K operands)", tile, tile_n ? tile_n : tile, variant);
+        set_error("no matrix kernel for tile %d x %d with variant %d (tiles: 256, 128, 64; 64, 32 with split K; wide: 32x32, 64x32, 64x64, N x K operands; convolutions with Cin a multiple of the K-block and at most 32 taps)", tile, tile_n ? tile_n : tile, variant);
         return GP_OUTOFRANGE;
     }
     int t = body == MB_PIPE256 ? 256 : (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
@@ -312,6 +321,7 @@ int plan_conv2d(const gp_conv_params *p, MatPlan *out) {
     GP_REQUIRE(Ho > 0 && Wo > 0, "conv: empty output");
     long M = (long)p->N * Ho * Wo;
     GP_REQUIRE(M < (1L << 31), "conv: too many output pixels");
+    GP_REQUIRE((long)p->N * (p->H + 2L * p->pad_h) * (p->W + 2L * p->pad_w) < (1L << 31), "conv: too many input pixels");
     GP_REQUIRE(!p->residual || p->res_pix_stride >= p->Cout, "conv: residual pixel stride");
     GP_REQUIRE(p->tile_m == p->tile_n || p->variant == GP_MAT_WIDE || p->variant == GP_MAT_WIDE8, "conv: square tiles only (the wide variants also take 64 x 32)");
     MatPlan &pl = *out;

@@ -61,6 +61,15 @@ static __device__ unsigned long long g_tile_prof[256 * 8];
 #define GP_PROBE(p) do { } while (0)
 #endif
 
+// a / b for 0 <= a < 2^22, 0 < b: a float multiply by a reciprocal taken once, and one correction step
+// either way (the integer division of this hardware is some sixty instructions per lane)
+__device__ __forceinline__ int small_div(int a, int b, float rcp_b) {
+    int q = (int)((float)a * rcp_b);
+    const int r = a - q * b;
+    q += (r >= b) - (r < 0);
+    return q;
+}
+
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
@@ -168,12 +177,15 @@ struct PipeKernel {
         const T *a_org[CONV ? A_PW : 1];         // CONV: the slot's window origin (may lie outside the image)
         int a_h0[CONV ? A_PW : 1], a_w0[CONV ? A_PW : 1];
         if (CONV) {
+            const int hw = g.Ho * g.Wo;
+            const bool small = g.M < (1 << 22);
+            const float rcp_hw = 1.0f / (float)hw, rcp_wo = 1.0f / (float)g.Wo;
 #pragma unroll
             for (int j = 0; j < A_PW; ++j) {
                 int m = a_row0 + j * 8;
                 int mm = m < g.M ? m : 0;
-                int n = mm / (g.Ho * g.Wo), rem = mm - n * (g.Ho * g.Wo);
-                int ho = rem / g.Wo, wo = rem - ho * g.Wo;
+                int n = small ? small_div(mm, hw, rcp_hw) : mm / hw, rem = mm - n * hw;
+                int ho = small ? small_div(rem, g.Wo, rcp_wo) : rem / g.Wo, wo = rem - ho * g.Wo;
                 a_h0[j] = ho * g.sh - g.ph; a_w0[j] = wo * g.sw - g.pw;
                 a_org[j] = A + ((long)n * g.H * g.W + (long)a_h0[j] * g.W + a_w0[j]) * g.lda;
             }

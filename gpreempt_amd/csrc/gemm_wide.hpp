@@ -22,15 +22,20 @@
 //
 // Measured (fp16, launch to launch): 128 x 768 x 3072 (BERT's second FFN layer) 10.2 -> 8.2 us,
 // 384 x 768 x 3072 11.9 -> 10.4 us; level with the four-wavefront bodies at K <= 1024, where the
-// longer wait for the first, larger stage costs what the faster stream saves.  A convolution form
-// (gathered A operand) was measured slower than the four-wavefront one at every ResNet-152 shape
-// and is not built.
+// longer wait for the first, larger stage costs what the faster stream saves.
+//
+// CONV = true: the A operand is gathered (implicit GEMM over NHWC pixels): row m is output pixel
+// (n, ho, wo), K element k is filter tap k / Cin, channel k % Cin.  Needs Cin to be a multiple of
+// BK (a block never straddles two taps) and at most 32 taps: which taps of a pixel's window lie
+// inside the image is worked out once per tile, as one bit per tap, so that a stage's loads cost a
+// shift, a select and an add per lane; the tap and channel of a wavefront group's next block
+// advance incrementally.
 #pragma once
 #include "gemm_pipe.hpp"
 
 namespace gp {
 
-template <typename T, int BM, int BN, int WAVES, int STAGES>
+template <typename T, int BM, int BN, int WAVES, int STAGES, bool CONV = false>
 struct WideKernel {
     using elem = T;
     static constexpr int bm = BM, bn = BN;
@@ -40,7 +45,8 @@ struct WideKernel {
     static constexpr int BK = RB / (int)sizeof(T);         // K elements per block: 64 (16-bit) or 32 (fp32)
     static constexpr int KB = WAVES / 4;                   // blocks per stage
     static constexpr int GROUPS = (BM + BN) / 8;           // 8-row load groups per block (A rows, then B rows)
-    static constexpr int LPW = GROUPS / 4;                 // load instructions per wavefront per stage
+    static constexpr int LPW_A = BM / 8 / 4, LPW_B = BN / 8 / 4;  // of a wavefront's loads per stage, the first LPW_A fetch A rows
+    static constexpr int LPW = LPW_A + LPW_B;              // load instructions per wavefront per stage
     static constexpr int A_BYTES = BM * RB, BLK_BYTES = (BM + BN) * RB, STAGE_BYTES = KB * BLK_BYTES;
     static constexpr int MI = BM / 32, NI = BN / 32;
     static constexpr int SLICES = MI * NI * 16;            // 64-float slices of one wavefront's accumulators
@@ -52,6 +58,8 @@ struct WideKernel {
     static constexpr bool early_stop = true;  // as PipeKernel::run: a second look at the stop index when the first stage has landed
     static_assert(WAVES % 4 == 0 && WAVES >= 4 && WAVES <= 16, "4, 8, 12 or 16 wavefronts");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && GROUPS % 4 == 0, "tile shape");
+    // slot j of wavefront wv (of its block group): row group wv*LPW_A + j of A, or wv*LPW_B + (j - LPW_A) of B
+    static __device__ __forceinline__ constexpr int group_of(int wv, int j) { return j < LPW_A ? wv * LPW_A + j : BM / 8 + wv * LPW_B + (j - LPW_A); }
     static_assert(STAGES >= 2 && (STAGES - 2) * LPW < 64, "pipeline depth");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 
@@ -79,20 +87,40 @@ struct WideKernel {
         const T *A = (const T *)g.A + offa, *B = (const T *)g.B + offb;
         const T *zero = (const T *)g_zero_page;
 
-        // ---- loader slots: slot j of this wavefront fetches row group wv*LPW + j of its block ------
+        // ---- loader slots: every wavefront fetches LPW_A row groups of A and LPW_B of B of its block (which
+        // kind a slot is is known at compile time: no branches in the stage's load sequence) ------
         // lane -> (row in the group, chunk position); the swizzle is applied on the source side:
         // the lane at position cpos of row r fetches chunk cpos ^ ((r >> 1) & 7) of that row
         const int rig = lane >> 3, cpos = lane & 7;
-        const T *base[LPW];    // the lane's row and chunk at k = 0
+        const int hw = CONV ? g.Ho * g.Wo : 1, ntap_rows = CONV ? g.K / (g.Cin * g.S) : 0;
+        const bool small = g.M < (1 << 22);
+        const float rcp_hw = 1.0f / (float)hw, rcp_wo = CONV ? 1.0f / (float)g.Wo : 1.0f;
+        const T *base[LPW];    // the lane's row and chunk at k = 0 (CONV, A rows: its window's origin, which may lie outside the image)
         bool row_ok[LPW];
         int kc[LPW];           // the lane's chunk offset in elements
+        unsigned taps[CONV ? LPW : 1];  // CONV, A rows: bit t set = tap t of the row's window is inside the image
 #pragma unroll
         for (int j = 0; j < LPW; ++j) {
-            const int gi = wv * LPW + j;              // group index in the block
-            const bool is_a = gi < BM / 8;
+            const int gi = group_of(wv, j);           // group index in the block
+            const bool is_a = j < LPW_A;
             const int r = (is_a ? gi : gi - BM / 8) * 8 + rig;   // row in its region
             kc[j] = (cpos ^ ((r >> 1) & 7)) * VEC;
-            if (is_a) {
+            if (is_a && CONV) {
+                const int m = m0 + r;
+                row_ok[j] = m < g.M;
+                const int mm = row_ok[j] ? m : 0;
+                const int n = small ? small_div(mm, hw, rcp_hw) : mm / hw, rem = mm - n * hw;
+                const int ho = small ? small_div(rem, g.Wo, rcp_wo) : rem / g.Wo, wo = rem - ho * g.Wo;
+                const int h0 = ho * g.sh - g.ph, w0 = wo * g.sw - g.pw;
+                base[j] = A + (long)((n * g.H + h0) * g.W + w0) * g.lda + kc[j];  // (pixel indices fit an int: checked by the planner)
+                // columns s of the window inside the image: s in [-w0, W - w0), clipped to [0, S); rows likewise
+                const int s_lo = w0 < 0 ? -w0 : 0, s_hi = g.W - w0 < g.S ? g.W - w0 : g.S;
+                const unsigned smask = (row_ok[j] && s_hi > s_lo) ? ((1u << s_hi) - 1u) & ~((1u << s_lo) - 1u) : 0u;
+                unsigned mask = 0;
+                for (int rr = 0; rr < ntap_rows; ++rr)  // (uniform trip count)
+                    if ((unsigned)(h0 + rr) < (unsigned)g.H) mask |= smask << (rr * g.S);
+                taps[CONV ? j : 0] = mask;
+            } else if (is_a) {
                 const int m = m0 + r;
                 row_ok[j] = m < g.M;
                 base[j] = A + (long)m * g.lda + kc[j];
@@ -104,16 +132,40 @@ struct WideKernel {
         }
         const int KT = (g.K + BK - 1) / BK;             // blocks along K
         const int NS = (KT + KB - 1) / KB;              // stages
+        // CONV: tap and channel of the block this wavefront group fetches next (stages are issued in order)
+        int nx_tap = 0, nx_r = 0, nx_s = 0, nx_ci = 0;
+        if (CONV) {
+            nx_tap = kb * BK / g.Cin;
+            nx_ci = kb * BK - nx_tap * g.Cin;
+            nx_r = nx_tap / g.S;
+            nx_s = nx_tap - nx_r * g.S;
+        }
         auto issue = [&](int s) {
             const int k0 = (s * KB + kb) * BK;          // first K element of this wavefront group's block
             const unsigned sbase = lds0 + (unsigned)(s % STAGES) * STAGE_BYTES + (unsigned)kb * BLK_BYTES;
+            const unsigned tap_bit = (k0 < g.K && nx_tap < 32) ? 1u << nx_tap : 0u;  // blocks past K have no tap
+            const int tap_off = (nx_r * g.W + nx_s) * (int)g.lda + nx_ci;  // elements from the window's origin
 #pragma unroll
             for (int j = 0; j < LPW; ++j) {
-                const int gi = wv * LPW + j;
-                // rows outside the problem and K-chunks past K (also whole blocks past the last one,
-                // when the stage is not full) come from the zero page
-                const bool ok = row_ok[j] & (k0 + kc[j] < g.K);
-                load_lds16(ok ? base[j] + k0 : zero, sbase + (unsigned)(gi * 8 * RB));
+                const int gi = group_of(wv, j);
+                if (CONV && j < LPW_A) {
+                    // taps outside the image, rows outside the problem and blocks past K come from the zero page
+                    const bool ok = (taps[CONV ? j : 0] & tap_bit) != 0;
+                    load_lds16(ok ? base[j] + tap_off : zero, sbase + (unsigned)(gi * 8 * RB));
+                } else {
+                    // rows outside the problem and K-chunks past K (also whole blocks past the last one,
+                    // when the stage is not full) come from the zero page
+                    const bool ok = row_ok[j] & (k0 + kc[j] < g.K);
+                    load_lds16(ok ? base[j] + k0 : zero, sbase + (unsigned)(gi * 8 * RB));
+                }
+            }
+            if (CONV) {
+                nx_ci += KB * BK;
+                while (nx_ci >= g.Cin) {
+                    nx_ci -= g.Cin;
+                    ++nx_tap;
+                    if (++nx_s == g.S) { nx_s = 0; ++nx_r; }
+                }
             }
         };
 

@@ -41,14 +41,19 @@ def test_conv2d_matches_oracle(gp, dt, case):
         got, info, _ = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=tile, variant=variant)
         assert np.isfinite(got).all(), (dt, case, tile, variant)
         assert rel_err(got, ref) < TOL[dt], (dt, case, tile, variant)
-    if k == 1 and stride == 1 and pad == 0:
-        # a pointwise convolution runs on the GEMM bodies, the wide split-K ones (16 or 8 wavefronts per tile) included
+    # the wide split-K bodies (16 or 8 wavefronts per tile): pointwise convolutions run on their GEMM form, the others
+    # on the gathered-operand form, which needs whole K-blocks per filter tap and at most 32 taps
+    bk = 32 if dt == "f32" else 64
+    if (k == 1 and stride == 1 and pad == 0) or (Cin % bk == 0 and k * k <= 32):
+        split_k = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=32, variant=3)[0]
         for tm, tn, variant in ((32, 32, gp.MAT_WIDE), (32, 32, gp.MAT_WIDE8), (64, 32, gp.MAT_WIDE), (64, 64, gp.MAT_WIDE8)):
             got, info, _ = gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=tm, tile_n=tn, variant=variant)
             assert info.total_tiles == -(-N * Ho * Wo // tm) * -(-Cout // tn) and info.block == (1024 if variant == gp.MAT_WIDE else 512)
             assert rel_err(got, ref) < TOL[dt], (dt, case, tm, tn, variant)
+            # the same summation as the four-wavefront split-K body: the same bits
+            assert got.tobytes() == split_k.tobytes(), (dt, case, tm, tn, variant)
     else:
-        with pytest.raises(gp.GpError):  # the wide bodies have no gathered-operand form
+        with pytest.raises(gp.GpError):
             gpu_conv2d(gp, dt, x, w, b, stride, pad, res, gp.ACT_RELU, tile=32, variant=gp.MAT_WIDE)
 
 
