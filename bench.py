@@ -29,7 +29,7 @@ HBM_PEAK_GBS = 8000.0
 # `bench.py --only roofline` (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads
 # for the copy of `--only copycal`); the figures and commands are in the hbm_traffic summary
 # under profiles/.  Counters cannot be collected from inside this process.
-HBM_TRAFFIC_PER_LAUNCH = {("resnet152", "f16"): 10.59e6}
+HBM_TRAFFIC_PER_LAUNCH = {("resnet152", "f16"): 10.57e6}
 
 
 def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
@@ -134,7 +134,7 @@ def roofline(workload, iters, dt):
             hbm_bound_layers += t_hbm > t_mfma
     ex.destroy()
     achieved = total_flop / (total_ms * 1e-3) / 1e12
-    return {"bound": "mfma", "kernel": "mat_kernel<PipeKernel<f16,conv>> (implicit-GEMM conv2d of " + workload + ", preemptible launches)",
+    return {"bound": "mfma", "kernel": "mat_kernel<PipeKernel | WideKernel<" + dt + ">> (the conv2d launches of " + workload + ", preemptible)",
             "achieved": achieved, "peak": PEAK[dt], "unit": "TFLOP/s", "frac": achieved / PEAK[dt],
             "traffic": HBM_TRAFFIC_PER_LAUNCH.get((workload, dt)),
             "launches": launches, "avg_launch_us": total_ms * 1e3 / launches, "event_bracket_us": bracket_ms * 1e3,

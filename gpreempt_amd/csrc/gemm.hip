@@ -241,7 +241,9 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
     } else if (variant == GP_MAT_AUTO) {
         // a tile wider than the problem multiplies zero columns: N <= 64 never takes the larger tiles
         if (!pl->conv && (tile == 256 || (tile == 0 && tiles(256) >= cus && g.N > 128 && g.M > 128))) body = MB_PIPE256;
-        else if (tile == 128 || (tile == 0 && tiles(128) >= cus && g.N > 64 && g.M > 64)) body = MB_PIPE128;
+        // (a problem of one or two K-steps is all epilogue, i.e. memory-bound: the 128 x 128 body runs one workgroup
+        // per CU, too few threads for that; 25088 x 256 x 64 with a residual: 19.8 us on 128 x 128, 15.0 on 64 x 64)
+        else if (tile == 128 || (tile == 0 && tiles(128) >= cus && g.N > 64 && g.M > 64 && g.K > 128)) body = MB_PIPE128;
         else if (tile == 0 && wide_ok && wide_pick(g, pl->batch, cus) >= 0) body = wide_pick(g, pl->batch, cus);
         else if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) body = MB_PIPE64;
         else if (tile == 0 && tiles(64) >= cus / 2) body = MB_PIPE64_SK;
