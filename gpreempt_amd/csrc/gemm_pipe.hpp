@@ -18,6 +18,7 @@
 //                 without making the result depend on scheduling.
 #pragma once
 #include "mma.hpp"
+#include "../../include/util/conv_addr.h"
 
 namespace gp {
 
@@ -60,15 +61,6 @@ static __device__ unsigned long long g_tile_prof[256 * 8];
 #else
 #define GP_PROBE(p) do { } while (0)
 #endif
-
-// a / b for 0 <= a < 2^22, 0 < b: a float multiply by a reciprocal taken once, and one correction step
-// either way (the integer division of this hardware is some sixty instructions per lane)
-__device__ __forceinline__ int small_div(int a, int b, float rcp_b) {
-    int q = (int)((float)a * rcp_b);
-    const int r = a - q * b;
-    q += (r >= b) - (r < 0);
-    return q;
-}
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");
@@ -178,7 +170,7 @@ struct PipeKernel {
         int a_h0[CONV ? A_PW : 1], a_w0[CONV ? A_PW : 1];
         if (CONV) {
             const int hw = g.Ho * g.Wo;
-            const bool small = g.M < (1 << 22);
+            const bool small = g.M < kSmallDivLimit;
             const float rcp_hw = 1.0f / (float)hw, rcp_wo = 1.0f / (float)g.Wo;
 #pragma unroll
             for (int j = 0; j < A_PW; ++j) {

@@ -93,7 +93,7 @@ struct WideKernel {
         // the lane at position cpos of row r fetches chunk cpos ^ ((r >> 1) & 7) of that row
         const int rig = lane >> 3, cpos = lane & 7;
         const int hw = CONV ? g.Ho * g.Wo : 1, ntap_rows = CONV ? g.K / (g.Cin * g.S) : 0;
-        const bool small = g.M < (1 << 22);
+        const bool small = g.M < kSmallDivLimit;
         const float rcp_hw = 1.0f / (float)hw, rcp_wo = CONV ? 1.0f / (float)g.Wo : 1.0f;
         const T *base[LPW];    // the lane's row and chunk at k = 0 (CONV, A rows: its window's origin, which may lie outside the image)
         bool row_ok[LPW];
@@ -113,12 +113,7 @@ struct WideKernel {
                 const int ho = small ? small_div(rem, g.Wo, rcp_wo) : rem / g.Wo, wo = rem - ho * g.Wo;
                 const int h0 = ho * g.sh - g.ph, w0 = wo * g.sw - g.pw;
                 base[j] = A + (long)((n * g.H + h0) * g.W + w0) * g.lda + kc[j];  // (pixel indices fit an int: checked by the planner)
-                // columns s of the window inside the image: s in [-w0, W - w0), clipped to [0, S); rows likewise
-                const int s_lo = w0 < 0 ? -w0 : 0, s_hi = g.W - w0 < g.S ? g.W - w0 : g.S;
-                const unsigned smask = (row_ok[j] && s_hi > s_lo) ? ((1u << s_hi) - 1u) & ~((1u << s_lo) - 1u) : 0u;
-                unsigned mask = 0;
-                for (int rr = 0; rr < ntap_rows; ++rr)  // (uniform trip count)
-                    if ((unsigned)(h0 + rr) < (unsigned)g.H) mask |= smask << (rr * g.S);
+                const unsigned mask = row_ok[j] ? window_tap_mask(h0, w0, g.H, g.W, ntap_rows, g.S) : 0u;
                 taps[CONV ? j : 0] = mask;
             } else if (is_a) {
                 const int m = m0 + r;
