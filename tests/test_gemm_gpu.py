@@ -447,7 +447,10 @@ def test_long_tiles_stopped_twice_then_finished(gp):
     stream.sync()
     second = st.checkpoint_headers(info.grid)
     assert st.stop_index() == 0
-    assert (second[:, 0] == first[:, 0]).all() and (second[second[:, 0] == 1][:, 3] >= first[first[:, 0] == 1][:, 3]).all()
+    # (a tile that no workgroup had started before the first stop may be started, and left, by the second launch:
+    # only the workgroups that already held a tile are compared)
+    held = first[:, 0] == 1
+    assert (second[held, 0] == 1).all() and (second[held, 2] == first[held, 2]).all() and (second[held, 3] >= first[held, 3]).all()
     flag.set(0)
     st.clear_stop()
     gp.launch("gp_launch_gemm", p, st.ctx(kernel_id=0), stream)
