@@ -74,6 +74,18 @@ def test_conv2d_channel_slices(gp):
     out = dbuf.download(gp.F32, (N, H, W, Cbuf))
     assert np.array_equal(out[..., :Cin], buf[..., :Cin]) and np.all(out[..., Cin:64] == 0)
     assert rel_err(nhwc_to_nchw(out[..., 64:]), O.conv2d(x, w, None, 1, 1)) < 1e-4
+    # the same through the wide bodies' gathered-operand form (Cin = 32 is one fp32 K-block per filter tap)
+    results = []
+    for tm, tn, variant in ((32, 32, gp.MAT_PIPE_SPLITK), (32, 32, gp.MAT_WIDE), (64, 64, gp.MAT_WIDE8)):
+        dbuf.upload(buf)
+        p.tile_m, p.tile_n, p.variant = tm, tn, variant
+        gp.launch("gp_launch_conv2d", p)
+        sync(gp)
+        results.append(dbuf.download(gp.F32, (N, H, W, Cbuf)).copy())
+        assert rel_err(nhwc_to_nchw(results[-1][..., 64:]), O.conv2d(x, w, None, 1, 1)) < 1e-4
+        assert np.array_equal(results[-1][..., :64], out[..., :64])
+    # the split-K summation of the four-wavefront body, bit for bit
+    assert np.array_equal(results[1], results[0]) and np.array_equal(results[2], results[0])
 
 
 @pytest.mark.parametrize("dt_in,dt_out", [("f32", "f32"), ("f32", "f16"), ("f16", "f16"), ("f32", "bf16")])
