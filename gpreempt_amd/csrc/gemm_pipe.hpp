@@ -366,22 +366,27 @@ struct PipeKernel {
         // SPREAD-th MFMA, so that their address arithmetic issues while the matrix pipe is busy
         // instead of in front of it, and the requests reach the memory system as a steady stream.
         constexpr int NM = MI * NI;
-        constexpr int EVEN = KSTEPS * NM / NLOADS > 0 ? KSTEPS * NM / NLOADS : 1;
+        // (the spacing is that of the operand loads alone: the stop-word load of a checkpointing body goes with
+        // the first of them, so that it has the whole stage to come back.  Counted with the others it halved
+        // the spacing of the 128 x 128 body, 2 -> 1, which bunched its eight operand loads at the start of the
+        // stage: 21 % of a VGG-16 layer)
+        constexpr int EVEN = KSTEPS * NM / LPS > 0 ? KSTEPS * NM / LPS : 1;
         // measured: slightly front-loaded beats even for the 256x256 tile; with eight wavefronts (each issues
         // half the loads) every second slot is better still: the last load of a stage then leaves 40 % into
         // the stage instead of 70 %, and the stage's end waits less for it (8192^3: 3-7 % of the launch)
         constexpr int SPREAD = GP_LOAD_SPREAD > 0 ? GP_LOAD_SPREAD : (BM == 256 && WAVES == 8 && EVEN >= 4) ? 2 : (EVEN >= 4 ? EVEN - 1 : EVEN);
-        static_assert(SPLITK || NLOADS <= KSTEPS * NM, "every load of a stage needs an MFMA slot");
+        static_assert(SPLITK || LPS <= KSTEPS * NM, "every operand load of a stage needs an MFMA slot");
         auto phase = [&](int buf, auto issue_c, const StageAddr &sa, auto p_c) {
             constexpr bool ISSUE = decltype(issue_c)::value != 0;
             constexpr int P = decltype(p_c)::value;
             static_for<0, NM>([&](auto qc) {
                 constexpr int q = decltype(qc)::value, slot = P * NM + q;
                 Elem<T>::mma(fa[buf][q / NI], fb[buf][q % NI], acc[q / NI][q % NI]);
-                if constexpr (ISSUE && slot % SPREAD == 0 && slot / SPREAD < NLOADS) issue_one(sa, slot / SPREAD);
+                if constexpr (ISSUE && slot % SPREAD == 0 && slot / SPREAD < LPS) issue_one(sa, slot / SPREAD);
+                if constexpr (ISSUE && slot == 0) static_for<LPS, NLOADS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
                 // the slots cannot hold every load at this spacing: the rest follow the last MFMA
-                if constexpr (ISSUE && slot == KSTEPS * NM - 1 && slot / SPREAD + 1 < NLOADS)
-                    static_for<slot / SPREAD + 1, NLOADS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
+                if constexpr (ISSUE && slot == KSTEPS * NM - 1 && slot / SPREAD + 1 < LPS)
+                    static_for<slot / SPREAD + 1, LPS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
                 if constexpr (ISSUE) __builtin_amdgcn_sched_barrier(0);
             });
         };
@@ -393,13 +398,6 @@ struct PipeKernel {
             else wait_vmcnt<0>();
             int stop_word = -1, flag_word = 0;
             __syncthreads();  // everyone's part of stage kt is visible; stage kt-1's buffer is free
-            if constexpr (CKPT) {
-                if (can_ckpt && (kt & (POLL_EVERY - 1)) == 0) {
-                    // the words that travelled with stage kt: the same two for every wave, looked at below
-                    stop_word = pollw[((kt % STAGES) * WAVES + 0) * 64];
-                    flag_word = pollw[((kt % STAGES) * WAVES + 1) * 64];
-                }
-            }
             if (kt == 0) GP_PROBE(2);
             const int stage = kt % STAGES;
             StageAddr sa = {};
@@ -417,12 +415,22 @@ struct PipeKernel {
                 } else if constexpr (ISSUE) {
                     static_for<0, NM>([&](auto qc) {  // first k-tile: phase 0 has loads but no MFMAs
                         constexpr int slot = decltype(qc)::value;
-                        if constexpr (slot % SPREAD == 0 && slot / SPREAD < NLOADS) issue_one(sa, slot / SPREAD);
+                        if constexpr (slot % SPREAD == 0 && slot / SPREAD < LPS) issue_one(sa, slot / SPREAD);
+                        if constexpr (slot == 0) static_for<LPS, NLOADS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
                     });
                 }
                 static_for<0, KSTEPS - 1>([&](auto kc) {
                     constexpr int ks = decltype(kc)::value;
                     __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (CKPT && ks == KSTEPS - 2) {
+                        // the words that travelled with stage kt: the same two for every wave, looked at after the
+                        // last phase, whose MFMAs cover the LDS latency (read at the top of the k-tile they cost
+                        // 12 % of a VGG-16 layer: the wait for them came in front of the first fragment reads)
+                        if (can_ckpt && (kt & (POLL_EVERY - 1)) == 0) {
+                            stop_word = pollw[((kt % STAGES) * WAVES + 0) * 64];
+                            flag_word = pollw[((kt % STAGES) * WAVES + 1) * 64];
+                        }
+                    }
                     read_frags((ks + 1) & 1, stage, ks + 1);
                     __builtin_amdgcn_sched_barrier(0);
                     phase(ks & 1, issue_c, sa, IntC<ks + 1>{});
