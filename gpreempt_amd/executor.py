@@ -16,7 +16,7 @@ SYMBOLS = """gpx_create gpx_destroy gpx_init gpx_set_input gpx_get_output gpx_ge
 gpx_launch_kernel gpx_get_kernel_num gpx_capture_graph gpx_uses_program gpx_clear gpx_set_flag gpx_set_running gpx_resume
 gpx_get_stop_point gpx_last_stop_index gpx_inject_preempt gpx_read_counters gpx_reset_counters gpx_storage_num gpx_storage_info
 gpx_kernel_info gpx_read_storage gpx_miniweather_reductions gpx_graph_info gpx_graph_result_bytes gpx_graph_result
-gpx_graph_inject_preempt gpx_set_lc_tasks gpx_set_graph_path gpx_write_synthetic_graph gpx_run_scenario gpx_preempt_probe gpx_parse_params gpx_parse_tvm_export gpx_set_priority gpx_domain_create gpx_domain_destroy gpx_get_fd gpx_domain_flag gpx_domain_flag_value
+gpx_graph_inject_preempt gpx_set_lc_tasks gpx_set_graph_path gpx_write_synthetic_graph gpx_run_scenario gpx_preempt_probe gpx_parse_params gpx_parse_tvm_export gpx_plan_tvm_export gpx_set_priority gpx_domain_create gpx_domain_destroy gpx_get_fd gpx_domain_flag gpx_domain_flag_value
 gpx_domain_begin gpx_domain_end gpx_suspend_streams gpx_resume_streams""".split()
 
 STATUS = ["Succ", "Fail", "Timeout", "NotFound", "OutOfRange", "Full"]

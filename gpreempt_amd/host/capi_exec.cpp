@@ -326,3 +326,76 @@ extern "C" int gpx_parse_tvm_export(const char *device_json, const char *host_js
         return copy_report(st, rep.dump(), report, report_len);
     });
 }
+
+// The native kernel list an exported model maps to, without touching a GPU.
+extern "C" int gpx_plan_tvm_export(const char *device_json, const char *host_json, const char *ops_json, const char *dtype, char *report, size_t report_len) {
+    return guarded("gpx_plan_tvm_export", [&] {
+        Model m;
+        json::Value rep = json::Value::object();
+        Status st = m.load_from_json(device_json ? device_json : "", host_json ? host_json : "");
+        std::string err = m.tvm_export() ? m.tvm_export()->error : "";
+        if (st == Status::Succ) {
+            std::ifstream f(ops_json ? ops_json : "", std::ios::binary);
+            if (!f.is_open()) { st = Status::NotFound; err = std::string("Cannot open the json file: ") + (ops_json ? ops_json : ""); }
+            else {
+                std::string text((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+                st = m.build_from_export(dtype && *dtype ? std::string("export@dtype=") + dtype : std::string("export"), text);
+                if (st != Status::Succ) err = m.tvm_export()->error;
+            }
+        }
+        rep.set("error") = err;
+        rep.set("dtype") = m.dtype();
+        json::Value &js = rep.set("storages");
+        js = json::Value::array();
+        for (size_t i = 0; st == Status::Succ && i < m.get_storage_num(); ++i) {
+            const StorageInfo &s = m.get_storage_info(i);
+            const ParamLayout &L = m.get_param_layout(i);
+            json::Value e = json::Value::object();
+            e.set("name") = s.name; e.set("stype") = s.stype; e.set("size") = s.size;
+            e.set("is_param") = L.is_param ? 1 : 0; e.set("kind") = (int)L.kind; e.set("disk_elems") = L.disk_elems;
+            js.push(e);
+        }
+        json::Value &jk = rep.set("kernels");
+        jk = json::Value::array();
+        for (size_t i = 0; st == Status::Succ && i < m.get_kernel_num(); ++i) {
+            const KernelInfo &k = m.get_kernel_info(i);
+            json::Value e = json::Value::object();
+            e.set("name") = k.name;
+            json::Value &ar = e.set("args");
+            ar = json::Value::array();
+            for (const ArgRef &r : k.refs) ar.push(r.storage == SIZE_MAX ? json::Value("") : json::Value(m.get_storage_info(r.storage).name));
+            json::Value &p = e.set("params");
+            p = json::Value::object();
+            switch (k.op) {
+                case OpKind::Conv: {
+                    const gp_conv_params &c = k.p.conv;
+                    p.set("N") = c.N; p.set("H") = c.H; p.set("W") = c.W; p.set("Cin") = c.Cin; p.set("Cout") = c.Cout; p.set("R") = c.R; p.set("S") = c.S;
+                    p.set("stride_h") = c.stride_h; p.set("stride_w") = c.stride_w; p.set("pad_h") = c.pad_h; p.set("pad_w") = c.pad_w; p.set("act") = c.act;
+                    p.set("in_pix_stride") = c.in_pix_stride; p.set("out_pix_stride") = c.out_pix_stride;
+                    break;
+                }
+                case OpKind::Gemm: {
+                    const gp_gemm_params &g = k.p.gemm;
+                    p.set("M") = g.M; p.set("N") = g.N; p.set("K") = g.K; p.set("lda") = g.lda; p.set("ldc") = g.ldc; p.set("act") = g.act;
+                    break;
+                }
+                case OpKind::Pool: {
+                    const gp_pool_params &q = k.p.pool;
+                    p.set("N") = q.N; p.set("H") = q.H; p.set("W") = q.W; p.set("C") = q.C; p.set("R") = q.R; p.set("stride") = q.stride; p.set("pad") = q.pad; p.set("mode") = q.mode;
+                    break;
+                }
+                case OpKind::Eltwise: {
+                    const gp_eltwise_params &q = k.p.eltwise;
+                    p.set("rows") = q.rows; p.set("cols") = q.cols; p.set("a_stride") = q.a_stride; p.set("out_stride") = q.out_stride; p.set("act") = q.act;
+                    break;
+                }
+                case OpKind::Softmax: p.set("rows") = k.p.softmax.rows; p.set("cols") = k.p.softmax.cols; break;
+                case OpKind::Layout: p.set("N") = k.p.layout.N; p.set("C") = k.p.layout.C; p.set("H") = k.p.layout.H; p.set("W") = k.p.layout.W; p.set("c_pad") = k.p.layout.c_pad; break;
+                default: break;
+            }
+            jk.push(e);
+        }
+        return copy_report(st, rep.dump(), report, report_len);
+    });
+}
+

@@ -10,6 +10,7 @@
 
 #include "numeric.h"
 #include "tvm_export.h"
+#include "graph_builder.h"
 #include "zoo.h"
 #include <sys/stat.h>
 
@@ -97,6 +98,16 @@ Status Model::load_model(const std::string &device_json, const std::string &host
             return s;
         }
     }
+    if (have_export) {
+        // with an operator sidecar next to it, the export itself is the graph that runs
+        const std::string ops_json = device_json.substr(0, device_json.find_last_of('/') + 1) + "ops.json";
+        std::ifstream oj(ops_json);
+        if (oj.is_open()) {
+            const std::string text((std::istreambuf_iterator<char>(oj)), std::istreambuf_iterator<char>());
+            RETURN_STATUS(build_from_export(name, text));
+            return allocate_and_bind();
+        }
+    }
     RETURN_STATUS(build(name));
     if (have_export) {
         // the native graph runs; the export must at least agree with it on what goes in and comes out
@@ -122,6 +133,38 @@ Status Model::load_model(const std::string &device_json, const std::string &host
 Status Model::load_from_json(const char *device_json, const char *host_json) {
     export_ = std::make_shared<TvmExport>();
     return load_tvm_export(device_json, host_json, *export_);
+}
+
+// The export's host functions replaced one for one by native operators (include/tvm_export.h).  The element type
+// is the export's own unless the workload name asks for another ("<directory>@dtype=f16").
+Status Model::build_from_export(const std::string &workload, const std::string &ops_json_text) {
+    if (is_loaded() || !export_) return Status::Fail;
+    ExportOps ops;
+    std::string err;
+    Status s = parse_export_ops(ops_json_text, ops);
+    if (s != Status::Succ) err = ops.error;
+    if (s == Status::Succ) s = check_export_ops(*export_, ops, err);
+    std::string dt;
+    size_t at = workload.find("dtype=");
+    if (at != std::string::npos && workload.find('@') < at) dt = workload.substr(at + 6, workload.find(',', at) == std::string::npos ? std::string::npos : workload.find(',', at) - at - 6);
+    if (s == Status::Succ && dt.empty()) {
+        for (const ExportNode &n : export_->nodes)
+            if (n.func.empty() && n.name == "data") dt = n.stype == "float32" ? "f32" : n.stype == "float16" ? "f16" : "";
+        if (dt.empty()) { err = "the export's data is neither float32 nor float16"; s = Status::Fail; }
+    }
+    if (s == Status::Succ && dt != "f32" && dt != "f16" && dt != "bf16") { err = "unknown dtype '" + dt + "'"; s = Status::Fail; }
+    if (s == Status::Succ) {
+        GraphBuilder b(*this, dt);
+        s = build_export_graph(b, *export_, ops, err);
+    }
+    if (s != Status::Succ) {
+        std::fprintf(stderr, "load_model: %s\n", err.c_str());
+        export_->error = err;
+        storage_infos.clear(); layouts.clear(); kernel_infos.clear();
+        return s;
+    }
+    workload_ = workload;
+    return Status::Succ;
 }
 
 Status Model::build(const std::string &workload) {
@@ -225,12 +268,14 @@ Status Model::upload_param(size_t idx, const float *disk, size_t n) {
                 for (int nn = 0; nn < L.o; ++nn) dev[(size_t)nn * L.i + k] = disk[(size_t)k * L.o + nn];
             break;
         case ParamLayout::DenseOverCHW: {
-            size_t feat = (size_t)L.c * L.h * L.w;
+            // rows of C x H x W features on disk, H x W x (C padded to i_pad) on the device
+            const size_t feat = (size_t)L.c * L.h * L.w, cp = L.i_pad > L.c ? (size_t)L.i_pad : (size_t)L.c, feat_dev = cp * L.h * L.w;
+            if ((size_t)L.o * feat_dev > dev_elems) return Status::OutOfRange;
             for (int o = 0; o < L.o; ++o)
                 for (int c = 0; c < L.c; ++c)
                     for (int h = 0; h < L.h; ++h)
                         for (int w = 0; w < L.w; ++w)
-                            dev[o * feat + ((size_t)h * L.w + w) * L.c + c] = disk[o * feat + ((size_t)c * L.h + h) * L.w + w];
+                            dev[o * feat_dev + ((size_t)h * L.w + w) * cp + c] = disk[o * feat + ((size_t)c * L.h + h) * L.w + w];
             break;
         }
     }

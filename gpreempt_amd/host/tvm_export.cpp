@@ -59,6 +59,10 @@ Status parse_tvm_export(const std::string &device_json_text, const std::string &
         if (es == 0) return fail(out.error, "device json: unknown dltype '" + s.stype + "' of node " + std::to_string(i));
         s.size = elems * es;
         out.storage_infos.push_back(s);
+        ExportNode n;
+        n.name = s.name; n.stype = s.stype;
+        for (const json::Value &dim : shapes.arr[i].arr) n.shape.push_back((long)dim.num);
+        out.nodes.push_back(n);
     }
     // temporary storages, typed float32 whatever they hold (src/model.cpp:176-183)
     for (const json::Value &t : h["temp_args"].arr) {
@@ -81,8 +85,10 @@ Status parse_tvm_export(const std::string &device_json_text, const std::string &
                 return fail(out.error, "device json: bad input of node " + std::to_string(i));
             args.push_back((size_t)in.arr[0].num);
         }
+        out.nodes[i].inputs = args;
+        out.nodes[i].func = node["attrs"]["func_name"].string();
         args.push_back(i);
-        func_args.emplace_back(node["attrs"]["func_name"].string(), args);
+        func_args.emplace_back(out.nodes[i].func, args);
     }
 
     auto push_nop = [&](const std::vector<size_t> &args) {

@@ -87,6 +87,12 @@ long gpx_parse_params(const char *path, const char *key, float *out, size_t n, s
  * (name, stype, size), "kernels" (name, func, launch_params, args_index), "global_len",
  * "heads_index", "ops" and "error".  Needs no GPU. */
 int gpx_parse_tvm_export(const char *device_json, const char *host_json, const char *ops_json, char *report, size_t report_len);
+/* The native kernel list that an export plus its sidecar maps to (foo::build_export_graph, include/tvm_export.h),
+ * in element type `dtype` ("f32" "f16" "bf16"; NULL or "" = the export's own): what Model::load_model runs when
+ * the model directory holds an ops.json, where the reference loads the export's own device code
+ * (src/model.cpp:84-98).  The JSON report holds "storages" (name, stype, size, is_param, kind, disk_elems),
+ * "kernels" (name, args = storage names, params) and "error".  Needs no GPU. */
+int gpx_plan_tvm_export(const char *device_json, const char *host_json, const char *ops_json, const char *dtype, char *report, size_t report_len);
 
 /* include/gpreempt.h through the C view.  gpx_set_priority = NvRmQuery + set_priority on the
  * tenant's stream (reference src/cuda-clients/gpreemptclient.cpp:170-177); 0 or -1 as the reference.

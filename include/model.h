@@ -31,7 +31,7 @@ public:
 struct ParamLayout {
     enum Kind { Plain, ConvOIHW, DenseOverCHW, MatKN } kind = Plain;
     int o = 0, i = 0, r = 0, s = 0, i_pad = 0;  // ConvOIHW; MatKN: a K x N matrix on disk (i = K, o = N), kept N x K on the device
-    int c = 0, h = 0, w = 0;                    // DenseOverCHW: input features were flattened from C x H x W
+    int c = 0, h = 0, w = 0;                    // DenseOverCHW: input features were flattened from C x H x W (device rows: H x W x max(C, i_pad))
     size_t disk_elems = 0;                      // fp32 values expected on disk
     bool is_param = false;
     // seeded initial value when no parameter file is given
@@ -86,11 +86,13 @@ public:
     // The three paths name files inside MODEL_PATH/<workload>/ as in the reference
     // (src/executor.cpp:110-113); the workload is the name of that directory and the graph is
     // built natively from it.  `workload` may carry options: "resnet152@b=8,dtype=f16".
-    // When mod.json and host.json exist they are read as the reference reads them (load_from_json)
-    // and must describe a model with the same input ("data") and output ("heads") sizes as the
-    // native graph of that workload name; a mismatch, or files that do not parse, is Status::Fail
-    // (a caller that brings a different graph under a known name must not silently get the built-in
-    // one).  The kernels that run are always the native ones.
+    // When mod.json and host.json exist they are read as the reference reads them (load_from_json).
+    // With an ops.json next to them (the operator sidecar of include/tvm_export.h) the exported graph
+    // is what runs, operator by operator on the native kernels, under whatever name the directory
+    // has.  Without one the native graph of that workload name runs, and the export must describe a
+    // model with the same input ("data") and output ("heads") sizes; a mismatch, or files that do
+    // not parse, is Status::Fail (a caller that brings a different graph under a known name must
+    // not silently get the built-in one).
     Status load_model(const std::string &device_json, const std::string &host_json, const std::string &cuda_module);
     // Model::load_from_json of the reference (src/model.cpp:128-235): storages and device kernels
     // of an exported model.  The result is kept for inspection (tvm_export()); it does not replace
@@ -98,6 +100,9 @@ public:
     Status load_from_json(const char *device_json, const char *host_json);
     const struct TvmExport *tvm_export() const { return export_.get(); }
     Status build(const std::string &workload);
+    // Fills the kernel list from the export read by load_from_json plus the text of its operator
+    // sidecar; allocates nothing (load_model does that next).
+    Status build_from_export(const std::string &workload, const std::string &ops_json_text);
 
     // Reads a "TVM_MODEL_PARAMS" file (format of reference src/model.cpp:15-55) and uploads every
     // tensor whose key names a storage.  Parameters missing from the file keep their seeded

@@ -17,7 +17,17 @@
 
 namespace foo {
 
+// One node of mod.json's graph: a tensor (an input or parameter when `func` is empty, else the result of
+// the host function `func`, "__nop" for a reshape).  The reference reads only the flattened view below;
+// the node view is what the native loader builds its kernels from.
+struct ExportNode {
+    std::string name, func, stype;
+    std::vector<long> shape;
+    std::vector<size_t> inputs;  // node ids
+};
+
 struct TvmExport {
+    std::vector<ExportNode> nodes;           // [0, global_len)
     std::vector<StorageInfo> storage_infos;  // [0, global_len): graph nodes; then one "temp" per host.json temp_args entry
     std::vector<KernelInfo> kernel_infos;    // name, launch_params, args_index as the reference fills them; "nop" for __nop nodes
     std::vector<std::string> kernel_func;    // host function (fused operator) each kernel belongs to; "__nop" for copies
@@ -54,5 +64,19 @@ struct ExportOps {
 Status parse_export_ops(const std::string &ops_json_text, ExportOps &out);
 // Every non-"__nop" host function of the export must be described exactly once, by name.
 Status check_export_ops(const TvmExport &ex, const ExportOps &ops, std::string &error);
+
+// ---- an export on the native operators ----------------------------------------------------------------
+// Appends to `m` the storages and kernels that compute the exported graph with the operators of
+// libgpreempt_hip.so, in the element type `dtype` ("f32" "f16" "bf16"; empty = the export's own).
+// Activations are kept NHWC; parameters keep the export's node names ("p0", "p1", ...) and are declared
+// in the export's on-disk convention (fp32; OIHW convolution weights; dense weights [units][features]
+// over an NCHW flatten), so that the export's own mod.params loads into them (src/model.cpp:263-282).
+// "data" and "heads" have the export's shapes (NCHW data).  Mapped: conv2d (groups 1, dilation 1,
+// symmetric padding), dense, max / average / global-average pooling, add, scale_shift, softmax over the
+// last axis, concatenate over channels, reshape / __nop between a 4-D tensor and its NCHW flatten.  Anything
+// else (the attention and layer-norm functions of a BERT export among them) is Status::Fail with `error`
+// naming the function: nothing is guessed.
+class GraphBuilder;
+Status build_export_graph(GraphBuilder &b, const TvmExport &ex, const ExportOps &ops, std::string &error);
 
 }  // namespace foo

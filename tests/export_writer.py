@@ -1,0 +1,231 @@
+"""Writes small models in the reference's export schema (mod.json as TVM's graph executor stores it,
+host.json as patch/tvm.patch:296-311 adds it, mod.params as scripts/compile/compile.py:73-83 writes
+it) plus the operator sidecar ops.json, and computes what the model must output with the oracle's
+operators on the way.  TEST INFRASTRUCTURE: the reference ships no exported model, so the tests
+build their own; names follow TVM's (parameters p0, p1, ...; one fused function per operator group,
+identical groups sharing a function, host.json listing one entry per operator node in graph order as
+src/model.cpp:199-229 walks it)."""
+import json
+import os
+
+import numpy as np
+
+from oracle import oracle as O
+from gpreempt_amd.executor import write_params
+
+
+class ExportWriter:
+    def __init__(self, dt="f32", seed=0):
+        self.dt = dt
+        self.rng = np.random.default_rng(seed)
+        self.nodes, self.shapes, self.values = [], [], []
+        self.params = {}
+        self.funcs = {}      # (base, key) -> function name
+        self.taken = {}      # base -> how many functions carry it
+        self.ops = []        # sidecar entries, one per function
+        self.host = []       # host.json entries, one per operator node
+        self.n_temp = 0
+
+    # ---- graph bookkeeping -------------------------------------------------------------------------
+    def _r(self, a):
+        return O.round_to(np.asarray(a, np.float32), self.dt)
+
+    def _node(self, name, inputs, value, func=None):
+        node = {"op": "tvm_op" if func else "null", "name": name, "inputs": [[i, 0, 0] for i in inputs]}
+        if func:
+            node["attrs"] = {"num_outputs": "1", "num_inputs": str(len(inputs)), "flatten_data": "0", "func_name": func}
+        self.nodes.append(node)
+        self.shapes.append(list(value.shape))
+        self.values.append(value)
+        return len(self.nodes) - 1
+
+    def _func(self, base, key, op, attrs, epilogue, inputs):
+        k = (base, key)
+        if k not in self.funcs:
+            n = self.taken.get(base, 0)
+            self.taken[base] = n + 1
+            name = "tvmgen_default_fused_" + base + (f"_{n}" if n else "")
+            self.funcs[k] = name
+            self.ops.append({"name": name, "op": op, "attrs": attrs, "epilogue": epilogue, "inputs": inputs})
+        return self.funcs[k]
+
+    def _op(self, base, key, op, attrs, epilogue, roles, inputs, value, temps=0):
+        func = self._func(base, key, op, attrs, epilogue, roles)
+        node = self._node(func.replace("tvmgen_default_", ""), inputs, value, func)
+        args = list(range(len(inputs) + 1))
+        kernels = [{"name": func + "_kernel0", "launch_params": [max(1, value.size // 256), 1, 1, 256, 1, 1], "args": args}]
+        if temps:  # a function whose first kernel leaves an intermediate in a temporary buffer
+            self.n_temp = max(self.n_temp, temps)
+            kernels = [{"name": func + "_kernel0", "launch_params": [1, 1, 1, 64, 1, 1], "args": args[:-1] + [-1]},
+                       {"name": func + "_kernel1", "launch_params": [1, 1, 1, 64, 1, 1], "args": [-1, args[-1]]}]
+        self.host.append({"name": func, "kernels": kernels})
+        return node
+
+    # ---- tensors -----------------------------------------------------------------------------------
+    def data(self, x):
+        return self._node("data", [], self._r(x))
+
+    def param(self, value):
+        name = f"p{len(self.params)}"
+        self.params[name] = np.asarray(value, np.float32)
+        return self._node(name, [], self._r(value))
+
+    def value(self, node):
+        return self.values[node]
+
+    # ---- operators ---------------------------------------------------------------------------------
+    def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, residual=None, relu=True, gain=1.0, temps=0):
+        kh, kw = (k, k) if isinstance(k, int) else k
+        sh, sw = (stride, stride) if isinstance(stride, int) else stride
+        ph, pw = (pad, pad) if isinstance(pad, int) else pad
+        cin = self.shapes[x][1]
+        w = self.param(self.rng.normal(0, gain * np.sqrt(2.0 / (cin * kh * kw)), (cout, cin, kh, kw)))
+        inputs, roles, epi, base = [x, w], {"data": 0, "weight": 1}, [], "nn_conv2d"
+        bv = None
+        if bias:
+            b = self.param(self.rng.normal(0, 0.1, (cout, 1, 1)))
+            bv = self.values[b].reshape(-1)
+            roles["bias"] = len(inputs); inputs.append(b); epi.append("bias"); base += "_add"
+        rv = None
+        if residual is not None:
+            rv = self.values[residual]
+            roles["residual"] = len(inputs); inputs.append(residual); epi.append("residual"); base += "_add"
+        if relu:
+            epi.append("relu"); base += "_nn_relu"
+        out = self._r(O.conv2d(self.values[x], self.values[w], bv, (sh, sw), (ph, pw), rv, O.ACT_RELU if relu else O.ACT_NONE))
+        attrs = {"strides": [sh, sw], "padding": [ph, pw, ph, pw], "dilation": [1, 1], "groups": 1}
+        key = (tuple(self.shapes[x]), cout, kh, kw, sh, sw, ph, pw, tuple(epi))
+        return self._op(base, key, "conv2d", attrs, epi, roles, inputs, out, temps)
+
+    def dense(self, x, units, bias=True, relu=False):
+        feat = self.shapes[x][1]
+        w = self.param(self.rng.normal(0, np.sqrt(1.0 / feat), (units, feat)))
+        inputs, roles, epi, base = [x, w], {"data": 0, "weight": 1}, [], "nn_dense"
+        bv = None
+        if bias:
+            b = self.param(self.rng.normal(0, 0.1, (units,)))
+            bv = self.values[b]
+            roles["bias"] = 2; inputs.append(b); epi.append("bias"); base += "_add"
+        if relu:
+            epi.append("relu"); base += "_nn_relu"
+        out = self._r(O.gemm_bias_act(self.values[x], self.values[w], bv, None, O.ACT_RELU if relu else O.ACT_NONE, b_is_nk=True))
+        return self._op(base, (tuple(self.shapes[x]), units, tuple(epi)), "dense", {}, epi, roles, inputs, out)
+
+    def pool(self, x, kind, k=2, stride=2, pad=0, count_include_pad=False):
+        if kind == "global_avg":
+            n, c = self.shapes[x][:2]
+            out = self._r(O.global_avgpool(self.values[x])).reshape(n, c, 1, 1)
+            return self._op("nn_global_avg_pool2d", tuple(self.shapes[x]), "global_avg_pool2d", {}, [], {"data": 0}, [x], out)
+        mode = "max" if kind == "max" else ("avg_pad" if count_include_pad else "avg")
+        out = self._r(O.pool2d(self.values[x], k, stride, pad, mode))
+        attrs = {"pool_size": [k, k], "strides": [stride, stride], "padding": [pad, pad, pad, pad], "ceil_mode": 0}
+        if kind == "avg":
+            attrs["count_include_pad"] = int(count_include_pad)
+        op = "max_pool2d" if kind == "max" else "avg_pool2d"
+        return self._op("nn_" + op, (tuple(self.shapes[x]), k, stride, pad, count_include_pad), op, attrs, [], {"data": 0}, [x], out)
+
+    def add(self, a, b, relu=False):
+        out = self._r(O.add_act(self.values[a], self.values[b], O.ACT_RELU if relu else O.ACT_NONE))
+        return self._op("add" + ("_nn_relu" if relu else ""), (tuple(self.shapes[a]), relu), "add", {}, ["relu"] if relu else [], {"lhs": 0, "rhs": 1}, [a, b], out)
+
+    def add_channel_constant(self, x, relu=False):
+        c = self.shapes[x][1]
+        p = self.param(self.rng.normal(0, 0.2, (c, 1, 1)))
+        out = self._r(O.scale_shift_act(self.values[x], np.ones(c, np.float32), self.values[p].reshape(-1), O.ACT_RELU if relu else O.ACT_NONE))
+        return self._op("add" + ("_nn_relu" if relu else ""), (tuple(self.shapes[x]), relu, "const"), "add", {}, ["relu"] if relu else [], {"lhs": 0, "rhs": 1}, [x, p], out)
+
+    def scale_shift(self, x, relu=True):
+        c = self.shapes[x][1]
+        s = self.param(self.rng.uniform(0.5, 1.5, (c, 1, 1)))
+        h = self.param(self.rng.normal(0, 0.2, (c, 1, 1)))
+        out = self._r(O.scale_shift_act(self.values[x], self.values[s].reshape(-1), self.values[h].reshape(-1), O.ACT_RELU if relu else O.ACT_NONE))
+        return self._op("multiply_add" + ("_nn_relu" if relu else ""), (tuple(self.shapes[x]), relu), "scale_shift", {}, ["relu"] if relu else [],
+                        {"data": 0, "scale": 1, "shift": 2}, [x, s, h], out)
+
+    def softmax(self, x):
+        return self._op("nn_softmax", tuple(self.shapes[x]), "softmax", {"axis": -1}, [], {"data": 0}, [x], self._r(O.softmax(self.values[x])))
+
+    def concatenate(self, xs):
+        out = np.concatenate([self.values[x] for x in xs], axis=1)
+        return self._op("concatenate", tuple(tuple(self.shapes[x]) for x in xs), "concatenate", {"axis": 1}, [], {}, list(xs), out)
+
+    def flatten(self, x):
+        """batch_flatten, which TVM turns into a __nop node (a reshape that shares its argument's memory)"""
+        v = self.values[x]
+        return self._node("reshape_nop", [x], v.reshape(v.shape[0], -1), "__nop")
+
+    # ---- files -------------------------------------------------------------------------------------
+    def write(self, directory, head, sidecar=True, params=True):
+        os.makedirs(directory, exist_ok=True)
+        stype = {"f32": "float32", "f16": "float16", "bf16": "float32"}[self.dt]
+        n = len(self.nodes)
+        mod = {"nodes": self.nodes, "arg_nodes": [i for i, nd in enumerate(self.nodes) if nd["op"] == "null"], "heads": [[head, 0, 0]],
+               "attrs": {"dltype": ["list_str", [stype] * n], "device_index": ["list_int", [2] * n], "storage_id": ["list_int", list(range(n))],
+                         "shape": ["list_shape", self.shapes]},
+               "node_row_ptr": list(range(n + 1))}
+        host = {"temp_args": [4096] * self.n_temp, "funcs": self.host}
+        with open(os.path.join(directory, "mod.json"), "w") as f:
+            json.dump(mod, f)
+        with open(os.path.join(directory, "host.json"), "w") as f:
+            json.dump(host, f)
+        if sidecar:
+            with open(os.path.join(directory, "ops.json"), "w") as f:
+                json.dump({"layout": "NCHW", "funcs": self.ops}, f)
+        if params:
+            write_params(os.path.join(directory, "mod.params"), self.params)
+        return self.values[head]
+
+
+def mini_resnet(dt, batch=2, hw=32, seed=1):
+    """stem, max-pool, two bottleneck blocks (one with a projected shortcut, one with the identity), a
+    concatenation, a per-channel scale and shift, average pool, global pool, classifier, softmax"""
+    w = ExportWriter(dt, seed)
+    x = w.data(w.rng.normal(0, 1, (batch, 3, hw, hw)))
+    y = w.conv2d(x, 16, 7, 2, 3, temps=1)
+    y = w.pool(y, "max", 3, 2, 1)
+    sc = w.conv2d(y, 32, 1, relu=False)
+    z = w.conv2d(y, 8, 1)
+    z = w.conv2d(z, 8, 3, 1, 1)
+    y = w.conv2d(z, 32, 1, residual=sc, gain=0.5)
+    z = w.conv2d(y, 8, 1)
+    z = w.conv2d(z, 8, 3, 1, 1)          # same shapes and attributes as the block before: the same function
+    y2 = w.conv2d(z, 32, 1, residual=y, gain=0.5)
+    br = w.conv2d(y2, 16, (1, 3), 1, (0, 1), bias=False)
+    cat = w.concatenate([y2, br])
+    y = w.pool(w.scale_shift(cat), "avg", 2, 2, 0)
+    y = w.add(y, w.pool(cat, "avg", 3, 2, 1, count_include_pad=True))
+    y = w.pool(y, "global_avg")
+    y = w.flatten(y)
+    y = w.dense(y, 10)
+    return w, w.softmax(y)
+
+
+def mini_vgg(dt, batch=1, hw=16, seed=2):
+    """convolutions without fused bias, a separate per-channel add, 2x2 max-pools, a flatten of a 4 x 4
+    image (dense weights stored over C x H x W) and two dense layers"""
+    w = ExportWriter(dt, seed)
+    x = w.data(w.rng.normal(0, 1, (batch, 3, hw, hw)))
+    y = w.conv2d(x, 8, 3, 1, 1, bias=False, relu=False)
+    y = w.add_channel_constant(y, relu=True)
+    y = w.pool(y, "max", 2, 2)
+    y = w.conv2d(y, 16, 3, 1, 1)
+    y = w.pool(y, "max", 2, 2)
+    y = w.flatten(y)
+    y = w.dense(y, 32, relu=True)
+    return w, w.dense(y, 10, bias=False)
+
+
+def padded_channels(dt, seed=3):
+    """channel counts that are no multiple of the 16-byte vector: 12 and 20 channels, the narrow one last
+    in a concatenation"""
+    w = ExportWriter(dt, seed)
+    x = w.data(w.rng.normal(0, 1, (1, 3, 12, 12)))
+    a = w.conv2d(x, 16, 3, 1, 1)
+    b = w.conv2d(a, 12, 3, 2, 1)
+    c = w.conv2d(b, 20, 1)
+    d = w.pool(w.conv2d(a, 16, 3, 2, 1), "max", 3, 1, 1)
+    y = w.concatenate([d, c])            # 16 + 20
+    y = w.conv2d(y, 24, 3, 1, 1)
+    y = w.pool(y, "global_avg")
+    y = w.flatten(y)
+    return w, w.dense(y, 5)

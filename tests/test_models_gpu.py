@@ -311,3 +311,58 @@ def test_exported_graph_next_to_the_model_is_read_and_checked(gp, ex_mod, tmp_pa
     # the model root is process-wide (an environment variable): leave one without exported files behind
     (d / "mod.json").unlink(); (d / "host.json").unlink()
     os.environ["GPREEMPT_MODEL_PATH"] = str(tmp_path)
+
+
+# ---- exported models on the native operators ------------------------------------------------------
+# The reference loads an export's own device code (src/model.cpp:84-98); here mod.json + host.json +
+# the operator sidecar ops.json become native kernels and the export's mod.params loads into them by the
+# export's parameter names.  The exports are written by tests/export_writer.py, which computes the expected
+# output with the oracle's operators while it writes.
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("maker", ["mini_resnet", "mini_vgg", "padded_channels"])
+def test_exported_model_matches_oracle(gp, ex_mod, tmp_path, maker, dt):
+    import export_writer as EW
+    w, head = getattr(EW, maker)(dt)
+    want = w.write(str(tmp_path / maker), head)
+    ex = ex_mod.Executor(maker, model_root=str(tmp_path))
+    dtype = gp.DTYPE_BY_NAME[dt]
+    got = run(gp, ex, gp.to_storage(w.value(0), dtype), dtype, want.shape)
+    assert rel_err(got, want) < TOL[dt], maker
+    names = {s["name"] for s in ex.storages() if s["is_param"]}
+    assert names == set(w.params)  # every parameter of the export, under the export's name
+    ex.destroy()
+
+
+def test_exported_model_in_another_element_type_and_without_parameters(gp, ex_mod, tmp_path):
+    import export_writer as EW
+    # an fp32 export run in bf16: the workload name carries the element type, as for the built-in models
+    w, head = EW.mini_vgg("bf16")
+    want = w.write(str(tmp_path / "mini_vgg@dtype=bf16"), head)
+    ex = ex_mod.Executor("mini_vgg@dtype=bf16", model_root=str(tmp_path))
+    got = run(gp, ex, gp.to_storage(w.value(0), gp.BF16), gp.BF16, want.shape)
+    assert rel_err(got, want) < TOL["bf16"]
+    ex.destroy()
+    # no mod.params: the seeded initialisation stays, the model still runs (src/model.cpp:263-282 copies only what the file holds)
+    w, head = EW.mini_resnet("f16")
+    w.write(str(tmp_path / "noparams"), head, params=False)
+    ex = ex_mod.Executor("noparams", model_root=str(tmp_path))
+    got = run(gp, ex, gp.to_storage(w.value(0), gp.F16), gp.F16, (2, 10))
+    assert np.isfinite(got).all() and np.allclose(got.sum(axis=1), 1, atol=1e-2)
+    ex.destroy()
+    # an export that cannot be mapped is refused at load time, by name
+    w, head = EW.mini_vgg("f32")
+    w.ops[0]["attrs"]["groups"] = 2
+    w.write(str(tmp_path / "grouped"), head)
+    with pytest.raises(ex_mod.StatusError) as e:
+        ex_mod.Executor("grouped", model_root=str(tmp_path))
+    assert e.value.status == 1
+
+
+@pytest.mark.parametrize("program", [False, True])
+def test_exported_model_preempt_resume_bit_exact(gp, ex_mod, tmp_path, program):
+    import export_writer as EW
+    w, head = EW.mini_resnet("f16", batch=4, hw=64)
+    w.write(str(tmp_path / "mini_resnet"), head)
+    x = gp.to_storage(w.value(0), gp.F16)
+    _blp_roundtrip(gp, ex_mod, tmp_path, "mini_resnet", x, [(1, 0), (6, 0), (9, 0)], graph=program)

@@ -121,3 +121,99 @@ def test_huge_counts_in_a_parameter_file_are_refused(tmp_path):
     assert lib.gpx_parse_params(path.encode(), None, None, C.c_size_t(0), None) == -1
     open(path, "wb").write(b"TVM_MODEL_PARAMS\0" + struct.pack("<Q", 1 << 60) + b"p0\0" + struct.pack("<Q", 4) + b"\0" * 16)
     assert lib.gpx_parse_params(path.encode(), None, None, C.c_size_t(0), None) == -1
+
+
+# ---- the export mapped onto the native operators (no GPU: the kernel list only) -----------------------------
+
+def plan(d, dtype=None):
+    from gpreempt_amd import executor as gx
+    buf = C.create_string_buffer(1 << 20)
+    rc = gx.lib().gpx_plan_tvm_export((d + "/mod.json").encode(), (d + "/host.json").encode(), (d + "/ops.json").encode(),
+                                      dtype.encode() if dtype else None, buf, C.c_size_t(len(buf)))
+    return rc, json.loads(buf.value.decode()) if buf.value else {}
+
+
+def test_tiny_export_maps_to_three_native_kernels():
+    rc, rep = plan(FIX)
+    assert rc == 0, rep
+    assert rep["dtype"] == "f32"
+    k = rep["kernels"]
+    assert [x["name"] for x in k] == ["nchw_to_nhwc", "conv2d", "dense"]  # the reshape is a view, not a copy
+    # 3 channels padded to one 16-byte vector; 3x3, stride 1, padding 1 from the sidecar; bias and ReLU fused
+    assert k[0]["params"] == {"N": 1, "C": 3, "H": 8, "W": 8, "c_pad": 4}
+    conv = k[1]["params"]
+    assert (conv["Cin"], conv["Cout"], conv["R"], conv["S"], conv["stride_h"], conv["pad_h"], conv["pad_w"], conv["act"]) == (4, 4, 3, 3, 1, 1, 1, 1)
+    assert k[1]["args"] == ["data.nhwc", "p0", "p1", "", "tvmgen_default_fused_nn_conv2d_add_nn_relu"]
+    # the dense layer reads the convolution's memory as one row of 256 and writes the renamed output
+    assert k[2]["params"] == {"M": 1, "N": 10, "K": 256, "lda": 256, "ldc": 10, "act": 0}
+    assert k[2]["args"] == ["tvmgen_default_fused_nn_conv2d_add_nn_relu", "p2", "", "", "heads"]
+    st = {s["name"]: s for s in rep["storages"]}
+    # parameters keep the export's names and its on-disk sizes: OIHW convolution weight, dense over C x H x W
+    assert (st["p0"]["is_param"], st["p0"]["kind"], st["p0"]["disk_elems"], st["p0"]["size"]) == (1, 1, 108, 4 * 4 * 3 * 3 * 4)
+    assert (st["p1"]["kind"], st["p1"]["disk_elems"]) == (0, 4)
+    assert (st["p2"]["kind"], st["p2"]["disk_elems"]) == (2, 2560)
+    assert st["data"]["size"] == 768 and st["heads"]["size"] == 40
+    rc, rep = plan(FIX, "f16")
+    assert rc == 0 and rep["dtype"] == "f16" and rep["kernels"][1]["params"]["Cin"] == 8
+    assert {s["name"]: s["size"] for s in rep["storages"]}["data"] == 384
+
+
+def test_generated_exports_map_operator_by_operator(tmp_path):
+    import export_writer as EW
+    w, head = EW.mini_resnet("f32")
+    d = str(tmp_path / "r")
+    w.write(d, head)
+    rc, rep = plan(d)
+    assert rc == 0, rep
+    names = [k["name"] for k in rep["kernels"]]
+    # layout, 9 convolutions, 4 pools, concat = 2 copies, scale-shift, add, classifier, softmax
+    assert names.count("conv2d") == 9 and names.count("pool2d") == 4 and names.count("eltwise") == 4
+    assert names[0] == "nchw_to_nhwc" and names[-2:] == ["dense", "softmax"]
+    stem = rep["kernels"][1]["params"]
+    assert (stem["R"], stem["stride_h"], stem["pad_h"], stem["Cout"], stem["act"]) == (7, 2, 3, 16, 1)
+    wide = [k["params"] for k in rep["kernels"] if k["name"] == "conv2d" and k["params"]["R"] == 1 and k["params"]["S"] == 3][0]
+    assert (wide["pad_h"], wide["pad_w"]) == (0, 1)
+    pools = [k["params"] for k in rep["kernels"] if k["name"] == "pool2d"]
+    assert [p["mode"] for p in pools] == [0, 1, 3, 2]   # max; average; average counting the padding; global
+    res = [k for k in rep["kernels"] if k["name"] == "conv2d" and k["args"][3]]
+    assert len(res) == 2                                  # the two residual inputs are fused into their convolutions
+    assert rep["storages"][-1]["name"] == "heads"
+    # channel counts that are no multiple of eight halves are padded; the padding is invisible to the export
+    w, head = EW.padded_channels("f16")
+    d = str(tmp_path / "p")
+    w.write(d, head)
+    rc, rep = plan(d)
+    assert rc == 0, rep
+    convs = [k["params"] for k in rep["kernels"] if k["name"] == "conv2d"]
+    assert [(c["Cin"], c["Cout"], c["out_pix_stride"]) for c in convs] == [(8, 16, 16), (16, 12, 16), (16, 20, 24), (16, 16, 16), (40, 24, 24)]
+    copies = [k["params"] for k in rep["kernels"] if k["name"] == "eltwise"]
+    assert [(c["cols"], c["out_stride"]) for c in copies] == [(16, 40), (24, 40)]
+
+
+def test_what_cannot_be_mapped_is_refused_by_name(tmp_path):
+    def conv_attr(key, value):
+        return lambda f, doc: doc["funcs"][0]["attrs"].__setitem__(key, value) if f == "ops.json" else None
+    for name, edit, text in [
+        ("groups", conv_attr("groups", 2), "grouped convolution is not mapped"),
+        ("dilation", conv_attr("dilation", [2, 2]), "dilated convolution is not mapped"),
+        ("asym", conv_attr("padding", [0, 0, 2, 2]), "asymmetric padding is not mapped"),
+        # the sidecar's attributes must reproduce the shapes the export states
+        ("stride", conv_attr("strides", [2, 2]), "the export says 1x4x8x8, the operator attributes give 1x4x4x4"),
+        ("tail", lambda f, doc: doc["funcs"][0].__setitem__("epilogue", ["relu", "bias"]) if f == "ops.json" else None, "in that order"),
+        ("role", lambda f, doc: doc["funcs"][0]["inputs"].__setitem__("weight", 0) if f == "ops.json" else None, "must be a parameter"),
+        ("bert", lambda f, doc: doc["funcs"][1].__setitem__("op", "layer_norm") if f == "ops.json" else None, "operator 'layer_norm' is not mapped"),
+        ("layout", lambda f, doc: doc.__setitem__("layout", "NHWC") if f == "ops.json" else None, "NCHW"),
+    ]:
+        d = _edited(tmp_path, name, edit)
+        rc, rep = plan(d)
+        assert rc == 1 and text in rep["error"], (name, rep["error"])
+        assert rep["kernels"] == [] and rep["storages"] == []
+
+    # an image as the model's output would have to be converted back to NCHW
+    def image_head(f, doc):
+        if f == "mod.json":
+            doc["heads"] = [[3, 0, 0]]
+    rc, rep = plan(_edited(tmp_path, "head", image_head))
+    assert rc == 1 and "an image as the model's output" in rep["error"]
+    rc, rep = plan(FIX, "f64")
+    assert rc == 1 and "unknown dtype" in rep["error"]
