@@ -25,6 +25,7 @@ class ExportWriter:
         self.ops = []        # sidecar entries, one per function
         self.host = []       # host.json entries, one per operator node
         self.n_temp = 0
+        self.alias = {}      # name of the same parameter in the built-in graphs -> export name
 
     # ---- graph bookkeeping -------------------------------------------------------------------------
     def _r(self, a):
@@ -74,16 +75,20 @@ class ExportWriter:
         return self.values[node]
 
     # ---- operators ---------------------------------------------------------------------------------
-    def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, residual=None, relu=True, gain=1.0, temps=0):
+    def conv2d(self, x, cout, k, stride=1, pad=0, bias=True, residual=None, relu=True, gain=1.0, temps=0, name=None):
         kh, kw = (k, k) if isinstance(k, int) else k
         sh, sw = (stride, stride) if isinstance(stride, int) else stride
         ph, pw = (pad, pad) if isinstance(pad, int) else pad
         cin = self.shapes[x][1]
         w = self.param(self.rng.normal(0, gain * np.sqrt(2.0 / (cin * kh * kw)), (cout, cin, kh, kw)))
         inputs, roles, epi, base = [x, w], {"data": 0, "weight": 1}, [], "nn_conv2d"
+        if name:
+            self.alias[name + ".weight"] = self.nodes[w]["name"]
         bv = None
         if bias:
             b = self.param(self.rng.normal(0, 0.1, (cout, 1, 1)))
+            if name:
+                self.alias[name + ".bias"] = self.nodes[b]["name"]
             bv = self.values[b].reshape(-1)
             roles["bias"] = len(inputs); inputs.append(b); epi.append("bias"); base += "_add"
         rv = None
@@ -97,13 +102,17 @@ class ExportWriter:
         key = (tuple(self.shapes[x]), cout, kh, kw, sh, sw, ph, pw, tuple(epi))
         return self._op(base, key, "conv2d", attrs, epi, roles, inputs, out, temps)
 
-    def dense(self, x, units, bias=True, relu=False):
+    def dense(self, x, units, bias=True, relu=False, name=None):
         feat = self.shapes[x][1]
         w = self.param(self.rng.normal(0, np.sqrt(1.0 / feat), (units, feat)))
         inputs, roles, epi, base = [x, w], {"data": 0, "weight": 1}, [], "nn_dense"
+        if name:
+            self.alias[name + ".weight"] = self.nodes[w]["name"]
         bv = None
         if bias:
             b = self.param(self.rng.normal(0, 0.1, (units,)))
+            if name:
+                self.alias[name + ".bias"] = self.nodes[b]["name"]
             bv = self.values[b]
             roles["bias"] = 2; inputs.append(b); epi.append("bias"); base += "_add"
         if relu:
@@ -229,3 +238,24 @@ def padded_channels(dt, seed=3):
     y = w.pool(y, "global_avg")
     y = w.flatten(y)
     return w, w.dense(y, 5)
+
+
+def resnet(dt, blocks, batch=1, hw=224, seed=4):
+    """ResNet v1 with bottleneck blocks as the built-in "resnet50" / "resnet101" / "resnet152" graphs hold it
+    (batch norm folded into the convolutions, stride on the first 1x1 of a down-sampling block);
+    `alias` maps the built-in graph's parameter names to the export's."""
+    w = ExportWriter(dt, seed)
+    x = w.data(w.rng.normal(0, 1, (batch, 3, hw, hw)))
+    x = w.conv2d(x, 64, 7, 2, 3, name="conv1")
+    x = w.pool(x, "max", 3, 2, 1)
+    for s in range(4):
+        width = 64 << s
+        for b in range(blocks[s]):
+            n = f"layer{s + 1}.{b}"
+            stride = 2 if (b == 0 and s > 0) else 1
+            shortcut = w.conv2d(x, 4 * width, 1, stride, 0, relu=False, name=n + ".downsample") if b == 0 else x
+            y = w.conv2d(x, width, 1, stride, 0, name=n + ".conv1")
+            y = w.conv2d(y, width, 3, 1, 1, name=n + ".conv2")
+            x = w.conv2d(y, 4 * width, 1, residual=shortcut, gain=0.5, name=n + ".conv3")
+    x = w.flatten(w.pool(x, "global_avg"))
+    return w, w.softmax(w.dense(x, 1000, name="fc"))

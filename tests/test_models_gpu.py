@@ -366,3 +366,23 @@ def test_exported_model_preempt_resume_bit_exact(gp, ex_mod, tmp_path, program):
     w.write(str(tmp_path / "mini_resnet"), head)
     x = gp.to_storage(w.value(0), gp.F16)
     _blp_roundtrip(gp, ex_mod, tmp_path, "mini_resnet", x, [(1, 0), (6, 0), (9, 0)], graph=program)
+
+
+def test_exported_resnet50_equals_the_builtin_graph(gp, ex_mod, tmp_path):
+    """A ResNet-50 written as an export maps onto the same kernels as the built-in graph of that name: the
+    same number of launches, and with the same parameters the same bits."""
+    import export_writer as EW
+    w, head = EW.resnet("f16", OM.RESNET_BLOCKS["resnet50"], batch=2, hw=64)
+    want = w.write(str(tmp_path / "exported_resnet"), head)
+    x = gp.to_storage(w.value(0), gp.F16)
+    ex = ex_mod.Executor("exported_resnet", model_root=str(tmp_path))
+    got = run(gp, ex, x, gp.F16, want.shape)
+    assert rel_err(got, want) < TOL["f16"]
+    builtin = "resnet50@b=2,hw=64,dtype=f16"
+    os.makedirs(str(tmp_path / builtin))
+    ex_mod.write_params(str(tmp_path / builtin / "mod.params"), {name: w.params[p] for name, p in w.alias.items()})
+    ref = ex_mod.Executor(builtin, model_root=str(tmp_path))
+    assert set(w.alias) == {s["name"] for s in ref.storages() if s["is_param"]}
+    assert ex.kernel_num() == ref.kernel_num()
+    assert np.array_equal(got, run(gp, ref, x, gp.F16, want.shape))
+    ex.destroy(); ref.destroy()
