@@ -34,6 +34,11 @@ struct Mapper {
     std::string &error;
     std::vector<Val> vals;
     std::map<std::string, const ExportOp *> by_func;
+    // concatenation without a copy: a tensor that a channel concatenation takes as an argument is written
+    // straight into its slice of the concatenation's buffer by the operator that computes it
+    struct Place { size_t into = SIZE_MAX; int off = 0; };
+    std::vector<Place> place;          // per node: the concatenation it lives in, and at which channel
+    std::map<size_t, Tensor> buffers;  // per root node: the buffer made for it, perhaps before its turn
 
     Mapper(GraphBuilder &b_, const TvmExport &e, const ExportOps &o, std::string &err) : b(b_), ex(e), ops(o), error(err) {}
 
@@ -115,11 +120,49 @@ struct Mapper {
                                   std::to_string(v.t.N) + "x" + std::to_string(c) + "x" + std::to_string(v.t.H) + "x" + std::to_string(v.t.W));
         return Status::Succ;
     }
-    Val fresh(const std::string &name, int N, int H, int W, int c_log) {
-        Val v;
+    const ExportOp *op_of(size_t node) const {
+        auto it = by_func.find(ex.nodes[node].func);
+        return it == by_func.end() ? nullptr : it->second;
+    }
+    // Which arguments of which concatenations can be computed in place.  An argument qualifies when one of
+    // the operators that can write a channel slice makes it, it is not already placed (a tensor lives in
+    // one place; a second concatenation of it copies), and its first channel falls on a 16-byte boundary.
+    void plan_concatenations() {
+        place.assign(ex.global_len, Place());
+        for (size_t i = 0; i < ex.global_len; ++i) {
+            const ExportOp *op = op_of(i);
+            if (!op || op->op != "concatenate" || attr(*op, "axis", 0, 1) != 1 || ex.nodes[i].shape.size() != 4) continue;
+            int off = 0;
+            for (size_t j : ex.nodes[i].inputs) {
+                const ExportOp *src = j < i ? op_of(j) : nullptr;
+                if (j >= ex.global_len || ex.nodes[j].shape.size() != 4) break;
+                const bool writes_slices = src && (src->op == "conv2d" || src->op == "max_pool2d" || src->op == "avg_pool2d" || src->op == "add" ||
+                                                   src->op == "scale_shift" || src->op == "concatenate");
+                if (writes_slices && place[j].into == SIZE_MAX && off % b.vec() == 0) { place[j].into = i; place[j].off = off; }
+                off += (int)ex.nodes[j].shape[1];
+            }
+        }
+    }
+    // where node `i` of the given shape is to be written: its slice of a concatenation's buffer, or a
+    // buffer of its own
+    Status out_for(size_t i, int N, int H, int W, int c_log, Val &v) {
+        size_t root = i;
+        int off = 0;
+        while (place[root].into != SIZE_MAX) { off += place[root].off; root = place[root].into; }
+        auto it = buffers.find(root);
+        if (it == buffers.end()) {
+            int rn, rc, rh, rw;
+            if (root == i) { rn = N; rc = c_log; rh = H; rw = W; }
+            else if (!nchw_of(root, rn, rc, rh, rw)) return fail(root, "tensors of 1, 2 or 4 dimensions only");
+            it = buffers.emplace(root, b.activation(ex.nodes[root].name, rn, rh, rw, b.pad_c(rc))).first;
+        }
+        const Tensor &buf = it->second;
+        if (buf.N != N || buf.H != H || buf.W != W || off + b.pad_c(c_log) > buf.C)
+            return fail(i, "the concatenation this result belongs to has another batch or image size");
+        v = Val();
         v.set = true; v.c_log = c_log;
-        v.t = b.activation(name, N, H, W, b.pad_c(c_log));
-        return v;
+        v.t = GraphBuilder::slice(buf, off, b.pad_c(c_log));
+        return Status::Succ;
     }
     Status need_act(size_t user, size_t node, const Val *&v) {
         if (node >= vals.size() || !vals[node].set || vals[node].is_param) return fail(user, "argument '" + ex.nodes[node].name + "' must be a tensor computed earlier in the graph");
@@ -165,7 +208,8 @@ struct Mapper {
             RETURN_STATUS(vector_param(i, bn, O, O, ParamLayout::InitZero, 0.f, 2, bias));
         }
         const Val *res = nullptr;
-        Val out = fresh(ex.nodes[i].name, in->t.N, Ho, Wo, O);
+        Val out;
+        RETURN_STATUS(out_for(i, in->t.N, Ho, Wo, O, out));
         if (has_tail(op, "residual")) {
             if (!input_of(i, op, "residual", 3, rn)) return fail(i, "the epilogue names a residual the function has no argument for");
             RETURN_STATUS(need_act(i, rn, res));
@@ -249,7 +293,8 @@ struct Mapper {
         }
         const int Ho = mode == 2 ? 1 : (in->t.H + 2 * pad - k) / stride + 1, Wo = mode == 2 ? 1 : (in->t.W + 2 * pad - k) / stride + 1;
         if (Ho <= 0 || Wo <= 0) return fail(i, "empty pooling output");
-        Val out = fresh(ex.nodes[i].name, in->t.N, Ho, Wo, in->c_log);
+        Val out;
+        RETURN_STATUS(out_for(i, in->t.N, Ho, Wo, in->c_log, out));
         const double bytes = b.es() * ((double)in->t.N * in->t.H * in->t.W * in->t.C + (double)in->t.N * Ho * Wo * in->t.C);
         KernelInfo &ki = b.add_kernel("pool2d", OpKind::Pool, {b.ref(in->t), b.ref(out.t)}, 0, bytes);
         gp_pool_params &p = ki.p.pool;
@@ -282,7 +327,8 @@ struct Mapper {
         int act;
         RETURN_STATUS(tail_act(i, op, act));
         if (has_tail(op, "bias") || has_tail(op, "residual")) return fail(i, "add takes an activation as its only epilogue step");
-        Val out = fresh(ex.nodes[i].name, a->t.N, a->t.H, a->t.W, a->c_log);
+        Val out;
+        RETURN_STATUS(out_for(i, a->t.N, a->t.H, a->t.W, a->c_log, out));
         out.fc = vals[an].fc; out.fh = vals[an].fh; out.fw = vals[an].fw;
         if (vals[bn].is_param) {  // a per-channel constant
             if (a->fc) return fail(i, "a per-channel constant added to a flattened tensor");
@@ -314,7 +360,8 @@ struct Mapper {
         size_t scale, shift;
         RETURN_STATUS(vector_param(i, sn, a->c_log, a->t.C, ParamLayout::InitConst, 1.f, 4, scale));
         RETURN_STATUS(vector_param(i, hn, a->c_log, a->t.C, ParamLayout::InitZero, 0.f, 2, shift));
-        Val out = fresh(ex.nodes[i].name, a->t.N, a->t.H, a->t.W, a->c_log);
+        Val out;
+        RETURN_STATUS(out_for(i, a->t.N, a->t.H, a->t.W, a->c_log, out));
         emit_eltwise(a->t, nullptr, scale, shift, out.t, act);
         vals[i] = out;
         return Status::Succ;
@@ -354,12 +401,15 @@ struct Mapper {
             total += v->c_log;
         }
         const Val &first = vals[ins[0]];
-        Val out = fresh(ex.nodes[i].name, first.t.N, first.t.H, first.t.W, total);
+        Val out;
+        RETURN_STATUS(out_for(i, first.t.N, first.t.H, first.t.W, total, out));
         int at = 0;
         for (size_t j : ins) {
             const Val &v = vals[j];
             Tensor slice = GraphBuilder::slice(out.t, at, v.t.C);
-            emit_eltwise(v.t, nullptr, SIZE_MAX, SIZE_MAX, slice, GP_ACT_NONE);
+            // an argument that was computed in place is already there
+            const bool in_place = v.t.st == slice.st && v.t.off == slice.off && v.t.ps == slice.ps;
+            if (!in_place) emit_eltwise(v.t, nullptr, SIZE_MAX, SIZE_MAX, slice, GP_ACT_NONE);
             at += v.c_log;
         }
         vals[i] = out;
@@ -400,6 +450,7 @@ struct Mapper {
         for (const ExportOp &o : ops.funcs) by_func[o.func] = &o;
         if (ops.layout != "NCHW") { error = "ops json: only exports in NCHW layout are mapped"; return Status::Fail; }
         vals.assign(ex.global_len, Val());
+        plan_concatenations();
         bool have_data = false;
         for (size_t i = 0; i < ex.global_len; ++i) {
             const ExportNode &n = ex.nodes[i];

@@ -73,7 +73,8 @@ Status check_export_ops(const TvmExport &ex, const ExportOps &ops, std::string &
 // over an NCHW flatten), so that the export's own mod.params loads into them (src/model.cpp:263-282).
 // "data" and "heads" have the export's shapes (NCHW data).  Mapped: conv2d (groups 1, dilation 1,
 // symmetric padding), dense, max / average / global-average pooling, add, scale_shift, softmax over the
-// last axis, concatenate over channels, reshape / __nop between a 4-D tensor and its NCHW flatten.  Anything
+// last axis, concatenate over channels (its arguments are computed in place in its buffer where they can
+// be, copied otherwise), reshape / __nop between a 4-D tensor and its NCHW flatten.  Anything
 // else (the attention and layer-norm functions of a BERT export among them) is Status::Fail with `error`
 // naming the function: nothing is guessed.
 class GraphBuilder;

@@ -143,10 +143,12 @@ class ExportWriter:
         out = self._r(O.scale_shift_act(self.values[x], np.ones(c, np.float32), self.values[p].reshape(-1), O.ACT_RELU if relu else O.ACT_NONE))
         return self._op("add" + ("_nn_relu" if relu else ""), (tuple(self.shapes[x]), relu, "const"), "add", {}, ["relu"] if relu else [], {"lhs": 0, "rhs": 1}, [x, p], out)
 
-    def scale_shift(self, x, relu=True):
+    def scale_shift(self, x, relu=True, name=None):
         c = self.shapes[x][1]
         s = self.param(self.rng.uniform(0.5, 1.5, (c, 1, 1)))
         h = self.param(self.rng.normal(0, 0.2, (c, 1, 1)))
+        if name:
+            self.alias[name + ".scale"], self.alias[name + ".shift"] = self.nodes[s]["name"], self.nodes[h]["name"]
         out = self._r(O.scale_shift_act(self.values[x], self.values[s].reshape(-1), self.values[h].reshape(-1), O.ACT_RELU if relu else O.ACT_NONE))
         return self._op("multiply_add" + ("_nn_relu" if relu else ""), (tuple(self.shapes[x]), relu), "scale_shift", {}, ["relu"] if relu else [],
                         {"data": 0, "scale": 1, "shift": 2}, [x, s, h], out)
@@ -259,3 +261,36 @@ def resnet(dt, blocks, batch=1, hw=224, seed=4):
             x = w.conv2d(y, 4 * width, 1, residual=shortcut, gain=0.5, name=n + ".conv3")
     x = w.flatten(w.pool(x, "global_avg"))
     return w, w.softmax(w.dense(x, 1000, name="fc"))
+
+
+def densenet(dt, layers=(2, 2, 2, 2), growth=8, init=16, batch=2, hw=32, classes=10, seed=5):
+    """DenseNet as the built-in "densenet" graph holds it: norm-ReLU in front of every convolution inside
+    the blocks, each layer's new channels concatenated behind everything before them."""
+    w = ExportWriter(dt, seed)
+    x = w.data(w.rng.normal(0, 1, (batch, 3, hw, hw)))
+    x = w.pool(w.conv2d(x, init, 7, 2, 3, name="conv0"), "max", 3, 2, 1)
+    for b, n_layers in enumerate(layers):
+        for l in range(n_layers):
+            n = f"block{b + 1}.layer{l + 1}"
+            t = w.scale_shift(x, name=n + ".norm1")
+            t = w.conv2d(t, 4 * growth, 1, name=n + ".conv1")
+            x = w.concatenate([x, w.conv2d(t, growth, 3, 1, 1, relu=False, name=n + ".conv2")])
+        if b + 1 < len(layers):
+            n = f"transition{b + 1}"
+            t = w.conv2d(w.scale_shift(x, name=n + ".norm"), w.shapes[x][1] // 2, 1, relu=False, name=n + ".conv")
+            x = w.pool(t, "avg", 2, 2, 0)
+    x = w.flatten(w.pool(w.scale_shift(x, name="norm5"), "global_avg"))
+    return w, w.softmax(w.dense(x, classes, name="classifier"))
+
+
+def shared_concat(dt, seed=6):
+    """one tensor in two concatenations: it is computed in place for the first and copied for the second;
+    an inception-style block whose four branches all land in place"""
+    w = ExportWriter(dt, seed)
+    x = w.data(w.rng.normal(0, 1, (1, 3, 8, 8)))
+    a = w.conv2d(x, 8, 3, 1, 1)
+    b = w.conv2d(x, 16, 1)
+    y = w.add(w.concatenate([a, b]), w.concatenate([b, a]))
+    y = w.concatenate([w.conv2d(y, 8, 1), w.conv2d(y, 8, 3, 1, 1), w.pool(y, "max", 3, 1, 1), w.pool(y, "avg", 3, 1, 1)])
+    y = w.flatten(w.pool(y, "global_avg"))
+    return w, w.dense(y, 6)

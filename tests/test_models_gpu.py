@@ -320,7 +320,7 @@ def test_exported_graph_next_to_the_model_is_read_and_checked(gp, ex_mod, tmp_pa
 # output with the oracle's operators while it writes.
 
 @pytest.mark.parametrize("dt", ["f32", "f16"])
-@pytest.mark.parametrize("maker", ["mini_resnet", "mini_vgg", "padded_channels"])
+@pytest.mark.parametrize("maker", ["mini_resnet", "mini_vgg", "padded_channels", "shared_concat", "densenet"])
 def test_exported_model_matches_oracle(gp, ex_mod, tmp_path, maker, dt):
     import export_writer as EW
     w, head = getattr(EW, maker)(dt)
@@ -384,5 +384,25 @@ def test_exported_resnet50_equals_the_builtin_graph(gp, ex_mod, tmp_path):
     ref = ex_mod.Executor(builtin, model_root=str(tmp_path))
     assert set(w.alias) == {s["name"] for s in ref.storages() if s["is_param"]}
     assert ex.kernel_num() == ref.kernel_num()
+    assert np.array_equal(got, run(gp, ref, x, gp.F16, want.shape))
+    ex.destroy(); ref.destroy()
+
+
+def test_exported_densenet_equals_the_builtin_graph(gp, ex_mod, tmp_path):
+    """The growing concatenations of a DenseNet export cost no copies: every layer writes its new channels
+    into the block's buffer, which is the built-in graph's layout; same launches, same bits."""
+    import export_writer as EW
+    w, head = EW.densenet("f16", layers=(2, 4, 2, 2), growth=16, init=32, batch=2, hw=64, classes=24)
+    want = w.write(str(tmp_path / "exported_densenet"), head)
+    x = gp.to_storage(w.value(0), gp.F16)
+    ex = ex_mod.Executor("exported_densenet", model_root=str(tmp_path))
+    got = run(gp, ex, x, gp.F16, want.shape)
+    assert rel_err(got, want) < TOL["f16"]
+    builtin = "densenet@b=2,hw=64,l1=2,l2=4,l3=2,l4=2,growth=16,init=32,classes=24,dtype=f16"
+    os.makedirs(str(tmp_path / builtin))
+    ex_mod.write_params(str(tmp_path / builtin / "mod.params"), {name: w.params[p] for name, p in w.alias.items()})
+    ref = ex_mod.Executor(builtin, model_root=str(tmp_path))
+    assert set(w.alias) == {s["name"] for s in ref.storages() if s["is_param"]}
+    assert [k["name"] for k in ex.kernels()] == [k["name"] for k in ref.kernels()]
     assert np.array_equal(got, run(gp, ref, x, gp.F16, want.shape))
     ex.destroy(); ref.destroy()

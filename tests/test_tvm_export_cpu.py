@@ -166,8 +166,11 @@ def test_generated_exports_map_operator_by_operator(tmp_path):
     rc, rep = plan(d)
     assert rc == 0, rep
     names = [k["name"] for k in rep["kernels"]]
-    # layout, 9 convolutions, 4 pools, concat = 2 copies, scale-shift, add, classifier, softmax
-    assert names.count("conv2d") == 9 and names.count("pool2d") == 4 and names.count("eltwise") == 4
+    # layout, 9 convolutions, 4 pools, scale-shift, add, classifier, softmax; the concatenation costs nothing:
+    # both of its arguments are written into their slices of its buffer by the convolutions that make them
+    assert names.count("conv2d") == 9 and names.count("pool2d") == 4 and names.count("eltwise") == 2
+    cat = [k["params"] for k in rep["kernels"] if k["name"] == "conv2d" and k["params"]["out_pix_stride"] == 48]
+    assert [c["Cout"] for c in cat] == [32, 16]
     assert names[0] == "nchw_to_nhwc" and names[-2:] == ["dense", "softmax"]
     stem = rep["kernels"][1]["params"]
     assert (stem["R"], stem["stride_h"], stem["pad_h"], stem["Cout"], stem["act"]) == (7, 2, 3, 16, 1)
@@ -185,9 +188,25 @@ def test_generated_exports_map_operator_by_operator(tmp_path):
     rc, rep = plan(d)
     assert rc == 0, rep
     convs = [k["params"] for k in rep["kernels"] if k["name"] == "conv2d"]
-    assert [(c["Cin"], c["Cout"], c["out_pix_stride"]) for c in convs] == [(8, 16, 16), (16, 12, 16), (16, 20, 24), (16, 16, 16), (40, 24, 24)]
-    copies = [k["params"] for k in rep["kernels"] if k["name"] == "eltwise"]
-    assert [(c["cols"], c["out_stride"]) for c in copies] == [(16, 40), (24, 40)]
+    assert [(c["Cin"], c["Cout"], c["out_pix_stride"]) for c in convs] == [(8, 16, 16), (16, 12, 16), (16, 20, 40), (16, 16, 16), (40, 24, 24)]
+    assert not [k for k in rep["kernels"] if k["name"] == "eltwise"]
+    # a tensor lives in one place: the second concatenation of the same two tensors copies them
+    w, head = EW.shared_concat("f16")
+    d = str(tmp_path / "s")
+    w.write(d, head)
+    rc, rep = plan(d)
+    assert rc == 0, rep
+    copies = [k for k in rep["kernels"] if k["name"] == "eltwise" and k["args"][1] == ""]
+    assert [(c["params"]["cols"], c["params"]["out_stride"]) for c in copies] == [(16, 24), (8, 24)]
+    assert len([k for k in rep["kernels"] if k["name"] == "eltwise"]) == 3   # the two copies and the add
+    # a DenseNet's growing concatenations: no copies at all, as in the built-in graph
+    w, head = EW.densenet("f16")
+    d = str(tmp_path / "d")
+    w.write(d, head)
+    rc, rep = plan(d)
+    assert rc == 0, rep
+    names = [k["name"] for k in rep["kernels"]]
+    assert names.count("eltwise") == 8 + 3 + 1 and names.count("conv2d") == 1 + 16 + 3   # the norms; stem, two per layer, transitions
 
 
 def test_what_cannot_be_mapped_is_refused_by_name(tmp_path):
