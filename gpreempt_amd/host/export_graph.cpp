@@ -129,6 +129,14 @@ struct Mapper {
     // one place; a second concatenation of it copies), and its first channel falls on a 16-byte boundary.
     void plan_concatenations() {
         place.assign(ex.global_len, Place());
+        // a tensor that is also flattened, soft-maxed or the model's output must lie in plain memory
+        std::vector<char> plain(ex.global_len, 0);
+        plain[ex.heads_index] = 1;
+        for (size_t i = 0; i < ex.global_len; ++i) {
+            const ExportOp *op = op_of(i);
+            if (ex.nodes[i].func == "__nop" || (op && (op->op == "reshape" || op->op == "softmax")))
+                for (size_t j : ex.nodes[i].inputs) if (j < ex.global_len) plain[j] = 1;
+        }
         for (size_t i = 0; i < ex.global_len; ++i) {
             const ExportOp *op = op_of(i);
             if (!op || op->op != "concatenate" || attr(*op, "axis", 0, 1) != 1 || ex.nodes[i].shape.size() != 4) continue;
@@ -136,9 +144,9 @@ struct Mapper {
             for (size_t j : ex.nodes[i].inputs) {
                 const ExportOp *src = j < i ? op_of(j) : nullptr;
                 if (j >= ex.global_len || ex.nodes[j].shape.size() != 4) break;
-                const bool writes_slices = src && (src->op == "conv2d" || src->op == "max_pool2d" || src->op == "avg_pool2d" || src->op == "add" ||
+                const bool writes_slices = src && (src->op == "conv2d" || src->op == "max_pool2d" || src->op == "avg_pool2d" || src->op == "global_avg_pool2d" || src->op == "add" ||
                                                    src->op == "scale_shift" || src->op == "concatenate");
-                if (writes_slices && place[j].into == SIZE_MAX && off % b.vec() == 0) { place[j].into = i; place[j].off = off; }
+                if (writes_slices && !plain[j] && place[j].into == SIZE_MAX && off % b.vec() == 0) { place[j].into = i; place[j].off = off; }
                 off += (int)ex.nodes[j].shape[1];
             }
         }

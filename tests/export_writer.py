@@ -292,5 +292,8 @@ def shared_concat(dt, seed=6):
     b = w.conv2d(x, 16, 1)
     y = w.add(w.concatenate([a, b]), w.concatenate([b, a]))
     y = w.concatenate([w.conv2d(y, 8, 1), w.conv2d(y, 8, 3, 1, 1), w.pool(y, "max", 3, 1, 1), w.pool(y, "avg", 3, 1, 1)])
-    y = w.flatten(w.pool(y, "global_avg"))
+    # a tensor that is both concatenated and flattened stays in plain memory (the concatenation copies it)
+    p = w.pool(y, "global_avg")
+    q = w.pool(w.conv2d(y, 8, 1), "global_avg")
+    y = w.add(w.dense(w.flatten(w.concatenate([p, q])), 8, bias=False), w.dense(w.flatten(q), 8))
     return w, w.dense(y, 6)
