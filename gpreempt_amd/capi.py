@@ -37,7 +37,8 @@ class GemmParams(C.Structure):
                 ("C", vp), ("ldc", C.c_long), ("stride_c", C.c_long),
                 ("bias", vp), ("residual", vp), ("alpha", C.c_float), ("act", C.c_int), ("batch", C.c_int),
                 ("batch_inner", C.c_int), ("stride_a_outer", C.c_long), ("stride_b_outer", C.c_long),
-                ("stride_c_outer", C.c_long), ("tile_m", C.c_int), ("tile_n", C.c_int), ("variant", C.c_int)]
+                ("stride_c_outer", C.c_long), ("tile_m", C.c_int), ("tile_n", C.c_int), ("variant", C.c_int),
+                ("ln_gamma", vp), ("ln_beta", vp), ("ln_out", vp), ("ln_eps", C.c_float)]
 
 
 class ConvParams(C.Structure):
@@ -99,7 +100,7 @@ SYMBOLS = """gp_init gp_last_error gp_device_info gp_stream_create gp_stream_des
 gp_stream_query gp_stream_priority gp_stream_set_priority gp_stream_native gp_event_create gp_event_destroy gp_event_record
 gp_event_sync gp_event_query gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free gp_memcpy_h2d gp_memcpy_d2h
 gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_flag_relay_start
-gp_launch_gemm gp_launch_gemm_noalloc gp_gemm_ckpt_bytes gp_conv_ckpt_bytes gp_ckpt_reset_async gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
+gp_launch_gemm gp_gemm_ln_supported gp_launch_gemm_noalloc gp_gemm_ckpt_bytes gp_conv_ckpt_bytes gp_ckpt_reset_async gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
 gp_launch_layernorm gp_launch_attention gp_launch_miniweather gp_launch_graph gp_launch_embed gp_launch_gate gp_launch_noop gp_graph_begin gp_graph_end gp_graph_launch
 gp_graph_destroy gp_program_create gp_program_destroy gp_program_add_gemm gp_program_add_conv2d
 gp_program_add_nchw_to_nhwc gp_program_add_pool2d gp_program_add_eltwise gp_program_add_softmax gp_program_add_layernorm

@@ -561,6 +561,91 @@ __global__ __launch_bounds__(NT) void softmax_kernel(gp_softmax_params p, BlpArg
 // ---- layer norm ----------------------------------------------------------------------------
 // one wavefront per RPW rows, 4 * RPW rows per tile; the rows (plus residual) are kept in registers
 // (up to MAXC 16-byte chunks per lane and row), so HBM sees one read and one write per element.
+// R rows, each held by one wavefront as 16-byte chunks lane, lane + 64, ...: mean, variance and the
+// normalised, packed rows.  The rows go through every step side by side, so that the cross-lane
+// reductions of one row hide behind those of the others; a row's own arithmetic is the same whatever R
+// is, and every kernel that normalises rows goes through this function, so that a row gets the same
+// bits wherever it is computed.
+// Sum over the 64 lanes, every lane getting the total.  The first four steps (partners 1, 2, 4 and 8 lanes
+// apart, inside a row of 16) are DPP moves, which run in the vector ALU; only the last two cross rows
+// and go through the LDS crossbar.  (Six crossbar shuffles per sum, from the sixteen wavefronts of a
+// workgroup that all normalise rows, made the layer-norm prologue of gemm_ln.hpp wait for the LDS pipe.)
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int R>
+__device__ __forceinline__ void wave_sum_rows(float (&s)[R]) {
+    // quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror: after each step the lanes of a
+    // group of 2, 4, 8, 16 hold the group's sum (a mirror pairs lane i with lane 7 - i or 15 - i, whose
+    // groups differ in the bit that the step adds)
+#pragma unroll
+    for (int q = 0; q < R; ++q) s[q] += dpp_mov<0xB1>(s[q]);
+#pragma unroll
+    for (int q = 0; q < R; ++q) s[q] += dpp_mov<0x4E>(s[q]);
+#pragma unroll
+    for (int q = 0; q < R; ++q) s[q] += dpp_mov<0x141>(s[q]);
+#pragma unroll
+    for (int q = 0; q < R; ++q) s[q] += dpp_mov<0x140>(s[q]);
+#pragma unroll
+    for (int o = 16; o <= 32; o <<= 1) {
+        float t[R];
+#pragma unroll
+        for (int q = 0; q < R; ++q) t[q] = __shfl_xor(s[q], o, 64);
+#pragma unroll
+        for (int q = 0; q < R; ++q) s[q] += t[q];
+    }
+}
+template <typename T, int MAXC, int R>
+__device__ __forceinline__ void ln_rows_math(const float (&v)[R][MAXC][VecIO<T>::VEC], int chunks, int lane, int cols, float eps,
+                                             const T *gamma, const T *beta, out_u32x4 (&y)[R][MAXC]) {
+    constexpr int VEC = VecIO<T>::VEC;
+    float sum[R], mean[R], sq[R], inv[R];
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+        sum[q] = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            const int ch = lane + i * 64;
+            if (ch < chunks) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) sum[q] += v[q][i][j];
+            }
+        }
+    }
+    wave_sum_rows<R>(sum);
+#pragma unroll
+    for (int q = 0; q < R; ++q) {
+        mean[q] = sum[q] / (float)cols;
+        sq[q] = 0.f;
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            const int ch = lane + i * 64;
+            if (ch < chunks) {
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) { float d = v[q][i][j] - mean[q]; sq[q] += d * d; }
+            }
+        }
+    }
+    wave_sum_rows<R>(sq);
+#pragma unroll
+    for (int q = 0; q < R; ++q) inv[q] = rsqrtf(sq[q] / (float)cols + eps);
+#pragma unroll
+    for (int i = 0; i < MAXC; ++i) {
+        const int ch = lane + i * 64;
+        if (ch < chunks) {
+            float ga[VEC], be[VEC];
+            VecIO<T>::load(gamma + ch * VEC, ga);
+            VecIO<T>::load(beta + ch * VEC, be);
+#pragma unroll
+            for (int q = 0; q < R; ++q) {
+                float o[VEC];
+#pragma unroll
+                for (int j = 0; j < VEC; ++j) o[j] = (v[q][i][j] - mean[q]) * inv[q] * ga[j] + be[j];
+                y[q][i] = VecIO<T>::pack(o);
+            }
+        }
+    }
+}
 // All loads of the wavefront's rows are issued before the first reduction.
 constexpr int kLnTwoRows = 0x100;  // flag in the plan's `sub`: RPW = 2
 template <typename T, int MAXC, int RPW, bool NTH>
@@ -589,49 +674,33 @@ __device__ __forceinline__ void layernorm_rows(const gp_layernorm_params &p, Til
             }
         }
     }
+    float v[RPW][MAXC][VEC];
 #pragma unroll
     for (int q = 0; q < RPW; ++q) {
-        float v[MAXC][VEC];
-        float sum = 0.f;
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
             const int ch = lane + i * 64;
             if (ch < chunks) {
-                VecIO<T>::unpack(rx[q][i], v[i]);
+                VecIO<T>::unpack(rx[q][i], v[q][i]);
                 if (p.residual) {
                     float r[VEC];
                     VecIO<T>::unpack(rr[q][i], r);
 #pragma unroll
-                    for (int j = 0; j < VEC; ++j) v[i][j] += r[j];
+                    for (int j = 0; j < VEC; ++j) v[q][i][j] += r[j];
                 }
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) sum += v[i][j];
             }
         }
-        const float mean = wave_sum(sum) / (float)p.cols;
-        float sq = 0.f;
+    }
+    out_u32x4 y[RPW][MAXC];
+    ln_rows_math<T, MAXC, RPW>(v, chunks, lane, p.cols, p.eps, (const T *)p.gamma, (const T *)p.beta, y);
 #pragma unroll
-        for (int i = 0; i < MAXC; ++i) {
-            const int ch = lane + i * 64;
-            if (ch < chunks) {
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) { float d = v[i][j] - mean; sq += d * d; }
-            }
-        }
-        const float inv = rsqrtf(wave_sum(sq) / (float)p.cols + p.eps);
+    for (int q = 0; q < RPW; ++q) {
         if (row0 + q >= p.rows) break;
         T *o = (T *)p.out + (row0 + q) * p.cols;
 #pragma unroll
         for (int i = 0; i < MAXC; ++i) {
             const int ch = lane + i * 64;
-            if (ch < chunks) {
-                float ga[VEC], be[VEC], y[VEC];
-                VecIO<T>::load((const T *)p.gamma + ch * VEC, ga);
-                VecIO<T>::load((const T *)p.beta + ch * VEC, be);
-#pragma unroll
-                for (int j = 0; j < VEC; ++j) y[j] = (v[i][j] - mean) * inv * ga[j] + be[j];
-                st_raw128<NTH>(o + ch * VEC, VecIO<T>::pack(y));
-            }
+            if (ch < chunks) st_raw128<NTH>(o + ch * VEC, y[q][i]);
         }
     }
 }

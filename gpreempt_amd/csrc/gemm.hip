@@ -17,6 +17,7 @@
 #include "gemm_tile.hpp"
 #include "gemm_pipe.hpp"
 #include "gemm_wide.hpp"
+#include "gemm_ln.hpp"
 #include "plans.hpp"
 
 namespace gp {
@@ -144,6 +145,9 @@ static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream 
         case MB_WIDE32x32_8: return wide_case<T, 32, 32, 8>(pl, ctx, s, info);
         case MB_WIDE64x32_16: return wide_case<T, 64, 32, 16>(pl, ctx, s, info);
         case MB_WIDE64x64_8: return wide_case<T, 64, 64, 8>(pl, ctx, s, info);
+        case MB_LNWIDE32x64_16:
+            if constexpr (sizeof(T) == 2) return launch_mat<LnWideKernel<T, 32, 64, 16, 3>>(pl, ctx, s, info);
+            break;
         case MB_STAGED128:
             if (pl.conv) return launch_mat<TK<T, 128, 128, SBK, 2, 2, true, false>>(pl, ctx, s, info);
             return pl.b_kn ? launch_mat<TK<T, 128, 128, SBK, 2, 2, false, true>>(pl, ctx, s, info)
@@ -179,6 +183,7 @@ static size_t body_lds_bytes(int body, int dtype) {
         case MB_WIDE32x32_8: return WideKernel<_Float16, 32, 32, 8, 3>::LDS_BYTES;
         case MB_WIDE64x32_16: return WideKernel<_Float16, 64, 32, 16, 3>::LDS_BYTES;
         case MB_WIDE64x64_8: return WideKernel<_Float16, 64, 64, 8, 3>::LDS_BYTES;
+        case MB_LNWIDE32x64_16: return LnWideKernel<_Float16, 32, 64, 16, 3>::LDS_BYTES;
         case MB_STAGED128: return (128 + 128) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
         case MB_STAGED64: return (64 + 64) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
     }
@@ -222,7 +227,8 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
     const int wide_bk = pl->dtype == GP_F32 ? 32 : 64;
     const bool wide_ok = !pl->b_kn && (!pl->conv || (g.Cin % wide_bk == 0 && g.K / g.Cin <= 32 && g.S < 32));
     int body = -1;
-    if (pl->b_kn || variant == GP_MAT_STAGED) {
+    if (g.ln_gamma) body = MB_LNWIDE32x64_16;  // (plan_gemm has checked that the shape fits)
+    else if (pl->b_kn || variant == GP_MAT_STAGED) {
         int tm = tile ? tile : (tiles(128) >= cus ? 128 : 64);
         body = tm == 128 ? MB_STAGED128 : tm == 64 ? MB_STAGED64 : -1;
     } else if (variant == GP_MAT_PIPE) {
@@ -256,6 +262,7 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
     int t = body == MB_PIPE256 ? 256 : (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
     int tn = t;
     if (const WideChoice *w = wide_of(body)) { t = w->bm; tn = w->bn; }
+    if (body == MB_LNWIDE32x64_16) { t = 32; tn = 64; }
     pl->body = body;
     pl->sx = (g.N + tn - 1) / tn;
     pl->sy = (g.M + t - 1) / t;
@@ -276,6 +283,28 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
 }
 
 static bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+// shapes the layer-norm prologue body takes (the tile count bounds how often a row is re-normalised)
+static bool ln_shape_ok(const gp_gemm_params *p) {
+    if (!p || (p->dtype != GP_F16 && p->dtype != GP_BF16) || p->batch > 1 || !p->b_is_nk) return false;
+    if (p->M <= 0 || p->N <= 0 || p->K <= 0 || p->lda != p->K || p->K % 64 != 0 || p->K > LnWideKernel<_Float16, 32, 64, 16, 3>::MAXK) return false;
+    // one round of workgroups: every workgroup normalises its own 32 rows, which pays while that hides
+    // behind the fetch of B and not when a compute unit does it twice
+    const long tiles = (long)((p->M + 31) / 32) * ((p->N + 63) / 64);
+    return tiles <= device_cus();
+}
+int plan_gemm(const gp_gemm_params *p, MatPlan *out);
+// ... and the body the launcher would pick for the plain GEMM sums K in the prologue body's order (K-steps
+// dealt to four wavefronts, partial tiles added in wavefront order), so that fusing changes no bit
+extern "C" int gp_gemm_ln_supported(const gp_gemm_params *p) {
+    if (!ln_shape_ok(p)) return 0;
+    gp_gemm_params q = *p;
+    q.ln_gamma = q.ln_beta = nullptr; q.ln_out = nullptr;
+    q.tile_m = q.tile_n = q.variant = 0;
+    MatPlan pl;
+    if (!q.A || !q.B || !q.C || plan_gemm(&q, &pl) != GP_SUCC) return 0;
+    return (is_wide_body(pl.body) || pl.body == MB_PIPE64_SK || pl.body == MB_PIPE32_SK) ? 1 : 0;
+}
 
 int plan_gemm(const gp_gemm_params *p, MatPlan *out) {
     GP_REQUIRE(p != nullptr, "null gemm params");
@@ -305,6 +334,12 @@ int plan_gemm(const gp_gemm_params *p, MatPlan *out) {
     g.alpha = p->alpha == 0.f ? 1.f : p->alpha;
     g.act = p->act; g.batch_inner = batch > 1 ? p->batch_inner : 0;
     pl.dtype = p->dtype; pl.conv = 0; pl.b_kn = !p->b_is_nk; pl.batch = batch;
+    if (p->ln_gamma) {
+        GP_REQUIRE(ln_shape_ok(p), "gemm: no layer-norm prologue for this shape (16-bit, batch 1, B as N x K, lda == K, K a multiple of 64 up to %d)", LnWideKernel<_Float16, 32, 64, 16, 3>::MAXK);
+        GP_REQUIRE(p->ln_beta && p->ln_out, "gemm: the layer-norm prologue needs gamma, beta and ln_out");
+        GP_REQUIRE(aligned16(p->ln_gamma) && aligned16(p->ln_beta) && aligned16(p->ln_out), "gemm: ln_gamma, ln_beta and ln_out must be 16-byte aligned");
+        g.ln_gamma = p->ln_gamma; g.ln_beta = p->ln_beta; g.ln_out = p->ln_out; g.ln_eps = p->ln_eps;
+    }
     return choose_body(&pl, p->tile_m, p->tile_n, p->variant);
 }
 

@@ -35,6 +35,100 @@
 
 namespace gp {
 
+// 1: ask for all STAGES buffers of the ring before the main loop instead of STAGES - 1 (every buffer is free
+// at the start of a tile).  Measured, launch to launch: 128 x 768 x 3072 8.04 -> 7.80 us, but 128 x 2304 x 768
+// 5.74 -> 5.85 and 128 x 768 x 768 4.84 -> 4.90: off.
+#ifndef GP_WIDE_PREFILL
+#define GP_WIDE_PREFILL 0
+#endif
+// waits until at most `stages` stages of LPW loads each are still in flight (stages = 0..3)
+template <int LPW> __device__ __forceinline__ void wait_stages(int stages) {
+    if (stages >= 3) wait_vmcnt<3 * LPW>();
+    else if (stages == 2) wait_vmcnt<2 * LPW>();
+    else if (stages == 1) wait_vmcnt<LPW>();
+    else wait_vmcnt<0>();
+}
+
+// The end of a tile of the wide bodies: the partial tiles of wavefronts 0..3 are summed through LDS in
+// wavefront order and the epilogue (alpha, bias, residual, activation) is applied on the way out.
+template <typename T, int BM, int BN, int NT>
+__device__ __forceinline__ void wide_reduce_store(const MatArgs &g, float *red, const f32x16 (&acc)[BM / 32][BN / 32], int m0, int n0, long offc,
+                                                  int tid, int wave, int lane, int kb) {
+    constexpr int MI = BM / 32, NI = BN / 32, SLICES = MI * NI * 16;
+    // ---- reduction and epilogue -------------------------------------------------------------
+    // partial tiles of wavefronts 0..3 -> LDS as [wavefront][slice][lane], slice = (i*NI + j)*16 + v,
+    // which is row 8*(v/4) + 4*(lane/32) + v%4, column 32*j + lane%32 of 32 x 32 block (i, j).
+    // The first BM*BN/4 threads then finish four consecutive columns of one row each, adding the
+    // partials in wavefront order.
+    T *C = (T *)g.C + offc;
+    const T *R = g.residual ? (const T *)g.residual + offc : nullptr;
+    const T *bias = (const T *)g.bias;
+    const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
+                        (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
+    __syncthreads();  // all wavefronts are done reading the stage buffers
+    if (kb == 0) {
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+    }
+    __syncthreads();
+    GP_PROBE(4);
+    constexpr int L4 = BN / 4;                        // threads per output row
+    constexpr int FIN = BM * L4 < NT ? BM * L4 : NT;  // threads that finish
+    constexpr int RPP = FIN / L4, PASSES = BM / RPP;
+    if (tid < FIN) {
+        const int c4 = tid % L4, r_in = tid / L4;
+        const int j = c4 >> 3, col = (c4 & 7) * 4;
+        const int n = n0 + j * 32 + col;
+        float bq[4] = {0.f, 0.f, 0.f, 0.f};
+        if (bias && n < g.N) {
+            if (vec_ok) {
+                const Vec4<T> b = *(const Vec4<T> *)(bias + n);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) bq[q] = Elem<T>::to_f(b.v[q]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (n + q < g.N) bq[q] = Elem<T>::to_f(bias[n + q]);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const int row = p * RPP + r_in, m = m0 + row;
+            const int i = row >> 5, r = row & 31;
+            const int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
+            const size_t o = ((size_t)(i * NI + j) * 16 + v) * 64 + hf * 32 + col;
+            f32x4 a = *(const f32x4 *)(red + o);
+#pragma unroll
+            for (int w = 1; w < 4; ++w) a += *(const f32x4 *)(red + (size_t)w * SLICES * 64 + o);
+            if (m >= g.M || n >= g.N) continue;
+            if (vec_ok) {
+                Vec4<T> rv;
+                if (R) rv = *(const Vec4<T> *)(R + (long)m * g.ldr + n);
+                Vec4<T> out;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    float x = a[q] * g.alpha + bq[q];
+                    if (R) x += Elem<T>::to_f(rv.v[q]);
+                    out.v[q] = Elem<T>::from_f(apply_act(x, g.act));
+                }
+                st_vec4<T>(&C[(long)m * g.ldc + n], out);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (n + q >= g.N) break;
+                    float x = a[q] * g.alpha + bq[q];
+                    if (R) x += Elem<T>::to_f(R[(long)m * g.ldr + n + q]);
+                    st_elem<T>(&C[(long)m * g.ldc + n + q], Elem<T>::from_f(apply_act(x, g.act)));
+                }
+            }
+        }
+    }
+}
+
 template <typename T, int BM, int BN, int WAVES, int STAGES, bool CONV = false>
 struct WideKernel {
     using elem = T;
@@ -56,11 +150,12 @@ struct WideKernel {
     static constexpr size_t CKPT_SLOT_BYTES = 0;
     static constexpr bool ckpt = false;
     static constexpr bool early_stop = true;  // as PipeKernel::run: a second look at the stop index when the first stage has landed
+    static constexpr int PRE = GP_WIDE_PREFILL ? STAGES : STAGES - 1;  // stages asked for before the main loop
     static_assert(WAVES % 4 == 0 && WAVES >= 4 && WAVES <= 16, "4, 8, 12 or 16 wavefronts");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && GROUPS % 4 == 0, "tile shape");
     // slot j of wavefront wv (of its block group): row group wv*LPW_A + j of A, or wv*LPW_B + (j - LPW_A) of B
     static __device__ __forceinline__ constexpr int group_of(int wv, int j) { return j < LPW_A ? wv * LPW_A + j : BM / 8 + wv * LPW_B + (j - LPW_A); }
-    static_assert(STAGES >= 2 && (STAGES - 2) * LPW < 64, "pipeline depth");
+    static_assert(STAGES >= 2 && STAGES <= 4 && (STAGES - 1) * LPW < 64, "pipeline depth");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 
     // Returns true when the early look found a stop recorded: the tile was not run.
@@ -180,13 +275,14 @@ struct WideKernel {
         GP_PROBE(1);
         __syncthreads();  // the previous tile of this workgroup may still be reading LDS
 #pragma unroll
-        for (int s = 0; s < STAGES - 1; ++s) {
+        for (int s = 0; s < PRE; ++s) {
             if (s < NS) issue(s);
             if (s == 0 && early && wave == 0) load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
         }
         for (int s = 0; s < NS; ++s) {
             // stage s has landed once at most the loads of the younger stages in flight remain
-            if (s + STAGES - 2 < NS) wait_vmcnt<(STAGES - 2) * LPW>();
+            if (s == 0) wait_stages<LPW>((NS < PRE ? NS : PRE) - 1);
+            else if (s + STAGES - 2 < NS) wait_vmcnt<(STAGES - 2) * LPW>();
             else wait_vmcnt<0>();
             __syncthreads();  // everyone's part of stage s is visible; the buffer of stage s-1 is free
             if (s == 0) GP_PROBE(2);
@@ -194,7 +290,7 @@ struct WideKernel {
                 wait_vmcnt<0>();  // loads still landing in LDS must not outlive the workgroup
                 return true;
             }
-            if (s + STAGES - 1 < NS) issue(s + STAGES - 1);
+            if (s >= PRE - (STAGES - 1) && s + STAGES - 1 < NS) issue(s + STAGES - 1);
             if (kb != 0) continue;  // (uniform) wavefronts 4.. only fetch
             const int stage = s % STAGES;
 #pragma unroll
@@ -214,80 +310,8 @@ struct WideKernel {
             }
         }
 
-        // ---- reduction and epilogue -------------------------------------------------------------
-        // partial tiles of wavefronts 0..3 -> LDS as [wavefront][slice][lane], slice = (i*NI + j)*16 + v,
-        // which is row 8*(v/4) + 4*(lane/32) + v%4, column 32*j + lane%32 of 32 x 32 block (i, j).
-        // The first BM*BN/4 threads then finish four consecutive columns of one row each, adding the
-        // partials in wavefront order.
         GP_PROBE(3);
-        float *red = (float *)lds_t;
-        T *C = (T *)g.C + offc;
-        const T *R = g.residual ? (const T *)g.residual + offc : nullptr;
-        const T *bias = (const T *)g.bias;
-        const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
-                            (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
-        __syncthreads();  // all wavefronts are done reading the stage buffers
-        if (kb == 0) {
-#pragma unroll
-            for (int i = 0; i < MI; ++i)
-#pragma unroll
-                for (int j = 0; j < NI; ++j)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + j) * 16 + v) * 64 + lane] = acc[i][j][v];
-        }
-        __syncthreads();
-        GP_PROBE(4);
-        constexpr int L4 = BN / 4;                        // threads per output row
-        constexpr int FIN = BM * L4 < NT ? BM * L4 : NT;  // threads that finish
-        constexpr int RPP = FIN / L4, PASSES = BM / RPP;
-        if (tid < FIN) {
-            const int c4 = tid % L4, r_in = tid / L4;
-            const int j = c4 >> 3, col = (c4 & 7) * 4;
-            const int n = n0 + j * 32 + col;
-            float bq[4] = {0.f, 0.f, 0.f, 0.f};
-            if (bias && n < g.N) {
-                if (vec_ok) {
-                    const Vec4<T> b = *(const Vec4<T> *)(bias + n);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) bq[q] = Elem<T>::to_f(b.v[q]);
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q)
-                        if (n + q < g.N) bq[q] = Elem<T>::to_f(bias[n + q]);
-                }
-            }
-#pragma unroll
-            for (int p = 0; p < PASSES; ++p) {
-                const int row = p * RPP + r_in, m = m0 + row;
-                const int i = row >> 5, r = row & 31;
-                const int v = 4 * (r >> 3) + (r & 3), hf = (r >> 2) & 1;
-                const size_t o = ((size_t)(i * NI + j) * 16 + v) * 64 + hf * 32 + col;
-                f32x4 a = *(const f32x4 *)(red + o);
-#pragma unroll
-                for (int w = 1; w < 4; ++w) a += *(const f32x4 *)(red + (size_t)w * SLICES * 64 + o);
-                if (m >= g.M || n >= g.N) continue;
-                if (vec_ok) {
-                    Vec4<T> rv;
-                    if (R) rv = *(const Vec4<T> *)(R + (long)m * g.ldr + n);
-                    Vec4<T> out;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        float x = a[q] * g.alpha + bq[q];
-                        if (R) x += Elem<T>::to_f(rv.v[q]);
-                        out.v[q] = Elem<T>::from_f(apply_act(x, g.act));
-                    }
-                    st_vec4<T>(&C[(long)m * g.ldc + n], out);
-                } else {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        if (n + q >= g.N) break;
-                        float x = a[q] * g.alpha + bq[q];
-                        if (R) x += Elem<T>::to_f(R[(long)m * g.ldr + n + q]);
-                        st_elem<T>(&C[(long)m * g.ldc + n + q], Elem<T>::from_f(apply_act(x, g.act)));
-                    }
-                }
-            }
-        }
+        wide_reduce_store<T, BM, BN, NT>(g, (float *)lds_t, acc, m0, n0, offc, tid, wave, lane, kb);
 #ifdef GP_TILE_PROF
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         GP_PROBE(5);

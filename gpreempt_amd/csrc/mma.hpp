@@ -67,6 +67,11 @@ struct MatArgs {
     int batch_inner;
     // convolution geometry (CONV only)
     int H, W, Cin, S, Ho, Wo, sh, sw, ph, pw;
+    // layer-norm prologue (gemm_ln.hpp; ln_gamma == nullptr: none): the rows of A are normalised over
+    // their K elements before they are multiplied, and written to ln_out (M x K)
+    const void *ln_gamma, *ln_beta;
+    void *ln_out;
+    float ln_eps;
 };
 
 }  // namespace gp

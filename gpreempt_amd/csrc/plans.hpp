@@ -10,7 +10,9 @@ namespace gp {
 
 enum MatBody { MB_PIPE128 = 0, MB_PIPE64 = 1, MB_PIPE64_SK = 2, MB_PIPE32_SK = 3, MB_STAGED128 = 4, MB_STAGED64 = 5, MB_PIPE256 = 6,
                // wide split-K bodies (gemm_wide.hpp): tile rows x columns _ wavefronts
-               MB_WIDE32x32_16 = 7, MB_WIDE32x32_8 = 8, MB_WIDE64x32_16 = 9, MB_WIDE64x64_8 = 10 };
+               MB_WIDE32x32_16 = 7, MB_WIDE32x32_8 = 8, MB_WIDE64x32_16 = 9, MB_WIDE64x64_8 = 10,
+               // a wide 32 x 64 body with a layer-norm prologue over the rows of A (gemm_ln.hpp)
+               MB_LNWIDE32x64_16 = 11 };
 inline bool is_wide_body(int b) { return b >= MB_WIDE32x32_16 && b <= MB_WIDE64x64_8; }
 
 struct MatPlan {

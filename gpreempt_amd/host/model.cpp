@@ -204,6 +204,7 @@ Status Model::allocate_and_bind() {
         bind_pointers(k);
     }
     loaded_ = true;
+    plan_fusions();
     // seeded random initialisation of every parameter (overwritten by load_param when a file exists)
     uint64_t seed = 0x5EEDull;
     for (size_t i = 0; i < storage_infos.size(); ++i) {
@@ -221,6 +222,30 @@ Status Model::allocate_and_bind() {
         RETURN_STATUS(upload_param(i, host.data(), host.size()));
     }
     return Status::Succ;
+}
+
+// layer_norm -> dense pairs that run as one launch (gp_gemm_params::ln_gamma).  Only where the device layer
+// says the fused launch has the bits of the two (gp_gemm_ln_supported), and only for kernels launched
+// one by one without preemption arguments: a preemptible tenant keeps one launch per kernel index, which
+// is what its stop index and its claim counters speak of.
+void Model::plan_fusions() {
+    const char *env = std::getenv("GPREEMPT_FUSE_LN");
+    fuse_launches_ = !(env && std::atoi(env) == 0);
+    for (size_t i = 0; i + 1 < kernel_infos.size(); ++i) {
+        KernelInfo &ln = kernel_infos[i], &mm = kernel_infos[i + 1];
+        ln.fused_away = false; mm.has_ln_gemm = false;
+        if (ln.op != OpKind::Layernorm || mm.op != OpKind::Gemm) continue;
+        const gp_layernorm_params &l = ln.p.layernorm;
+        const gp_gemm_params &g = mm.p.gemm;
+        if (l.residual || g.A != l.out || g.K != l.cols || g.lda != l.cols || (long)g.M != l.rows || g.batch > 1 || g.dtype != l.dtype) continue;
+        if (g.C == l.out || g.residual == l.out || g.C == l.x || l.out == l.x) continue;
+        if (gp_gemm_ln_supported(&g) != 1) continue;
+        mm.ln_gemm = g;
+        mm.ln_gemm.A = l.x;
+        mm.ln_gemm.ln_gamma = l.gamma; mm.ln_gemm.ln_beta = l.beta; mm.ln_gemm.ln_out = l.out; mm.ln_gemm.ln_eps = l.eps;
+        mm.has_ln_gemm = true;
+        ln.fused_away = true;
+    }
 }
 
 // Slot order per operator is fixed by the builders in zoo.cpp.
@@ -415,6 +440,8 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         CUDA_RETURN_STATUS(gp_memcpy_d2d_async(k.args[1], k.args[0], size, stream));
         return Status::Succ;
     }
+    const bool fuse = fuse_launches_ && !k.preemptible;
+    if (fuse && k.fused_away) return Status::Succ;  // the next kernel's prologue does this one's work
     gp_preempt_ctx ctx{};
     const gp_preempt_ctx *pc = nullptr;
     if (k.preemptible) {
@@ -435,7 +462,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
     gp_launch_info info{};
     int rc = GP_FAIL;
     switch (k.op) {
-        case OpKind::Gemm: rc = gp_launch_gemm(&k.p.gemm, pc, stream, &info); break;
+        case OpKind::Gemm: rc = gp_launch_gemm(fuse && k.has_ln_gemm ? &k.ln_gemm : &k.p.gemm, pc, stream, &info); break;
         case OpKind::Conv: rc = gp_launch_conv2d(&k.p.conv, pc, stream, &info); break;
         case OpKind::Layout: rc = gp_launch_nchw_to_nhwc(&k.p.layout, pc, stream, &info); break;
         case OpKind::Pool: rc = gp_launch_pool2d(&k.p.pool, pc, stream, &info); break;

@@ -177,8 +177,22 @@ typedef struct gp_gemm_params {
     int batch_inner; long stride_a_outer, stride_b_outer, stride_c_outer;
     int tile_m, tile_n; /* 0 = chosen by the launcher; 256, 128, 64 or 32 (square; 64 x 32 with the wide variants) */
     int variant;        /* enum gp_mat_variant; 0 = chosen by the launcher */
+    /* Layer-norm prologue (ln_gamma == NULL: none): C = act(alpha * LN(A) * op(B) + bias + residual), where
+     * LN normalises every row of A over its K elements (gamma, beta: K elements of A's dtype; eps), rounds it
+     * to A's dtype and also writes it to ln_out (M x K, row stride K).  One launch where the exported graph
+     * has two (layer_norm, then dense): at batch 1 a launch costs more than the layer-norm's arithmetic.
+     * The result has the bits of gp_launch_layernorm followed by gp_launch_gemm.  Only for shapes that
+     * gp_gemm_ln_supported accepts; ln_out must not overlap A, B, C, bias or residual. */
+    const void *ln_gamma; const void *ln_beta; void *ln_out; float ln_eps;
 } gp_gemm_params;
 int gp_launch_gemm(const gp_gemm_params *p, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info);
+/* 1 when a layer-norm launch followed by the GEMM `p` (its ln_* fields are not looked at) can be replaced by
+ * one launch with the prologue without changing a bit: 16-bit dtype, batch 1, B stored N x K, lda == K, K a
+ * multiple of 64 and at most 832, at most one 32 x 64 tile per compute unit (every workgroup of a tile row
+ * normalises the rows again, which must stay cheaper than a launch), and a plain GEMM of this shape would be summed in the prologue body's order
+ * (K split over four wavefronts).  gp_launch_gemm itself takes the prologue for any shape that passes the
+ * first five conditions. */
+int gp_gemm_ln_supported(const gp_gemm_params *p);
 /* No counterpart in the reference: gp_launch_gemm for callers that cannot allocate device memory
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  The
  * preemption state that gp_preempt_ctx otherwise brings in (32 claim counters per kernel, the stop

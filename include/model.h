@@ -75,6 +75,13 @@ public:
     GPUdeviceptr executed = nullptr;
     int kernel_id = 0;
     double flops = 0, bytes = 0;          // algorithmic work of one launch
+    // Launch fusion (Model::plan_fusions): a layer-norm whose only job before the next kernel is to feed
+    // that kernel's A operand is not launched (`fused_away`); the dense layer behind it runs `ln_gemm`,
+    // the same GEMM with the layer-norm as its prologue.  The kernel list, its indices and the
+    // whole-model program keep the two-kernel form.
+    bool fused_away = false;
+    bool has_ln_gemm = false;
+    gp_gemm_params ln_gemm;
 };
 
 class Model {
@@ -187,6 +194,8 @@ private:
     std::unordered_map<std::string, size_t> storages_idx;
 
     Status allocate_and_bind();
+    void plan_fusions();
+    bool fuse_launches_ = true;  // GPREEMPT_FUSE_LN=0 in the environment keeps every launch of the kernel list
     Status upload_param(size_t idx, const float *disk, size_t n);
     void bind_pointers(KernelInfo &k);
 };

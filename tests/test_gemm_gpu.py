@@ -624,3 +624,77 @@ def test_config5_gemm8192_bf16_full_size(gp):
             relaunches += 1
             assert relaunches < 4
         assert np.array_equal(dC.download(np_dtype=np.uint16).reshape(n, n), base), f"resume after {frac:.0%} differs"
+
+
+# ---- layer-norm prologue -----------------------------------------------------------------------------
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K,act", [(128, 2304, 768, 0), (128, 3072, 768, 2), (100, 72, 256, 1), (384, 200, 832, 0)])
+def test_gemm_with_layernorm_prologue_has_the_bits_of_two_launches(gp, dt, M, N, K, act):
+    """gp_launch_gemm with ln_gamma set = gp_launch_layernorm, then gp_launch_gemm: same C, same normalised
+    rows, bit for bit (BERT-base's QKV and first FFN projection at sequence 128 among the shapes); within
+    tolerance of the oracle's layer-norm and GEMM; stopped at a tile boundary and resumed, still the same."""
+    rng = np.random.default_rng(M + N + K)
+    dtype = gp.DTYPE_BY_NAME[dt]
+    es = gp.DTYPE_SIZE[dtype]
+    X = O.round_to(rng.normal(0.1, 1.5, (M, K)).astype(np.float32), dt)
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32) * 0.05, dt)
+    gamma = O.round_to(rng.uniform(0.5, 1.5, K).astype(np.float32), dt)
+    beta = O.round_to(rng.normal(0, 0.2, K).astype(np.float32), dt)
+    bias = O.round_to(rng.uniform(-0.1, 0.1, N).astype(np.float32), dt)
+    res = O.round_to(rng.uniform(-1, 1, (M, N)).astype(np.float32), dt)
+    dX, dB, dg, dbeta, dbias, dres = (gp.DevBuf.from_array(a, dtype) for a in (X, B, gamma, beta, bias, res))
+    dLN, dC = gp.DevBuf(M * K * es), gp.DevBuf(M * N * es)
+    # two launches
+    gp.launch("gp_launch_layernorm", gp.LayernormParams(dtype, M, K, dX.ptr, None, dg.ptr, dbeta.ptr, dLN.ptr, 1e-12))
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dLN.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, bias=dbias.ptr,
+                      residual=dres.ptr, alpha=1.0, act=act, batch=1)
+    # the model loader fuses only where the launcher's own choice for the plain GEMM sums K as the prologue body does
+    assert gp.lib().gp_gemm_ln_supported(C.byref(p)) == (1 if K >= 768 else 0)  # K = 256 runs on a body that keeps K in one wavefront
+    p.tile_m = p.tile_n = 32
+    p.variant = gp.MAT_PIPE_SPLITK  # K split over four wavefronts: the order of the wide bodies and of the prologue body
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    ln_two, c_two = dLN.download().copy(), dC.download().copy()
+    ln_ref = O.round_to(O.layernorm(X, gamma, beta, 1e-12), dt)
+    assert rel_err(dLN.download(dtype, (M, K)), ln_ref) < TOL[dt]
+    assert rel_err(dC.download(dtype, (M, N)), O.gemm_bias_act(ln_ref, B, bias, res, act, b_is_nk=True)) < TOL[dt]
+    # one launch
+    dLN.fill32(0x7E007E00); dC.fill32(0x7E007E00)
+    p.A = dX.ptr
+    p.tile_m = p.tile_n = p.variant = 0
+    p.ln_gamma, p.ln_beta, p.ln_out, p.ln_eps = dg.ptr, dbeta.ptr, dLN.ptr, 1e-12
+    info = gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert info.total_tiles == ((M + 31) // 32) * ((N + 63) // 64)
+    assert np.array_equal(dLN.download(), ln_two) and np.array_equal(dC.download(), c_two)
+    # preempted and resumed
+    flag = gp.Flag()
+    total = info.total_tiles
+    for groups, wgs in ((1, 4), (32, 0)):
+        st = gp.BlpState(1, flag, groups)
+        for frac in (0.3, 0.8):
+            st.reset(); st.clear_stop(); flag.set(0)
+            dLN.fill32(0); dC.fill32(0)
+            gp.launch("gp_launch_gemm", p, st.ctx(inject_at=int(frac * total), max_workgroups=wgs, fresh=1))
+            gp.check(gp.lib().gp_stream_sync(None))
+            assert flag.get() == 1
+            flag.set(0)
+            st.clear_stop()
+            gp.launch("gp_launch_gemm", p, st.ctx())
+            gp.check(gp.lib().gp_stream_sync(None))
+            assert np.array_equal(dLN.download(), ln_two) and np.array_equal(dC.download(), c_two), (groups, frac)
+
+
+def test_layernorm_prologue_is_refused_where_it_does_not_fit(gp):
+    dA = gp.DevBuf(1 << 20)
+    def params(**kw):
+        base = dict(dtype=gp.F16, M=128, N=256, K=768, A=dA.ptr, lda=768, B=dA.ptr, ldb=768, b_is_nk=1, C=dA.ptr, ldc=256, alpha=1.0, batch=1)
+        base.update(kw)
+        return gp.GemmParams(**base)
+    assert gp.lib().gp_gemm_ln_supported(C.byref(params())) == 1
+    for kw in (dict(dtype=gp.F32), dict(K=1024, lda=1024, ldb=1024), dict(K=72, lda=72, ldb=72), dict(lda=776), dict(b_is_nk=0, ldb=256), dict(batch=2), dict(M=1 << 16)):
+        p = params(**kw)
+        assert gp.lib().gp_gemm_ln_supported(C.byref(p)) == 0, kw
+        p.ln_gamma = p.ln_beta = p.ln_out = dA.ptr
+        with pytest.raises(gp.GpError):
+            gp.launch("gp_launch_gemm", p)
