@@ -477,6 +477,28 @@ def cpu_baseline(runs):
             "legs": legs}
 
 
+def hp_request(model, runs=50):
+    """The high-priority request alone, submitted as the harness submits it (a non-preemptible executor,
+    one launch per kernel of its list): `--only hp` under rocprofv3 --kernel-trace shows which kernels it
+    consists of, how long each takes and the gaps between them."""
+    import numpy as np
+    from gpreempt_amd import capi as gp, executor as E
+    ex = E.Executor(model, blp=False)
+    stream = gp.Stream(0)
+    ids = np.random.default_rng(0).integers(0, 30000, ex.data_size("data") // 8).astype(np.int64)
+    ex.set_input("data", ids, stream)
+    e0, e1 = gp.Event(), gp.Event()
+    ts = []
+    for i in range(runs + 5):
+        e0.record(stream)
+        ex.execute(stream)
+        e1.record(stream); e1.sync()
+        if i >= 5:
+            ts.append(e0.elapsed_ms(e1))
+    ts.sort()
+    return {"model": model, "kernels_in_list": ex.kernel_num(), "runs": runs, "device_ms": {"p50": ts[len(ts) // 2], "min": ts[0], "max": ts[-1]}}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -486,7 +508,7 @@ def main():
     ap.add_argument("--hp-rate", type=float, default=200.0)
     ap.add_argument("--hp-model", default="bert")
     ap.add_argument("--be-model", default="resnet152")
-    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal | vendor")
+    ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal | vendor | hp")
     ap.add_argument("--cpu-requests", type=int, default=10, help="timed submissions per graph in the cpu_baseline leg")
     ap.add_argument("--gemm-operands", default="random", choices=("random", "const"), help="operands of the 8192^3 GEMM leg (--only gemm)")
     args = ap.parse_args()
@@ -541,6 +563,8 @@ def main():
         out["graph_workloads"] = graph_workloads()
     if args.only == "copycal":
         out["copy_calibration"] = copy_calibration()
+    if args.only == "hp":
+        out["hp_request_alone"] = hp_request(args.hp_model)
     if args.only in ("", "cpu"):
         out["cpu_baseline"] = cpu_baseline(args.cpu_requests)
     print(json.dumps(out))
