@@ -457,6 +457,11 @@ struct Mapper {
     Status run() {
         for (const ExportOp &o : ops.funcs) by_func[o.func] = &o;
         if (ops.layout != "NCHW") { error = "ops json: only exports in NCHW layout are mapped"; return Status::Fail; }
+        for (size_t i = 0; i < ex.global_len; ++i) {
+            if (ex.nodes[i].shape.empty() || ex.nodes[i].shape.size() > 4) return fail(i, "tensors of 1 to 4 dimensions only");
+            for (long d : ex.nodes[i].shape) if (d <= 0 || d >= (1L << 31)) return fail(i, "a dimension of " + std::to_string(d));
+            if (prod(ex.nodes[i].shape) >= (1L << 40)) return fail(i, "more than 2^40 elements");
+        }
         vals.assign(ex.global_len, Val());
         plan_concatenations();
         bool have_data = false;

@@ -237,3 +237,14 @@ def test_what_cannot_be_mapped_is_refused_by_name(tmp_path):
     assert rc == 1 and "an image as the model's output" in rep["error"]
     rc, rep = plan(FIX, "f64")
     assert rc == 1 and "unknown dtype" in rep["error"]
+    # shapes that no tensor can have
+    def zero_dim(f, doc):
+        if f == "mod.json":
+            doc["attrs"]["shape"][1][1] = [4, 0, 3, 3]
+    rc, rep = plan(_edited(tmp_path, "zero", zero_dim))
+    assert rc == 1 and "a dimension of 0" in rep["error"]
+    def huge_dim(f, doc):
+        if f == "mod.json":
+            doc["attrs"]["shape"][1][5] = [10, 1 << 33]
+    rc, rep = plan(_edited(tmp_path, "huge", huge_dim))
+    assert rc == 1 and "a dimension of" in rep["error"]
