@@ -23,6 +23,37 @@ constexpr int ATT_QB = 128;      // query rows per tile (32 per wave)
 __host__ __device__ inline int attention_key_blocks(int seq) { return (seq + 31) / 32; }
 __host__ __device__ inline size_t attention_lds_bytes(int nb) { return (size_t)ATT_D * (nb * 32 + 4) * 2; }
 
+// V^T into LDS: vt[d][key] for NB * 32 keys, keys past the sequence zero-filled.  A thread moves
+// NB * 32 * 8 / 256 chunks of eight d values; a wavefront takes 64 consecutive keys of one chunk, so
+// its transposing 2-byte writes are 128 contiguous bytes per d, free of bank conflicts.  The chunks
+// are fetched up to eight at a time before any is written (as one loop over the chunks, every
+// iteration waited for its own load; 384 keys: 12.95 -> 12.3 us per launch).
+template <typename T, int NB>
+__device__ __forceinline__ void stage_vt(const T *V, long ld, int S, T *vt, int tid) {
+    constexpr int SP = NB * 32 + 4;
+    constexpr int ITER = NB * 32 * (ATT_D / 8) / 256;   // NB
+    constexpr int BATCH = ITER % 8 == 0 ? 8 : ITER % 4 == 0 ? 4 : ITER;
+    const u32x4 zero4 = {0, 0, 0, 0};
+#pragma unroll
+    for (int b0 = 0; b0 < ITER; b0 += BATCH) {
+        u32x4 raw[BATCH];
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) {
+            const int idx = tid + (b0 + b) * 256;
+            const int key = idx % (NB * 32), dc = idx / (NB * 32);
+            raw[b] = key < S ? *(const u32x4 *)(V + (long)key * ld + dc * 8) : zero4;
+        }
+#pragma unroll
+        for (int b = 0; b < BATCH; ++b) {
+            const int idx = tid + (b0 + b) * 256;
+            const int key = idx % (NB * 32), dc = idx / (NB * 32);
+            const unsigned short *e = (const unsigned short *)&raw[b];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) ((unsigned short *)vt)[(dc * 8 + j) * SP + key] = e[j];
+        }
+    }
+}
+
 template <typename T, int NB>
 __device__ __forceinline__ void attention_tile(const AttnArgs &a, TileIdx t, T *vt) {
     const gp_attention_params &p = a.p;
@@ -56,18 +87,10 @@ __device__ __forceinline__ void attention_tile(const AttnArgs &a, TileIdx t, T *
         }
     }
 
-    // ---- V^T into LDS: vt[d][key], keys past the sequence zero-filled (their probability is 0,
-    // but 0 * garbage could be NaN) -----------------------------------------------------------
+    // ---- V^T into LDS (keys past the sequence zero-filled: their probability is 0, but 0 * garbage
+    // could be NaN) ---------------------------------------------------------------------------
     __syncthreads();  // the previous tile of this workgroup may still be reading vt
-    for (int idx = tid; idx < NB * 32 * (ATT_D / 8); idx += 256) {
-        // a wavefront takes 64 consecutive keys of one 8-wide d chunk: its transposing 2-byte
-        // writes are then 128 contiguous bytes per d, free of bank conflicts
-        const int key = idx % (NB * 32), dc = idx / (NB * 32);
-        u32x4 raw = key < S ? *(const u32x4 *)(V + (long)key * p.ld_qkv + dc * 8) : zero4;
-        const unsigned short *e = (const unsigned short *)&raw;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) ((unsigned short *)vt)[(dc * 8 + j) * SP + key] = e[j];
-    }
+    stage_vt<T, NB>(V, p.ld_qkv, S, vt, tid);
     __syncthreads();
 
     // ---- scores (transposed): s[nb][v] = <K[key], Q[query]> ------------------------------------
@@ -177,13 +200,7 @@ __device__ __forceinline__ void attention_tile_split(const AttnArgs &a, TileIdx 
     for (int ks = 0; ks < 4; ++ks) bq[ks] = q < S ? *(const u32x4 *)(Q + (long)q * p.ld_qkv + ks * 16 + half * 8) : zero4;
 
     __syncthreads();  // the previous tile of this workgroup may still be reading vt or the merge area
-    for (int idx = tid; idx < NB * 32 * (ATT_D / 8); idx += 256) {
-        const int key = idx % (NB * 32), dc = idx / (NB * 32);
-        u32x4 raw = key < S ? *(const u32x4 *)(V + (long)key * p.ld_qkv + dc * 8) : zero4;
-        const unsigned short *e = (const unsigned short *)&raw;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) ((unsigned short *)vt)[(dc * 8 + j) * SP + key] = e[j];
-    }
+    stage_vt<T, NB>(V, p.ld_qkv, S, vt, tid);
     __syncthreads();
 
     const int nb0 = kh * NBH;
@@ -261,15 +278,50 @@ __device__ __forceinline__ void attention_tile_split(const AttnArgs &a, TileIdx 
         const float den = a1 * sum + a2 * sum2;
         const float f1 = a1 / den, f2 = a2 / den;  // this lane's query (row l32 of the group)
         const int q0 = t.x * ATT_QB_SPLIT + qg * 32;
+        // The accumulator registers of a lane belong to four runs of four consecutive query rows, whose
+        // factors sit in other lanes: they go through LDS (the slots of m2 and sum2, read above) and
+        // come back as 16-byte reads, one per run.  The wavefront is alone in this part of LDS, and its
+        // LDS operations complete in order.
+        float *fac = merge + 32 * ATT_D;
+        if (half == 0) {
+            fac[l32] = f1;
+            fac[32 + l32] = f2;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int vq = 0; vq < 4; ++vq) {
+            const f32x4 g1 = *(const f32x4 *)(fac + 8 * vq + 4 * half), g2 = *(const f32x4 *)(fac + 32 + 8 * vq + 4 * half);
+#pragma unroll
+            for (int db = 0; db < 2; ++db)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int v = 4 * vq + e, r = 8 * vq + 4 * half + e;
+                    o[db][v] = g1[e] * o[db][v] + g2[e] * merge[r * ATT_D + db * 32 + l32];
+                }
+        }
+        // The 32 x 64 block of results is laid out in LDS (over the partial block, which has been read)
+        // and leaves as 16-byte stores, four per lane, instead of sixty-four 2-byte ones.
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        T *ob = (T *)merge;
+        const bool vec_out = p.ld_out % 8 == 0 && (size_t)p.out % 16 == 0;  // rows of 64 values start on 16-byte boundaries
 #pragma unroll
         for (int db = 0; db < 2; ++db)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = 8 * (v / 4) + 4 * half + (v % 4);  // the accumulator's query row: its factors sit in lane r
-                const float g1 = __shfl(f1, r, 64), g2 = __shfl(f2, r, 64);
-                const float val = g1 * o[db][v] + g2 * merge[r * ATT_D + db * 32 + l32];
-                if (q0 + r < S) st_elem<T>(O + (long)(q0 + r) * p.ld_out + db * 32 + l32, Elem<T>::from_f(val));
+            for (int v = 0; v < 16; ++v) ob[(8 * (v / 4) + 4 * half + (v % 4)) * ATT_D + db * 32 + l32] = Elem<T>::from_f(o[db][v]);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int c0 = 0; c0 < 32 * ATT_D / 8; c0 += 64) {
+            const int c = c0 + lane, r = c >> 3, d8 = (c & 7) * 8;
+            const u32x4 chunk = *(const u32x4 *)(ob + r * ATT_D + d8);
+            if (q0 + r >= S) continue;
+            T *dst = O + (long)(q0 + r) * p.ld_out + d8;
+            if (vec_out) st_out128(dst, __builtin_bit_cast(out_u32x4, chunk));
+            else {
+                const T *e = (const T *)&chunk;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) st_elem<T>(dst + j, e[j]);
             }
+        }
     }
 }
 
