@@ -595,9 +595,12 @@ __device__ __forceinline__ void wave_sum_rows(float (&s)[R]) {
         for (int q = 0; q < R; ++q) s[q] += t[q];
     }
 }
-template <typename T, int MAXC, int R>
+// PRE: gamma and beta come as the lane's raw chunks (chunk lane + 64 i in slot i), fetched by the caller when
+// it suits it; otherwise they are read here, chunk by chunk (long rows: no registers to spare for them).
+template <typename T, int MAXC, int R, bool PRE>
 __device__ __forceinline__ void ln_rows_math(const float (&v)[R][MAXC][VecIO<T>::VEC], int chunks, int lane, int cols, float eps,
-                                             const T *gamma, const T *beta, out_u32x4 (&y)[R][MAXC]) {
+                                             const T *gamma_p, const T *beta_p, const out_u32x4 (&gamma)[PRE ? MAXC : 1],
+                                             const out_u32x4 (&beta)[PRE ? MAXC : 1], out_u32x4 (&y)[R][MAXC]) {
     constexpr int VEC = VecIO<T>::VEC;
     float sum[R], mean[R], sq[R], inv[R];
 #pragma unroll
@@ -634,8 +637,13 @@ __device__ __forceinline__ void ln_rows_math(const float (&v)[R][MAXC][VecIO<T>:
         const int ch = lane + i * 64;
         if (ch < chunks) {
             float ga[VEC], be[VEC];
-            VecIO<T>::load(gamma + ch * VEC, ga);
-            VecIO<T>::load(beta + ch * VEC, be);
+            if constexpr (PRE) {
+                VecIO<T>::unpack(gamma[i], ga);
+                VecIO<T>::unpack(beta[i], be);
+            } else {
+                VecIO<T>::load(gamma_p + ch * VEC, ga);
+                VecIO<T>::load(beta_p + ch * VEC, be);
+            }
 #pragma unroll
             for (int q = 0; q < R; ++q) {
                 float o[VEC];
@@ -655,7 +663,19 @@ __device__ __forceinline__ void layernorm_rows(const gp_layernorm_params &p, Til
     const int lane = threadIdx.x & 63;
     const long row0 = ((long)t.x * 4 + (threadIdx.x >> 6)) * RPW;
     if (row0 >= p.rows) return;
-    out_u32x4 rx[RPW][MAXC], rr[RPW][MAXC];
+    constexpr bool PRE = MAXC <= 2;  // short rows: gamma and beta are fetched with the row
+    out_u32x4 rx[RPW][MAXC], rr[RPW][MAXC], graw[PRE ? MAXC : 1], braw[PRE ? MAXC : 1];
+    if constexpr (PRE) {
+#pragma unroll
+        for (int i = 0; i < MAXC; ++i) {
+            const int ch = lane + i * 64;
+            graw[i] = braw[i] = out_u32x4{0, 0, 0, 0};
+            if (ch < chunks) {
+                graw[i] = *(const out_u32x4 *)((const T *)p.gamma + ch * VEC);
+                braw[i] = *(const out_u32x4 *)((const T *)p.beta + ch * VEC);
+            }
+        }
+    }
 #pragma unroll
     for (int q = 0; q < RPW; ++q) {
         const long row = row0 + q < p.rows ? row0 + q : row0;  // a missing second row re-reads the first and is not stored
@@ -692,7 +712,7 @@ __device__ __forceinline__ void layernorm_rows(const gp_layernorm_params &p, Til
         }
     }
     out_u32x4 y[RPW][MAXC];
-    ln_rows_math<T, MAXC, RPW>(v, chunks, lane, p.cols, p.eps, (const T *)p.gamma, (const T *)p.beta, y);
+    ln_rows_math<T, MAXC, RPW, PRE>(v, chunks, lane, p.cols, p.eps, (const T *)p.gamma, (const T *)p.beta, graw, braw, y);
 #pragma unroll
     for (int q = 0; q < RPW; ++q) {
         if (row0 + q >= p.rows) break;

@@ -53,6 +53,7 @@ struct LnWideKernel {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 
     static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0}) {
+        GP_PROBE(0);
         __shared__ int early_slot[64];
         const bool early = cc.stop_index != nullptr;
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
@@ -112,10 +113,23 @@ struct LnWideKernel {
                     if (ch < chunks) rx[q][i] = *(const out_u32x4 *)(x + ch * VEC);
                 }
             }
+            // gamma and beta with them: a wait for them later would be a wait for B as well
+            out_u32x4 graw[MAXC], braw[MAXC];
 #pragma unroll
-            for (int q = 0; q < RPW; ++q)
+            for (int i = 0; i < MAXC; ++i) {
+                const int ch = lane + i * 64;
+                graw[i] = braw[i] = out_u32x4{0, 0, 0, 0};
+                if (ch < chunks) {
+                    graw[i] = *(const out_u32x4 *)((const T *)g.ln_gamma + ch * VEC);
+                    braw[i] = *(const out_u32x4 *)((const T *)g.ln_beta + ch * VEC);
+                }
+            }
 #pragma unroll
-                for (int i = 0; i < MAXC; ++i) asm volatile("" : "+v"(rx[q][i]) :: "memory");  // the rows have arrived
+            for (int i = 0; i < MAXC; ++i) {
+#pragma unroll
+                for (int q = 0; q < RPW; ++q) asm volatile("" : "+v"(rx[q][i]) :: "memory");  // the rows have arrived
+                asm volatile("" : "+v"(graw[i]), "+v"(braw[i]) :: "memory");
+            }
 #pragma unroll
             for (int s = 0; s < PRE; ++s) {
                 if (s < NS) issue(s);
@@ -130,7 +144,7 @@ struct LnWideKernel {
                     if (ch < chunks) VecIO<T>::unpack(rx[q][i], v[q][i]);
                 }
             out_u32x4 y[RPW][MAXC];
-            ln_rows_math<T, MAXC, RPW>(v, chunks, lane, g.K, g.ln_eps, (const T *)g.ln_gamma, (const T *)g.ln_beta, y);
+            ln_rows_math<T, MAXC, RPW, true>(v, chunks, lane, g.K, g.ln_eps, (const T *)g.ln_gamma, (const T *)g.ln_beta, graw, braw, y);
 #pragma unroll
             for (int q = 0; q < RPW; ++q) {
                 const int r = wave + q * WAVES, m = m0 + r;
@@ -147,6 +161,7 @@ struct LnWideKernel {
             }
         }
 
+        GP_PROBE(1);
         f32x16 acc[MI][NI];
 #pragma unroll
         for (int i = 0; i < MI; ++i)
@@ -169,6 +184,7 @@ struct LnWideKernel {
             else if (s + STAGES - 2 < NS) wait_vmcnt<(STAGES - 2) * LPW>();
             else wait_vmcnt<0>();
             __syncthreads();  // stage s of B (and, the first time, the rows of A) visible; the buffer of stage s-1 is free
+            if (s == 0) GP_PROBE(2);
             if (s == 0 && early && __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1) {
                 wait_vmcnt<0>();  // loads still landing in LDS must not outlive the workgroup
                 return true;
@@ -190,7 +206,12 @@ struct LnWideKernel {
                     for (int j = 0; j < NI; ++j) Elem<T>::mma(fa[i], fb[j], acc[i][j]);
             }
         }
+        GP_PROBE(3);
         wide_reduce_store<T, BM, BN, NT>(g, (float *)lds_t, acc, m0, n0, 0, tid, wave, lane, kb);
+#ifdef GP_TILE_PROF
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        GP_PROBE(5);
+#endif
         return false;
     }
 };
