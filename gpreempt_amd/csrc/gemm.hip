@@ -124,10 +124,19 @@ static int pipe_case_ckpt(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_strea
     return launch_mat<PipeKernel<T, TILE, TILE, STAGES, false, false, true>>(pl, ctx, s, info);
 }
 
+// Ring depth of a wide body: three stages, four for the GEMM form of the 32 x 32 tile on 16 wavefronts (a
+// stage is (WAVES / 4) K-blocks of BM + BN rows of 128 bytes: 32 KB there).  128 x 768 x 3072 went from
+// 7.96 to 7.67 us per launch with the fourth stage; given to every body that has room for it, it cost the
+// convolution chain of ResNet-152 1 us per launch (10.2 -> 11.2); two stages instead of three for the
+// convolution form changed nothing (10.27 either way).
+constexpr int wide_stages(int bm, int bn, int waves, bool conv) { return (!conv && bm == 32 && bn == 32 && waves == 16) ? 4 : 3; }
+template <typename T, int BM, int BN, int WAVES, bool CONV = false>
+using WideK = WideKernel<T, BM, BN, WAVES, wide_stages(BM, BN, WAVES, CONV), CONV>;
+
 template <typename T, int BM, int BN, int WAVES>
 static int wide_case(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
-    if (pl.conv) return launch_mat<WideKernel<T, BM, BN, WAVES, 3, true>>(pl, ctx, s, info);
-    return launch_mat<WideKernel<T, BM, BN, WAVES, 3, false>>(pl, ctx, s, info);
+    if (pl.conv) return launch_mat<WideK<T, BM, BN, WAVES, true>>(pl, ctx, s, info);
+    return launch_mat<WideK<T, BM, BN, WAVES, false>>(pl, ctx, s, info);
 }
 
 template <typename T>
@@ -179,10 +188,10 @@ static size_t body_lds_bytes(int body, int dtype) {
         case MB_PIPE64: return GP_S64 * (64 + 64) * 128;
         case MB_PIPE64_SK: return GP_S64 * (64 + 64) * 128;   // at least the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4 = 64 KB)
         case MB_PIPE32_SK: return GP_S32 * (32 + 32) * 128;
-        case MB_WIDE32x32_16: return WideKernel<_Float16, 32, 32, 16, 3>::LDS_BYTES;
-        case MB_WIDE32x32_8: return WideKernel<_Float16, 32, 32, 8, 3>::LDS_BYTES;
-        case MB_WIDE64x32_16: return WideKernel<_Float16, 64, 32, 16, 3>::LDS_BYTES;
-        case MB_WIDE64x64_8: return WideKernel<_Float16, 64, 64, 8, 3>::LDS_BYTES;
+        case MB_WIDE32x32_16: return WideK<_Float16, 32, 32, 16>::LDS_BYTES;
+        case MB_WIDE32x32_8: return WideK<_Float16, 32, 32, 8>::LDS_BYTES;
+        case MB_WIDE64x32_16: return WideK<_Float16, 64, 32, 16>::LDS_BYTES;
+        case MB_WIDE64x64_8: return WideK<_Float16, 64, 64, 8>::LDS_BYTES;
         case MB_LNWIDE32x64_16: return LnWideKernel<_Float16, 32, 64, 16, 3>::LDS_BYTES;
         case MB_STAGED128: return (128 + 128) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
         case MB_STAGED64: return (64 + 64) * ((es == 4 ? 16 : 32) + (es == 4 ? 4 : 8)) * es;
@@ -197,10 +206,10 @@ static size_t body_lds_bytes(int body, int dtype) {
 // the wide split-K bodies (gemm_wide.hpp) and their tiles
 struct WideChoice { int body, bm, bn, waves; size_t lds; };
 static const WideChoice kWide[4] = {
-    {MB_WIDE32x32_16, 32, 32, 16, WideKernel<_Float16, 32, 32, 16, 3>::LDS_BYTES},
-    {MB_WIDE32x32_8, 32, 32, 8, WideKernel<_Float16, 32, 32, 8, 3>::LDS_BYTES},
-    {MB_WIDE64x32_16, 64, 32, 16, WideKernel<_Float16, 64, 32, 16, 3>::LDS_BYTES},
-    {MB_WIDE64x64_8, 64, 64, 8, WideKernel<_Float16, 64, 64, 8, 3>::LDS_BYTES}};
+    {MB_WIDE32x32_16, 32, 32, 16, WideK<_Float16, 32, 32, 16>::LDS_BYTES},
+    {MB_WIDE32x32_8, 32, 32, 8, WideK<_Float16, 32, 32, 8>::LDS_BYTES},
+    {MB_WIDE64x32_16, 64, 32, 16, WideK<_Float16, 64, 32, 16>::LDS_BYTES},
+    {MB_WIDE64x64_8, 64, 64, 8, WideK<_Float16, 64, 64, 8>::LDS_BYTES}};
 static const WideChoice *wide_of(int body) {
     for (const WideChoice &w : kWide) if (w.body == body) return &w;
     return nullptr;
