@@ -15,7 +15,8 @@
 // kb = w / 4 and fetches a quarter of the rows of that group's block.  One barrier per stage.  The
 // arithmetic stays with wavefronts 0..3 (there is little of it: these layers wait for operands):
 // wavefront w multiplies MFMA k-step w of every block, block after block, for the whole BM x BN
-// tile, and at the end the four partial tiles are summed through LDS in the order 0, 1, 2, 3.  That
+// tile (the code lets G groups of four share the output blocks between them; G = 1, see there), and at the end
+// the four partial tiles are summed through LDS in the order 0, 1, 2, 3.  That
 // is exactly the summation of the four-wavefront split-K bodies of gemm_pipe.hpp, so the result
 // has the same bits as theirs (the whole-model program, whose workgroups have four wavefronts,
 // uses those) and does not depend on scheduling: a preempted-then-resumed run stays bit-identical.
@@ -51,10 +52,10 @@ template <int LPW> __device__ __forceinline__ void wait_stages(int stages) {
 
 // The end of a tile of the wide bodies: the partial tiles of wavefronts 0..3 are summed through LDS in
 // wavefront order and the epilogue (alpha, bias, residual, activation) is applied on the way out.
-template <typename T, int BM, int BN, int NT>
-__device__ __forceinline__ void wide_reduce_store(const MatArgs &g, float *red, const f32x16 (&acc)[BM / 32][BN / 32], int m0, int n0, long offc,
-                                                  int tid, int wave, int lane, int kb) {
-    constexpr int MI = BM / 32, NI = BN / 32, SLICES = MI * NI * 16;
+template <typename T, int BM, int BN, int NT, int G>
+__device__ __forceinline__ void wide_reduce_store(const MatArgs &g, float *red, const f32x16 (&acc)[(BM / 32) * (BN / 32) / G], int m0, int n0, long offc,
+                                                  int tid, int wv, int lane, int kb) {
+    constexpr int MI = BM / 32, NI = BN / 32, SLICES = MI * NI * 16, BPW = MI * NI / G;
     // ---- reduction and epilogue -------------------------------------------------------------
     // partial tiles of wavefronts 0..3 -> LDS as [wavefront][slice][lane], slice = (i*NI + j)*16 + v,
     // which is row 8*(v/4) + 4*(lane/32) + v%4, column 32*j + lane%32 of 32 x 32 block (i, j).
@@ -66,13 +67,11 @@ __device__ __forceinline__ void wide_reduce_store(const MatArgs &g, float *red, 
     const bool vec_ok = (g.N % 4 == 0) && (g.ldc % 4 == 0) && (offc % 4 == 0) && ((size_t)g.C % 16 == 0) &&
                         (!R || (g.ldr % 4 == 0 && (size_t)g.residual % 16 == 0)) && (!bias || (size_t)bias % 16 == 0);
     __syncthreads();  // all wavefronts are done reading the stage buffers
-    if (kb == 0) {
+    if (kb < G) {  // wavefront (kb, wv) holds k-step wv of the 32 x 32 blocks kb, kb + G, ...
 #pragma unroll
-        for (int i = 0; i < MI; ++i)
+        for (int q = 0; q < BPW; ++q)
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) red[((size_t)wave * SLICES + (i * NI + j) * 16 + v) * 64 + lane] = acc[i][j][v];
+            for (int v = 0; v < 16; ++v) red[((size_t)wv * SLICES + (kb + q * G) * 16 + v) * 64 + lane] = acc[q][v];
     }
     __syncthreads();
     GP_PROBE(4);
@@ -143,7 +142,16 @@ struct WideKernel {
     static constexpr int LPW = LPW_A + LPW_B;              // load instructions per wavefront per stage
     static constexpr int A_BYTES = BM * RB, BLK_BYTES = (BM + BN) * RB, STAGE_BYTES = KB * BLK_BYTES;
     static constexpr int MI = BM / 32, NI = BN / 32;
-    static constexpr int SLICES = MI * NI * 16;            // 64-float slices of one wavefront's accumulators
+    // Which wavefronts multiply: group kb < G takes the 32 x 32 output blocks kb, kb + G, ... (k-step wv of every
+    // K-block: whose registers a partial sum lives in does not change what is added to what).  G = 1 here:
+    // two multiplying groups (one per output block of a 64 x 32 tile) were measured and changed nothing or
+    // cost a little (1568 x 256 x 2304: 8.50 -> 8.54 us, 128 x 2304 x 768: 5.16 -> 5.43; each group re-reads
+    // the fragments it shares with the other); the layer-norm prologue body, whose A operand stays in LDS,
+    // gains from two (gemm_ln.hpp).
+    static constexpr int G = 1;
+    static constexpr int BPW = MI * NI / G;
+    static_assert(MI * NI % G == 0, "output blocks divide among the multiplying groups");
+    static constexpr int SLICES = MI * NI * 16;            // 64-float slices of one k-step's partial tile
     static constexpr size_t RED_BYTES = (size_t)4 * SLICES * 64 * 4;   // the partial tiles of wavefronts 0..3
     static constexpr size_t RING_BYTES = (size_t)STAGES * STAGE_BYTES;
     static constexpr size_t LDS_BYTES = RING_BYTES > RED_BYTES ? RING_BYTES : RED_BYTES;
@@ -259,13 +267,11 @@ struct WideKernel {
             }
         };
 
-        f32x16 acc[MI][NI];
+        f32x16 acc[BPW];
 #pragma unroll
-        for (int i = 0; i < MI; ++i)
+        for (int q = 0; q < BPW; ++q)
 #pragma unroll
-            for (int j = 0; j < NI; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+            for (int v = 0; v < 16; ++v) acc[q][v] = 0.f;
         auto frag = [&](int stage, int blk, int region_bytes, int row, int chunk) -> u32x4 {
             const int phys = chunk ^ ((row >> 1) & 7);
             return *(const u32x4 *)(lds_c + (size_t)stage * STAGE_BYTES + (size_t)blk * BLK_BYTES + region_bytes + row * RB + phys * 16);
@@ -291,27 +297,25 @@ struct WideKernel {
                 return true;
             }
             if (s >= PRE - (STAGES - 1) && s + STAGES - 1 < NS) issue(s + STAGES - 1);
-            if (kb != 0) continue;  // (uniform) wavefronts 4.. only fetch
+            if (kb >= G) continue;  // (uniform) the other wavefronts only fetch
             const int stage = s % STAGES;
 #pragma unroll
             for (int b = 0; b < KB; ++b) {
                 // a block past the last one holds zeros; it is skipped, not multiplied, so that the sum
                 // has the bits of a K loop that ends at the last block
                 if (s * KB + b >= KT) break;
-                u32x4 fa[MI], fb[NI];
 #pragma unroll
-                for (int i = 0; i < MI; ++i) fa[i] = frag(stage, b, 0, i * 32 + l32, wv * 2 + half);
-#pragma unroll
-                for (int j = 0; j < NI; ++j) fb[j] = frag(stage, b, A_BYTES, j * 32 + l32, wv * 2 + half);
-#pragma unroll
-                for (int i = 0; i < MI; ++i)
-#pragma unroll
-                    for (int j = 0; j < NI; ++j) Elem<T>::mma(fa[i], fb[j], acc[i][j]);
+                for (int q = 0; q < BPW; ++q) {
+                    const int blk = kb + q * G, i = blk / NI, j = blk % NI;
+                    const u32x4 fa = frag(stage, b, 0, i * 32 + l32, wv * 2 + half);
+                    const u32x4 fb = frag(stage, b, A_BYTES, j * 32 + l32, wv * 2 + half);
+                    Elem<T>::mma(fa, fb, acc[q]);
+                }
             }
         }
 
         GP_PROBE(3);
-        wide_reduce_store<T, BM, BN, NT>(g, (float *)lds_t, acc, m0, n0, offc, tid, wave, lane, kb);
+        wide_reduce_store<T, BM, BN, NT, G>(g, (float *)lds_t, acc, m0, n0, offc, tid, wv, lane, kb);
 #ifdef GP_TILE_PROF
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         GP_PROBE(5);
