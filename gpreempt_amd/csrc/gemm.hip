@@ -219,8 +219,13 @@ static const WideChoice *wide_of(int body) {
 // enough to pay for the larger first stage.  128 x 768 x 3072: 10.2 -> 7.9 us; 392 x 512 x 4608:
 // 14.0 -> 10.4; 1568 x 256 x 2304: 10.0 -> 8.3; 1568 x 256 x 1024: 6.6 -> 6.1; 128 x 768 x 768: 5.1 -> 4.7;
 // 6272 x 128 x 1152: 8.9 -> 8.0; 392 x 2048 x 512: 6.4 -> 5.9.
-static int wide_pick(const MatArgs &g, int batch, long cus) {
+static int wide_pick(const MatArgs &g, int batch, long cus, int dtype) {
     auto tiles = [&](int tm, int tn) { return (long)((g.M + tm - 1) / tm) * ((g.N + tn - 1) / tn) * batch; };
+    // fp32 runs on MFMAs an eighth as fast, so a small layer is bound by them and not by its operands: as many
+    // tiles as there are compute units to take them (ResNet-50 b1 fp32, launch to launch: 7 x 7 x 512 -> 2048
+    // 13.1 -> 6.7 us, 3 x 3 at 56 x 56 x 64 16.2 -> 9.1 us; these tiles are also what a preempted tenant
+    // finishes before it leaves)
+    if (dtype == GP_F32 && tiles(32, 32) <= cus) return g.K >= 768 ? MB_WIDE32x32_16 : MB_WIDE32x32_8;
     if (g.K >= 768 && tiles(32, 32) <= cus) return MB_WIDE32x32_16;
     if (g.K >= 768 && tiles(64, 32) <= cus) return MB_WIDE64x32_16;
     if (g.K >= 512 && tiles(64, 64) <= cus && g.N > 32) return MB_WIDE64x64_8;
@@ -259,7 +264,7 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
         // (a problem of one or two K-steps is all epilogue, i.e. memory-bound: the 128 x 128 body runs one workgroup
         // per CU, too few threads for that; 25088 x 256 x 64 with a residual: 19.8 us on 128 x 128, 15.0 on 64 x 64)
         else if (tile == 128 || (tile == 0 && tiles(128) >= cus && g.N > 64 && g.M > 64 && g.K > 128)) body = MB_PIPE128;
-        else if (tile == 0 && wide_ok && wide_pick(g, pl->batch, cus) >= 0) body = wide_pick(g, pl->batch, cus);
+        else if (tile == 0 && wide_ok && wide_pick(g, pl->batch, cus, pl->dtype) >= 0) body = wide_pick(g, pl->batch, cus, pl->dtype);
         else if (tile == 64 || (tile == 0 && (tiles(64) >= cus || g.K < 512))) body = MB_PIPE64;
         else if (tile == 0 && tiles(64) >= cus / 2) body = MB_PIPE64_SK;
         else if (tile == 0 || tile == 32) body = MB_PIPE32_SK;
