@@ -210,6 +210,9 @@ def gemm_roofline(iters=10, operands="random"):
     flag = gp.Flag()
     stream = gp.Stream(1)
     st = gp.BlpState(1, flag, 32)
+    # the first dozen launches of a process run 15-20 % slower than those after them, whichever form comes
+    # first (measured in all orders): they are warm-up, not a property of the form that is timed first
+    _time_gemm(gp, p, stream, None, 12)
     t, info = _time_gemm(gp, p, stream, st, iters)
     t_plain, _ = _time_gemm(gp, p, stream, None, iters)
     st_ck = gp.BlpState(1, flag, 32)
