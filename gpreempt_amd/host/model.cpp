@@ -224,10 +224,12 @@ Status Model::allocate_and_bind() {
     return Status::Succ;
 }
 
-// layer_norm -> dense pairs that run as one launch (gp_gemm_params::ln_gamma).  Only where the device layer
-// says the fused launch has the bits of the two (gp_gemm_ln_supported), and only for kernels launched
-// one by one without preemption arguments: a preemptible tenant keeps one launch per kernel index, which
-// is what its stop index and its claim counters speak of.
+// layer_norm -> dense pairs that run as one launch (gp_gemm_params::ln_gamma), where the device layer says the
+// fused launch has the bits of the two (gp_gemm_ln_supported).  For a preemptible tenant the fused launch
+// carries the dense layer's kernel index, claim counters and tiles: the layer-norm's index is never launched,
+// so it never appears as a stop index, its counters stay zero, and a preemption injected at it (a test hook)
+// does not fire; a run stopped inside the fused launch resumes there, and the tiles that are left redo
+// their rows (the workgroups of tile column 0 are the ones that store them).
 void Model::plan_fusions() {
     const char *env = std::getenv("GPREEMPT_FUSE_LN");
     fuse_launches_ = !(env && std::atoi(env) == 0);
@@ -440,7 +442,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         CUDA_RETURN_STATUS(gp_memcpy_d2d_async(k.args[1], k.args[0], size, stream));
         return Status::Succ;
     }
-    const bool fuse = fuse_launches_ && !k.preemptible;
+    const bool fuse = fuse_launches_;
     if (fuse && k.fused_away) return Status::Succ;  // the next kernel's prologue does this one's work
     gp_preempt_ctx ctx{};
     const gp_preempt_ctx *pc = nullptr;

@@ -77,8 +77,8 @@ public:
     double flops = 0, bytes = 0;          // algorithmic work of one launch
     // Launch fusion (Model::plan_fusions): a layer-norm whose only job before the next kernel is to feed
     // that kernel's A operand is not launched (`fused_away`); the dense layer behind it runs `ln_gemm`,
-    // the same GEMM with the layer-norm as its prologue.  The kernel list, its indices and the
-    // whole-model program keep the two-kernel form.
+    // the same GEMM with the layer-norm as its prologue (preemptible or not).  The kernel list, its
+    // indices and the whole-model program keep the two-kernel form.
     bool fused_away = false;
     bool has_ln_gemm = false;
     gp_gemm_params ln_gemm;
