@@ -297,3 +297,11 @@ def shared_concat(dt, seed=6):
     q = w.pool(w.conv2d(y, 8, 1), "global_avg")
     y = w.add(w.dense(w.flatten(w.concatenate([p, q])), 8, bias=False), w.dense(w.flatten(q), 8))
     return w, w.dense(y, 6)
+
+
+def mlp(dt, seed=7):
+    """a model whose input is a matrix: two dense layers and a softmax"""
+    w = ExportWriter(dt, seed)
+    x = w.data(w.rng.normal(0, 1, (6, 64)))
+    y = w.dense(x, 48, relu=True)
+    return w, w.softmax(w.dense(y, 16))

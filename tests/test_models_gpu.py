@@ -321,7 +321,7 @@ def test_exported_graph_next_to_the_model_is_read_and_checked(gp, ex_mod, tmp_pa
 # output with the oracle's operators while it writes.
 
 @pytest.mark.parametrize("dt", ["f32", "f16"])
-@pytest.mark.parametrize("maker", ["mini_resnet", "mini_vgg", "padded_channels", "shared_concat", "densenet"])
+@pytest.mark.parametrize("maker", ["mini_resnet", "mini_vgg", "padded_channels", "shared_concat", "densenet", "mlp"])
 def test_exported_model_matches_oracle(gp, ex_mod, tmp_path, maker, dt):
     import export_writer as EW
     w, head = getattr(EW, maker)(dt)
