@@ -118,3 +118,32 @@ def test_trace_load_serves_the_newest_arrival(gp):
     n = rep["tasks"]["hp"]["requests"]
     assert 7 <= n <= 11, n  # the burst at 200 ms collapses; nothing is served after the end
     assert rep["tasks"]["be"]["requests"] > 10
+
+
+def test_exported_model_as_best_effort_tenant(gp, tmp_path):
+    """A model directory in the reference's export format (plus the operator sidecar) takes the place of a
+    built-in workload name in a task file: it is preempted by the high-priority tenant and every one of its
+    outputs afterwards has the bits of its output when run alone."""
+    import os
+    import export_writer as EW
+    from gpreempt_amd import executor as gx
+    w, head = EW.resnet("f16", (1, 1, 1, 1), batch=4, hw=96)
+    w.write(str(tmp_path / "exported_net"), head)
+    os.environ["GPREEMPT_MODEL_PATH"] = str(tmp_path)
+    cfg = {
+        "time": 2.0, "policy": "wb-chunk-async", "hp_requests": 40, "warmups": 3, "standalone_runs": 10, "verify_outputs": True,
+        "tasks": [
+            {"id": "hp", "load": {"type": "poisson", "frequency": 400, "seed": 3},
+             "client": {"name": "hp", "model_name": "bert@layers=2", "priority": 0, "use_cuda_graph": False, "launch_mode": "launch", "preprocess_time": 0}},
+            {"id": "be", "load": {"type": "continuous"},
+             "client": {"name": "be", "model_name": "exported_net", "priority": 1, "use_cuda_graph": False, "launch_mode": "launch", "preprocess_time": 0}},
+        ],
+    }
+    buf = C.create_string_buffer(1 << 20)
+    rc = gx.lib().gpx_run_scenario(json.dumps(cfg).encode(), buf, C.c_size_t(len(buf)))
+    assert rc == 0, buf.value[:400]
+    rep = json.loads(buf.value.decode())
+    hp, be = rep["tasks"]["hp"], rep["tasks"]["be"]
+    assert hp["requests"] >= 40 and be["requests"] > 0 and be["preemptions"] > 0
+    assert be["kernels"] == 1 + 1 + 1 + 4 * 4 + 1 + 1 + 1   # layout, stem, pool, four blocks of four convolutions, pool, classifier, softmax
+    assert hp["outputMismatches"] == 0 and be["outputMismatches"] == 0
