@@ -428,3 +428,41 @@ def test_fused_attention_preempt_resume_bit_exact(gp):
     gp.launch("gp_launch_attention", p, st.ctx(max_workgroups=4))
     sync(gp)
     assert np.array_equal(do.download(), want)
+
+
+def test_deep_preemptible_convolution_takes_small_tiles_with_the_same_bits(gp):
+    """A preemptible launch finishes the tiles it holds before it leaves: where the rule would run 128 x 128 tiles
+    over K >= 2304 (VGG-16's 256 -> 256 layers at 56 x 56), a launch with claim counters takes 64 x 64 tiles,
+    and the result has the bits of the plain launch; stopped and resumed, still the same.  A tile chosen by
+    the caller is respected."""
+    rng = np.random.default_rng(11)
+    N, H, Cc = 16, 56, 256
+    x = O.round_to(rng.normal(0, 1, (N, Cc, H, H)).astype(np.float32), "f16")
+    w = O.round_to((rng.normal(0, 1, (Cc, Cc, 3, 3)) * 0.03).astype(np.float32), "f16")
+    bias = O.round_to(rng.normal(0, 0.1, Cc).astype(np.float32), "f16")
+    plain, info, (p, do, keep) = gpu_conv2d(gp, "f16", x, w, bias, 1, 1, act=gp.ACT_RELU)
+    M = N * H * H
+    assert info.total_tiles == (M // 128) * (Cc // 128)
+    base = do.download().copy()
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag, 32)
+    do.fill32(0)
+    info = gp.launch("gp_launch_conv2d", p, st.ctx(fresh=1))
+    sync(gp)
+    assert info.total_tiles == (M // 64) * (Cc // 64)
+    assert np.array_equal(do.download(), base)
+    for frac in (0.2, 0.7):
+        st.reset(); st.clear_stop(); flag.set(0)
+        do.fill32(0)
+        gp.launch("gp_launch_conv2d", p, st.ctx(inject_at=int(frac * info.total_tiles), fresh=1))
+        sync(gp)
+        assert flag.get() == 1 and not np.array_equal(do.download(), base)
+        flag.set(0); st.clear_stop()
+        gp.launch("gp_launch_conv2d", p, st.ctx())
+        sync(gp)
+        assert np.array_equal(do.download(), base), frac
+    p.tile_m = p.tile_n = 128
+    st.reset(); st.clear_stop()
+    info = gp.launch("gp_launch_conv2d", p, st.ctx(fresh=1))
+    sync(gp)
+    assert info.total_tiles == (M // 128) * (Cc // 128) and np.array_equal(do.download(), base)
