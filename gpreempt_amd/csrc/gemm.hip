@@ -127,8 +127,8 @@ static int pipe_case_ckpt(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_strea
 // Ring depth of a wide body: three stages, four for the GEMM form of the 32 x 32 tile on 16 wavefronts (a
 // stage is (WAVES / 4) K-blocks of BM + BN rows of 128 bytes: 32 KB there).  128 x 768 x 3072 went from
 // 7.96 to 7.67 us per launch with the fourth stage; given to every body that has room for it, it cost the
-// convolution chain of ResNet-152 1 us per launch (10.2 -> 11.2); two stages instead of three for the
-// convolution form changed nothing (10.27 either way).
+// convolution chain of ResNet-152 1 us per launch (10.2 -> 11.2), and so did two stages instead of three for
+// the convolution form (10.05 -> 10.98).
 constexpr int wide_stages(int bm, int bn, int waves, bool conv) { return (!conv && bm == 32 && bn == 32 && waves == 16) ? 4 : 3; }
 template <typename T, int BM, int BN, int WAVES, bool CONV = false>
 using WideK = WideKernel<T, BM, BN, WAVES, wide_stages(BM, BN, WAVES, CONV), CONV>;
@@ -147,7 +147,14 @@ static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream 
             if (ctx && ctx->ckpt) return launch_mat<PipeKernel<T, 256, 256, 2, false, false, true, GP_W256>>(pl, ctx, s, info);
             return launch_mat<PipeKernel<T, 256, 256, 2, false, false, false, GP_W256>>(pl, ctx, s, info);
         case MB_PIPE128: return pipe_case_ckpt<T, 128, GP_S128>(pl, ctx, s, info);
-        case MB_PIPE64: return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
+        case MB_PIPE64:
+            // A layer of at most four K-steps is all prologue and epilogue, and what hides those is more workgroups
+            // per compute unit: with a ring of two stages (32 KB of LDS instead of 64) four fit instead of two.
+            // 25088 x 256 x 64 with a residual (ResNet-152 b8, 56 x 56): 15.5 -> 10.7 us plain, 19.4 -> 13.6 us
+            // preemptible; 6272 x 512 x 128: 10.0 -> 7.6 us.  Deep layers keep four stages (K = 4608 on 392 tiles:
+            // 22.5 us with four, 38.6 with two).
+            if (pl.g.K <= 256) return pipe_case<T, 64, 2, false>(pl, ctx, s, info);
+            return pipe_case<T, 64, GP_S64, false>(pl, ctx, s, info);
         case MB_PIPE64_SK: return pipe_case<T, 64, GP_S64, true>(pl, ctx, s, info);
         case MB_PIPE32_SK: return pipe_case<T, 32, GP_S32, true>(pl, ctx, s, info);
         case MB_WIDE32x32_16: return wide_case<T, 32, 32, 16>(pl, ctx, s, info);
