@@ -88,9 +88,14 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
             blp->spare = 4;
             *grid += 4;
         }
+        // where claims go through several counters, counters 0..3 read the flag; the others need the
+        // lengths of those four slices to tell when to take over (reads_flag in tile_loop.hpp)
+        for (int g = 0; g < 4; ++g)
+            blp->poll_n[g] = ng > 1 && g < ng ? group_slice_begin((int)total, g + 1, ng, *grid) - group_slice_begin((int)total, g, ng, *grid) : 0;
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
         blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0; blp->spare = 0;
+        for (int g = 0; g < 4; ++g) blp->poll_n[g] = 0;
         *grid = (int)total;
     }
     if (info) {

@@ -55,6 +55,7 @@ struct BlpArgs {
     int tiles;        // number of tiles (total = ceil(tiles / batch) claims)
     int fresh;        // the host vouches that no claim of this kernel has been made since its counters were cleared
     int spare;        // fixed claims only: the last `spare` workgroups of the grid have no claim and read the flag
+    int poll_n[4];    // several counters, claims through them: the number of claims in the slices of counters 0..3
 };
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
@@ -109,6 +110,19 @@ __device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy, int orde
 // kernel of the same submission leaves too until the host re-arms it, even if the flag has been
 // lowered in between; otherwise a kernel queued behind a stopped one could run to completion on
 // incomplete inputs.
+//
+// Who reads the flag: with several counters, the first four groups do, for everybody.  Their slices
+// end when everybody's do, give or take the skew between XCDs (all four are served by XCD 0), and a
+// relaunch may find them handed out while other slices are not.  So a group beyond the four reads
+// the flag at the same cadence once the counter of its counterpart among them (grp & 3) has passed
+// the end of that group's slice (BlpArgs::poll_n, from the host: the slice arithmetic is too much
+// code for every kernel to carry); until then it pays one more read of device memory on those claims.
+__device__ __forceinline__ bool reads_flag(const BlpArgs &b, int grp) {
+    if (grp < 4 || b.poll_mask == 0) return true;   // (poll_mask == 0: the flag is cheap device memory)
+    const int g = grp & 3;
+    return __hip_atomic_load(b.executed + g * COUNTER_STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= b.poll_n[g];
+}
+
 __device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_lo, int slice_n) {
     int claim = -1;
     int stop = __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
@@ -118,9 +132,7 @@ __device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_l
             claim = slice_lo + c;
             if (claim == b.inject_at && b.flag)
                 __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            // with several counters only the first four groups read the flag, unless it is read on
-            // every claim (poll_mask == 0: the flag is cheap device memory)
-            if ((grp < 4 || b.poll_mask == 0) && (c & b.poll_mask) == 0 && b.flag &&
+            if ((c & b.poll_mask) == 0 && b.flag && reads_flag(b, grp) &&
                 __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
                 atomicCAS(b.stop_index, -1, b.kernel_id);
             // the polling workgroup still owes the tile it has just claimed

@@ -198,6 +198,51 @@ def test_flag_set_before_launch(gp):
         gp.launch("gp_launch_gemm", p, st.ctx(poll_every=3))
 
 
+def test_flag_is_seen_after_the_first_four_counter_groups_ran_out(gp):
+    """With 32 claim counters the first four groups read the flag for everybody.  A relaunch that finds their
+    slices handed out (here: their counters set past the end by the test) while the flag is up must still
+    stop: the other groups take the reading over.  Lowering the flag and relaunching completes the work
+    with the bits of an uninterrupted run."""
+    rng = np.random.default_rng(21)
+    M = N = 4096
+    K = 256
+    A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), "f16")
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32), "f16")
+    dA, dB = (gp.DevBuf.from_array(x, gp.F16) for x in (A, B))
+    dC = gp.DevBuf(2 * M * N)
+    p = gp.GemmParams(dtype=gp.F16, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, alpha=1.0, batch=1,
+                      tile_m=64, tile_n=64)
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    base = dC.download().copy()
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag, 32)   # fewer workgroups than tiles below, so that claims go through the counters
+    S = st.COUNTER_STRIDE
+    gone = np.zeros(32 * S, np.int32)
+    gone[[0, S, 2 * S, 3 * S]] = 1 << 20
+    st.executed.upload(gone)
+    flag.set(1)
+    dC.fill32(0)
+    info = gp.launch("gp_launch_gemm", p, st.ctx(max_workgroups=512))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert info.total_tiles == 4096 and info.grid < info.total_tiles and info.fixed_claims == 0
+    assert st.stop_index() == 0
+    c = st.counters()[::S]
+    # the first claim of every group has a number that reads the flag: at most one tile per workgroup
+    assert 0 < int(c[4:].sum()) <= info.grid, c
+    assert not np.array_equal(dC.download(), base)
+    # the four groups get their slices back; the flag comes down; the relaunch finishes everything
+    now = st.counters()
+    now[[0, S, 2 * S, 3 * S]] = 0
+    st.executed.upload(now)
+    flag.set(0)
+    st.clear_stop()
+    gp.launch("gp_launch_gemm", p, st.ctx(max_workgroups=512))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert st.stop_index() == -1
+    assert np.array_equal(dC.download(), base)
+
+
 def test_fixed_claims_of_a_one_claim_per_workgroup_launch(gp):
     """With several counters per kernel and at least as many workgroups as claims, a workgroup's
     claim is fixed by its index and a bit per workgroup (ints 1..15 of the counter's line) says

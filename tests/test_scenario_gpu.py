@@ -28,17 +28,20 @@ def _run(policy, hp_requests=60, be_mode="program", hp_model="bert", be_model="r
 
 @pytest.mark.parametrize("policy", ["wb", "wb-async", "wb-chunk", "wb-chunk-async"])
 def test_preempting_policies_serve_hp_and_preempt_be(gp, policy):
-    rep = _run(policy)
+    rep = _run(policy, hp_requests=200)
     hp, be = rep["tasks"]["hp"], rep["tasks"]["be"]
     assert rep["policy"] == policy
-    assert hp["requests"] >= 60
+    assert hp["requests"] >= 200
     assert be["requests"] > 0
     assert be["preemptions"] > 0, "the best-effort tenant was never interrupted"
     assert rep["preemptLatency(us)"]["count"] > 0
     # a drain is bounded by queued kernels x launch turnaround: far below a millisecond here
     assert 0 < rep["preemptLatency(us)"]["p50"] < 1000
-    # co-run latency stays within a small factor of the isolated latency (np is ~50x on this pair)
-    assert 0.5 < rep["hp_p99_vs_isolated"] < 4.0, rep["hp_p99_vs_isolated"]
+    # co-run latency stays within a small factor of the isolated latency (np is ~50x on this pair): the
+    # typical request tightly, the tail (arrivals queue behind one another at 300 Hz, and 1 request in 100
+    # is two requests here) loosely
+    assert hp["inferLatency(us)"]["p50"] < 2.5 * hp["standAloneTotalLatency(us)"], (hp["inferLatency(us)"], hp["standAloneTotalLatency(us)"])
+    assert 0.5 < rep["hp_p99_vs_isolated"] < 8.0, rep["hp_p99_vs_isolated"]
     assert hp["preemptions"] == 0
 
 

@@ -63,8 +63,11 @@ def test_noalloc_gemm_preempt_and_resume(gp):
     the uninterrupted run; another slot is untouched by it."""
     flag = gp.Flag()
     stop_out = gp.DevBuf(4)
-    p, dC, bufs, ref, dtype = _problem(gp, "f16", 4096, 4096, 256, 5)
-    p.tile_m = p.tile_n = 64  # 4096 tiles: more than the GPU holds at once, claims go through the counters
+    # 4096 tiles, more than the GPU holds at once, so claims go through the counters; deep enough that the
+    # tiles left after the injection outlast the flag's trip through host memory.  Claim 2064 is the 16th
+    # of 128 in its counter's slice: the flag goes up with most of every slice still to be handed out.
+    p, dC, bufs, ref, dtype = _problem(gp, "f16", 4096, 4096, 1024, 5)
+    p.tile_m = p.tile_n = 64
     flag.set(0)
     gp.launch("gp_launch_gemm", p)
     gp.check(gp.lib().gp_stream_sync(None))
@@ -72,7 +75,7 @@ def test_noalloc_gemm_preempt_and_resume(gp):
     for slot in (3, 63):
         dC.fill32(0)
         flag.set(0)
-        info = _noalloc(gp, p, flag, slot, CLEAR | REARM, 2000, stop_out)
+        info = _noalloc(gp, p, flag, slot, CLEAR | REARM, 2064, stop_out)
         gp.check(gp.lib().gp_stream_sync(None))
         assert flag.get() == 1 and stop_out.download(np_dtype=np.int32)[0] == slot
         assert not np.array_equal(dC.download(), want), "the kernel was not interrupted"
