@@ -59,7 +59,8 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
         blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;
         blp->kernel_id = ctx->kernel_id; blp->inject_at = ctx->inject_at;
-        blp->fresh = ctx->fresh != 0;
+        GP_REQUIRE(ctx->fresh >= 0 && ctx->fresh <= 2, "fresh is 0, 1 or 2");
+        blp->fresh = ctx->fresh;
         int pe = ctx->poll_every > 0 ? ctx->poll_every : 8;
         GP_REQUIRE((pe & (pe - 1)) == 0, "poll_every must be a power of two");
         blp->poll_mask = pe - 1;

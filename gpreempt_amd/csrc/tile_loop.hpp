@@ -53,7 +53,7 @@ struct BlpArgs {
     void *ckpt;       // checkpoint workspace of kernels that can leave a tile half-way, or nullptr
     int batch;        // tiles per claim (>= 1): a claim of index u stands for tiles [u*batch, (u+1)*batch)
     int tiles;        // number of tiles (total = ceil(tiles / batch) claims)
-    int fresh;        // the host vouches that no claim of this kernel has been made since its counters were cleared
+    int fresh;        // nonzero: the host vouches that no claim of this kernel has been made since its counters were cleared; 2: eager start (tile_fixed_early)
     int spare;        // fixed claims only: the last `spare` workgroups of the grid have no claim and read the flag
     int poll_n[4];    // several counters, claims through them: the number of claims in the slices of counters 0..3
 };
@@ -156,9 +156,10 @@ __device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_l
 // operand load of every launch).
 static_assert(kFixedClaimBits == (COUNTER_STRIDE - 1) * 32, "a bit per workgroup in ints 1..15 of the counter's line");
 
+template <bool LOOK = true>
 __device__ __forceinline__ int claim_fixed(const BlpArgs &b, int grp) {
     if ((int)blockIdx.x >= b.total) return -1;
-    if (__hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1) return -1;
+    if (LOOK && __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1) return -1;
     const int j = (int)blockIdx.x >> log2_pow2(b.groups);  // this workgroup's rank among those of its group
     int *line = b.executed + grp * COUNTER_STRIDE;
     const int bit = 1 << (j & 31);
@@ -274,11 +275,35 @@ __device__ __forceinline__ void unclaim_fixed(const BlpArgs &b) {
     __hip_atomic_fetch_and(line + 1 + (j >> 5), ~(1 << (j & 31)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_fetch_add(line, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+//
+// Eager start (BlpArgs::fresh == 2).  On a kernel's first launch after its counters were cleared
+// nothing has to come back from memory before the tile starts: the claim is known from the
+// workgroup's number, its bit cannot be set yet, and the body's look at the stop word, which travels
+// with the first operands, stands in for the look in front of the claim.  The bit and the count go
+// out without waiting for their old values and are withdrawn like any claim if the body finds the
+// stop recorded.  A launch saves the wait for the stop index that way (0.2 us of a 10 us
+// convolution); a kernel queued behind a stop leaves a first operand fetch later than it would
+// have, which adds 4 us to the drain of a chunk of launches.  That trade is the caller's.
+// Everything the body is handed is computed from kernel arguments and the workgroup's number alone:
+// a stop word that reaches the body in a vector register (a value merged from two branches does)
+// makes the compiler treat the body's control flow as divergent, and the body, whose barriers and
+// hand-placed waits assume uniform flow, then computes garbage for K of one step.
 template <class Body>
 __device__ __forceinline__ void tile_fixed_early(const BlpArgs &b, Body &&body) {
-    const int idx = fixed_claim_of_workgroup(b);
+    const bool eager = b.fresh > 1;
+    int idx;
+    if (eager) {
+        const bool leader = threadIdx.x == 0;
+        if (spare_workgroup(b, true, leader)) return;
+        if ((int)blockIdx.x >= b.total) return;
+        if (leader) claim_fixed<false>(b, wg_group((int)blockIdx.x, b.groups));
+        idx = xcd_contiguous((int)blockIdx.x, b.total);
+    } else {
+        idx = fixed_claim_of_workgroup(b);
+    }
     if (idx < 0) return;
-    const bool left = body(decode_tile(idx, b.sx, b.sy, b.order), b.spare ? b.stop_index : nullptr);
+    int *word = (eager || b.spare) ? b.stop_index : nullptr;
+    const bool left = body(decode_tile(idx, b.sx, b.sy, b.order), word);
     if (left && threadIdx.x == 0) unclaim_fixed(b);
 }
 

@@ -233,6 +233,8 @@ Status Model::allocate_and_bind() {
 void Model::plan_fusions() {
     const char *env = std::getenv("GPREEMPT_FUSE_LN");
     fuse_launches_ = !(env && std::atoi(env) == 0);
+    env = std::getenv("GPREEMPT_EAGER_TILES");
+    eager_tiles_ = !(env && std::atoi(env) == 0);
     for (size_t i = 0; i + 1 < kernel_infos.size(); ++i) {
         KernelInfo &ln = kernel_infos[i], &mm = kernel_infos[i + 1];
         ln.fused_away = false; mm.has_ln_gemm = false;
@@ -456,7 +458,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.max_workgroups = 0;
         ctx.poll_every = poll_every_;
         ctx.counter_groups = counter_groups_;
-        ctx.fresh = idx < fresh_.size() && fresh_[idx];
+        ctx.fresh = idx < fresh_.size() && fresh_[idx] ? (eager_tiles_ ? 2 : 1) : 0;
         ctx.ckpt = ckpt_;
         ctx.ckpt_bytes = ckpt_bytes_;
         pc = &ctx;

@@ -196,6 +196,7 @@ private:
     Status allocate_and_bind();
     void plan_fusions();
     bool fuse_launches_ = true;  // GPREEMPT_FUSE_LN=0 in the environment keeps every launch of the kernel list
+    bool eager_tiles_ = true;    // first launches start their tiles before the stop index has come back (gp_preempt_ctx::fresh = 2); GPREEMPT_EAGER_TILES=0 makes them wait for it
     Status upload_param(size_t idx, const float *disk, size_t n);
     void bind_pointers(KernelInfo &k);
 };

@@ -243,6 +243,41 @@ def test_flag_is_seen_after_the_first_four_counter_groups_ran_out(gp):
     assert np.array_equal(dC.download(), base)
 
 
+@pytest.mark.parametrize("K", [64, 128, 256])
+@pytest.mark.parametrize("N,res", [(256, True), (64, False)])
+def test_shallow_gemm_plain_and_preemptible_launches_agree(gp, N, K, res):
+    """One to four K-steps over many rows (the first pointwise layers of a CNN at batch 8): the 64 x 64 body
+    with its two-stage ring, launched plainly, with fixed claims on fresh counters (waiting for the stop
+    index, and starting the tile without waiting) and on counters that may hold claims; each against the
+    oracle and all four with the same bits."""
+    M = 8192
+    rng = np.random.default_rng(K + N)
+    A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), "f16")
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32), "f16")
+    bias = O.round_to(rng.uniform(-1, 1, N).astype(np.float32), "f16")
+    R = O.round_to(rng.uniform(-1, 1, (M, N)).astype(np.float32), "f16")
+    dA, dB, db, dR = (gp.DevBuf.from_array(x, gp.F16) for x in (A, B, bias, R))
+    dC = gp.DevBuf(2 * M * N)
+    p = gp.GemmParams(dtype=gp.F16, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, bias=db.ptr,
+                      residual=dR.ptr if res else None, ldr=N, alpha=1.0, act=gp.ACT_RELU, batch=1)
+    ref = O.gemm_bias_act(A, B, bias, act=O.ACT_RELU, b_is_nk=True, residual=R if res else None)
+    flag = gp.Flag()
+    flag.set(0)
+    outs = []
+    for fresh in (None, 1, 2, 0):
+        dC.fill32(0)
+        if fresh is None:
+            gp.launch("gp_launch_gemm", p)
+        else:
+            st = gp.BlpState(1, flag, 32)
+            info = gp.launch("gp_launch_gemm", p, st.ctx(fresh=fresh))
+            assert info.fixed_claims == 1
+        gp.check(gp.lib().gp_stream_sync(None))
+        outs.append(dC.download().copy())
+        assert rel_err(gp.from_storage(outs[-1], gp.F16).reshape(M, N), ref) < 1e-2, fresh
+    assert all(np.array_equal(outs[0], o) for o in outs[1:])
+
+
 def test_fixed_claims_of_a_one_claim_per_workgroup_launch(gp):
     """With several counters per kernel and at least as many workgroups as claims, a workgroup's
     claim is fixed by its index and a bit per workgroup (ints 1..15 of the counter's line) says

@@ -244,11 +244,15 @@ def test_bert_preempt_resume_bit_exact(gp, ex_mod, tmp_path):
     _blp_roundtrip(gp, ex_mod, tmp_path, "bert", ids, [(0, 3), (2, 17), (58, 0), (-1, 10)])
 
 
-@pytest.mark.parametrize("program", [False, True])
-def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path, program):
+@pytest.mark.parametrize("program,eager", [(False, True), (True, True), (False, False)])
+def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path, program, eager, monkeypatch):
     """src/tests/test-dnn-blp.cpp:36-42 verbatim: execute; set the flag from the host right
-    away; sync; clear; resume; sync.  Where the flag lands is up to timing; the result is not."""
+    away; sync; clear; resume; sync.  Where the flag lands is up to timing; the result is not.
+    (eager, the default: first launches start their tiles before the stop index has come back;
+    GPREEMPT_EAGER_TILES=0 makes them wait for it)"""
     root = str(tmp_path)
+    if not eager:
+        monkeypatch.setenv("GPREEMPT_EAGER_TILES", "0")
     x = gp.to_storage(np.full((8, 3, 224, 224), 10.0, np.float32), gp.F16)  # the reference's all-10.0 image
     base = ex_mod.Executor("resnet152", model_root=root)
     base.set_input("data", x)
