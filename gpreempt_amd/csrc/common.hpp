@@ -89,6 +89,11 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
             blp->spare = 4;
             *grid += 4;
         }
+        // An eager start (fresh = 2, tile_fixed_early) makes a kernel queued behind a stop leave one operand
+        // fetch later per round of workgroups: kept for launches whose workgroups all start at once, where that
+        // is half a microsecond; a launch of several rounds waits for the stop index as before (VGG-16 b16 next
+        // to two higher levels: drain 41 / 77 us mean / p99 with the wait, 48 / 94 without).
+        if (blp->fresh > 1 && (long)*grid > resident) blp->fresh = 1;
         // where claims go through several counters, counters 0..3 read the flag; the others need the
         // lengths of those four slices to tell when to take over (reads_flag in tile_loop.hpp)
         for (int g = 0; g < 4; ++g)

@@ -130,7 +130,8 @@ typedef struct gp_preempt_ctx {
                      /* for the old values; 0 is always safe.  Clear all 16 ints of every counter.     */
                      /* 2: as 1, and the GEMM and convolution bodies start their tile without waiting   */
                      /* for the stop index (they look at it when their first operands have landed):     */
-                     /* shorter launches, a longer drain of launches queued behind a stop.              */
+                     /* shorter launches, a longer drain of launches queued behind a stop.  Honoured    */
+                     /* for launches whose workgroups all start at once; others behave as with 1.       */
     int *left_host;  /* programs only, may be NULL: device-visible address of a gp_flag_create    */
                      /* word; the last workgroup to leave a launch stores that launch's number    */
                      /* (info->shape[1] of gp_program_launch) there, so the host learns that the  */
