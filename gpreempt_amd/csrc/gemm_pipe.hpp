@@ -134,7 +134,9 @@ struct PipeKernel {
                                                int tile_index = 0, int kt0 = 0) {
         GP_PROBE(0);
         __shared__ int early_slot[64];  // landing place of the early-stop word (lane 0's dword)
-        const bool early = !CKPT && cc.stop_index != nullptr;
+        // (made wave-uniform by force: handed over in a vector register, the word would make the compiler treat every branch
+        // that depends on it as divergent, and the barriers and hand-placed waits below assume uniform control flow)
+        const bool early = !CKPT && __builtin_amdgcn_readfirstlane((int)(cc.stop_index != nullptr)) != 0;
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
         const int tid = threadIdx.x, lane = tid & 63;

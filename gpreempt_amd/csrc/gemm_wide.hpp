@@ -170,7 +170,7 @@ struct WideKernel {
     static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0}) {
         GP_PROBE(0);
         __shared__ int early_slot[64];
-        const bool early = cc.stop_index != nullptr;
+        const bool early = __builtin_amdgcn_readfirstlane((int)(cc.stop_index != nullptr)) != 0;
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
         const int tid = threadIdx.x, lane = tid & 63;
