@@ -228,8 +228,9 @@ def test_flag_is_seen_after_the_first_four_counter_groups_ran_out(gp):
     assert info.total_tiles == 4096 and info.grid < info.total_tiles and info.fixed_claims == 0
     assert st.stop_index() == 0
     c = st.counters()[::S]
-    # the first claim of every group has a number that reads the flag: at most one tile per workgroup
-    assert 0 < int(c[4:].sum()) <= info.grid, c
+    # the first claim of every group has a number that reads the flag: about one tile per workgroup (a second
+    # one where a tile ends before the read of host memory has come back), of the 3584 these groups own
+    assert 0 < int(c[4:].sum()) <= 2 * info.grid, c
     assert not np.array_equal(dC.download(), base)
     # the four groups get their slices back; the flag comes down; the relaunch finishes everything
     now = st.counters()
