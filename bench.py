@@ -25,6 +25,7 @@ sys.path.insert(0, ROOT)
 
 PEAK = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}  # dense MFMA TFLOP/s, MI355X
 HBM_PEAK_GBS = 8000.0
+CORUN_DISCARD = 5  # co-run requests of the high-priority tenant served before the counted ones
 # HBM bytes per launch of the dominant kernel, from two `rocprofv3 --pmc` runs of
 # `bench.py --only roofline` (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads
 # for the copy of `--only copycal`); the figures and commands are in the hbm_traffic summary
@@ -32,7 +33,7 @@ HBM_PEAK_GBS = 8000.0
 HBM_TRAFFIC_PER_LAUNCH = {("resnet152", "f16"): 10.57e6}
 
 
-def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
+def scenario(steps, warmup, policy, hp_rate, be_model, hp_model, extra=None):
     """Two tenants through the C++ harness (gpx_run_scenario).  The high-priority tenant submits
     launch by launch (it is never preempted and plain launches are its fastest path); the
     best-effort tenant runs as one persistent, preemptible program kernel, except under
@@ -43,6 +44,10 @@ def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
     cfg = {
         "time": max(5.0, 4.0 * steps / hp_rate), "policy": policy, "hp_requests": steps,
         "warmups": warmup, "standalone_runs": 300,
+        # the first co-run requests find a cold best-effort tenant and cold caches (0.60 ms against 0.52-0.57 ms for
+        # every later one): they are served but not counted, as DISB lets a run settle before it measures
+        # (third_party/disb/include/benchmark.h:41); `steps` requests are counted after them
+        "corun_discard": CORUN_DISCARD,
         "tasks": [
             {"id": "hp", "load": {"type": "poisson", "frequency": hp_rate, "seed": 2025},
              "client": {"name": "hp", "model_name": hp_model, "priority": 0, "use_cuda_graph": False, "launch_mode": "launch", "preprocess_time": 0}},
@@ -50,6 +55,12 @@ def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
              "client": {"name": "be", "model_name": be_model, "priority": 1, "use_cuda_graph": True, "launch_mode": "program", "preprocess_time": 0}},
         ],
     }
+    cfg.update(extra or {})
+    return run_config(cfg)
+
+
+def run_config(cfg):
+    from gpreempt_amd import executor as gx
     buf = C.create_string_buffer(1 << 20)
     rc = gx.lib().gpx_run_scenario(json.dumps(cfg).encode(), buf, C.c_size_t(len(buf)))
     if rc != 0:
@@ -57,11 +68,44 @@ def scenario(steps, warmup, policy, hp_rate, be_model, hp_model):
     return json.loads(buf.value.decode())
 
 
+def config_leg(name, seconds):
+    """One of the scenario files under gpreempt_amd/config/ (BASELINE configs 4 and 5) for a bounded time:
+    high-priority p99 against isolated, preemption latency, and what every lower level kept."""
+    with open(os.path.join(ROOT, "gpreempt_amd", "config", name)) as f:
+        cfg = json.load(f)
+    cfg.update({"time": seconds, "standalone_runs": 60, "warmups": 5})
+    rep = run_config(cfg)
+    out = {"config": name, "seconds": seconds, "policy": rep["policy"], "hp_p99_vs_isolated": rep["hp_p99_vs_isolated"],
+           "preemption_latency_us": {k: rep["preemptLatency(us)"][k] for k in ("count", "mean", "p99", "max")},
+           "be_throughput_kept": rep["be_throughput_kept"], "levels": {}}
+    for tid, t in rep["tasks"].items():
+        e = {"priority": t["priority"], "model": t["model"], "requests": t["requests"], "req_s": t["avgThroughput(req/s)"],
+             "isolated_ms": t["standAlone(us)"]["mean"] / 1e3, "p99_ms": t["totalLatency(us)"]["p99"] / 1e3, "preemptions": t["preemptions"]}
+        if "throughput_kept" in t:
+            e["throughput_kept"] = t["throughput_kept"]
+            e["isolated_req_s"] = t["standAloneThroughput(req/s)"]
+        if "p99_vs_isolated" in t:
+            e["p99_vs_isolated"] = t["p99_vs_isolated"]
+        out["levels"][tid] = e
+    return out
+
+
+def stamps_leg(steps, warmup, policy, hp_rate, be_model, hp_model):
+    """The headline scenario once more with the GPU's own time stamps switched on (a measurement mode: the kernels
+    of the best-effort tenant write the device clock when the stop is recorded, when their last workgroup leaves
+    and at the first claim after a resubmission), next to the host-clock figure of the same run."""
+    rep = scenario(steps, warmup, policy, hp_rate, be_model, hp_model, {"device_stamps": True})
+    ds = rep.get("deviceStamps(us)", {})
+    return {"requests": rep["tasks"]["hp"]["requests"],
+            "host_flagStore_to_streamIdle_us": {k: rep["preemptLatency(us)"][k] for k in ("count", "mean", "p99", "max")},
+            **{k: {q: v[q] for q in ("count", "mean", "p50", "p99", "max")} for k, v in ds.items()}}
+
+
 def summarize(rep):
     hp, be = rep["tasks"]["hp"], rep["tasks"]["be"]
     return {
         "hp_p99_vs_isolated": rep["hp_p99_vs_isolated"],
-        "hp_requests": hp["requests"],
+        "hp_requests": hp["requests"], "hp_requests_served_before_counting": hp.get("discardedRequests", 0),
         "hp_isolated_ms": {k: hp["standAlone(us)"][k] / 1e3 for k in ("mean", "p50", "p99")},
         "hp_corun_ms": {k: hp["totalLatency(us)"][k] / 1e3 for k in ("mean", "p50", "p99", "max")},
         "hp_throughput_req_s": hp["avgThroughput(req/s)"],
@@ -69,7 +113,8 @@ def summarize(rep):
         "be_throughput_kept": rep["be_throughput_kept"],
         "be_throughput_req_s": be["avgThroughput(req/s)"], "be_isolated_req_s": be["standAloneThroughput(req/s)"],
         "be_preemptions": be["preemptions"], "hp_busy_fraction": rep["hp_busy_fraction"],
-        "hp_kernels": hp["kernels"], "be_kernels": be["kernels"]}
+        "hp_kernels": hp["kernels"], "be_kernels": be["kernels"],
+        "hp_first_corun_latencies_ms": [round(v / 1e3, 4) for v in hp.get("firstLatencies(us)", [])[:24]]}
 
 
 def probe(workload, trials):
@@ -85,6 +130,7 @@ def probe(workload, trials):
             "isolated_ms": r["isolated(us)"]["mean"] / 1e3,
             "preemption_latency_us": {k: r["preemptLatency(us)"][k] for k in ("mean", "p50", "p99", "max")},
             "resume_call_us": {k: r["resumeCall(us)"][k] for k in ("mean", "p99", "max")},
+            "device_stamps_us": {k: {q: v[q] for q in ("count", "mean", "p99", "max")} for k, v in r.get("deviceStamps(us)", {}).items()},
             "slowest_kernels": [{"kernel": k["kernel"], "name": k["name"], "preempt_max_us": k["preempt_max(us)"]} for k in worst]}
 
 
@@ -502,6 +548,42 @@ def hp_request(model, runs=50):
     return {"model": model, "kernels_in_list": ex.kernel_num(), "runs": runs, "device_ms": {"p50": ts[len(ts) // 2], "min": ts[0], "max": ts[-1]}}
 
 
+def summary_of(out):
+    """The figures the legs above produced, once more in a few hundred characters at the END of the line."""
+    r2 = lambda v: round(v, 2)
+    r3 = lambda v: round(v, 3)
+    s = {}
+    h = out.get("headline_600")
+    if h:
+        s["headline_600"] = {"value": r3(h["value"]), "hp_p99_ms_isolated_corun": [r3(h["hp_isolated_ms"]["p99"]), r3(h["hp_corun_ms"]["p99"])],
+                             "preempt_us_mean_p99": [r2(h["preemption_latency_us"]["mean"]), r2(h["preemption_latency_us"]["p99"])],
+                             "be_kept": r3(h["be_throughput_kept"]), "be_req_s_corun_isolated": [r2(h["be_throughput_req_s"]), r2(h["be_isolated_req_s"])]}
+    for key, tag in (("config4_three_tenants", "config4"), ("config5_bert384_over_gemm8192", "config5")):
+        c = out.get(key)
+        if c:
+            s[tag] = {"hp_p99_vs_isolated": r3(c["hp_p99_vs_isolated"]), "preempt_us_mean_p99": [r2(c["preemption_latency_us"]["mean"]), r2(c["preemption_latency_us"]["p99"])],
+                      "kept": {k: r3(v["throughput_kept"]) for k, v in c["levels"].items() if "throughput_kept" in v},
+                      "req_s": {k: r2(v["req_s"]) for k, v in c["levels"].items() if v["priority"] > 0}}
+    d = out.get("device_stamps")
+    if d:
+        s["device_stamps_us_mean_p99"] = {k: [r2(v["mean"]), r2(v["p99"])] for k, v in d.items() if isinstance(v, dict) and "mean" in v}
+    c2 = out.get("config2_resnet50_fp32_b1")
+    if c2:
+        s["config2_preempt_us_mean_p99"] = [r2(c2["preemption_latency_us"]["mean"]), r2(c2["preemption_latency_us"]["p99"])]
+        s["config2_stamps_us_mean_p99"] = {k: [r2(v["mean"]), r2(v["p99"])] for k, v in c2.get("device_stamps_us", {}).items()}
+    if "roofline" in out:
+        s["conv_launch_us"] = r2(out["roofline"]["avg_launch_us"])
+        s["conv_frac"] = round(out["roofline"]["frac"], 4)
+    g = out.get("config5_gemm8192_bf16")
+    if g:
+        s["gemm8192_frac_preemptible_plain_ckpt"] = [r3(g["frac"]), r3(g["plain_launch"]["frac"]), r3(g["with_checkpoint_workspace"]["frac"])]
+    if "config1_gemm1024_f32" in out:
+        s["gemm1024_f32_us_plain_preemptible"] = [r2(out["config1_gemm1024_f32"]["plain_us"]), r2(out["config1_gemm1024_f32"]["preemptible_us"])]
+    if "miniweather" in out:
+        s["miniweather_frac_hbm"] = r3(out["miniweather"]["frac_of_hbm_peak"])
+    return s
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -513,6 +595,7 @@ def main():
     ap.add_argument("--be-model", default="resnet152")
     ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal | vendor | hp")
     ap.add_argument("--cpu-requests", type=int, default=10, help="timed submissions per graph in the cpu_baseline leg")
+    ap.add_argument("--config-seconds", type=float, default=3.5, help="co-run time of the config 4 and config 5 scenario legs")
     ap.add_argument("--gemm-operands", default="random", choices=("random", "const"), help="operands of the 8192^3 GEMM leg (--only gemm)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -553,6 +636,10 @@ def main():
             alone = scenario(max(200, args.steps // 2), args.warmup, "lco", args.hp_rate, args.be_model, args.hp_model)["tasks"]["hp"]
             out["hp_alone_same_arrivals_ms"] = {k: alone["totalLatency(us)"][k] / 1e3 for k in ("mean", "p50", "p99")}
             out["hp_p99_vs_alone_same_arrivals"] = out["hp_corun_ms"]["p99"] / out["hp_alone_same_arrivals_ms"]["p99"]
+            # BASELINE configs 4 and 5 for a few seconds each, and the headline scenario with device time stamps
+            out["config4_three_tenants"] = config_leg("config4_bert_densenet201_vgg16.json", args.config_seconds)
+            out["config5_bert384_over_gemm8192"] = config_leg("config5_bert384_gemm8192.json", args.config_seconds)
+            out["device_stamps"] = stamps_leg(300, args.warmup, args.policy, args.hp_rate, args.be_model, args.hp_model)
     if args.only in ("", "roofline"):
         out["roofline"] = roofline(args.be_model, 10, "f16")
     if args.only in ("", "gemm"):
@@ -570,6 +657,8 @@ def main():
         out["hp_request_alone"] = hp_request(args.hp_model)
     if args.only in ("", "cpu"):
         out["cpu_baseline"] = cpu_baseline(args.cpu_requests)
+    if not args.only:
+        out["summary"] = summary_of(out)  # last on purpose: whoever keeps only the end of the line keeps this
     print(json.dumps(out))
 
 

@@ -23,7 +23,7 @@ vp = C.c_void_p
 class PreemptCtx(C.Structure):
     _fields_ = [("flag", vp), ("stop_index", vp), ("executed", vp), ("kernel_id", C.c_int),
                 ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("fresh", C.c_int), ("left_host", vp),
-                ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong)]
+                ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong), ("stamps", vp)]
 
 
 class LaunchInfo(C.Structure):
@@ -96,7 +96,7 @@ class EmbedParams(C.Structure):
 
 
 # every symbol include/gpreempt_hip.h declares
-SYMBOLS = """gp_init gp_last_error gp_device_info gp_stream_create gp_stream_destroy gp_stream_sync
+SYMBOLS = """gp_init gp_last_error gp_device_info gp_device_clock gp_stream_create gp_stream_destroy gp_stream_sync
 gp_stream_query gp_stream_priority gp_stream_set_priority gp_stream_native gp_event_create gp_event_destroy gp_event_record
 gp_event_sync gp_event_query gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free gp_memcpy_h2d gp_memcpy_d2h
 gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_flag_relay_start
@@ -302,7 +302,22 @@ class BlpState:
     def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0, fresh=0):
         ck = getattr(self, "ckpt", None)
         return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id * self.ints_per_kernel, kernel_id, inject_at, max_workgroups,
-                          poll_every, self.groups if self.groups > 1 else 0, fresh, None, ck.ptr if ck else None, ck.nbytes if ck else 0)
+                          poll_every, self.groups if self.groups > 1 else 0, fresh, None, ck.ptr if ck else None, ck.nbytes if ck else 0,
+                          self.stamps.ptr if getattr(self, "stamps", None) else None)
+
+    STAMP_WORDS = 8 + 1024
+
+    def enable_stamps(self):
+        """Device time stamps of the preemption (gp_preempt_ctx::stamps), cleared."""
+        self.stamps = DevBuf(8 * self.STAMP_WORDS)
+        self.stamps.upload(np.zeros(self.STAMP_WORDS, np.uint64))
+
+    def read_stamps(self):
+        """(stop recorded, first claim, latest exit, number of exit stamps) in device clock ticks; 0 = not written."""
+        raw = np.empty(self.STAMP_WORDS, np.uint64)
+        check(lib().gp_memcpy_d2h(raw.ctypes.data_as(vp), vp(self.stamps.ptr), C.c_size_t(raw.nbytes)))
+        ex = raw[8:]
+        return int(raw[0]), int(raw[1]), int(ex.max()), int((ex != 0).sum())
 
     def enable_checkpoints(self, params):
         """Allocates the workspace that lets the GEMM `params` leave its tiles half-way (if it can)."""

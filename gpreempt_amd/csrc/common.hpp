@@ -42,6 +42,15 @@ inline size_t dtype_size(int dt) {
     }
 }
 
+// Where claims go through several counters, counters 0..3 read the flag; the others need the lengths of
+// those four slices to tell when to take over (reads_flag in tile_loop.hpp).  The slices depend on the
+// grid, so a launcher that changes the grid after plan_launch calls this again.
+inline void set_poll_slices(BlpArgs *blp, int grid) {
+    const int ng = blp->groups;
+    for (int g = 0; g < 4; ++g)
+        blp->poll_n[g] = ng > 1 && g < ng ? group_slice_begin(blp->total, g + 1, ng, grid) - group_slice_begin(blp->total, g, ng, grid) : 0;
+}
+
 // Resolves the launch geometry of one preemptible kernel, as Model::add_block_preemption_param
 // does in the reference (src/model.cpp:366-396): total_block = sx*sy*sz; persistent grid =
 // min(total_block, resident workgroups the device can hold); a NULL context keeps one
@@ -58,7 +67,7 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
     if (ctx) {
         GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
         blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;
-        blp->kernel_id = ctx->kernel_id; blp->inject_at = ctx->inject_at;
+        blp->kernel_id = ctx->kernel_id; blp->inject_at = ctx->inject_at; blp->stamps = ctx->stamps;
         GP_REQUIRE(ctx->fresh >= 0 && ctx->fresh <= 2, "fresh is 0, 1 or 2");
         blp->fresh = ctx->fresh;
         int pe = ctx->poll_every > 0 ? ctx->poll_every : 8;
@@ -94,13 +103,10 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         // is half a microsecond; a launch of several rounds waits for the stop index as before (VGG-16 b16 next
         // to two higher levels: drain 41 / 77 us mean / p99 with the wait, 48 / 94 without).
         if (blp->fresh > 1 && (long)*grid > resident) blp->fresh = 1;
-        // where claims go through several counters, counters 0..3 read the flag; the others need the
-        // lengths of those four slices to tell when to take over (reads_flag in tile_loop.hpp)
-        for (int g = 0; g < 4; ++g)
-            blp->poll_n[g] = ng > 1 && g < ng ? group_slice_begin((int)total, g + 1, ng, *grid) - group_slice_begin((int)total, g, ng, *grid) : 0;
+        set_poll_slices(blp, *grid);
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
-        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0; blp->spare = 0;
+        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0; blp->spare = 0; blp->stamps = nullptr;
         for (int g = 0; g < 4; ++g) blp->poll_n[g] = 0;
         *grid = (int)total;
     }

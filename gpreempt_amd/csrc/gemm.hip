@@ -38,7 +38,7 @@ template <class TK>
 __global__ __launch_bounds__(TK::NT) void mat_kernel_ckpt(MatArgs g, BlpArgs blp) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     auto *lds = reinterpret_cast<typename TK::elem *>(lds_raw);
-    const CkptCtx cc = {blp.executed && blp.ckpt ? blp.stop_index : nullptr, blp.flag, blp.ckpt, blp.kernel_id};
+    const CkptCtx cc = {blp.executed && blp.ckpt ? blp.stop_index : nullptr, blp.flag, blp.ckpt, blp.kernel_id, blp.stamps};
     tile_loop_ckpt(blp, [&](TileIdx t, int tile_index, int kt0) { return TK::run(g, t, lds, cc, tile_index, kt0); });
 }
 
@@ -85,7 +85,7 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
     blp.order = pl.order;
     if constexpr (K_is_ckpt<K>::value) {
         if (info) info->fixed_claims = 0;  // tile_loop_ckpt always claims through the counters
-        if (blp.spare) { grid -= blp.spare; blp.spare = 0; if (info) info->grid = grid; }
+        if (blp.spare) { grid -= blp.spare; blp.spare = 0; set_poll_slices(&blp, grid); if (info) info->grid = grid; }
         // mid-tile checkpoints need the caller's workspace and a slot per workgroup
         if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES, grid) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
     }

@@ -159,7 +159,6 @@ struct LnWideKernel {
                         // chunk ch of the row is chunk ch % 8 of K-block ch / 8, at the swizzled position
                         const int blk = ch >> 3, phys = (ch & 7) ^ ((r >> 1) & 7);
                         *(out_u32x4 *)(a_res + (size_t)blk * A_BLK_BYTES + r * RB + phys * 16) = y[q][i];
-                        if (t.x == 0 && m < g.M) st_out128((T *)g.ln_out + (long)m * g.K + ch * VEC, y[q][i]);
                     }
                 }
             }
@@ -190,6 +189,24 @@ struct LnWideKernel {
             if (s == 0 && early && __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1) {
                 wait_vmcnt<0>();  // loads still landing in LDS must not outlive the workgroup
                 return true;
+            }
+            // The workgroups of tile column 0 store the normalised rows, and only now: a launch that started
+            // eagerly behind a stopped kernel normalised rows of an incomplete x, and must leave (above) without
+            // having written anything.  Every wavefront stores the rows it normalised, from their copy in LDS.
+            if (s == 0 && t.x == 0) {
+                const int chunks = g.K / VEC;
+#pragma unroll
+                for (int q = 0; q < BM / WAVES; ++q) {
+                    const int r = wave + q * WAVES, m = m0 + r;
+#pragma unroll
+                    for (int i = 0; i < MAXC; ++i) {
+                        const int ch = lane + i * 64;
+                        if (ch < chunks && m < g.M) {
+                            const int blk = ch >> 3, phys = (ch & 7) ^ ((r >> 1) & 7);
+                            st_out128((T *)g.ln_out + (long)m * g.K + ch * VEC, *(const out_u32x4 *)(a_res + (size_t)blk * A_BLK_BYTES + r * RB + phys * 16));
+                        }
+                    }
+                }
             }
             if (s >= PRE - (STAGES - 1) && s + STAGES - 1 < NS) issue(s + STAGES - 1);
             if (kb >= G) continue;  // (uniform) the other wavefronts only fetch

@@ -86,6 +86,7 @@ struct CkptCtx {       // what a checkpointing body needs from the dispatcher, p
     int *flag;
     void *ckpt;
     int kernel_id;
+    unsigned long long *stamps = nullptr;  // BlpArgs::stamps (the measurement mode of tile_loop.hpp)
 };
 
 // NWAVES: wavefronts per workgroup.  With eight (two per SIMD, 128 accumulator registers each) the
@@ -445,7 +446,7 @@ struct PipeKernel {
             }
             if constexpr (CKPT) {
                 const int sw = __builtin_amdgcn_readfirstlane(stop_word), fw = __builtin_amdgcn_readfirstlane(flag_word);
-                if (fw != 0 && tid == 0) atomicCAS(cc.stop_index, -1, cc.kernel_id);  // pass the host flag on
+                if (fw != 0 && tid == 0) record_stop(cc.stop_index, cc.kernel_id, cc.stamps);  // pass the host flag on
                 stop_now = (sw != -1) | (fw != 0);
             }
             return stop_now;

@@ -73,6 +73,7 @@ struct ProgArgs {
     int *left_host;    // optional host-visible word: set to `launch_tag` by the last workgroup to leave
     int launch_tag;
     unsigned long long *prof;  // optional: 4 cycle counters per workgroup (claim, acquire, body, publish)
+    unsigned long long *stamps;  // optional: time stamps of the preemption (tile_loop.hpp, "time stamps")
 };
 
 template <typename T>
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(256, GP_EXP_WGS) void program_kernel(ProgArgs p) {
             unsigned spins = 0;
             for (;;) {
                 if (stop_word != -1) {
-                    if (leader) atomicCAS(p.stop_index, -1, L < p.n_layers ? L : p.n_layers - 1);
+                    if (leader) record_stop(p.stop_index, L < p.n_layers ? L : p.n_layers - 1, p.stamps);
                     claim = -1;
                     break;
                 }
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(256, GP_EXP_WGS) void program_kernel(ProgArgs p) {
                             int f = 0;
                             if (leader) f = __hip_atomic_load(p.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                             if (__builtin_amdgcn_readfirstlane(f) != 0) {
-                                if (leader) atomicCAS(p.stop_index, -1, L);
+                                if (leader) record_stop(p.stop_index, L, p.stamps);
                                 stop_word = L;
                             }
                         }
@@ -230,7 +231,8 @@ __global__ __launch_bounds__(256, GP_EXP_WGS) void program_kernel(ProgArgs p) {
                         __hip_atomic_store(p.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
                     if (grp < p.poll_groups && (c & p.poll_mask) == 0 && p.flag &&
                         __hip_atomic_load(p.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
-                        atomicCAS(p.stop_index, -1, L);
+                        record_stop(p.stop_index, L, p.stamps);
+                    stamp_first_claim(p.stamps);
                 }
                 break;
             }
@@ -245,6 +247,7 @@ __global__ __launch_bounds__(256, GP_EXP_WGS) void program_kernel(ProgArgs p) {
         const int claim = __builtin_amdgcn_readfirstlane(mailbox[it & 1][1]);
         if (p.prof) { unsigned long long t1 = wall_clock64(); t_claim += t1 - t0; t0 = t1; }
         if (claim < 0) {
+            if (leader && p.stamps) stamp_exit_leader(p.stamps);
             if (leader && p.left_host) {
                 // every workgroup of this launch has stopped touching the model's buffers once the
                 // count is complete: tell the host without waiting for the queue to report it
@@ -468,6 +471,7 @@ extern "C" int gp_program_launch(gp_program p, const gp_preempt_ctx *ctx, int re
     a.launch_tag = ++p->launches;
     if (a.left_host) { int rc = gp_fill32_async(p->exited(), 0, 1, s); if (rc) return rc; }
     a.prof = p->d_prof;
+    a.stamps = ctx ? ctx->stamps : nullptr;
     long grid = p->max_tiles < p->resident ? p->max_tiles : p->resident;
     if (ctx) {
         GP_REQUIRE(ctx->stop_index != nullptr, "preempt context needs stop_index");

@@ -1,6 +1,7 @@
 // Device, stream, event, memory, flag, gate and graph entry points of the C ABI.
 #include "common.hpp"
 #include <atomic>
+#include <ctime>
 #include <mutex>
 
 namespace gp {
@@ -45,6 +46,11 @@ __global__ void gate_kernel(const int *stop, unsigned long long spin_limit, int 
 }
 
 __global__ void noop_kernel() {}
+
+// stores the device's constant-rate clock where the host can see it
+__global__ void clock_probe_kernel(unsigned long long *host_word) {
+    if (threadIdx.x == 0) __hip_atomic_store(host_word, (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 struct RelayArgs { const int *flags[8]; int *mirror; int n; const int *quit; unsigned long long spin_limit; };
 
@@ -230,6 +236,50 @@ extern "C" int gp_launch_gate(const int *stop, unsigned long long spin_limit, in
 extern "C" int gp_launch_noop(gp_stream s) {
     hipLaunchKernelGGL(noop_kernel, dim3(1), dim3(64), 0, native(s));
     GP_HIP(hipGetLastError());
+    return GP_SUCC;
+}
+
+// Device clock against the host's: a kernel stores wall_clock64() into fine-grained host memory and the
+// host, spinning on the word, notes its own clock when the value appears.  host - device is the offset plus
+// the store's way to the host; the minimum over the rounds keeps the shortest way (1-2 us).
+extern "C" int gp_device_clock(gp_stream s, int rounds, double *tick_ns, double *offset_ns, unsigned long long *ticks) {
+    GP_REQUIRE(tick_ns && offset_ns, "null clock out");
+    if (rounds < 1) rounds = 16;
+    int dev = 0, khz = 0;
+    GP_HIP(hipGetDevice(&dev));
+    GP_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    GP_REQUIRE(khz > 0, "the device reports no wall clock rate");
+    const double tick = 1e6 / (double)khz;
+    volatile unsigned long long *word = nullptr;
+    GP_HIP(hipHostMalloc((void **)&word, 64, hipHostMallocCoherent | hipHostMallocMapped));
+    void *word_dev = nullptr;
+    if (hipHostGetDevicePointer(&word_dev, (void *)word, 0) != hipSuccess) { hipHostFree((void *)word); set_error("gp_device_clock: no device address for the probe word"); return GP_FAIL; }
+    double best = 0;
+    unsigned long long best_ticks = 0;
+    bool have = false;
+    for (int r = 0; r < rounds; ++r) {
+        *word = 0;
+        hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, native(s), (unsigned long long *)word_dev);
+        hipError_t e = hipGetLastError();
+        unsigned long long d = 0;
+        // bounded: a kernel that never ran must not hang the caller (about two seconds of polls)
+        for (long spins = 0; e == hipSuccess && (d = *word) == 0 && spins < (1L << 31); ++spins) { }
+        struct timespec ts;
+        clock_gettime(CLOCK_MONOTONIC, &ts);
+        const double host_ns = (double)ts.tv_sec * 1e9 + (double)ts.tv_nsec;
+        hipError_t e2 = hipStreamSynchronize(native(s));
+        if (e != hipSuccess || e2 != hipSuccess || d == 0) {
+            hipHostFree((void *)word);
+            set_error("gp_device_clock: the probe kernel did not report (%s)", hipGetErrorString(e != hipSuccess ? e : e2));
+            return GP_FAIL;
+        }
+        const double off = host_ns - (double)d * tick;
+        if (!have || off < best) { best = off; best_ticks = d; have = true; }
+    }
+    GP_HIP(hipHostFree((void *)word));
+    *tick_ns = tick;
+    *offset_ns = best;
+    if (ticks) *ticks = best_ticks;
     return GP_SUCC;
 }
 

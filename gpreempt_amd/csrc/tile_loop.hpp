@@ -56,6 +56,7 @@ struct BlpArgs {
     int fresh;        // nonzero: the host vouches that no claim of this kernel has been made since its counters were cleared; 2: eager start (tile_fixed_early)
     int spare;        // fixed claims only: the last `spare` workgroups of the grid have no claim and read the flag
     int poll_n[4];    // several counters, claims through them: the number of claims in the slices of counters 0..3
+    unsigned long long *stamps;  // nullptr (the default) or device time stamps of the preemption (see "time stamps" below)
 };
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
@@ -98,6 +99,35 @@ __device__ __forceinline__ TileIdx decode_tile(int idx, int sx, int sy, int orde
     return t;
 }
 
+// ---- time stamps ----------------------------------------------------------------------------------
+// A measurement mode (BlpArgs::stamps != nullptr), off by default.  The reference measures a preemption
+// from the host (src/cuda-clients/blpclient.cpp:185-195: flag store, then a spin on the best-effort
+// tenant's counter); what the host sees includes its own polling and the PCIe round trips.  With a stamp
+// buffer the kernels write the device's constant-rate clock (wall_clock64) at the three moments that
+// bound a preemption on the GPU:
+//   word 0                 the workgroup whose compare-and-swap recorded the stop (flag seen on the device)
+//   word 1                 the first claim made while the word was zero (the host clears it before a resume)
+//   words 8 .. 8 + 1023    workgroup b, when it leaves, writes word 8 + (b mod 1024): the largest of them is
+//                          the moment the last workgroup of the tenant's latest kernel left the GPU (a stop
+//                          is often honoured without being recorded: the few kernels in flight simply end)
+// Plain stores to distinct words: no atomic is added to the leaving path (an atomic on one word from every
+// leaving workgroup serialises the exit of a large grid).
+constexpr int STAMP_STOP = 0, STAMP_FIRST_CLAIM = 1, STAMP_EXIT0 = 8, STAMP_EXIT_SLOTS = 1024;
+constexpr int STAMP_WORDS = STAMP_EXIT0 + STAMP_EXIT_SLOTS;
+
+// records the stop (first writer wins) and, in the measurement mode, when
+__device__ __forceinline__ void record_stop(int *stop_index, int kernel_id, unsigned long long *stamps) {
+    if (atomicCAS(stop_index, -1, kernel_id) == -1 && stamps) stamps[STAMP_STOP] = wall_clock64();
+}
+__device__ __forceinline__ void stamp_first_claim(unsigned long long *stamps) {
+    if (stamps && __hip_atomic_load(stamps + STAMP_FIRST_CLAIM, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0)
+        atomicCAS(stamps + STAMP_FIRST_CLAIM, 0ull, (unsigned long long)wall_clock64());
+}
+// the leader of a leaving workgroup, once all its threads are done
+__device__ __forceinline__ void stamp_exit_leader(unsigned long long *stamps) {
+    stamps[STAMP_EXIT0 + ((int)blockIdx.x & (STAMP_EXIT_SLOTS - 1))] = wall_clock64();
+}
+
 // One claim by the workgroup's leader: -1 when the workgroup has to leave (stop requested or the
 // slice is handed out).
 //
@@ -134,8 +164,9 @@ __device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_l
                 __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             if ((c & b.poll_mask) == 0 && b.flag && reads_flag(b, grp) &&
                 __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
-                atomicCAS(b.stop_index, -1, b.kernel_id);
+                record_stop(b.stop_index, b.kernel_id, b.stamps);
             // the polling workgroup still owes the tile it has just claimed
+            stamp_first_claim(b.stamps);
         }
     }
     // (a workgroup that finds the stop index set has nothing to record: the first writer won.
@@ -175,7 +206,8 @@ __device__ __forceinline__ int claim_fixed(const BlpArgs &b, int grp) {
     // (with spare workgroups the flag is theirs to read: nobody's tile waits for host memory)
     if (b.spare == 0 && (grp < 4 || b.poll_mask == 0) && (j & b.poll_mask) == 0 && b.flag &&
         __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
-        atomicCAS(b.stop_index, -1, b.kernel_id);
+        record_stop(b.stop_index, b.kernel_id, b.stamps);
+    stamp_first_claim(b.stamps);
     return claim;
 }
 
@@ -186,8 +218,16 @@ __device__ __forceinline__ bool spare_workgroup(const BlpArgs &b, bool fixed, bo
     if (!fixed || b.spare == 0 || (int)blockIdx.x < (int)gridDim.x - b.spare) return false;
     if (leader && b.flag && __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0 &&
         __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == -1)
-        atomicCAS(b.stop_index, -1, b.kernel_id);
+        record_stop(b.stop_index, b.kernel_id, b.stamps);
+    if (leader && b.stamps) stamp_exit_leader(b.stamps);
     return true;
+}
+
+// A workgroup of a preemptible launch leaves (every thread calls this; measurement mode only).
+__device__ __forceinline__ void leave_stamped(const BlpArgs &b) {
+    if (!b.stamps || !b.executed) return;
+    __syncthreads();
+    if ((threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0)) stamp_exit_leader(b.stamps);
 }
 
 // Runs body(TileIdx) for every tile this workgroup obtains.  All threads of the workgroup must
@@ -226,12 +266,12 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
             idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1]);  // wave-uniform: tile coordinates stay scalar
         }
         if (it == 0) GP_DISP_PROBE(3);
-        if (idx < 0) return;
+        if (idx < 0) { leave_stamped(b); return; }
         // Streaming kernels have tiles of a few KB; handing them out several at a time keeps the
         // claim (an atomic and a barrier, 1-2 us) off their critical path.
         const int first = idx * b.batch, last = first + b.batch < b.tiles ? first + b.batch : b.tiles;
         for (int tile = first; tile < last; ++tile) body(decode_tile(tile, b.sx, b.sy, b.order));
-        if (single) return;
+        if (single) { leave_stamped(b); return; }
     }
 }
 
@@ -301,17 +341,19 @@ __device__ __forceinline__ void tile_fixed_early(const BlpArgs &b, Body &&body) 
     } else {
         idx = fixed_claim_of_workgroup(b);
     }
-    if (idx < 0) return;
+    if (idx < 0) { leave_stamped(b); return; }
     int *word = (eager || b.spare) ? b.stop_index : nullptr;
     const bool left = body(decode_tile(idx, b.sx, b.sy, b.order), word);
     if (left && threadIdx.x == 0) unclaim_fixed(b);
+    leave_stamped(b);
 }
 
 template <class Body>
 __device__ __forceinline__ void tile_fixed(const BlpArgs &b, Body &&body) {
     const int idx = fixed_claim_of_workgroup(b);
-    if (idx < 0) return;
+    if (idx < 0) { leave_stamped(b); return; }
     body(decode_tile(idx, b.sx, b.sy, b.order));
+    leave_stamped(b);
 }
 
 // body(first_tile, last_tile) forms, for kernels built on tile_loop_span
@@ -325,8 +367,9 @@ __device__ __forceinline__ void span_plain(const BlpArgs &b, Body &&body) {
 template <class Body>
 __device__ __forceinline__ void span_fixed(const BlpArgs &b, Body &&body) {
     const int idx = fixed_claim_of_workgroup(b);
-    if (idx < 0) return;
+    if (idx < 0) { leave_stamped(b); return; }
     body(idx, idx + 1);
+    leave_stamped(b);
 }
 
 // which of the loops a kernel instantiation is built around
@@ -365,10 +408,10 @@ __device__ __forceinline__ void tile_loop_span(const BlpArgs &b, Body &&body) {
             __syncthreads();
             idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1]);
         }
-        if (idx < 0) return;
+        if (idx < 0) { leave_stamped(b); return; }
         const int first = idx * b.batch;
         body(first, first + b.batch < b.tiles ? first + b.batch : b.tiles);
-        if ((int)gridDim.x >= b.total) return;  // one claim per workgroup at most (see tile_loop)
+        if ((int)gridDim.x >= b.total) { leave_stamped(b); return; }  // one claim per workgroup at most (see tile_loop)
     }
 }
 
@@ -429,11 +472,11 @@ __device__ __forceinline__ void tile_loop_ckpt(const BlpArgs &b, Body &&body) {
             idx = __builtin_amdgcn_readfirstlane(mailbox[it & 1][0]);  // wave-uniform: tile coordinates and
             kt0 = __builtin_amdgcn_readfirstlane(mailbox[it & 1][1]);  // K position stay scalar
         }
-        if (idx < 0) return;
-        if (body(decode_tile(idx, b.sx, b.sy, b.order), idx, kt0)) return;
+        if (idx < 0) { leave_stamped(b); return; }
+        if (body(decode_tile(idx, b.sx, b.sy, b.order), idx, kt0)) { leave_stamped(b); return; }
         // one claim per workgroup at most (see tile_loop); a relaunch may continue a stored tile and
         // then still owe its slice a claim, so the shortcut holds on the fresh path only
-        if ((int)gridDim.x >= b.total && kt0 == 0 && !(it == 0 && b.ckpt)) return;
+        if ((int)gridDim.x >= b.total && kt0 == 0 && !(it == 0 && b.ckpt)) { leave_stamped(b); return; }
     }
 }
 

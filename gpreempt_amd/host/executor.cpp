@@ -164,6 +164,8 @@ BLPExecutor::~BLPExecutor() {
     if (dpStopIndex) gp_free(dpStopIndex);
     if (executed) gp_free(executed);
     if (ckpt) gp_free(ckpt);
+    if (stamps) gp_free(stamps);
+    if (stamps_host) gp_host_free(stamps_host);
     if (stop_host) gp_host_free(stop_host);
     if (left_host) gp_flag_destroy(left_host);
 }
@@ -292,6 +294,59 @@ Status BLPExecutor::resume(GPUstream stream) {
     if (use_program) return model->launch_program(stream, false, inject_kernel, inject_claim);
     for (size_t i = (size_t)stopIndex; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
     return Status::Succ;
+}
+
+Status BLPExecutor::enable_device_stamps(GPUstream stream) {
+    if (graph_compute || !model) return Status::Fail;
+    if (stamps) return Status::Succ;
+    RETURN_STATUS(calibrate_device_clock(stream));
+    CUDA_RETURN_STATUS(gp_malloc(&stamps, sizeof(unsigned long long) * GP_STAMP_WORDS));
+    CUDA_RETURN_STATUS(gp_host_alloc((void **)&stamps_host, sizeof(unsigned long long) * GP_STAMP_WORDS));
+    RETURN_STATUS(clear_device_stamps(stream));
+    CUDA_RETURN_STATUS(gp_stream_sync(stream));
+    model->set_stamps(stamps);
+    return Status::Succ;
+}
+
+Status BLPExecutor::clear_device_stamps(GPUstream stream) {
+    if (!stamps) return Status::Fail;
+    CUDA_RETURN_STATUS(gp_fill32_async(stamps, 0, 2 * (size_t)GP_STAMP_WORDS, stream));
+    return Status::Succ;
+}
+
+Status BLPExecutor::read_device_stamps(GPUstream stream, DeviceStamps &out) {
+    if (!stamps) return Status::Fail;
+    CUDA_RETURN_STATUS(gp_memcpy_d2h_async(stamps_host, stamps, sizeof(unsigned long long) * GP_STAMP_WORDS, stream));
+    CUDA_RETURN_STATUS(gp_stream_sync(stream));
+    unsigned long long last = 0;
+    out = DeviceStamps();
+    for (int i = 0; i < GP_STAMP_EXIT_SLOTS; ++i) {
+        const unsigned long long v = stamps_host[GP_STAMP_EXIT0 + i];
+        if (v) ++out.exits;
+        if (v > last) last = v;
+    }
+    out.stop_recorded = stamps_host[GP_STAMP_STOP];
+    out.first_claim = stamps_host[GP_STAMP_FIRST_CLAIM];
+    out.last_exit = last;
+    return Status::Succ;
+}
+
+Status BLPExecutor::calibrate_device_clock(GPUstream stream) {
+    double offset = 0;
+    unsigned long long ticks = 0;
+    CUDA_RETURN_STATUS(gp_device_clock(stream, 32, &stamp_tick_ns, &offset, &ticks));
+    const int slot = cal_ticks[0] ? 1 : 0;
+    cal_ticks[slot] = ticks;
+    cal_host_ns[slot] = (double)ticks * stamp_tick_ns + offset;
+    return Status::Succ;
+}
+
+int64_t BLPExecutor::device_ticks_to_ns(unsigned long long ticks) const {
+    if (!ticks || !cal_ticks[0]) return 0;
+    // between two calibrations the measured rate, with one the nominal rate
+    double rate = stamp_tick_ns;
+    if (cal_ticks[1] > cal_ticks[0] + 1000000ull) rate = (cal_host_ns[1] - cal_host_ns[0]) / (double)(cal_ticks[1] - cal_ticks[0]);
+    return (int64_t)(cal_host_ns[0] + ((double)ticks - (double)cal_ticks[0]) * rate);
 }
 
 Status BLPExecutor::reset_counters(GPUstream stream) {

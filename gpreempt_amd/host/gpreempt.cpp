@@ -49,7 +49,10 @@ int hipGetFd() {
 }
 
 static int each_level(int fd, std::vector<int> &ids, bool suspend) {
-    foo::PreemptDomain *d = domain_of(fd);
+    // the table's lock is held across the calls: a domain destroyed on another thread unregisters itself
+    // under the same lock first, so the pointer cannot go stale in between
+    std::lock_guard<std::mutex> g(g_fd_mu);
+    foo::PreemptDomain *d = fd >= 0 && (size_t)fd < g_fds.size() ? g_fds[fd] : nullptr;
     if (!d) return -1;
     for (int p : ids)
         if (p < 1 || p >= d->levels()) return -1;

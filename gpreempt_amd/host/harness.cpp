@@ -223,6 +223,11 @@ struct Shared {
     std::mutex seq_mu;
     std::mutex stats_mu;
     Stats preempt_latency;                  // flag store -> lower-priority stream drained
+    // the same preemptions split by device time stamps ("device_stamps": true): flag store -> stop recorded
+    // on the GPU -> last workgroup of the tenant gone -> the host notices; and, after the higher level has
+    // finished, resubmission -> first tile claimed
+    bool device_stamps = false;
+    long corun_discard = 0;                 // the first requests of every priority-0 tenant are served but not counted
     // busy_above[L]: time during which at least one request of a level above L (a smaller number)
     // was being served: what a continuous tenant of level L could not have used
     std::mutex busy_mu;
@@ -282,6 +287,12 @@ struct Tenant {
     uint64_t ref_hash = 0;
     long output_mismatches = 0;
     int64_t preemptions = 0, requests = 0;
+    std::vector<double> first_latencies;    // total latency of the first co-run requests, in arrival order
+    long discarded = 0;
+    int64_t resubmitted_ns = 0;             // device stamps: when the kernels of a stopped model were submitted again
+    // one preemption (or resubmission) as the host and the GPU saw it: host clock nanoseconds and raw device ticks
+    struct StampSample { int64_t raised = 0, drained = 0, resubmitted = 0; unsigned long long stop = 0, exit = 0, claim = 0; };
+    std::vector<StampSample> stamp_samples;
     int64_t first_ns = 0, last_ns = 0;
     Status error = Status::Succ;
     gp_event chunk_events[3] = {nullptr, nullptr, nullptr};
@@ -335,6 +346,7 @@ Status init_tenant(Tenant &t, Shared &sh) {
         t.ex->capture_graph(t.stream);
     }
     if (chunked) for (int i = 0; i < 3; ++i) CUDA_RETURN_STATUS(gp_event_create(&t.chunk_events[i]));
+    if (chunked && sh.device_stamps && !t.ex->graph_workload()) RETURN_STATUS(t.blp->enable_device_stamps(t.stream));
     return Status::Succ;
 }
 
@@ -401,6 +413,21 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             if (st != Status::Succ) { sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel); break; }
             const int stop = ex->last_stop_index();
             const int64_t raised = sh.domain->raised_ns(p);
+            if (ex->device_stamps_enabled()) {
+                // the GPU's own account of this preemption (and of the resume before it, if there was one)
+                BLPExecutor::DeviceStamps ds;
+                st = ex->read_device_stamps(t.stream, ds);
+                if (st == Status::Succ) st = ex->clear_device_stamps(t.stream);
+                if (st != Status::Succ) { sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel); break; }
+                Tenant::StampSample smp;
+                if ((queued > 0 || stop >= 0) && raised > 0 && drained >= raised && ds.last_exit) {
+                    smp.raised = raised; smp.drained = drained; smp.exit = ds.last_exit;
+                    smp.stop = stop >= 0 ? ds.stop_recorded : 0;
+                }
+                if (t.resubmitted_ns && ds.first_claim) { smp.resubmitted = t.resubmitted_ns; smp.claim = ds.first_claim; }
+                if (smp.raised || smp.resubmitted) t.stamp_samples.push_back(smp);
+                t.resubmitted_ns = 0;
+            }
             // a preemption-latency sample needs something to have been preempted: kernels in flight
             // when the request was noticed, or a kernel recorded as stopped.  (A request that finds
             // this tenant between two submissions waits for nothing.)
@@ -415,6 +442,7 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             while (sh.active_above(p) > 0) spin_pause();
             sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
             if (stop >= 0) { next = (size_t)stop; ++t.preemptions; }  // kernels from the stopped one on are submitted again
+            if (stop >= 0 && ex->device_stamps_enabled()) t.resubmitted_ns = now_ns();
             continue;
         }
         if (next < n && inflight < 2) {
@@ -436,6 +464,16 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             st = ex->getStopPoint(t.stream);
             if (st == Status::Succ && ex->last_stop_index() >= 0) { next = (size_t)ex->last_stop_index(); ++t.preemptions; }
         }
+    }
+    if (st == Status::Succ && t.resubmitted_ns && ex->device_stamps_enabled()) {
+        BLPExecutor::DeviceStamps ds;
+        if (ex->read_device_stamps(t.stream, ds) == Status::Succ && ds.first_claim) {
+            Tenant::StampSample smp;
+            smp.resubmitted = t.resubmitted_ns; smp.claim = ds.first_claim;
+            t.stamp_samples.push_back(smp);
+        }
+        ex->clear_device_stamps(t.stream);
+        t.resubmitted_ns = 0;
     }
     ex->running = false;
     sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
@@ -624,6 +662,8 @@ void tenant_thread(Tenant *t, Shared *sh, std::atomic<int> *ready, int n_tasks, 
         int64_t start = now_ns();
         Status s = infer_once(*t, *sh, &total, &inf);
         if (s != Status::Succ) { t->error = s; break; }
+        if (t->first_latencies.size() < 32) t->first_latencies.push_back(total);
+        if (t->priority == 0 && t->discarded < sh->corun_discard) { ++t->discarded; continue; }
         if (t->requests == 0) t->first_ns = start;
         t->last_ns = now_ns();
         ++t->requests;
@@ -656,6 +696,8 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     sh.hp_requests = (long)cfg["hp_requests"].number(0);
     sh.verify_outputs = cfg["verify_outputs"].boolean(false);
     sh.hp_gate = cfg["hp_gate"].boolean(false);
+    sh.device_stamps = cfg["device_stamps"].boolean(false);
+    sh.corun_discard = (long)cfg["corun_discard"].number(0);
     const json::Value &tasks = cfg["tasks"];
     std::vector<std::unique_ptr<Tenant>> tenants;
     // Declared after `tenants`, so it runs first on every exit path: executors free device memory
@@ -797,6 +839,12 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
                 sd.push(e);
             }
         }
+        {
+            json::Value &fl = o.set("firstLatencies(us)");
+            fl = json::Value::array();
+            for (double v : t->first_latencies) fl.push(json::Value(v));
+            if (t->discarded) o.set("discardedRequests") = (long)t->discarded;
+        }
         if (sh.verify_outputs) o.set("outputMismatches") = t->output_mismatches;
         if (t->error != Status::Succ) { o.set("error") = status_name(t->error); result = t->error; }
     }
@@ -850,6 +898,34 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     rep.set("be_throughput_kept") = n_be ? be_kept / n_be : 0.0;
     rep.set("preemptLatency(us)") = sh.preempt_latency.to_json();
     rep.set("hints_fired") = (double)(sh.hints ? sh.hints->fired() : 0);
+    if (sh.device_stamps) {
+        // device ticks -> host clock through a second calibration now, a run's length after the first
+        Stats raise_to_stop, stop_to_exit, raise_to_exit, exit_to_host, resub_to_claim;
+        for (auto &t : tenants) {
+            if (!t->blp || !t->blp->device_stamps_enabled()) continue;
+            if (t->blp->calibrate_device_clock(t->stream) != Status::Succ) continue;
+            for (const Tenant::StampSample &m : t->stamp_samples) {
+                if (m.raised && m.exit) {
+                    const int64_t ex_ns = t->blp->device_ticks_to_ns(m.exit);
+                    raise_to_exit.add((ex_ns - m.raised) / 1e3);
+                    exit_to_host.add((m.drained - ex_ns) / 1e3);
+                    if (m.stop && m.exit >= m.stop) {
+                        const int64_t st_ns = t->blp->device_ticks_to_ns(m.stop);
+                        raise_to_stop.add((st_ns - m.raised) / 1e3);
+                        stop_to_exit.add((ex_ns - st_ns) / 1e3);
+                    }
+                }
+                if (m.resubmitted && m.claim) resub_to_claim.add((t->blp->device_ticks_to_ns(m.claim) - m.resubmitted) / 1e3);
+            }
+        }
+        json::Value &ds = rep.set("deviceStamps(us)");
+        ds = json::Value::object();
+        ds.set("flagStore_to_lastWorkgroupExit") = raise_to_exit.to_json();
+        ds.set("lastWorkgroupExit_to_hostNotices") = exit_to_host.to_json();
+        ds.set("flagStore_to_stopRecorded") = raise_to_stop.to_json();
+        ds.set("stopRecorded_to_lastWorkgroupExit") = stop_to_exit.to_json();
+        ds.set("resubmission_to_firstTileClaimed") = resub_to_claim.to_json();
+    }
     report_text = rep.dump();
 
     sh.hints.reset();         // joins the daemon before the domain goes
@@ -883,6 +959,11 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
     GPUstream stream;
     CUDA_RETURN_STATUS(gp_stream_create(1, &stream));
     if (use_graph) ex.capture_graph(stream);
+    // the GPU's own time stamps ride along (GPREEMPT_PROBE_STAMPS=0 switches them off)
+    const char *ps = getenv("GPREEMPT_PROBE_STAMPS");
+    const bool stamps = !(ps && *ps == '0') && ex.enable_device_stamps(stream) == Status::Succ;
+    struct ProbeSample { int64_t raised, drained, r0; unsigned long long stop, exit, claim; };
+    std::vector<ProbeSample> probe_samples;
     size_t n = ex.get_kernel_num();
     // isolated duration of one inference
     Stats iso;
@@ -908,11 +989,23 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
         RETURN_STATUS(drain(stream));
         int64_t drained = now_ns();
         *flag_host = 0;
+        BLPExecutor::DeviceStamps ds;
+        if (stamps) {
+            RETURN_STATUS(ex.read_device_stamps(stream, ds));
+            RETURN_STATUS(ex.clear_device_stamps(stream));
+            RETURN_STATUS(drain(stream));
+        }
         int64_t r0 = now_ns();
         RETURN_STATUS(ex.resume(stream));
         int64_t r1 = now_ns();
         int stop = ex.last_stop_index();
         RETURN_STATUS(drain(stream));
+        if (stamps && stop >= 0) {
+            BLPExecutor::DeviceStamps rs;
+            RETURN_STATUS(ex.read_device_stamps(stream, rs));
+            probe_samples.push_back({raised, drained, r0, ds.stop_recorded, ds.last_exit, rs.first_claim});
+            RETURN_STATUS(ex.clear_device_stamps(stream));
+        }
         if (stop >= 0 && (size_t)stop < n) {
             ++hits;
             per_kernel[stop].add((drained - raised) / 1e3);
@@ -930,6 +1023,24 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
     rep.set("isolated(us)") = iso.to_json();
     rep.set("preemptLatency(us)") = all.to_json();
     rep.set("resumeCall(us)") = all_resume.to_json();
+    if (stamps && ex.calibrate_device_clock(stream) == Status::Succ) {
+        Stats st_raise_to_stop, st_stop_to_exit, st_exit_to_host, st_resume_to_claim;
+        for (const ProbeSample &m : probe_samples) {
+            if (m.stop && m.exit >= m.stop) {
+                const int64_t st_ns = ex.device_ticks_to_ns(m.stop), ex_ns = ex.device_ticks_to_ns(m.exit);
+                st_raise_to_stop.add((st_ns - m.raised) / 1e3);
+                st_stop_to_exit.add((ex_ns - st_ns) / 1e3);
+                st_exit_to_host.add((m.drained - ex_ns) / 1e3);
+            }
+            if (m.claim) st_resume_to_claim.add((ex.device_ticks_to_ns(m.claim) - m.r0) / 1e3);  // resume() entered -> first tile claimed
+        }
+        json::Value &dsj = rep.set("deviceStamps(us)");
+        dsj = json::Value::object();
+        dsj.set("flagStore_to_stopRecorded") = st_raise_to_stop.to_json();
+        dsj.set("stopRecorded_to_lastWorkgroupExit") = st_stop_to_exit.to_json();
+        dsj.set("lastWorkgroupExit_to_hostNotices") = st_exit_to_host.to_json();
+        dsj.set("resumeEntered_to_firstTileClaimed") = st_resume_to_claim.to_json();
+    }
     json::Value &pk = rep.set("perKernel");
     pk = json::Value::array();
     auto model = ex.get_model();

@@ -111,15 +111,20 @@ Status Model::load_model(const std::string &device_json, const std::string &host
     RETURN_STATUS(build(name));
     if (have_export) {
         // the native graph runs; the export must at least agree with it on what goes in and comes out
-        auto size_of = [](const std::vector<StorageInfo> &v, const std::string &key) -> long {
-            for (const StorageInfo &s : v) if (s.name == key) return (long)s.size;
-            return -1;
+        // (in ELEMENTS: the reference's exports are float32 while the native graphs default to 16-bit
+        // types, and the same model in another element type is still the same model)
+        auto find = [](std::vector<StorageInfo> &v, const std::string &key) -> StorageInfo * {
+            for (StorageInfo &s : v) if (s.name == key) return &s;
+            return nullptr;
         };
         for (const char *key : {"data", "heads"}) {
-            const long a = size_of(export_->storage_infos, key), b = size_of(storage_infos, key);
-            if (a != b) {
-                std::fprintf(stderr, "load_model: %s describes a model whose \"%s\" is %ld bytes; the native graph of workload '%s' has %ld: refusing to run a different model under this name\n",
-                             device_json.c_str(), key, a, name.c_str(), b);
+            StorageInfo *a = find(export_->storage_infos, key), *b = find(storage_infos, key);
+            const size_t ea = a ? get_stype_size(a->stype) : 0, eb = b ? get_stype_size(b->stype) : 0;
+            const long na = ea ? (long)(a->size / ea) : -1, nb = eb ? (long)(b->size / eb) : -1;
+            if (na != nb) {
+                std::fprintf(stderr, "load_model: %s describes a model whose \"%s\" holds %ld elements (%s); the native graph of workload '%s' has %ld (%s): "
+                                     "refusing to run a different model under this name (name the directory with the options that match the export, e.g. '%s@b=1')\n",
+                             device_json.c_str(), key, na, a ? a->stype.c_str() : "absent", name.c_str(), nb, b ? b->stype.c_str() : "absent", name.substr(0, name.find('@')).c_str());
                 clear();
                 return Status::Fail;
             }
@@ -461,6 +466,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.fresh = idx < fresh_.size() && fresh_[idx] ? (eager_tiles_ ? 2 : 1) : 0;
         ctx.ckpt = ckpt_;
         ctx.ckpt_bytes = ckpt_bytes_;
+        ctx.stamps = (unsigned long long *)stamps_;
         pc = &ctx;
     }
     gp_launch_info info{};
@@ -540,6 +546,7 @@ Status Model::launch_program(GPUstream stream, bool reset, int inject_layer, int
         ctx.inject_at = inject_layer >= 0 ? inject_claim : -1;
         ctx.poll_every = poll_every_;
         ctx.left_host = (int *)left_word_;
+        ctx.stamps = (unsigned long long *)stamps_;
         pc = &ctx;
     }
     gp_launch_info info{};

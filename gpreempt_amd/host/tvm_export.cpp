@@ -23,7 +23,8 @@ Status fail(std::string &err, const std::string &what) {
     return Status::Fail;
 }
 
-bool is_uint(const json::Value &v) { return v.type == json::Value::Number && v.num >= 0 && v.num == (double)(uint64_t)v.num; }
+// a non-negative integer a double holds exactly (below 2^53: beyond that the cast back is not defined for every value)
+bool is_uint(const json::Value &v) { return v.type == json::Value::Number && v.num >= 0 && v.num < 9007199254740992.0 && v.num == (double)(uint64_t)v.num; }
 
 }  // namespace
 
@@ -52,8 +53,10 @@ Status parse_tvm_export(const std::string &device_json_text, const std::string &
         s.stype = dltypes.arr[i].string();
         size_t elems = 1;
         for (const json::Value &dim : shapes.arr[i].arr) {
-            if (!is_uint(dim)) return fail(out.error, "device json: bad shape of node " + std::to_string(i));
+            // every dimension below 2^31 and every tensor below 2^40 elements: the product cannot wrap
+            if (!is_uint(dim) || dim.num >= 2147483648.0) return fail(out.error, "device json: bad shape of node " + std::to_string(i));
             elems *= (size_t)dim.num;
+            if (elems >= ((size_t)1 << 40)) return fail(out.error, "device json: node " + std::to_string(i) + " holds more than 2^40 elements");
         }
         const size_t es = Model::get_stype_size(s.stype);
         if (es == 0) return fail(out.error, "device json: unknown dltype '" + s.stype + "' of node " + std::to_string(i));
@@ -66,7 +69,7 @@ Status parse_tvm_export(const std::string &device_json_text, const std::string &
     }
     // temporary storages, typed float32 whatever they hold (src/model.cpp:176-183)
     for (const json::Value &t : h["temp_args"].arr) {
-        if (!is_uint(t)) return fail(out.error, "host json: bad temp_args entry");
+        if (!is_uint(t) || t.num >= 1099511627776.0) return fail(out.error, "host json: bad temp_args entry");
         StorageInfo s;
         s.name = "temp"; s.stype = "float32"; s.size = (size_t)t.num;
         out.storage_infos.push_back(s);

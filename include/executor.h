@@ -105,6 +105,21 @@ public:
     // word the kernel sets; cheaper and earlier than a stream query).  Always false when the
     // executor is not in program mode.
     bool program_vacated() const;
+    // Device-side time stamps of preemptions, a measurement mode (per-kernel launches only; off by default).
+    // What src/cuda-clients/blpclient.cpp:185-195 measures with the host's clock around a spin, taken on the
+    // GPU: when the stop was recorded, when the tenant's last workgroup left, when the first tile was claimed
+    // after a resume.  Raw device clock ticks; 0 = not written since the last clear.  The device clock drifts
+    // against the host's by tens of microseconds per second, so the ticks are converted afterwards:
+    // calibrate_device_clock() notes a (ticks, host time) pair (enable_device_stamps takes the first one), and
+    // device_ticks_to_ns() interpolates between the first and the latest pair (CLOCK_MONOTONIC nanoseconds, good to
+    // 1-2 us once two pairs a run apart exist).
+    struct DeviceStamps { unsigned long long stop_recorded = 0, last_exit = 0, first_claim = 0; int exits = 0; };
+    Status enable_device_stamps(GPUstream stream);
+    Status read_device_stamps(GPUstream stream, DeviceStamps &out);   // blocks on `stream`
+    Status clear_device_stamps(GPUstream stream);                      // a fill kernel on `stream`
+    Status calibrate_device_clock(GPUstream stream);                   // blocks on `stream`
+    int64_t device_ticks_to_ns(unsigned long long ticks) const;
+    bool device_stamps_enabled() const { return stamps != nullptr; }
 
     // Claim counters per kernel.  The reference keeps one int per kernel (src/executor.cpp:333);
     // claims from several hundred workgroups serialise on a single address, so each kernel gets
@@ -132,6 +147,11 @@ private:
     void *left_dev = nullptr;
     GPUdeviceptr ckpt = nullptr;         // owned: checkpoint workspace of long GEMM tiles, or null
     size_t ckpt_bytes = 0;
+    GPUdeviceptr stamps = nullptr;       // owned: GP_STAMP_WORDS 64-bit words, or null
+    unsigned long long *stamps_host = nullptr;  // pinned landing area
+    double stamp_tick_ns = 10.0;
+    unsigned long long cal_ticks[2] = {0, 0};   // first and latest calibration: device ticks ...
+    double cal_host_ns[2] = {0, 0};             // ... and the host clock at that moment
     int inject_kernel = -1, inject_claim = -1, inject_iteration = -2;
     std::atomic<int> *lc_tasks = nullptr;
     std::atomic<int> *be_tasks = nullptr;

@@ -143,7 +143,22 @@ typedef struct gp_preempt_ctx {
                      /* with gp_ckpt_reset_async whenever the claim counters are cleared.  No       */
                      /* counterpart in the reference, whose tiles are never long enough to matter.  */
     unsigned long long ckpt_bytes;
+    unsigned long long *stamps; /* may be NULL (the default).  A measurement mode: GP_STAMP_WORDS 64-bit words of   */
+                     /* device memory that the kernels fill with the device's constant-rate clock             */
+                     /* (gp_device_clock gives its rate and its offset to the host's monotonic clock):        */
+                     /* word 0 when the stop was recorded, word 1 at the first claim made while it was zero,   */
+                     /* words 8 + (workgroup mod 1024) whenever a workgroup of a preemptible launch leaves.    */
+                     /* What                                                                                  */
+                     /* src/cuda-clients/blpclient.cpp:185-195 measures from the host, measured on the GPU.    */
 } gp_preempt_ctx;
+enum { GP_STAMP_STOP = 0, GP_STAMP_FIRST_CLAIM = 1, GP_STAMP_EXIT0 = 8, GP_STAMP_EXIT_SLOTS = 1024, GP_STAMP_WORDS = 8 + 1024 };
+/* The device clock the stamps are taken from: *tick_ns = nominal nanoseconds per tick; *offset_ns = what to
+ * add to ticks * tick_ns to get the host's CLOCK_MONOTONIC in nanoseconds, as of now (the minimum over
+ * `rounds` exchanges of "a kernel stores its clock to host memory, the host notes when it sees it": good to
+ * the one-way latency of such a store, 1-2 us); *ticks (may be NULL) = the device clock of that exchange.
+ * The two clocks drift apart by tens of microseconds per second: to convert stamps taken over seconds, call
+ * this before and after and interpolate between the two (ticks, host time) pairs. */
+int gp_device_clock(gp_stream s, int rounds, double *tick_ns, double *offset_ns, unsigned long long *ticks);
 
 /* What a launch did: filled when the `info` argument of a launcher is non-NULL. */
 typedef struct gp_launch_info {

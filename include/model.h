@@ -154,6 +154,8 @@ public:
     void set_left_word(GPUdeviceptr p) { left_word_ = p; }
     // workspace that lets long GEMM tiles be left between two K-steps (gp_preempt_ctx::ckpt)
     void set_checkpoint_workspace(GPUdeviceptr p, size_t bytes) { ckpt_ = p; ckpt_bytes_ = bytes; }
+    // device time stamps of preemptions (gp_preempt_ctx::stamps); null = off
+    void set_stamps(GPUdeviceptr p) { stamps_ = p; }
     // largest such workspace any kernel of the model can use (0: none can)
     size_t checkpoint_bytes_wanted() const;
     int last_launch_tag() const { return last_launch_tag_; }
@@ -184,6 +186,7 @@ private:
     GPUdeviceptr left_word_ = nullptr;
     GPUdeviceptr ckpt_ = nullptr;
     size_t ckpt_bytes_ = 0;
+    GPUdeviceptr stamps_ = nullptr;
     int last_launch_tag_ = 0;
     std::string workload_, dtype_;
     std::shared_ptr<struct TvmExport> export_;

@@ -37,7 +37,7 @@ class _Ctx:
         return self.R(O.gemm_bias_act(x, self.P(name + ".weight"), self.P(name + ".bias"), residual, act, b_is_nk=True))
 
 
-def resnet(params, x, blocks, dt="f32"):
+def resnet(params, x, blocks, dt="f32", logits=False):
     """ResNet v1, bottleneck blocks, stride on the first 1x1 of a down-sampling block, BN folded."""
     c = _Ctx(params, dt)
     x = c.R(x)
@@ -52,10 +52,11 @@ def resnet(params, x, blocks, dt="f32"):
             y = c.conv(n + ".conv2", y, 1, 1, O.ACT_RELU)
             x = c.conv(n + ".conv3", y, 1, 0, O.ACT_RELU, residual=shortcut)
     gap = c.R(O.global_avgpool(x))
-    return c.R(O.softmax(c.dense("fc", gap)))
+    lg = c.dense("fc", gap)
+    return (c.R(O.softmax(lg)), lg) if logits else c.R(O.softmax(lg))
 
 
-def vgg16(params, x, dt="f16", wdiv=1):
+def vgg16(params, x, dt="f16", wdiv=1, logits=False):
     c = _Ctx(params, dt)
     x = c.R(x)
     ci = 0
@@ -68,10 +69,11 @@ def vgg16(params, x, dt="f16", wdiv=1):
     x = x.reshape(x.shape[0], -1)  # NCHW flatten, as relay's batch_flatten
     x = c.dense("fc1", x, O.ACT_RELU)
     x = c.dense("fc2", x, O.ACT_RELU)
-    return c.R(O.softmax(c.dense("fc3", x)))
+    lg = c.dense("fc3", x)
+    return (c.R(O.softmax(lg)), lg) if logits else c.R(O.softmax(lg))
 
 
-def densenet(params, x, dt="f16", blocks=(6, 12, 48, 32), growth=32):
+def densenet(params, x, dt="f16", blocks=(6, 12, 48, 32), growth=32, logits=False):
     c = _Ctx(params, dt)
     x = c.R(x)
     x = c.conv("conv0", x, 2, 3, O.ACT_RELU)
@@ -90,10 +92,11 @@ def densenet(params, x, dt="f16", blocks=(6, 12, 48, 32), growth=32):
             x = c.R(O.pool2d(t, 2, 2, 0, "avg"))
     t = c.R(O.scale_shift_act(x, c.P("norm5.scale"), c.P("norm5.shift"), O.ACT_RELU))
     gap = c.R(O.global_avgpool(t))
-    return c.R(O.softmax(c.dense("classifier", gap)))
+    lg = c.dense("classifier", gap)
+    return (c.R(O.softmax(lg)), lg) if logits else c.R(O.softmax(lg))
 
 
-def inception_v3(params, x, dt="f16"):
+def inception_v3(params, x, dt="f16", logits=False):
     """Inception-v3 as relay.testing.inception_v3 lays it out: stem, 3 x A, B, 4 x C, D, 2 x E,
     global average pool, FC, softmax; every convolution with folded batch-norm and ReLU; average
     pools count their padding."""
@@ -153,7 +156,8 @@ def inception_v3(params, x, dt="f16"):
         b3 = cv(n + ".proj", c.R(O.pool2d(x, 3, 1, 1, mode)))
         x = np.concatenate([b0, b1, b2, b3], axis=1)
     gap = c.R(O.global_avgpool(x))
-    return c.R(O.softmax(c.dense("fc1", gap)))
+    lg = c.dense("fc1", gap)
+    return (c.R(O.softmax(lg)), lg) if logits else c.R(O.softmax(lg))
 
 
 def bert(params, ids, dt="f16", batch=1, seq=128, layers=12, hidden=768, heads=12, fused_attention=None):

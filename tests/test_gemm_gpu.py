@@ -779,3 +779,132 @@ def test_layernorm_prologue_is_refused_where_it_does_not_fit(gp):
         p.ln_gamma = p.ln_beta = p.ln_out = dA.ptr
         with pytest.raises(gp.GpError):
             gp.launch("gp_launch_gemm", p)
+
+
+# ---- a kernel started eagerly behind a stopped one -------------------------------------------------
+
+def _chain_second(gp, family, dX_ptr, M, K, dtype, es, rng, dt):
+    """The second kernel of a two-kernel chain, reading the first one's output (M x K): (params, output buffer, kept buffers)."""
+    N = 256
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32) * 0.05, dt)
+    dB, dC = gp.DevBuf.from_array(B, dtype), gp.DevBuf(M * N * es)
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dX_ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, alpha=1.0, act=gp.ACT_RELU, batch=1)
+    keep = [dB]
+    if family == "pipe":
+        p.tile_m = p.tile_n = 64; p.variant = gp.MAT_PIPE
+    elif family == "wide":
+        p.tile_m = p.tile_n = 32; p.variant = gp.MAT_WIDE
+    elif family == "ln":
+        gamma = O.round_to(rng.uniform(0.5, 1.5, K).astype(np.float32), dt)
+        beta = O.round_to(rng.normal(0, 0.2, K).astype(np.float32), dt)
+        dg, dbeta, dLN = gp.DevBuf.from_array(gamma, dtype), gp.DevBuf.from_array(beta, dtype), gp.DevBuf(M * K * es)
+        p.ln_gamma, p.ln_beta, p.ln_out, p.ln_eps = dg.ptr, dbeta.ptr, dLN.ptr, 1e-12
+        keep += [dg, dbeta, dLN]
+    return p, dC, keep
+
+
+@pytest.mark.parametrize("family,K", [("pipe", 512), ("pipe", 64), ("wide", 768), ("wide", 64), ("ln", 768), ("ln", 64)])
+def test_kernel_started_eagerly_behind_a_stopped_one_withdraws_every_claim(gp, family, K):
+    """Kernel N is stopped late by an injected flag; kernel N+1, which reads N's output, is queued behind it as a first
+    launch with an eager start (fresh = 2): its workgroups begin their tiles before they know of the stop, find it with
+    their first operands, withdraw their claims (every count back to zero, every bit clear) and write nothing.
+    After the resume of both the chain's output has the bits of an uninterrupted run.  In every body family with an
+    early look (pipelined, wide, layer-norm prologue), also with a K of one step."""
+    dt = "f16"
+    dtype, es = gp.DTYPE_BY_NAME[dt], 2
+    rng = np.random.default_rng(K + len(family))
+    M, K0 = 1024, 256  # kernel N: 32 x K/32 tiles of 32 x 32 on 32 workgroups, so that its claims go through the counters
+    A = O.round_to(rng.uniform(-1, 1, (M, K0)).astype(np.float32), dt)
+    W0 = O.round_to(rng.uniform(-1, 1, (K, K0)).astype(np.float32) * 0.1, dt)
+    dA, dW0, dX = gp.DevBuf.from_array(A, dtype), gp.DevBuf.from_array(W0, dtype), gp.DevBuf(M * K * es)
+    p0 = gp.GemmParams(dtype=dtype, M=M, N=K, K=K0, A=dA.ptr, lda=K0, B=dW0.ptr, ldb=K0, b_is_nk=1, C=dX.ptr, ldc=K, alpha=1.0, batch=1,
+                       tile_m=32, tile_n=32, variant=gp.MAT_PIPE_SPLITK)
+    p1, dC, keep = _chain_second(gp, family, dX.ptr, M, K, dtype, es, rng, dt)
+    # uninterrupted chain, plain launches
+    gp.launch("gp_launch_gemm", p0); gp.launch("gp_launch_gemm", p1)
+    gp.check(gp.lib().gp_stream_sync(None))
+    want_x, want_c = dX.download().copy(), dC.download().copy()
+    want_ln = keep[-1].download().copy() if family == "ln" else None
+    flag = gp.Flag()
+    st = gp.BlpState(2, flag, 32)
+    G = 32
+    # kernel N: few workgroups, claims through the counters, so that its polls see the flag it raises itself
+    dX.fill32(0); dC.fill32(0x7E007E00)
+    if family == "ln":
+        keep[-1].fill32(0x7E007E00)
+    info0 = gp.launch("gp_launch_gemm", p0, st.ctx(kernel_id=0, inject_at=info_total(M, K) // 2, max_workgroups=8, fresh=1, poll_every=1))
+    assert info0.fixed_claims == 0 and info0.total_tiles == info_total(M, K)
+    info1 = gp.launch("gp_launch_gemm", p1, st.ctx(kernel_id=1, fresh=2))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert info1.fixed_claims == 1, "the second kernel must have a workgroup per claim for this test"
+    assert flag.get() == 1 and st.stop_index() == 0
+    lines1 = st.counters().reshape(2, G, 16)[1]
+    assert not lines1.any(), "every eager claim of the queued kernel must have been withdrawn"
+    assert np.all(dC.download(np_dtype=np.uint16) == 0x7E00), "the queued kernel wrote output on incomplete input"
+    if family == "ln":
+        assert np.all(keep[-1].download(np_dtype=np.uint16) == 0x7E00), "the queued kernel stored normalised rows of incomplete input"
+    x_part = dX.download(np_dtype=np.uint16).reshape(M // 32, 32, K // 32, 32)
+    assert (x_part == 0).all(axis=(1, 3)).any(), "kernel N was not really interrupted"
+    # resume (executor.cpp:280-298): stop index re-armed, counters kept, kernels from the stopped one on
+    flag.set(0)
+    st.clear_stop()
+    gp.launch("gp_launch_gemm", p0, st.ctx(kernel_id=0, max_workgroups=8, poll_every=1))
+    gp.launch("gp_launch_gemm", p1, st.ctx(kernel_id=1))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert st.stop_index() == -1
+    assert np.array_equal(dX.download(), want_x) and np.array_equal(dC.download(), want_c)
+    if family == "ln":
+        assert np.array_equal(keep[-1].download(), want_ln)
+    assert st.counters().reshape(2, G, 16)[1][:, 0].sum() == info1.total_tiles
+
+
+def info_total(M, N, tile=32):
+    return -(-M // tile) * -(-N // tile)
+
+
+def test_device_time_stamps_of_a_preemption(gp):
+    """gp_preempt_ctx::stamps: the stop is stamped by the workgroup that records it, every workgroup that leaves
+    with a stop recorded stamps its exit, the first claim after the stamps were cleared is stamped; all on the
+    device's constant-rate clock, which gp_device_clock ties to the host's monotonic clock."""
+    import time
+    A, B, bias, p, dC, keep = _config1(gp, 64)
+    gp.launch("gp_launch_gemm", p)
+    gp.check(gp.lib().gp_stream_sync(None))
+    base = dC.download(gp.F32, (1024, 1024)).copy()
+    tick, off = C.c_double(0), C.c_double(0)
+    gp.check(gp.lib().gp_device_clock(None, 16, C.byref(tick), C.byref(off), None))
+    assert 1.0 <= tick.value <= 100.0  # 100 MHz on this GPU: 10 ns
+    to_host_ns = lambda ticks: ticks * tick.value + off.value
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag, 32)
+    st.enable_stamps()
+    WGS = 32
+    t0 = time.monotonic_ns()
+    info = gp.launch("gp_launch_gemm", p, st.ctx(inject_at=100, max_workgroups=WGS, fresh=1, poll_every=1))
+    gp.check(gp.lib().gp_stream_sync(None))
+    t1 = time.monotonic_ns()
+    assert st.stop_index() == 0 and info.fixed_claims == 0
+    stop, first, last_exit, exits = st.read_stamps()
+    assert stop and first and last_exit
+    assert first <= stop <= last_exit           # claims began before the stop; the tiles owed were finished after it
+    assert 1 <= exits <= WGS
+    assert (last_exit - stop) * tick.value < 5e6  # the drain of 64 x 64 tiles: far below 5 ms
+    slack = 200e3  # the offset is good to a few microseconds; host-side launch and sync cost tens
+    assert t0 - slack <= to_host_ns(first) <= to_host_ns(last_exit) <= t1 + slack
+    # resume with cleared stamps: a first claim, no stop, every workgroup stamps its exit
+    st.stamps.upload(np.zeros(st.STAMP_WORDS, np.uint64))
+    flag.set(0)
+    st.clear_stop()
+    info = gp.launch("gp_launch_gemm", p, st.ctx(max_workgroups=WGS, poll_every=1))
+    gp.check(gp.lib().gp_stream_sync(None))
+    stop2, first2, last2, exits2 = st.read_stamps()
+    assert stop2 == 0 and exits2 == info.grid and last_exit < first2 < last2
+    assert np.array_equal(dC.download(gp.F32, (1024, 1024)), base)
+    # fixed claims (a workgroup per tile) with the flag already up: the spare workgroups record and stamp the stop
+    st.reset(); st.stamps.upload(np.zeros(st.STAMP_WORDS, np.uint64))
+    flag.set(1)
+    info = gp.launch("gp_launch_gemm", p, st.ctx(fresh=1))
+    gp.check(gp.lib().gp_stream_sync(None))
+    assert info.fixed_claims == 1 and st.stop_index() == 0
+    stop3, first3, last3, exits3 = st.read_stamps()
+    assert stop3 and first3 and last3 >= stop3 and exits3 >= 1

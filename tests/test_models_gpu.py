@@ -38,6 +38,12 @@ def run(gp, ex, x_raw, dtype, out_shape):
     return gp.from_storage(ex.get_output("heads"), dtype).reshape(out_shape).copy()
 
 
+def logits_of(gp, ex, storage, dtype, shape):
+    """The classifier's output in front of the softmax, read from its storage by name (Model::get): probabilities
+    alone can hide a wrong logit that does not move the top class."""
+    return gp.from_storage(ex.get_output(storage), dtype).reshape(shape).copy()
+
+
 def test_gemm1024_workload_matches_oracle(gp, ex_mod, tmp_path):
     ex, params = make_model(ex_mod, tmp_path, "gemm1024", "gemm", 1)
     A = np.random.default_rng(0xC0FFEE).uniform(-1, 1, (1024, 1024)).astype(np.float32)
@@ -57,10 +63,11 @@ def test_resnet_matches_oracle(gp, ex_mod, tmp_path, workload, dt, blocks):
     hw = 64 if "hw=64" in workload else 224
     x = O.round_to(np.random.default_rng(3).normal(0, 1, (n, 3, hw, hw)).astype(np.float32), dt)
     got = run(gp, ex, gp.to_storage(x, dtype), dtype, (n, 1000))
-    ref = OM.resnet(params, x, blocks, dt)
+    ref, ref_logits = OM.resnet(params, x, blocks, dt, logits=True)
     assert np.isfinite(got).all()
     assert rel_err(got, ref) < TOL[dt]
     assert abs(got.sum(axis=1) - 1).max() < 2e-2
+    assert rel_err(logits_of(gp, ex, "fc.out", dtype, (n, 1000)), ref_logits) < TOL[dt]
 
 
 def test_vgg16_matches_oracle(gp, ex_mod, tmp_path):
@@ -68,7 +75,22 @@ def test_vgg16_matches_oracle(gp, ex_mod, tmp_path):
     ex, params = make_model(ex_mod, tmp_path, wl, "cnn", 4)
     x = O.round_to(np.random.default_rng(5).normal(0, 1, (2, 3, 64, 64)).astype(np.float32), "f16")
     got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (2, 1000))
-    assert rel_err(got, OM.vgg16(params, x, "f16")) < TOL["f16"]
+    ref, ref_logits = OM.vgg16(params, x, "f16", logits=True)
+    assert rel_err(got, ref) < TOL["f16"]
+    assert rel_err(logits_of(gp, ex, "fc3.out", gp.F16, (2, 1000)), ref_logits) < TOL["f16"]
+
+
+def test_vgg16_full_size_logits_match_oracle(gp, ex_mod, tmp_path):
+    """BASELINE config 4's best-effort model at its real shape (224 x 224, 4096-wide classifier), one image:
+    the 25088 -> 4096 dense layer (K = 25088, M = 1) and the 224 x 224 x 64 convolutions, on the logits."""
+    wl = "vgg16@b=1"
+    ex, params = make_model(ex_mod, tmp_path, wl, "cnn", 14)
+    x = O.round_to(np.random.default_rng(15).normal(0, 1, (1, 3, 224, 224)).astype(np.float32), "f16")
+    got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (1, 1000))
+    ref, ref_logits = OM.vgg16(params, x, "f16", logits=True)
+    assert np.isfinite(got).all() and abs(got.sum() - 1) < 2e-2
+    assert rel_err(logits_of(gp, ex, "fc3.out", gp.F16, (1, 1000)), ref_logits) < TOL["f16"]
+    assert rel_err(got, ref) < TOL["f16"]
 
 
 def test_densenet_matches_oracle(gp, ex_mod, tmp_path):
@@ -76,7 +98,21 @@ def test_densenet_matches_oracle(gp, ex_mod, tmp_path):
     ex, params = make_model(ex_mod, tmp_path, wl, "cnn", 6)
     x = O.round_to(np.random.default_rng(7).normal(0, 1, (1, 3, 64, 64)).astype(np.float32), "f16")
     got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (1, 1000))
-    assert rel_err(got, OM.densenet(params, x, "f16", (2, 4, 5, 3))) < TOL["f16"]
+    ref, ref_logits = OM.densenet(params, x, "f16", (2, 4, 5, 3), logits=True)
+    assert rel_err(got, ref) < TOL["f16"]
+    assert rel_err(logits_of(gp, ex, "classifier.out", gp.F16, (1, 1000)), ref_logits) < TOL["f16"]
+
+
+def test_densenet201_full_size_logits_match_oracle(gp, ex_mod, tmp_path):
+    """BASELINE config 4's mid-priority model at its real shape (blocks 6 / 12 / 48 / 32, 224 x 224), one image."""
+    wl = "densenet201@b=1"
+    ex, params = make_model(ex_mod, tmp_path, wl, "cnn", 16)
+    x = O.round_to(np.random.default_rng(17).normal(0, 1, (1, 3, 224, 224)).astype(np.float32), "f16")
+    got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (1, 1000))
+    ref, ref_logits = OM.densenet(params, x, "f16", logits=True)
+    assert np.isfinite(got).all() and abs(got.sum() - 1) < 2e-2
+    assert rel_err(logits_of(gp, ex, "classifier.out", gp.F16, (1, 1000)), ref_logits) < TOL["f16"]
+    assert rel_err(got, ref) < TOL["f16"]
 
 
 def test_inception_v3_matches_oracle(gp, ex_mod, tmp_path):
@@ -87,7 +123,9 @@ def test_inception_v3_matches_oracle(gp, ex_mod, tmp_path):
     x = O.round_to(np.random.default_rng(9).normal(0, 1, (1, 3, 107, 107)).astype(np.float32), "f16")
     got = run(gp, ex, gp.to_storage(x, gp.F16), gp.F16, (1, 1000))
     assert np.isfinite(got).all() and abs(got.sum() - 1) < 2e-2
-    assert rel_err(got, OM.inception_v3(params, x, "f16")) < TOL["f16"]
+    ref, ref_logits = OM.inception_v3(params, x, "f16", logits=True)
+    assert rel_err(got, ref) < TOL["f16"]
+    assert rel_err(logits_of(gp, ex, "fc1.out", gp.F16, (1, 1000)), ref_logits) < TOL["f16"]
 
 
 @pytest.mark.parametrize("workload,kw", [
@@ -283,6 +321,43 @@ def test_host_timed_preempt_like_reference_test(gp, ex_mod, tmp_path, program, e
     ex.resume(stream)  # running == false: no-op (executor.cpp:281)
 
 
+def test_vgg16_b16_full_size_host_timed_preempt_bit_exact(gp, ex_mod, tmp_path):
+    """The same protocol on BASELINE config 4's best-effort tenant at its real shape (VGG-16, batch 16, 224 x 224):
+    its deep 3 x 3 layers take 64 x 64 tiles when preemptible (K >= 2304) and run in several rounds of workgroups,
+    its 25088 -> 4096 layer is the longest K of any model here."""
+    root = str(tmp_path)
+    os.environ["GPREEMPT_USE_HIPGRAPH"] = "0"
+    x = gp.to_storage(np.random.default_rng(21).normal(0, 1, (16, 3, 224, 224)).astype(np.float32), gp.F16)
+    base = ex_mod.Executor("vgg16", model_root=root)
+    base.set_input("data", x)
+    base.execute()
+    want = base.get_output("heads").copy()
+    want_logits = base.get_output("fc3.out").copy()
+    base.destroy()
+    ex = ex_mod.Executor("vgg16", blp=True, model_root=root)
+    flag = gp.Flag()
+    ex.set_flag(flag)
+    stream = gp.Stream(1)
+    ex.set_input("data", x, stream)
+    stream.sync()
+    import time
+    stops = []
+    for i in range(4):
+        ex.execute(stream)
+        ex.set_running(True)
+        time.sleep(0.0002 * i)  # the flag lands in another part of the network every time
+        flag.set(1)
+        stream.sync()
+        flag.set(0)
+        ex.resume(stream)
+        stops.append(ex.last_stop_index())
+        stream.sync()
+        assert np.array_equal(ex.get_output("heads", stream), want)
+        assert np.array_equal(ex.get_output("fc3.out", stream), want_logits)
+    assert any(s != -1 for s in stops), stops
+    ex.set_running(False)
+
+
 def test_exported_graph_next_to_the_model_is_read_and_checked(gp, ex_mod, tmp_path):
     """mod.json + host.json in the model directory are read as the reference reads them; an export
     that describes another model than the native graph of that name is refused, not ignored."""
@@ -304,6 +379,14 @@ def test_exported_graph_next_to_the_model_is_read_and_checked(gp, ex_mod, tmp_pa
     ex = ex_mod.Executor("toy", model_root=str(root))  # agrees with the native toy graph (64 x 64 fp32 in and out)
     x = np.arange(64 * 64, dtype=np.float32)
     assert np.array_equal(run(gp, ex, x, gp.F32, (64 * 64,)), 8 * x)
+    # the reference's exports are float32; the same model run in a 16-bit type is still the same model:
+    # what must agree is the number of elements, not of bytes
+    d16 = root / "toy@dtype=f16"
+    d16.mkdir()
+    (d16 / "mod.json").write_text(json.dumps(mod)); (d16 / "host.json").write_text(json.dumps(host))
+    ex16 = ex_mod.Executor("toy@dtype=f16", model_root=str(root))
+    x16 = (np.arange(64 * 64) % 128).astype(np.float32)
+    assert np.array_equal(run(gp, ex16, gp.to_storage(x16, gp.F16), gp.F16, (64 * 64,)), 8 * x16)
     mod, host = export(100)
     (d / "mod.json").write_text(json.dumps(mod))
     with pytest.raises(ex_mod.StatusError) as e:

@@ -185,6 +185,32 @@ def test_three_priority_levels(gp, policy):
     assert "beginTime" in rep and "endTime" in rep and isinstance(rep["benchmarkTime(s)"], int)
 
 
+def test_config4_at_full_size_with_verified_outputs(gp):
+    """BASELINE config 4 as the scenario file states it (BERT-base at 100 req/s over DenseNet-201 b4 at 50 req/s over
+    VGG-16 b16 back to back, all at 224 x 224 and full width) for two seconds: every request of every tenant returns
+    the bits of that tenant's uninterrupted run, and both lower levels were really stopped."""
+    import os
+    with open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpreempt_amd", "config", "config4_bert_densenet201_vgg16.json")) as f:
+        cfg = json.load(f)
+    cfg.update({"time": 2.0, "warmups": 2, "standalone_runs": 5, "verify_outputs": True, "device_stamps": True})
+    rep = _scenario(cfg)
+    t = rep["tasks"]
+    hp, mid, be = t["bert_rt"], t["densenet201_mid"], t["vgg16_be"]
+    assert hp["requests"] > 100 and mid["requests"] > 40 and be["requests"] > 100
+    assert mid["preemptions"] > 3 and be["preemptions"] > 50
+    for k, v in t.items():
+        assert v["outputMismatches"] == 0, (k, v["outputMismatches"])
+    # the GPU's own account of the preemptions: the stop is recorded after the flag store, the last workgroup
+    # leaves after that, and the host notices later still
+    # (the two clocks are tied together to a few microseconds: hence the slack)
+    ds = rep["deviceStamps(us)"]
+    assert ds["flagStore_to_lastWorkgroupExit"]["count"] > 50
+    assert -5 < ds["flagStore_to_lastWorkgroupExit"]["p50"] < rep["preemptLatency(us)"]["p50"] + 5
+    assert -5 < ds["lastWorkgroupExit_to_hostNotices"]["p50"] < 100
+    assert ds["stopRecorded_to_lastWorkgroupExit"]["count"] > 10 and ds["flagStore_to_stopRecorded"]["p50"] > -5
+    assert ds["resubmission_to_firstTileClaimed"]["count"] > 50 and 0 < ds["resubmission_to_firstTileClaimed"]["p50"] < 500
+
+
 def test_hp_gate_policy_option(gp):
     """The reference's blocking stream (gpreemptclient.cpp:74-81,232-235) as a scenario option: the
     high-priority tenant queues its kernels behind two gate kernels and releases them at once."""

@@ -247,4 +247,14 @@ def test_what_cannot_be_mapped_is_refused_by_name(tmp_path):
         if f == "mod.json":
             doc["attrs"]["shape"][1][5] = [10, 1 << 33]
     rc, rep = plan(_edited(tmp_path, "huge", huge_dim))
-    assert rc == 1 and "a dimension of" in rep["error"]
+    assert rc == 1 and "bad shape of node 5" in rep["error"]  # the reader itself bounds every dimension (< 2^31)
+    def huge_tensor(f, doc):
+        if f == "mod.json":
+            doc["attrs"]["shape"][1][5] = [1 << 20, 1 << 20]
+    rc, rep = plan(_edited(tmp_path, "huge2", huge_tensor))
+    assert rc == 1 and "more than 2^40 elements" in rep["error"]  # ... and every tensor: a storage size cannot wrap
+    def not_an_integer(f, doc):
+        if f == "mod.json":
+            doc["attrs"]["shape"][1][5] = [10, 1e300]
+    rc, rep = plan(_edited(tmp_path, "huge3", not_an_integer))
+    assert rc == 1 and "bad shape of node 5" in rep["error"]
