@@ -377,6 +377,11 @@ extern "C" int gpx_plan_tvm_export(const char *device_json, const char *host_jso
                 case OpKind::Gemm: {
                     const gp_gemm_params &g = k.p.gemm;
                     p.set("M") = g.M; p.set("N") = g.N; p.set("K") = g.K; p.set("lda") = g.lda; p.set("ldc") = g.ldc; p.set("act") = g.act;
+                    if (g.batch > 1) {  // a batched product: how the heads are laid out
+                        p.set("batch") = g.batch; p.set("batch_inner") = g.batch_inner; p.set("ldb") = g.ldb; p.set("b_is_nk") = g.b_is_nk; p.set("alpha") = (double)g.alpha;
+                        p.set("stride_a") = g.stride_a; p.set("stride_b") = g.stride_b; p.set("stride_c") = g.stride_c;
+                        p.set("stride_a_outer") = g.stride_a_outer; p.set("stride_b_outer") = g.stride_b_outer; p.set("stride_c_outer") = g.stride_c_outer;
+                    }
                     break;
                 }
                 case OpKind::Pool: {
@@ -390,6 +395,8 @@ extern "C" int gpx_plan_tvm_export(const char *device_json, const char *host_jso
                     break;
                 }
                 case OpKind::Softmax: p.set("rows") = k.p.softmax.rows; p.set("cols") = k.p.softmax.cols; break;
+                case OpKind::Layernorm: p.set("rows") = k.p.layernorm.rows; p.set("cols") = k.p.layernorm.cols; p.set("eps") = (double)k.p.layernorm.eps; break;
+                case OpKind::Embed: p.set("tokens") = k.p.embed.tokens; p.set("seq") = k.p.embed.seq; p.set("hidden") = k.p.embed.hidden; p.set("vocab") = k.p.embed.vocab; break;
                 case OpKind::Layout: p.set("N") = k.p.layout.N; p.set("C") = k.p.layout.C; p.set("H") = k.p.layout.H; p.set("W") = k.p.layout.W; p.set("c_pad") = k.p.layout.c_pad; break;
                 default: break;
             }

@@ -16,8 +16,24 @@ namespace foo {
 
 namespace {
 
+// A strided view of a storage, for the tensors of a transformer between its matrix products: [batch, sequence,
+// heads, head size] and its transposes.  Always held as four dimensions (leading ones of size 1 where the
+// export has fewer); `merged` says the export sees the first two as one ([batch * heads, rows, columns]).
+struct SeqView {
+    bool on = false, merged = false;
+    long dim[4] = {1, 1, 1, 1}, str[4] = {0, 0, 0, 0};  // elements
+    bool contiguous() const {
+        long want = 1;
+        for (int i = 3; i >= 0; --i) { if (dim[i] != 1 && str[i] != want) return false; want *= dim[i]; }
+        return true;
+    }
+    long elems() const { return dim[0] * dim[1] * dim[2] * dim[3]; }
+};
+
 struct Val {
     bool set = false, is_param = false;
+    bool is_ids = false;  // int64 token ids (a transformer's "data")
+    SeqView sv;           // on: `t` only names the storage and the offset
     Tensor t;           // t.C = channels held in memory (>= c_log), t.ps = pixel stride
     int c_log = 0;      // channels the export knows about
     int fc = 0, fh = 0, fw = 0;  // a flattened fh x fw x fc tensor (t.H = t.W = 1, c_log = fh * fw * fc, t.C counts the padding channels too); 0 = not one
@@ -107,13 +123,15 @@ struct Mapper {
         const std::vector<long> &s = ex.nodes[i].shape;
         for (long d : s) if (d <= 0 || d >= (1L << 31)) return false;
         if (s.size() == 4) { N = (int)s[0]; C = (int)s[1]; H = (int)s[2]; W = (int)s[3]; return true; }
+        if (s.size() == 3) { if (s[0] * s[1] >= (1L << 31)) return false; N = (int)(s[0] * s[1]); C = (int)s[2]; H = W = 1; return true; }  // [batch, sequence, width]: rows of a matrix
         if (s.size() == 2) { N = (int)s[0]; C = (int)s[1]; H = W = 1; return true; }
         if (s.size() == 1) { N = 1; C = (int)s[0]; H = W = 1; return true; }
         return false;
     }
     Status check_shape(size_t node, const Val &v) {
+        if (v.sv.on) return check_view_shape(node, v.sv);
         int N, C, H, W;
-        if (!nchw_of(node, N, C, H, W)) return fail(node, "tensors of 1, 2 or 4 dimensions only");
+        if (!nchw_of(node, N, C, H, W)) return fail(node, "tensors of 1 to 4 dimensions only");
         const int c = v.c_log;
         if (N != v.t.N || C != c || H != v.t.H || W != v.t.W)
             return fail(node, "the export says " + std::to_string(N) + "x" + std::to_string(C) + "x" + std::to_string(H) + "x" + std::to_string(W) + ", the operator attributes give " +
@@ -161,7 +179,7 @@ struct Mapper {
         if (it == buffers.end()) {
             int rn, rc, rh, rw;
             if (root == i) { rn = N; rc = c_log; rh = H; rw = W; }
-            else if (!nchw_of(root, rn, rc, rh, rw)) return fail(root, "tensors of 1, 2 or 4 dimensions only");
+            else if (!nchw_of(root, rn, rc, rh, rw)) return fail(root, "tensors of 1 to 4 dimensions only");
             it = buffers.emplace(root, b.activation(ex.nodes[root].name, rn, rh, rw, b.pad_c(rc))).first;
         }
         const Tensor &buf = it->second;
@@ -174,6 +192,7 @@ struct Mapper {
     }
     Status need_act(size_t user, size_t node, const Val *&v) {
         if (node >= vals.size() || !vals[node].set || vals[node].is_param) return fail(user, "argument '" + ex.nodes[node].name + "' must be a tensor computed earlier in the graph");
+        if (vals[node].is_ids) return fail(user, "argument '" + ex.nodes[node].name + "' holds token ids: only take reads those");
         v = &vals[node];
         return Status::Succ;
     }
@@ -240,6 +259,7 @@ struct Mapper {
         if (!input_of(i, op, "data", 0, dn) || !input_of(i, op, "weight", 1, wn)) return fail(i, "dense needs data and weight");
         const Val *in;
         RETURN_STATUS(need_act(i, dn, in));
+        if (in->sv.on) return fail(i, "dense over a view of a matrix (reshape it back to rows x features first)");
         if (in->t.H != 1 || in->t.W != 1) return fail(i, "dense over a tensor that was not flattened");
         const std::vector<long> &ws = ex.nodes[wn].shape;
         if (ws.size() != 2) return fail(i, "dense weight must be units x features");
@@ -247,9 +267,16 @@ struct Mapper {
         if (feat != in->c_log) return fail(i, "weight has " + std::to_string(feat) + " input features, the data " + std::to_string(in->c_log));
         const int K = in->t.C;  // features as they lie in memory: padding channels take zero weights
         if (K % b.vec() || in->t.ps % b.vec()) return fail(i, "dense over " + std::to_string(feat) + " features, which is not a multiple of " + std::to_string(b.vec()));
-        if (has_tail(op, "residual")) return fail(i, "a residual in a dense epilogue is not mapped");
         int act;
         RETURN_STATUS(tail_act(i, op, act));
+        const Val *res = nullptr;
+        if (has_tail(op, "residual")) {
+            size_t rn;
+            if (!input_of(i, op, "residual", 3, rn)) return fail(i, "the epilogue names a residual the function has no argument for");
+            RETURN_STATUS(need_act(i, rn, res));
+            // the GEMM reads the residual with the output's row stride
+            if (!plain_matrix(*res) || res->t.N != in->t.N || res->t.C != units) return fail(i, "the residual of a dense layer must be a plain rows x units matrix");
+        }
         ParamLayout L;
         const int fc = in->fc ? in->fc : feat, fh = in->fc ? in->fh : 1, fw = in->fc ? in->fw : 1;
         if (fh * fw > 1 || K != feat) { L.kind = ParamLayout::DenseOverCHW; L.c = fc; L.h = fh; L.w = fw; L.i_pad = K / (fh * fw); }
@@ -269,7 +296,7 @@ struct Mapper {
         const long rows = in->t.N;
         const double flops = 2.0 * rows * units * (double)feat;
         const double bytes = b.es() * ((double)rows * feat + (double)units * feat + units + (double)rows * units);
-        KernelInfo &ki = b.add_kernel("dense", OpKind::Gemm, {b.ref(in->t), GraphBuilder::ref(w), bias == SIZE_MAX ? GraphBuilder::none() : GraphBuilder::ref(bias), GraphBuilder::none(), b.ref(out.t)}, flops, bytes);
+        KernelInfo &ki = b.add_kernel("dense", OpKind::Gemm, {b.ref(in->t), GraphBuilder::ref(w), bias == SIZE_MAX ? GraphBuilder::none() : GraphBuilder::ref(bias), res ? b.ref(res->t) : GraphBuilder::none(), b.ref(out.t)}, flops, bytes);
         gp_gemm_params &p = ki.p.gemm;
         p.dtype = b.gp_dtype(); p.M = (int)rows; p.N = units; p.K = K; p.lda = in->t.ps; p.ldb = K; p.b_is_nk = 1; p.ldc = units; p.alpha = 1.f; p.act = act; p.batch = 1;
         vals[i] = out;
@@ -321,6 +348,7 @@ struct Mapper {
         p.dtype = b.gp_dtype(); p.rows = (long)a.N * a.H * a.W; p.cols = a.C; p.a_stride = a.ps; p.b_stride = other ? other->ps : 0; p.out_stride = out.ps; p.act = act;
     }
     Status elementwise_ready(size_t i, const Val &v) {
+        if (v.sv.on) return fail(i, "an element-wise operator over a view of a matrix (reshape it back first)");
         if (v.t.C % b.vec() || v.t.ps % b.vec() || v.t.off % b.vec()) return fail(i, "an element-wise operator over rows of " + std::to_string(v.t.C) + " values, which is not a multiple of " + std::to_string(b.vec()));
         return Status::Succ;
     }
@@ -380,6 +408,7 @@ struct Mapper {
         if (!input_of(i, op, "data", 0, dn)) return fail(i, "softmax needs data");
         const Val *a;
         RETURN_STATUS(need_act(i, dn, a));
+        if (a->sv.on) return softmax_view(i, op, *a);
         const long axis = attr(op, "axis", 0, -1);
         const long rank = (long)ex.nodes[dn].shape.size();
         if (a->t.H != 1 || a->t.W != 1 || (axis != -1 && axis != rank - 1)) return fail(i, "softmax over the last axis of a matrix only");
@@ -430,8 +459,10 @@ struct Mapper {
         const size_t dn = ex.nodes[i].inputs[0];
         const Val *a;
         RETURN_STATUS(need_act(i, dn, a));
+        // a view of a transformer's tensors, or a plain matrix about to become one
+        if (a->sv.on || (plain_matrix(*a) && ex.nodes[i].shape.size() == 4)) return reshape_seq(i, *a);
         int N, C, H, W;
-        if (!nchw_of(i, N, C, H, W)) return fail(i, "tensors of 1, 2 or 4 dimensions only");
+        if (!nchw_of(i, N, C, H, W)) return fail(i, "tensors of 1 to 4 dimensions only");
         const long have = (long)a->t.N * a->t.H * a->t.W * a->c_log;
         if ((long)N * C * H * W != have) return fail(i, "a reshape that changes the number of elements");
         Val out = *a;
@@ -454,6 +485,277 @@ struct Mapper {
         return Status::Succ;
     }
 
+    // ---- transformer operators (the functions of a BERT export, scripts/compile/compile-bert.py:76-77) -----------
+    // A plain matrix: rows x columns in unpadded, unsliced memory (what the dense layers and layer-norms of a
+    // transformer read and write).
+    static bool plain_matrix(const Val &v) { return !v.sv.on && !v.is_ids && v.t.H == 1 && v.t.W == 1 && v.t.off == 0 && v.t.ps == v.t.C && v.t.C == v.c_log && !v.fc; }
+    Val matrix_val(const std::string &name, long rows, int cols) {
+        Val out;
+        out.set = true; out.c_log = cols;
+        out.t.st = b.add_storage(name, (size_t)rows * cols, b.stype_);
+        out.t.N = (int)rows; out.t.H = out.t.W = 1; out.t.C = cols; out.t.ps = cols;
+        return out;
+    }
+    // the shape the export states for node i, as four dimensions (leading ones)
+    bool dims4_of(size_t i, long d[4], int &rank) const {
+        const std::vector<long> &s = ex.nodes[i].shape;
+        rank = (int)s.size();
+        if (rank < 1 || rank > 4) return false;
+        for (int k = 0; k < 4; ++k) d[k] = 1;
+        for (int k = 0; k < rank; ++k) d[4 - rank + k] = s[k];
+        return true;
+    }
+    Status check_view_shape(size_t i, const SeqView &v) {
+        long d[4]; int rank;
+        if (!dims4_of(i, d, rank)) return fail(i, "tensors of 1 to 4 dimensions only");
+        bool ok;
+        if (v.merged) ok = rank == 3 && d[1] == v.dim[0] * v.dim[1] && d[2] == v.dim[2] && d[3] == v.dim[3];
+        else ok = d[0] == v.dim[0] && d[1] == v.dim[1] && d[2] == v.dim[2] && d[3] == v.dim[3];
+        if (!ok) return fail(i, "the export's shape differs from what the operator attributes give (" + std::to_string(v.dim[0]) + "x" + std::to_string(v.dim[1]) + "x" +
+                                    std::to_string(v.dim[2]) + "x" + std::to_string(v.dim[3]) + (v.merged ? ", first two merged)" : ")"));
+        return Status::Succ;
+    }
+    static float attr_eps(const ExportOp &op) {  // "epsilon": [mantissa, decimal exponent], e.g. [1, -12]
+        auto it = op.attrs.find("epsilon");
+        if (it == op.attrs.end() || it->second.size() != 2) return 1e-5f;
+        return (float)((double)it->second[0] * std::pow(10.0, (double)it->second[1]));
+    }
+
+    // take(table, indices) [+ position rows] [+ one segment row]: the embedding sum of a BERT encoder
+    Status take(size_t i, const ExportOp &op) {
+        size_t tn, in, pn = SIZE_MAX, sn = SIZE_MAX;
+        if (!input_of(i, op, "table", 0, tn) || !input_of(i, op, "indices", 1, in)) return fail(i, "take needs a table and indices");
+        if (!vals[in].is_ids) return fail(i, "take: the indices must be the model's int64 input");
+        if (attr(op, "axis", 0, 0) != 0) return fail(i, "take along axis 0 only");
+        const std::vector<long> &ts = ex.nodes[tn].shape, &is = ex.nodes[in].shape;
+        if (ts.size() != 2) return fail(i, "take: the table must be rows x width");
+        const long vocab = ts[0]; const int Hd = (int)ts[1];
+        if (Hd % b.vec()) return fail(i, "take: rows of " + std::to_string(Hd) + " values, which is not a multiple of " + std::to_string(b.vec()));
+        const long T = prod(is), S = is.empty() ? 1 : is.back();
+        ParamLayout L; L.o = (int)vocab; L.disk_elems = (size_t)vocab * Hd; L.init = ParamLayout::InitNormal; L.init_a = 0.02f;
+        size_t tab, pos, seg = SIZE_MAX;
+        RETURN_STATUS(param(i, tn, (size_t)vocab * Hd, L, 5, tab));
+        if (op.inputs.count("position")) {
+            if (!input_of(i, op, "position", 2, pn)) return fail(i, "take: no argument for the position rows");
+            const long rows = prod(ex.nodes[pn].shape) / Hd;
+            if (prod(ex.nodes[pn].shape) != rows * Hd || rows < S) return fail(i, "take: the position rows must be (at least) sequence x width");
+            ParamLayout P; P.o = (int)rows; P.disk_elems = (size_t)rows * Hd; P.init = ParamLayout::InitNormal; P.init_a = 0.02f;
+            RETURN_STATUS(param(i, pn, (size_t)rows * Hd, P, 6, pos));
+        } else {
+            // a bare gather: position rows of zeros (never on disk, so they stay zero)
+            ParamLayout Z; Z.disk_elems = (size_t)S * Hd; Z.init = ParamLayout::InitZero;
+            pos = b.add_param(ex.nodes[i].name + ".zero_rows", (size_t)S * Hd, Z);
+        }
+        if (op.inputs.count("segment")) {
+            if (!input_of(i, op, "segment", 3, sn)) return fail(i, "take: no argument for the segment row");
+            if (prod(ex.nodes[sn].shape) != Hd) return fail(i, "take: the segment row must hold one row of the table's width");
+            ParamLayout G; G.o = 1; G.disk_elems = (size_t)Hd; G.init = ParamLayout::InitNormal; G.init_a = 0.02f;
+            RETURN_STATUS(param(i, sn, (size_t)Hd, G, 7, seg));
+        }
+        Val out = matrix_val(ex.nodes[i].name, T, Hd);
+        KernelInfo &k = b.add_kernel("embed", OpKind::Embed, {b.ref(vals[in].t), GraphBuilder::ref(tab), GraphBuilder::ref(pos), seg == SIZE_MAX ? GraphBuilder::none() : GraphBuilder::ref(seg), b.ref(out.t)},
+                                     2.0 * T * Hd, 8.0 * T + b.es() * 4.0 * T * Hd);
+        gp_embed_params &p = k.p.embed;
+        p.dtype = b.gp_dtype(); p.tokens = T; p.seq = (int)S; p.hidden = Hd; p.vocab = vocab;
+        vals[i] = out;
+        return Status::Succ;
+    }
+
+    Status layer_norm(size_t i, const ExportOp &op) {
+        size_t dn, gn, bn, rn;
+        if (!input_of(i, op, "data", 0, dn) || !input_of(i, op, "gamma", 1, gn) || !input_of(i, op, "beta", 2, bn)) return fail(i, "layer_norm needs data, gamma and beta");
+        const Val *a, *res = nullptr;
+        RETURN_STATUS(need_act(i, dn, a));
+        if (!plain_matrix(*a)) return fail(i, "layer_norm over the rows of a plain matrix only");
+        const long axis = attr(op, "axis", 0, -1);
+        if (axis != -1 && axis != (long)ex.nodes[dn].shape.size() - 1) return fail(i, "layer_norm over the last axis only");
+        if (!op.epilogue.empty()) return fail(i, "layer_norm takes no epilogue");
+        if (a->t.C % b.vec()) return fail(i, "layer_norm over rows of " + std::to_string(a->t.C) + " values, which is not a multiple of " + std::to_string(b.vec()));
+        if (op.inputs.count("residual")) {  // layer_norm(data + residual): the add in front of it fused in
+            if (!input_of(i, op, "residual", 3, rn)) return fail(i, "layer_norm: no argument for the residual");
+            RETURN_STATUS(need_act(i, rn, res));
+            if (!plain_matrix(*res) || res->t.N != a->t.N || res->t.C != a->t.C) return fail(i, "layer_norm: the residual's shape differs from the data's");
+        }
+        size_t ga, be;
+        RETURN_STATUS(vector_param(i, gn, a->t.C, a->t.C, ParamLayout::InitConst, 1.f, 4, ga));
+        RETURN_STATUS(vector_param(i, bn, a->t.C, a->t.C, ParamLayout::InitZero, 0.f, 2, be));
+        Val out = matrix_val(ex.nodes[i].name, a->t.N, a->t.C);
+        const double e = (double)a->t.N * a->t.C;
+        KernelInfo &k = b.add_kernel("layernorm", OpKind::Layernorm, {b.ref(a->t), res ? b.ref(res->t) : GraphBuilder::none(), GraphBuilder::ref(ga), GraphBuilder::ref(be), b.ref(out.t)},
+                                     8 * e, b.es() * e * (res ? 3 : 2));
+        gp_layernorm_params &p = k.p.layernorm;
+        p.dtype = b.gp_dtype(); p.rows = a->t.N; p.cols = a->t.C; p.eps = attr_eps(op);
+        vals[i] = out;
+        return Status::Succ;
+    }
+
+    // erf-GELU as a function of its own
+    Status gelu(size_t i, const ExportOp &op) {
+        size_t dn;
+        if (!input_of(i, op, "data", 0, dn)) return fail(i, "gelu needs data");
+        const Val *a;
+        RETURN_STATUS(need_act(i, dn, a));
+        if (!plain_matrix(*a)) return fail(i, "gelu over a plain matrix only");
+        RETURN_STATUS(elementwise_ready(i, *a));
+        if (!op.epilogue.empty()) return fail(i, "gelu takes no epilogue");
+        Val out = matrix_val(ex.nodes[i].name, a->t.N, a->t.C);
+        emit_eltwise(a->t, nullptr, SIZE_MAX, SIZE_MAX, out.t, GP_ACT_GELU);
+        vals[i] = out;
+        return Status::Succ;
+    }
+
+    // transpose: a new view of the same memory (the matrix products read and write through strides)
+    Status transpose(size_t i, const ExportOp &op) {
+        if (ex.nodes[i].inputs.size() != 1) return fail(i, "a transpose has one argument");
+        const Val *a;
+        RETURN_STATUS(need_act(i, ex.nodes[i].inputs[0], a));
+        if (!a->sv.on) return fail(i, "transpose of a tensor that is not a view of a matrix (reshape it to its dimensions first)");
+        auto it = op.attrs.find("axes");
+        if (it == op.attrs.end()) return fail(i, "transpose needs axes");
+        const std::vector<long> &ax = it->second;
+        const int rank = a->sv.merged ? 3 : 4;
+        // fewer axes than four: the leading dimensions of size 1 stay in front
+        int lead = 0;
+        if (!a->sv.merged) while (lead < 4 && (int)ax.size() < 4 - lead && a->sv.dim[lead] == 1) ++lead;
+        if ((int)ax.size() != rank - lead) return fail(i, "transpose: " + std::to_string(ax.size()) + " axes for a tensor of " + std::to_string(rank - lead) + " dimensions");
+        Val out = *a;
+        if (a->sv.merged) {
+            if (ax[0] != 0 || !((ax[1] == 1 && ax[2] == 2) || (ax[1] == 2 && ax[2] == 1))) return fail(i, "of a [batch x heads, rows, columns] tensor only the last two axes can be swapped");
+            if (ax[1] == 2) { std::swap(out.sv.dim[2], out.sv.dim[3]); std::swap(out.sv.str[2], out.sv.str[3]); }
+        } else {
+            bool seen[4] = {false, false, false, false};
+            for (size_t k = 0; k < ax.size(); ++k) {
+                if (ax[k] < 0 || ax[k] >= (long)ax.size() || seen[ax[k]]) return fail(i, "transpose: axes must be a permutation");
+                seen[ax[k]] = true;
+                out.sv.dim[lead + k] = a->sv.dim[lead + ax[k]];
+                out.sv.str[lead + k] = a->sv.str[lead + ax[k]];
+            }
+        }
+        vals[i] = out;
+        return check_view_shape(i, out.sv);
+    }
+
+    // which batch_matmul results are read back as [batch, rows, heads x columns] (reshape, transpose (0,2,1,3),
+    // reshape): those are written in that order, so that the way back costs nothing
+    std::vector<char> interleave;
+    void plan_batch_matmuls() {
+        interleave.assign(ex.global_len, 0);
+        std::vector<std::vector<size_t>> users(ex.global_len);
+        for (size_t i = 0; i < ex.global_len; ++i) for (size_t j : ex.nodes[i].inputs) if (j < ex.global_len) users[j].push_back(i);
+        auto is_reshape = [&](size_t n) { const ExportOp *o = op_of(n); return ex.nodes[n].func == "__nop" || (o && o->op == "reshape"); };
+        for (size_t i = 0; i < ex.global_len; ++i) {
+            const ExportOp *o = op_of(i);
+            if (!o || o->op != "batch_matmul" || users[i].size() != 1 || (size_t)ex.heads_index == i) continue;
+            const size_t r = users[i][0];
+            if (!is_reshape(r) || ex.nodes[r].shape.size() != 4 || users[r].size() != 1) continue;
+            const ExportOp *t = op_of(users[r][0]);
+            if (!t || t->op != "transpose") continue;
+            auto it = t->attrs.find("axes");
+            if (it != t->attrs.end() && it->second == std::vector<long>{0, 2, 1, 3}) interleave[i] = 1;
+        }
+    }
+
+    // batch_matmul(lhs [b, M, K], rhs [b, N, K]) -> [b, M, N] (relay's nn.batch_matmul; "transpose_b": 0 for rhs [b, K, N]);
+    // "scale_rsqrt": d multiplies the products by 1 / sqrt(d)
+    Status batch_matmul(size_t i, const ExportOp &op) {
+        size_t an, bn;
+        if (!input_of(i, op, "lhs", 0, an) || !input_of(i, op, "rhs", 1, bn)) return fail(i, "batch_matmul needs two arguments");
+        const Val *A, *B;
+        RETURN_STATUS(need_act(i, an, A));
+        RETURN_STATUS(need_act(i, bn, B));
+        if (!A->sv.on || !B->sv.on) return fail(i, "batch_matmul over tensors that are not views of matrices (reshape them to their dimensions first)");
+        if (!op.epilogue.empty()) return fail(i, "batch_matmul takes no epilogue");
+        const bool tb = attr(op, "transpose_b", 0, 1) != 0;
+        const SeqView &a = A->sv, &r = B->sv;
+        const long bo = a.dim[0], bi = a.dim[1], M = a.dim[2], K = a.dim[3];
+        const long N = tb ? r.dim[2] : r.dim[3], Kb = tb ? r.dim[3] : r.dim[2];
+        if (r.dim[0] != bo || r.dim[1] != bi || Kb != K) return fail(i, "batch_matmul: the arguments' batch or inner dimensions differ");
+        if (a.str[3] != 1) return fail(i, "batch_matmul: the rows of the first argument must be contiguous");
+        // the second argument as the GEMM wants it: N x K with K contiguous, or K x N with N contiguous
+        const long k_str = tb ? r.str[3] : r.str[2], n_str = tb ? r.str[2] : r.str[3];
+        int b_is_nk; long ldb;
+        if (k_str == 1) { b_is_nk = 1; ldb = n_str; }
+        else if (n_str == 1) { b_is_nk = 0; ldb = k_str; }
+        else return fail(i, "batch_matmul: neither dimension of the second argument is contiguous");
+        const int vec = b.vec();
+        if (K % vec || a.str[2] % vec || ldb % vec || a.str[0] % vec || a.str[1] % vec || r.str[0] % vec || r.str[1] % vec || (!b_is_nk && N % vec) ||
+            A->t.off % vec || B->t.off % vec)
+            return fail(i, "batch_matmul: dimensions and strides must be multiples of " + std::to_string(vec) + " elements");
+        if (M >= (1L << 31) || N >= (1L << 31) || bo * bi >= (1L << 24)) return fail(i, "batch_matmul: too large");
+        Val out;
+        out.set = true; out.c_log = (int)N;
+        out.t.st = b.add_storage(ex.nodes[i].name, (size_t)(bo * bi * M * N), b.stype_);
+        out.sv.on = true; out.sv.merged = true;
+        out.sv.dim[0] = bo; out.sv.dim[1] = bi; out.sv.dim[2] = M; out.sv.dim[3] = N;
+        if (interleave[i]) { out.sv.str[0] = M * bi * N; out.sv.str[1] = N; out.sv.str[2] = bi * N; out.sv.str[3] = 1; }
+        else { out.sv.str[0] = bi * M * N; out.sv.str[1] = M * N; out.sv.str[2] = N; out.sv.str[3] = 1; }
+        const long scale = attr(op, "scale_rsqrt", 0, 0);
+        const double flops = 2.0 * bo * bi * M * N * (double)K;
+        const double bytes = b.es() * ((double)bo * bi * (M * K + N * K + M * N));
+        KernelInfo &k = b.add_kernel("batch_matmul", OpKind::Gemm, {b.ref(A->t), b.ref(B->t), GraphBuilder::none(), GraphBuilder::none(), b.ref(out.t)}, flops, bytes);
+        gp_gemm_params &p = k.p.gemm;
+        p.dtype = b.gp_dtype(); p.M = (int)M; p.N = (int)N; p.K = (int)K; p.lda = a.str[2]; p.ldb = ldb; p.b_is_nk = b_is_nk; p.ldc = out.sv.str[2];
+        p.alpha = scale > 0 ? 1.f / std::sqrt((float)scale) : 1.f; p.act = GP_ACT_NONE;
+        p.batch = (int)(bo * bi);
+        if (bi > 1) {
+            p.batch_inner = (int)bi;
+            p.stride_a = a.str[1]; p.stride_b = r.str[1]; p.stride_c = out.sv.str[1];
+            p.stride_a_outer = a.str[0]; p.stride_b_outer = r.str[0]; p.stride_c_outer = out.sv.str[0];
+        } else {
+            p.batch_inner = 0;
+            p.stride_a = a.str[0]; p.stride_b = r.str[0]; p.stride_c = out.sv.str[0];
+        }
+        vals[i] = out;
+        return check_view_shape(i, out.sv);
+    }
+
+    // softmax over the last axis of a contiguous view (the attention scores)
+    Status softmax_view(size_t i, const ExportOp &op, const Val &a) {
+        const long axis = attr(op, "axis", 0, -1);
+        const long rank = (long)ex.nodes[i].shape.size();
+        if (axis != -1 && axis != rank - 1) return fail(i, "softmax over the last axis only");
+        if (!a.sv.contiguous() || a.t.off != 0) return fail(i, "softmax over a transposed or sliced tensor");
+        if (!op.epilogue.empty()) return fail(i, "softmax takes no epilogue");
+        Val out = a;
+        out.t.st = b.add_storage(ex.nodes[i].name, (size_t)a.sv.elems(), b.stype_);
+        b.softmax(a.t.st, out.t.st, a.sv.elems() / a.sv.dim[3], (int)a.sv.dim[3], 1.f);
+        vals[i] = out;
+        return check_view_shape(i, out.sv);
+    }
+
+    // reshapes of a transformer: a matrix seen as [batch, sequence, heads, head size] and back
+    Status reshape_seq(size_t i, const Val &a) {
+        long d[4]; int rank;
+        if (!dims4_of(i, d, rank)) return fail(i, "tensors of 1 to 4 dimensions only");
+        Val out = a;
+        if (!a.sv.on) {
+            // a plain matrix seen as four dimensions: a contiguous view
+            if (prod(ex.nodes[i].shape) != (long)a.t.N * a.c_log) return fail(i, "a reshape that changes the number of elements");
+            out.sv.on = true; out.sv.merged = false;
+            long st = 1;
+            for (int k = 3; k >= 0; --k) { out.sv.dim[k] = d[k]; out.sv.str[k] = st; st *= d[k]; }
+            vals[i] = out;
+            return Status::Succ;
+        }
+        if (prod(ex.nodes[i].shape) != a.sv.elems()) return fail(i, "a reshape that changes the number of elements");
+        const SeqView &v = a.sv;
+        // the same four dimensions, the first two seen as one or as two again
+        if (rank == 3 && d[1] == v.dim[0] * v.dim[1] && d[2] == v.dim[2] && d[3] == v.dim[3]) { out.sv.merged = true; vals[i] = out; return Status::Succ; }
+        if (rank == 4 && d[0] == v.dim[0] && d[1] == v.dim[1] && d[2] == v.dim[2] && d[3] == v.dim[3]) { out.sv.merged = false; vals[i] = out; return Status::Succ; }
+        if (!v.contiguous()) return fail(i, "a reshape of a transposed tensor that is more than joining its first two dimensions");
+        if (rank <= 3) {  // contiguous memory read as a matrix again: rows x last dimension
+            out.sv = SeqView();
+            out.c_log = (int)d[3];
+            out.t.N = (int)(a.sv.elems() / d[3]); out.t.H = out.t.W = 1; out.t.C = (int)d[3]; out.t.ps = d[3];
+        } else {
+            out.sv.merged = false;
+            long st = 1;
+            for (int k = 3; k >= 0; --k) { out.sv.dim[k] = d[k]; out.sv.str[k] = st; st *= d[k]; }
+        }
+        vals[i] = out;
+        return Status::Succ;
+    }
+
     Status run() {
         for (const ExportOp &o : ops.funcs) by_func[o.func] = &o;
         if (ops.layout != "NCHW") { error = "ops json: only exports in NCHW layout are mapped"; return Status::Fail; }
@@ -464,6 +766,7 @@ struct Mapper {
         }
         vals.assign(ex.global_len, Val());
         plan_concatenations();
+        plan_batch_matmuls();
         bool have_data = false;
         for (size_t i = 0; i < ex.global_len; ++i) {
             const ExportNode &n = ex.nodes[i];
@@ -472,10 +775,14 @@ struct Mapper {
                 if (have_data) return fail(i, "two inputs named data");
                 have_data = true;
                 int N, C, H, W;
-                if (!nchw_of(i, N, C, H, W)) return fail(i, "tensors of 1, 2 or 4 dimensions only");
+                if (!nchw_of(i, N, C, H, W)) return fail(i, "tensors of 1 to 4 dimensions only");
                 Val v;
                 v.set = true; v.c_log = C;
-                if (n.shape.size() == 4) v.t = b.input_nchw(N, C, H, W);
+                if (n.stype == "int64") {  // token ids (src/tests/test-dnn.cpp:21-23): read by take only
+                    v.is_ids = true;
+                    v.t.st = b.add_storage("data", (size_t)prod(n.shape), "int64");
+                    v.t.N = (int)prod(n.shape); v.t.H = v.t.W = 1; v.t.C = v.t.ps = 1; v.c_log = 1;
+                } else if (n.shape.size() == 4) v.t = b.input_nchw(N, C, H, W);
                 else {
                     v.t.st = b.add_storage("data", (size_t)N * C, b.stype_);
                     v.t.N = N; v.t.H = v.t.W = 1; v.t.C = v.t.ps = C;
@@ -496,6 +803,11 @@ struct Mapper {
             else if (op.op == "softmax") s = softmax(i, op);
             else if (op.op == "concatenate") s = concatenate(i, op);
             else if (op.op == "reshape") s = reshape(i);
+            else if (op.op == "take") s = take(i, op);
+            else if (op.op == "layer_norm") s = layer_norm(i, op);
+            else if (op.op == "gelu") s = gelu(i, op);
+            else if (op.op == "transpose") s = transpose(i, op);
+            else if (op.op == "batch_matmul") s = batch_matmul(i, op);
             else s = fail(i, "operator '" + op.op + "' is not mapped onto the native kernels");
             RETURN_STATUS(s);
             RETURN_STATUS(check_shape(i, vals[i]));

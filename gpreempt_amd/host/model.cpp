@@ -153,9 +153,12 @@ Status Model::build_from_export(const std::string &workload, const std::string &
     size_t at = workload.find("dtype=");
     if (at != std::string::npos && workload.find('@') < at) dt = workload.substr(at + 6, workload.find(',', at) == std::string::npos ? std::string::npos : workload.find(',', at) - at - 6);
     if (s == Status::Succ && dt.empty()) {
+        auto type_of = [](const std::string &stype) { return stype == "float32" ? "f32" : stype == "float16" ? "f16" : ""; };
         for (const ExportNode &n : export_->nodes)
-            if (n.func.empty() && n.name == "data") dt = n.stype == "float32" ? "f32" : n.stype == "float16" ? "f16" : "";
-        if (dt.empty()) { err = "the export's data is neither float32 nor float16"; s = Status::Fail; }
+            if (n.func.empty() && n.name == "data") dt = type_of(n.stype);
+        // a model fed token ids (int64 "data"): the element type is that of its output
+        if (dt.empty() && export_->heads_index < export_->nodes.size()) dt = type_of(export_->nodes[export_->heads_index].stype);
+        if (dt.empty()) { err = "neither the export's data nor its output is float32 or float16"; s = Status::Fail; }
     }
     if (s == Status::Succ && dt != "f32" && dt != "f16" && dt != "bf16") { err = "unknown dtype '" + dt + "'"; s = Status::Fail; }
     if (s == Status::Succ) {

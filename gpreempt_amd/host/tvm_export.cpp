@@ -165,7 +165,7 @@ Status parse_export_ops(const std::string &text, ExportOps &out) {
     out.layout = v["layout"].string("NCHW");
     if (out.layout != "NCHW" && out.layout != "NHWC") return fail(out.error, "ops json: layout must be NCHW or NHWC");
     static const std::set<std::string> known = {"conv2d", "dense", "max_pool2d", "avg_pool2d", "global_avg_pool2d", "add", "softmax", "layer_norm",
-                                                "batch_matmul", "take", "scale_shift", "concatenate", "reshape"};
+                                                "batch_matmul", "take", "scale_shift", "concatenate", "reshape", "transpose", "gelu"};
     static const std::set<std::string> tails = {"bias", "residual", "relu", "gelu"};
     for (const json::Value &f : v["funcs"].arr) {
         ExportOp op;

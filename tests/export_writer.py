@@ -19,6 +19,7 @@ class ExportWriter:
         self.dt = dt
         self.rng = np.random.default_rng(seed)
         self.nodes, self.shapes, self.values = [], [], []
+        self.dtypes = {}     # node -> dltype, where it is not the model's element type (int64 token ids)
         self.params = {}
         self.funcs = {}      # (base, key) -> function name
         self.taken = {}      # base -> how many functions carry it
@@ -102,9 +103,9 @@ class ExportWriter:
         key = (tuple(self.shapes[x]), cout, kh, kw, sh, sw, ph, pw, tuple(epi))
         return self._op(base, key, "conv2d", attrs, epi, roles, inputs, out, temps)
 
-    def dense(self, x, units, bias=True, relu=False, name=None):
+    def dense(self, x, units, bias=True, relu=False, name=None, gelu=False, residual=None, std=None):
         feat = self.shapes[x][1]
-        w = self.param(self.rng.normal(0, np.sqrt(1.0 / feat), (units, feat)))
+        w = self.param(self.rng.normal(0, std if std else np.sqrt(1.0 / feat), (units, feat)))
         inputs, roles, epi, base = [x, w], {"data": 0, "weight": 1}, [], "nn_dense"
         if name:
             self.alias[name + ".weight"] = self.nodes[w]["name"]
@@ -115,10 +116,82 @@ class ExportWriter:
                 self.alias[name + ".bias"] = self.nodes[b]["name"]
             bv = self.values[b]
             roles["bias"] = 2; inputs.append(b); epi.append("bias"); base += "_add"
+        rv = None
+        if residual is not None:
+            rv = self.values[residual]
+            roles["residual"] = len(inputs); inputs.append(residual); epi.append("residual"); base += "_add"
         if relu:
             epi.append("relu"); base += "_nn_relu"
-        out = self._r(O.gemm_bias_act(self.values[x], self.values[w], bv, None, O.ACT_RELU if relu else O.ACT_NONE, b_is_nk=True))
+        if gelu:
+            epi.append("gelu"); base += "_multiply_erf_add_multiply_multiply"
+        act = O.ACT_RELU if relu else O.ACT_GELU if gelu else O.ACT_NONE
+        out = self._r(O.gemm_bias_act(self.values[x], self.values[w], bv, rv, act, b_is_nk=True))
         return self._op(base, (tuple(self.shapes[x]), units, tuple(epi)), "dense", {}, epi, roles, inputs, out)
+
+    # ---- transformer operators (the functions of a BERT export) -------------------------------------
+    def data_ids(self, ids):
+        n = self._node("data", [], np.asarray(ids, np.int64))
+        self.dtypes[n] = "int64"
+        return n
+
+    def take_embed(self, ids, vocab, hidden, position=True, segment=True, names=None):
+        """take(word table, ids) + position rows + segment row: one fused function, as TVM fuses a gather with the
+        broadcast additions behind it"""
+        B, S = self.shapes[ids]
+        word = self.param(self.rng.normal(0, 0.02, (vocab, hidden)))
+        inputs, roles, base = [word, ids], {"table": 0, "indices": 1}, "take"
+        pos_v = np.zeros((S, hidden), np.float32)
+        seg_v = None
+        if position:
+            pos = self.param(self.rng.normal(0, 0.02, (1, S, hidden)))  # the first S position rows, folded to a constant
+            pos_v = self.values[pos].reshape(S, hidden)
+            roles["position"] = len(inputs); inputs.append(pos); base += "_add"
+        if segment:
+            seg = self.param(self.rng.normal(0, 0.02, (1, 1, hidden)))
+            seg_v = self.values[seg].reshape(hidden)
+            roles["segment"] = len(inputs); inputs.append(seg); base += "_add"
+        if names:
+            self.alias[names[0]] = self.nodes[word]["name"]
+            if position: self.alias[names[1]] = self.nodes[pos]["name"]
+            if segment: self.alias[names[2]] = self.nodes[seg]["name"]
+        out = self._r(O.embed(self.values[ids], self.values[word], pos_v, seg_v, S)).reshape(B, S, hidden)
+        return self._op(base, (B, S, vocab, hidden, position, segment), "take", {"axis": 0}, [], roles, inputs, out)
+
+    def layer_norm(self, x, eps=(1, -12), residual=None, name=None):
+        c = self.shapes[x][-1]
+        g = self.param(self.rng.uniform(0.8, 1.2, (c,)))
+        bt = self.param(self.rng.uniform(-0.1, 0.1, (c,)))
+        if name:
+            self.alias[name + ".gamma"], self.alias[name + ".beta"] = self.nodes[g]["name"], self.nodes[bt]["name"]
+        inputs, roles = [x, g, bt], {"data": 0, "gamma": 1, "beta": 2}
+        rv = None
+        if residual is not None:
+            rv = self.values[residual]
+            roles["residual"] = 3; inputs.append(residual)
+        out = self._r(O.layernorm(self.values[x], self.values[g], self.values[bt], eps[0] * 10.0 ** eps[1], rv))
+        return self._op("add_layer_norm" if residual is not None else "layer_norm", (tuple(self.shapes[x]), eps, residual is not None), "layer_norm",
+                        {"axis": -1, "epsilon": list(eps)}, [], roles, inputs, out)
+
+    def gelu(self, x):
+        out = self._r(O.add_act(self.values[x], None, O.ACT_GELU))
+        return self._op("multiply_erf_add_multiply_multiply", tuple(self.shapes[x]), "gelu", {}, [], {"data": 0}, [x], out)
+
+    def reshape(self, x, shape):
+        """a reshape that TVM turns into a __nop node (it shares its argument's memory)"""
+        return self._node("reshape_nop", [x], self.values[x].reshape(shape), "__nop")
+
+    def transpose(self, x, axes):
+        out = np.ascontiguousarray(np.transpose(self.values[x], axes))
+        return self._op("transpose", (tuple(self.shapes[x]), tuple(axes)), "transpose", {"axes": list(axes)}, [], {"data": 0}, [x], out)
+
+    def batch_matmul(self, a, b, scale_rsqrt=0, transpose_b=True):
+        alpha = 1.0 / np.sqrt(scale_rsqrt) if scale_rsqrt else 1.0
+        out = self._r(O.bmm(self.values[a], self.values[b], alpha=alpha, b_is_nk=transpose_b))
+        attrs = {"transpose_b": int(transpose_b)}
+        if scale_rsqrt:
+            attrs["scale_rsqrt"] = int(scale_rsqrt)
+        return self._op("nn_batch_matmul" + ("_multiply" if scale_rsqrt else ""), (tuple(self.shapes[a]), tuple(self.shapes[b]), scale_rsqrt, transpose_b), "batch_matmul", attrs, [],
+                        {"lhs": 0, "rhs": 1}, [a, b], out)
 
     def pool(self, x, kind, k=2, stride=2, pad=0, count_include_pad=False):
         if kind == "global_avg":
@@ -171,7 +244,7 @@ class ExportWriter:
         stype = {"f32": "float32", "f16": "float16", "bf16": "float32"}[self.dt]
         n = len(self.nodes)
         mod = {"nodes": self.nodes, "arg_nodes": [i for i, nd in enumerate(self.nodes) if nd["op"] == "null"], "heads": [[head, 0, 0]],
-               "attrs": {"dltype": ["list_str", [stype] * n], "device_index": ["list_int", [2] * n], "storage_id": ["list_int", list(range(n))],
+               "attrs": {"dltype": ["list_str", [self.dtypes.get(i, stype) for i in range(n)]], "device_index": ["list_int", [2] * n], "storage_id": ["list_int", list(range(n))],
                          "shape": ["list_shape", self.shapes]},
                "node_row_ptr": list(range(n + 1))}
         host = {"temp_args": [4096] * self.n_temp, "funcs": self.host}
@@ -305,3 +378,58 @@ def mlp(dt, seed=7):
     x = w.data(w.rng.normal(0, 1, (6, 64)))
     y = w.dense(x, 48, relu=True)
     return w, w.softmax(w.dense(y, 16))
+
+
+def bert(dt, layers=2, batch=2, seq=32, hidden=128, heads=2, ffn=256, vocab=96, seed=8, separate_tail=False):
+    """A BERT encoder as a PyTorch model reaches TVM (scripts/compile/compile-bert.py:33-52): embedding gather with
+    the position and segment rows added, layer-norm, then per layer separate query / key / value projections,
+    [batch, sequence, heads, size] reshapes and transposes around two batch_matmul functions and a softmax, the
+    output projection with the residual, layer-norm, and the feed-forward pair with erf-GELU.  separate_tail:
+    GELU and the residual additions as functions of their own (the add in front of a layer-norm fused into it)
+    instead of dense epilogues.  Returns (writer, head node, parameters under the built-in "bert" graph's names)."""
+    w = ExportWriter(dt, seed)
+    d = hidden // heads
+    T = batch * seq
+    ids = w.data_ids(w.rng.integers(0, vocab, (batch, seq)))
+    x = w.take_embed(ids, vocab, hidden, names=("embeddings.word", "embeddings.position", "embeddings.token_type"))
+    x = w.layer_norm(x, name="embeddings.ln")
+    x = w.reshape(x, (T, hidden))
+    builtin = {}
+    for l in range(layers):
+        n = f"layer{l}"
+        def heads_of(t):  # [T, hidden] -> [batch * heads, seq, d]
+            t = w.reshape(t, (batch, seq, heads, d))
+            t = w.transpose(t, (0, 2, 1, 3))
+            return w.reshape(t, (batch * heads, seq, d))
+        qkv = [w.dense(x, hidden, std=0.02, name=f"{n}.attn.{r}") for r in ("q", "k", "v")]
+        q, k, v = (heads_of(t) for t in qkv)
+        scores = w.batch_matmul(q, k, scale_rsqrt=d)
+        probs = w.softmax(scores)
+        vt = w.transpose(v, (0, 2, 1))                 # relay's batch_matmul wants [b, N, K]
+        ctx = w.batch_matmul(probs, vt)
+        ctx = w.reshape(ctx, (batch, heads, seq, d))
+        ctx = w.transpose(ctx, (0, 2, 1, 3))
+        ctx = w.reshape(ctx, (T, hidden))
+        if separate_tail:
+            ao = w.dense(ctx, hidden, std=0.02, name=n + ".attn.proj")
+            x1 = w.layer_norm(ao, residual=x, name=n + ".ln1")
+            f1 = w.gelu(w.dense(x1, ffn, std=0.02, name=n + ".ffn1"))
+            f2 = w.add(w.dense(f1, hidden, std=0.02, name=n + ".ffn2"), x1)
+            x = w.layer_norm(f2, name=n + ".ln2")
+        else:
+            ao = w.dense(ctx, hidden, std=0.02, residual=x, name=n + ".attn.proj")
+            x1 = w.layer_norm(ao, name=n + ".ln1")
+            f1 = w.dense(x1, ffn, std=0.02, gelu=True, name=n + ".ffn1")
+            f2 = w.dense(f1, hidden, std=0.02, residual=x1, name=n + ".ffn2")
+            x = w.layer_norm(f2, name=n + ".ln2")
+        # the built-in graph holds the three projections as one matrix
+        for part in ("weight", "bias"):
+            builtin[f"{n}.attn.qkv.{part}"] = np.concatenate([w.params[w.alias[f"{n}.attn.{r}.{part}"]] for r in ("q", "k", "v")], axis=0)
+    for name, pname in w.alias.items():
+        if ".attn.q." in name or ".attn.k." in name or ".attn.v." in name:
+            continue
+        builtin[name] = w.params[pname]
+    builtin["embeddings.position"] = builtin["embeddings.position"].reshape(seq, hidden)
+    builtin["embeddings.token_type"] = builtin["embeddings.token_type"].reshape(1, hidden)
+    head = w.reshape(x, (batch, seq, hidden))
+    return w, head, builtin

@@ -494,3 +494,52 @@ def test_exported_densenet_equals_the_builtin_graph(gp, ex_mod, tmp_path):
     assert [k["name"] for k in ex.kernels()] == [k["name"] for k in ref.kernels()]
     assert np.array_equal(got, run(gp, ref, x, gp.F16, want.shape))
     ex.destroy(); ref.destroy()
+
+
+@pytest.mark.parametrize("dt", ["f16", "f32"])
+@pytest.mark.parametrize("separate_tail", [False, True])
+def test_exported_bert_matches_oracle(gp, ex_mod, tmp_path, dt, separate_tail):
+    """A BERT encoder written as an export (take, layer_norm, three projections, reshapes and transposes around two
+    batch_matmul functions and a softmax, erf-GELU): against the oracle's operators applied node by node as the
+    writer goes, and against the oracle's own BERT composition on the same parameters."""
+    import export_writer as EW
+    w, head, builtin = EW.bert(dt, layers=2, separate_tail=separate_tail)
+    want = w.write(str(tmp_path / "bert_export"), head)
+    ex = ex_mod.Executor("bert_export", model_root=str(tmp_path))
+    dtype = gp.DTYPE_BY_NAME[dt]
+    ids = w.value(0).astype(np.int64)
+    got = run(gp, ex, ids, dtype, (64, 128))
+    assert rel_err(got, want.reshape(64, 128)) < TOL[dt]
+    ref = OM.bert(builtin, ids.reshape(-1), dt, batch=2, seq=32, layers=2, hidden=128, heads=2, fused_attention=False)
+    assert rel_err(got, ref) < TOL[dt]
+    assert {s["name"] for s in ex.storages() if s["is_param"]} == set(w.params)
+    ex.destroy()
+
+
+def test_exported_bert_equals_the_builtin_graph(gp, ex_mod, tmp_path):
+    """The same encoder from the export and from the built-in "bert" graph (its attention as batch_matmul, softmax,
+    batch_matmul; the three projections there are one matrix) on the same parameters: the same bits."""
+    import export_writer as EW
+    w, head, builtin_params = EW.bert("f16", layers=2)
+    w.write(str(tmp_path / "bert_export"), head)
+    ids = w.value(0).astype(np.int64)
+    ex = ex_mod.Executor("bert_export", model_root=str(tmp_path))
+    got = run(gp, ex, ids, gp.F16, (64, 128))
+    builtin = "bert@b=2,s=32,layers=2,hidden=128,heads=2,ffn=256,vocab=96,maxpos=32,fused_attention=0,dtype=f16"
+    os.makedirs(str(tmp_path / builtin))
+    ex_mod.write_params(str(tmp_path / builtin / "mod.params"), builtin_params)
+    ref = ex_mod.Executor(builtin, model_root=str(tmp_path))
+    assert set(builtin_params) == {s["name"] for s in ref.storages() if s["is_param"]}
+    assert ex.kernel_num() == ref.kernel_num() + 2 * 2  # three projections per layer where the built-in graph has one
+    assert np.array_equal(got, run(gp, ref, ids, gp.F16, (64, 128)))
+    ex.destroy(); ref.destroy()
+
+
+@pytest.mark.parametrize("program", [False, True])
+def test_exported_bert_preempt_resume_bit_exact(gp, ex_mod, tmp_path, program):
+    import export_writer as EW
+    w, head, _ = EW.bert("f16", layers=2, batch=4, seq=64)
+    w.write(str(tmp_path / "bert_export"), head)
+    ids = w.value(0).astype(np.int64)
+    # the embedding, a projection, both batched products, a dense layer with a residual, the last layer-norm
+    _blp_roundtrip(gp, ex_mod, tmp_path, "bert_export", ids, [(0, 0), (3, 1), (5, 2), (7, 1), (8, 0), (-1, 1)], graph=program)

@@ -221,7 +221,8 @@ def test_what_cannot_be_mapped_is_refused_by_name(tmp_path):
         ("stride", conv_attr("strides", [2, 2]), "the export says 1x4x8x8, the operator attributes give 1x4x4x4"),
         ("tail", lambda f, doc: doc["funcs"][0].__setitem__("epilogue", ["relu", "bias"]) if f == "ops.json" else None, "in that order"),
         ("role", lambda f, doc: doc["funcs"][0]["inputs"].__setitem__("weight", 0) if f == "ops.json" else None, "must be a parameter"),
-        ("bert", lambda f, doc: doc["funcs"][1].__setitem__("op", "layer_norm") if f == "ops.json" else None, "operator 'layer_norm' is not mapped"),
+        ("bert", lambda f, doc: doc["funcs"][1].__setitem__("op", "layer_norm") if f == "ops.json" else None, "layer_norm needs data, gamma and beta"),
+        ("view", lambda f, doc: doc["funcs"][1].update(op="transpose", attrs={"axes": [1, 0]}) if f == "ops.json" else None, "a transpose has one argument"),
         ("layout", lambda f, doc: doc.__setitem__("layout", "NHWC") if f == "ops.json" else None, "NCHW"),
     ]:
         d = _edited(tmp_path, name, edit)
@@ -258,3 +259,59 @@ def test_what_cannot_be_mapped_is_refused_by_name(tmp_path):
             doc["attrs"]["shape"][1][5] = [10, 1e300]
     rc, rep = plan(_edited(tmp_path, "huge3", not_an_integer))
     assert rc == 1 and "bad shape of node 5" in rep["error"]
+
+
+def test_bert_export_maps_onto_the_transformer_kernels(tmp_path):
+    """The functions of a BERT export (scripts/compile/compile-bert.py:76-77: take, layer_norm, dense, reshape /
+    transpose around batch_matmul, softmax, erf-GELU) become embed, layernorm, dense and batched GEMM launches; the
+    reshapes and transposes between them cost no kernel: the batched products read the heads through strides and
+    the second one writes its result where the transpose back would have put it."""
+    import export_writer as EW
+    B, S, H, heads, d, F = 2, 32, 128, 2, 64, 256
+    w, head, builtin = EW.bert("f16", layers=2, batch=B, seq=S, hidden=H, heads=heads, ffn=F)
+    dd = str(tmp_path / "bert")
+    w.write(dd, head)
+    rc, rep = plan(dd)
+    assert rc == 0, rep
+    assert rep["dtype"] == "f16"  # "data" holds int64 token ids: the element type is the output's
+    k = rep["kernels"]
+    per_layer = ["dense", "dense", "dense", "batch_matmul", "softmax", "batch_matmul", "dense", "layernorm", "dense", "dense", "layernorm"]
+    assert [x["name"] for x in k] == ["embed", "layernorm"] + per_layer * 2
+    assert k[0]["params"] == {"tokens": B * S, "seq": S, "hidden": H, "vocab": 96} and k[0]["args"][0] == "data"
+    assert abs(k[1]["params"]["eps"] - 1e-12) < 1e-18
+    qk, sm, pv, proj, ln1, f1, f2 = k[5], k[6], k[7], k[8], k[9], k[10], k[11]
+    # Q K^T per head: rows of the [tokens, hidden] projections, a head every 64 columns, a batch every S rows
+    assert qk["params"] == {"M": S, "N": S, "K": d, "lda": H, "ldc": S, "act": 0, "batch": B * heads, "batch_inner": heads, "ldb": H, "b_is_nk": 1, "alpha": 0.125,
+                            "stride_a": d, "stride_b": d, "stride_c": S * S, "stride_a_outer": S * H, "stride_b_outer": S * H, "stride_c_outer": heads * S * S}
+    assert sm["params"] == {"rows": B * heads * S, "cols": S}
+    # P V: V is read untransposed (K x N with the model's row stride); the result lands as [tokens, hidden]
+    assert pv["params"]["b_is_nk"] == 0 and pv["params"]["ldb"] == H and pv["params"]["ldc"] == H
+    assert (pv["params"]["stride_c"], pv["params"]["stride_c_outer"]) == (d, S * H)
+    assert proj["args"][3] != "" and f2["args"][3] != ""      # the residuals ride in the dense epilogues
+    assert f1["params"]["act"] == 2                              # erf-GELU in the epilogue
+    assert proj["params"]["lda"] == H and k[-1]["args"][-1] == "heads"
+    st = {x["name"]: x for x in rep["storages"]}
+    assert st["data"]["stype"] == "int64" and st["data"]["size"] == 8 * B * S
+    assert st["heads"]["size"] == 2 * B * S * H
+    assert {x["name"] for x in rep["storages"] if x["is_param"]} == set(w.params)
+    # GELU and the residual additions as functions of their own: an element-wise launch each, the add in front of a
+    # layer-norm inside it
+    w, head, _ = EW.bert("f32", layers=1, separate_tail=True)
+    dd = str(tmp_path / "bert_sep")
+    w.write(dd, head)
+    rc, rep = plan(dd)
+    assert rc == 0, rep
+    names = [x["name"] for x in rep["kernels"]]
+    assert names == ["embed", "layernorm", "dense", "dense", "dense", "batch_matmul", "softmax", "batch_matmul", "dense", "layernorm", "dense", "eltwise", "dense", "eltwise", "layernorm"]
+    assert rep["kernels"][9]["args"][1] != ""  # layer_norm(data + residual)
+    assert rep["kernels"][11]["params"]["act"] == 2
+    # what the views cannot express is refused by name
+    w, head, _ = EW.bert("f16", layers=1)
+    for fn in w.ops:
+        if fn["op"] == "transpose" and fn["attrs"]["axes"] == [0, 2, 1, 3]:
+            fn["attrs"]["axes"] = [0, 1, 3, 2]
+            break
+    dd = str(tmp_path / "bert_bad")
+    w.write(dd, head)
+    rc, rep = plan(dd)
+    assert rc == 1 and "the export's shape differs" in rep["error"]
