@@ -73,11 +73,13 @@ def config_leg(name, seconds):
     high-priority p99 against isolated, preemption latency, and what every lower level kept."""
     with open(os.path.join(ROOT, "gpreempt_amd", "config", name)) as f:
         cfg = json.load(f)
-    cfg.update({"time": seconds, "standalone_runs": 60, "warmups": 5})
+    # (with the GPU's own time stamps switched on: a workgroup of the lower levels writes the device clock when it leaves)
+    cfg.update({"time": seconds, "standalone_runs": 60, "warmups": 5, "device_stamps": True})
     rep = run_config(cfg)
     out = {"config": name, "seconds": seconds, "policy": rep["policy"], "hp_p99_vs_isolated": rep["hp_p99_vs_isolated"],
            "preemption_latency_us": {k: rep["preemptLatency(us)"][k] for k in ("count", "mean", "p99", "max")},
-           "be_throughput_kept": rep["be_throughput_kept"], "levels": {}}
+           "be_throughput_kept": rep["be_throughput_kept"], "levels": {},
+           "device_stamps_us": {k: {q: v[q] for q in ("count", "mean", "p50", "p99", "max")} for k, v in rep.get("deviceStamps(us)", {}).items()}}
     for tid, t in rep["tasks"].items():
         e = {"priority": t["priority"], "model": t["model"], "requests": t["requests"], "req_s": t["avgThroughput(req/s)"],
              "isolated_ms": t["standAlone(us)"]["mean"] / 1e3, "p99_ms": t["totalLatency(us)"]["p99"] / 1e3, "preemptions": t["preemptions"]}
@@ -86,6 +88,8 @@ def config_leg(name, seconds):
             e["isolated_req_s"] = t["standAloneThroughput(req/s)"]
         if "p99_vs_isolated" in t:
             e["p99_vs_isolated"] = t["p99_vs_isolated"]
+        if t.get("slowestDrains"):
+            e["slowest_drains"] = [{"us": d["us"], "kernel": d["stopKernel"], "name": d.get("name", ""), "tiles": d.get("tiles", 0)} for d in t["slowestDrains"][:3]]
         out["levels"][tid] = e
     return out
 
@@ -558,19 +562,20 @@ def summary_of(out):
         s["headline_600"] = {"value": r3(h["value"]), "hp_p99_ms_isolated_corun": [r3(h["hp_isolated_ms"]["p99"]), r3(h["hp_corun_ms"]["p99"])],
                              "preempt_us_mean_p99": [r2(h["preemption_latency_us"]["mean"]), r2(h["preemption_latency_us"]["p99"])],
                              "be_kept": r3(h["be_throughput_kept"]), "be_req_s_corun_isolated": [r2(h["be_throughput_req_s"]), r2(h["be_isolated_req_s"])]}
-    for key, tag in (("config4_three_tenants", "config4"), ("config5_bert384_over_gemm8192", "config5")):
+    for key, tag in (("config2_resnet50_fp32_b1_preempted", "config2"), ("config4_three_tenants", "config4"), ("config5_bert384_over_gemm8192", "config5")):
         c = out.get(key)
         if c:
             s[tag] = {"hp_p99_vs_isolated": r3(c["hp_p99_vs_isolated"]), "preempt_us_mean_p99": [r2(c["preemption_latency_us"]["mean"]), r2(c["preemption_latency_us"]["p99"])],
                       "kept": {k: r3(v["throughput_kept"]) for k, v in c["levels"].items() if "throughput_kept" in v},
-                      "req_s": {k: r2(v["req_s"]) for k, v in c["levels"].items() if v["priority"] > 0}}
+                      "req_s": {k: r2(v["req_s"]) for k, v in c["levels"].items() if v["priority"] > 0},
+                      "gpu_drain_us_mean_p99": [r2(c["device_stamps_us"]["flagStore_to_lastWorkgroupExit"][q]) for q in ("mean", "p99")] if c.get("device_stamps_us") else None}
     d = out.get("device_stamps")
     if d:
         s["device_stamps_us_mean_p99"] = {k: [r2(v["mean"]), r2(v["p99"])] for k, v in d.items() if isinstance(v, dict) and "mean" in v}
     c2 = out.get("config2_resnet50_fp32_b1")
     if c2:
-        s["config2_preempt_us_mean_p99"] = [r2(c2["preemption_latency_us"]["mean"]), r2(c2["preemption_latency_us"]["p99"])]
-        s["config2_stamps_us_mean_p99"] = {k: [r2(v["mean"]), r2(v["p99"])] for k, v in c2.get("device_stamps_us", {}).items()}
+        s["config2_as_one_program_preempt_us_mean_p99"] = [r2(c2["preemption_latency_us"]["mean"]), r2(c2["preemption_latency_us"]["p99"])]
+        s["config2_as_one_program_stamps_us_mean_p99"] = {k: [r2(v["mean"]), r2(v["p99"])] for k, v in c2.get("device_stamps_us", {}).items()}
     if "roofline" in out:
         s["conv_launch_us"] = r2(out["roofline"]["avg_launch_us"])
         s["conv_frac"] = round(out["roofline"]["frac"], 4)
@@ -637,6 +642,9 @@ def main():
             out["hp_alone_same_arrivals_ms"] = {k: alone["totalLatency(us)"][k] / 1e3 for k in ("mean", "p50", "p99")}
             out["hp_p99_vs_alone_same_arrivals"] = out["hp_corun_ms"]["p99"] / out["hp_alone_same_arrivals_ms"]["p99"]
             # BASELINE configs 4 and 5 for a few seconds each, and the headline scenario with device time stamps
+            # config 2's tenant as the default policy runs a best-effort tenant (per-kernel launches, two chunks ahead),
+            # stopped at random instants by a high-priority tenant that does next to nothing
+            out["config2_resnet50_fp32_b1_preempted"] = config_leg("config2_resnet50_fp32_preempted.json", args.config_seconds)
             out["config4_three_tenants"] = config_leg("config4_bert_densenet201_vgg16.json", args.config_seconds)
             out["config5_bert384_over_gemm8192"] = config_leg("config5_bert384_gemm8192.json", args.config_seconds)
             out["device_stamps"] = stamps_leg(300, args.warmup, args.policy, args.hp_rate, args.be_model, args.hp_model)

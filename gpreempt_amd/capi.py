@@ -23,11 +23,11 @@ vp = C.c_void_p
 class PreemptCtx(C.Structure):
     _fields_ = [("flag", vp), ("stop_index", vp), ("executed", vp), ("kernel_id", C.c_int),
                 ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("fresh", C.c_int), ("left_host", vp),
-                ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong), ("stamps", vp)]
+                ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong), ("done", vp), ("done_launches", C.c_int), ("stamps", vp)]
 
 
 class LaunchInfo(C.Structure):
-    _fields_ = [("total_tiles", C.c_int), ("shape", C.c_int * 3), ("grid", C.c_int), ("block", C.c_int), ("fixed_claims", C.c_int)]
+    _fields_ = [("total_tiles", C.c_int), ("shape", C.c_int * 3), ("grid", C.c_int), ("block", C.c_int), ("fixed_claims", C.c_int), ("front", C.c_int)]
 
 
 class GemmParams(C.Structure):
@@ -298,12 +298,20 @@ class BlpState:
 
     def reset(self):
         self.executed.upload(np.zeros(self.n * self.ints_per_kernel, np.int32))
+        if getattr(self, "done", None):
+            self.done.upload(np.zeros(self.n * self.ints_per_kernel, np.int32))
 
-    def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0, fresh=0):
+    def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0, fresh=0, done_launches=0):
         ck = getattr(self, "ckpt", None)
         return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id * self.ints_per_kernel, kernel_id, inject_at, max_workgroups,
                           poll_every, self.groups if self.groups > 1 else 0, fresh, None, ck.ptr if ck else None, ck.nbytes if ck else 0,
+                          (self.done.ptr + 4 * kernel_id * self.ints_per_kernel) if getattr(self, "done", None) else None, done_launches,
                           self.stamps.ptr if getattr(self, "stamps", None) else None)
+
+    def enable_done_counters(self):
+        """Counters of the workers that have left (gp_preempt_ctx::done), cleared by reset()."""
+        self.done = DevBuf(4 * self.n * self.ints_per_kernel)
+        self.done.upload(np.zeros(self.n * self.ints_per_kernel, np.int32))
 
     STAMP_WORDS = 8 + 1024
 

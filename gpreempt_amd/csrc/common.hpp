@@ -57,7 +57,7 @@ inline void set_poll_slices(BlpArgs *blp, int grid) {
 // workgroup per tile.
 template <class Kernel>
 int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int sz,
-                const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info, int batch = 1, int waves = 1) {
+                const gp_preempt_ctx *ctx, BlpArgs *blp, int *grid, gp_launch_info *info, int batch = 1, int waves = 1, bool long_tiles = false) {
     long tiles = (long)sx * sy * sz;
     GP_REQUIRE(tiles > 0 && tiles < (1L << 31), "tile count %ld out of range", tiles);
     if (batch < 1) batch = 1;
@@ -86,7 +86,15 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         // by the hardware as others retire) beats a persistent grid that claims through the
         // counters: 4 % on ResNet-152 b8.  The caller allows it where tiles are short; with
         // VGG-16 b16's 128 x 128 tiles it lengthened the drain (p99 130 -> 178 us).
-        if (ng > 1 && ctx->max_workgroups == 0 && total > resident && total <= (long)waves * resident && total + 4 <= (long)ng * kFixedClaimBits)
+        // Long tiles that can be given up (see below) always get a workgroup per claim, up to eight rounds of them: a
+        // persistent grid would finish the tiles it is in.  (Not where the front workgroup, which keeps one place until
+        // the launch ends, would cost a round of its own: a compute unit holds one workgroup of the kernel and the
+        // rounds are full.)
+        bool long_ok = long_tiles && ctx->done && ctx->flag && blp->poll_mask != 0 && ng > 1;
+        if (long_ok && per_cu < 2 && total > resident && (ctx->max_workgroups != 0 || (total + resident - 2) / (resident - 1) != (total + resident - 1) / resident))
+            long_ok = false;
+        if (long_ok && waves < 8) waves = 8;
+        if (ng > 1 && ctx->max_workgroups == 0 && total > resident && total <= (long)waves * resident && total + 8 <= (long)ng * kFixedClaimBits)
             *grid = (int)total;
         if (*grid < blp->groups) *grid = blp->groups;  // every counter needs a workgroup to serve its slice
         // a launch with fixed claims gets four workgroups more, which only read the flag (tile_loop.hpp)
@@ -103,17 +111,45 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         // is half a microsecond; a launch of several rounds waits for the stop index as before (VGG-16 b16 next
         // to two higher levels: drain 41 / 77 us mean / p99 with the wait, 48 / 94 without).
         if (blp->fresh > 1 && (long)*grid > resident) blp->fresh = 1;
+        // A launch with more claims than the device holds workgroups gets eight workgroups in front of its workers, the
+        // first of which reads the flag for as long as claims are still being made (front_workgroup in tile_loop.hpp);
+        // the workers then leave the flag alone.  (Kept out of the slices' arithmetic: the workers are counted without them.)
+        // (Not where a compute unit holds a single workgroup of this kernel: the one that stays would cost a whole
+        // compute unit, a fifth round of tiles for 8192^3 on 256 x 256 tiles.)
+        blp->front = 0; blp->done = nullptr; blp->done_target = 0;
+#ifndef GP_NO_FRONT
+        if (ctx->flag && blp->poll_mask != 0 && blp->spare == 0 && ng > 1 && per_cu >= 2 && total > resident &&
+            (!fixed_claims(true, ng, *grid, (int)total) || fixed_claims(true, ng, *grid + 8, (int)total)))
+            blp->front = 8;
+#endif
+        // Long tiles with fixed claims: the front workgroup stays until the workers have left (they count themselves
+        // in ctx->done), whatever the number of rounds, and takes the place of the spare ones; the tile bodies look at
+        // the stop index every few K-stages and give their tile up when a stop is recorded (tile_fixed_early).
+        const int workers = *grid - blp->spare;
+        if (long_ok && fixed_claims(true, ng, workers, (int)total) && fixed_claims(true, ng, workers + 8, (int)total)) {
+            *grid = workers;
+            blp->spare = 0; blp->front = 8;
+            blp->done = ctx->done;
+            // (the front workgroup leaves when half of the last round of workers has counted itself, which a worker does a
+            // few K-stages before the end of its tile: the microsecond or two in which the front workgroup notices and
+            // gets its last read of the flag back would otherwise come on top of every launch, 2.5 us on each of
+            // ResNet-50's fp32 kernels)
+            const int last_round = (int)(workers < resident ? workers : resident);
+            blp->done_target = ctx->done_launches * workers + workers - last_round / 2;
+        }
         set_poll_slices(blp, *grid);
+        *grid += blp->front;
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
-        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0; blp->spare = 0; blp->stamps = nullptr;
+        blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0; blp->spare = 0; blp->stamps = nullptr; blp->front = 0; blp->done = nullptr; blp->done_target = 0;
         for (int g = 0; g < 4; ++g) blp->poll_n[g] = 0;
         *grid = (int)total;
     }
     if (info) {
         info->total_tiles = (int)total; info->shape[0] = sx; info->shape[1] = sy; info->shape[2] = sz;
         info->grid = *grid; info->block = block;
-        info->fixed_claims = fixed_claims(ctx != nullptr, blp->groups, *grid, (int)total);
+        info->front = blp->front;
+        info->fixed_claims = fixed_claims(ctx != nullptr, blp->groups, *grid - blp->front, (int)total);
     }
     return GP_SUCC;
 }

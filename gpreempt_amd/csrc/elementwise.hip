@@ -30,7 +30,7 @@ static int launch_tiles(KernelSet<Kernel> ks, int sx, int sy, const gp_preempt_c
     Kernel kern = ks.any;
     if (batch == 1) {  // the special forms call the body once: one tile per claim only
         if (!ctx) kern = ks.plain;
-        else if (fixed_claims(true, blp.groups, grid, blp.total)) kern = ks.fixed;
+        else if (fixed_claims(true, blp.groups, grid - blp.front, blp.total)) kern = ks.fixed;
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds_bytes, native(s), arg, blp);
     GP_HIP(hipGetLastError());

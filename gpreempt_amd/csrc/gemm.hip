@@ -23,11 +23,18 @@
 namespace gp {
 
 // LOOP: which dispatcher loop the instantiation is built around (tile_loop.hpp)
+constexpr int LOOP_LOOKS = 3;
 template <class TK, int LOOP>
 __global__ __launch_bounds__(TK::NT) void mat_kernel(MatArgs g, BlpArgs blp) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
     auto *lds = reinterpret_cast<typename TK::elem *>(lds_raw);
-    if constexpr (LOOP == LOOP_FIXED && TK::early_stop)
+    if constexpr (LOOP == LOOP_LOOKS)  // long tiles: fixed claims, and the body looks at the stop word every few K-stages
+        tile_fixed_early<true>(blp, [&](TileIdx t, int *stop) {
+            CkptCtx cc{stop, nullptr, nullptr, 0};
+            if (stop && blp.done) cc.announce = done_counter(blp);
+            return TK::template run<true>(g, t, lds, cc);
+        });
+    else if constexpr (LOOP == LOOP_FIXED && TK::early_stop)
         tile_fixed_early(blp, [&](TileIdx t, int *stop) { return TK::run(g, t, lds, CkptCtx{stop, nullptr, nullptr, 0}); });
     else
         tiles<LOOP>(blp, [&](TileIdx t) { TK::run(g, t, lds); });
@@ -51,11 +58,17 @@ template <class K> struct KernelOf {
     static constexpr auto fn = mat_kernel<K, LOOP_ANY>;
     static constexpr auto plain = mat_kernel<K, LOOP_PLAIN>;
     static constexpr auto fixed = mat_kernel<K, LOOP_FIXED>;
+#ifdef GP_NO_LOOKS  // (experiment switch: no instantiations that look more than once)
+    static constexpr auto looks = fixed;
+#else
+    static constexpr auto looks = mat_kernel<K, K::can_look ? LOOP_LOOKS : LOOP_FIXED>;
+#endif
 };
 template <typename T, int BM, int BN, int ST, bool CV, int W> struct KernelOf<PipeKernel<T, BM, BN, ST, CV, false, true, W>> {
     static constexpr auto fn = mat_kernel_ckpt<PipeKernel<T, BM, BN, ST, CV, false, true, W>>;
     static constexpr auto plain = fn;
     static constexpr auto fixed = fn;
+    static constexpr auto looks = fn;
 };
 
 // bytes of checkpoint workspace a launch of body K needs (0: the body always finishes its tiles)
@@ -73,25 +86,32 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
         static std::once_flag once;
         static hipError_t once_rc = hipSuccess;
         std::call_once(once, [] {
-            for (const void *f : {(const void *)KernelOf<K>::fn, (const void *)KernelOf<K>::plain, (const void *)KernelOf<K>::fixed}) {
+            for (const void *f : {(const void *)KernelOf<K>::fn, (const void *)KernelOf<K>::plain, (const void *)KernelOf<K>::fixed, (const void *)KernelOf<K>::looks}) {
                 hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)K::LDS_BYTES);
                 if (e != hipSuccess) once_rc = e;
             }
         });
         GP_HIP(once_rc);
     }
-    int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info, 1, K::LDS_BYTES <= 64 * 1024 ? 4 : 1);
+    // Long tiles (2 * 10^7 multiply-adds of the 16-bit rate and more, 10-40 us depending on how many workgroups share a
+    // compute unit): what a stopped tenant would otherwise finish before it leaves.  The bodies that look at the stop
+    // word every few K-stages can give such a tile up (tile_fixed_early).  Measured with the threshold at 0.8 / 2 / 4 * 10^7:
+    // ResNet-50 fp32 b1 under a 500 req/s probe drains in 35 / 42 / 57 us (p99) and keeps 1046 / 1095 / 1094 req/s
+    // (a launch in this mode is about a microsecond longer).  GPREEMPT_LONG_TILE_MACS overrides it.
+    static const double long_macs = [] { const char *e = getenv("GPREEMPT_LONG_TILE_MACS"); return e && atof(e) > 0 ? atof(e) : 2e7; }();
+    const bool long_tiles = K::can_look && (double)K::bm * K::bn * pl.g.K * (pl.dtype == GP_F32 ? 8.0 : 1.0) >= long_macs;
+    int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info, 1, K::LDS_BYTES <= 64 * 1024 ? 4 : 1, long_tiles);
     if (rc) return rc;
     blp.order = pl.order;
     if constexpr (K_is_ckpt<K>::value) {
         if (info) info->fixed_claims = 0;  // tile_loop_ckpt always claims through the counters
-        if (blp.spare) { grid -= blp.spare; blp.spare = 0; set_poll_slices(&blp, grid); if (info) info->grid = grid; }
+        if (blp.spare || blp.front) { grid -= blp.spare + blp.front; blp.spare = blp.front = 0; blp.done = nullptr; set_poll_slices(&blp, grid); if (info) { info->grid = grid; info->front = 0; } }
         // mid-tile checkpoints need the caller's workspace and a slot per workgroup
         if (ctx && ctx->ckpt && ctx->ckpt_bytes >= ckpt_workspace_bytes(K::CKPT_SLOT_BYTES, grid) && grid <= CKPT_MAX_WGS) blp.ckpt = ctx->ckpt;
     }
     // one tile per claim here (plan_launch's default), which is what the two special forms assume
     if (!ctx) kern = KernelOf<K>::plain;
-    else if (fixed_claims(true, blp.groups, grid, blp.total)) kern = KernelOf<K>::fixed;  // (not for checkpointing bodies: theirs is fn)
+    else if (fixed_claims(true, blp.groups, grid - blp.front, blp.total)) kern = blp.done ? KernelOf<K>::looks : KernelOf<K>::fixed;  // (not for checkpointing bodies: theirs is fn)
     hipLaunchKernelGGL(kern, dim3(grid), dim3(K::NT), K::LDS_BYTES, native(s), pl.g, blp);
     GP_HIP(hipGetLastError());
     return GP_SUCC;
@@ -110,6 +130,14 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
 #ifndef GP_S32
 #define GP_S32 4
 #endif
+// The large-GEMM body.  Experiment switch GP_BIG_BM / GP_BIG_BN / GP_BIG_STAGES: another tile shape and ring depth
+// for it (128 x 256 with three stages has a prefetch distance of two stages in 144 KB of LDS).
+#ifndef GP_BIG_BM
+#define GP_BIG_BM 256
+#define GP_BIG_BN 256
+#define GP_BIG_STAGES 2
+#endif
+template <typename T, bool CK> using BigPipe = PipeKernel<T, GP_BIG_BM, GP_BIG_BN, GP_BIG_STAGES, false, false, CK, GP_W256>;
 template <typename T, int TILE, int STAGES, bool SPLITK>
 static int pipe_case(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, gp_launch_info *info) {
     if (pl.conv) return launch_mat<PipeKernel<T, TILE, TILE, STAGES, true, SPLITK>>(pl, ctx, s, info);
@@ -144,8 +172,8 @@ static int launch_typed(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream 
     constexpr int SBK = sizeof(T) == 4 ? 16 : 32;
     switch (pl.body) {
         case MB_PIPE256:  // GEMM only: the gathered A operand of a convolution does not fit its register budget
-            if (ctx && ctx->ckpt) return launch_mat<PipeKernel<T, 256, 256, 2, false, false, true, GP_W256>>(pl, ctx, s, info);
-            return launch_mat<PipeKernel<T, 256, 256, 2, false, false, false, GP_W256>>(pl, ctx, s, info);
+            if (ctx && ctx->ckpt) return launch_mat<BigPipe<T, true>>(pl, ctx, s, info);
+            return launch_mat<BigPipe<T, false>>(pl, ctx, s, info);
         case MB_PIPE128: return pipe_case_ckpt<T, 128, GP_S128>(pl, ctx, s, info);
         case MB_PIPE64:
             // A layer of at most four K-steps is all prologue and epilogue, and what hides those is more workgroups
@@ -190,7 +218,7 @@ int launch_mat_plan(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s, g
 static size_t body_lds_bytes(int body, int dtype) {
     const size_t es = dtype == GP_F32 ? 4 : 2;
     switch (body) {
-        case MB_PIPE256: return 2 * (256 + 256) * 128;
+        case MB_PIPE256: return BigPipe<_Float16, false>::LDS_BYTES;
         case MB_PIPE128: return GP_S128 * (128 + 128) * 128;
         case MB_PIPE64: return GP_S64 * (64 + 64) * 128;
         case MB_PIPE64_SK: return GP_S64 * (64 + 64) * 128;   // at least the reduction buffer (4 waves x 4 blocks x 16 x 64 x 4 = 64 KB)
@@ -280,8 +308,8 @@ static int choose_body(MatPlan *pl, int tile, int tile_n, int variant) {
         set_error("no matrix kernel for tile %d x %d with variant %d (tiles: 256, 128, 64; 64, 32 with split K; wide: 32x32, 64x32, 64x64, N x K operands; convolutions with Cin a multiple of the K-block and at most 32 taps)", tile, tile_n ? tile_n : tile, variant);
         return GP_OUTOFRANGE;
     }
-    int t = body == MB_PIPE256 ? 256 : (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
-    int tn = t;
+    int t = body == MB_PIPE256 ? GP_BIG_BM : (body == MB_PIPE128 || body == MB_STAGED128) ? 128 : (body == MB_PIPE32_SK ? 32 : 64);
+    int tn = body == MB_PIPE256 ? GP_BIG_BN : t;
     if (const WideChoice *w = wide_of(body)) { t = w->bm; tn = w->bn; }
     if (body == MB_LNWIDE32x64_16) { t = 32; tn = 64; }
     pl->body = body;
@@ -455,7 +483,7 @@ extern "C" int gp_debug_tile_prof(unsigned long long *out, int n) {
 // bodies): headers plus one accumulator slot per resident workgroup.
 namespace gp {
 static size_t plan_ckpt_bytes(const MatPlan &pl) {
-    if (pl.body == MB_PIPE256) return ckpt_workspace_bytes(PipeKernel<float, 256, 256, 2, false, false, true, GP_W256>::CKPT_SLOT_BYTES, (int)device_cus());
+    if (pl.body == MB_PIPE256) return ckpt_workspace_bytes(BigPipe<float, true>::CKPT_SLOT_BYTES, (int)device_cus());
     if (pl.body == MB_PIPE128) return ckpt_workspace_bytes(PipeKernel<float, 128, 128, GP_S128, false, false, true>::CKPT_SLOT_BYTES, 2 * (int)device_cus());
     return 0;
 }

@@ -50,6 +50,7 @@ struct LnWideKernel {
     static constexpr size_t CKPT_SLOT_BYTES = 0;
     static constexpr bool ckpt = false;
     static constexpr bool early_stop = true;
+    static constexpr bool can_look = false;
     static constexpr int PRE = GP_WIDE_PREFILL ? STAGES : STAGES - 1;
     static_assert(sizeof(T) == 2, "16-bit element types");
     static_assert(WAVES == 16 && BM % WAVES == 0 && BN % 32 == 0 && BM % 32 == 0, "tile shape");

@@ -87,6 +87,8 @@ struct CkptCtx {       // what a checkpointing body needs from the dispatcher, p
     void *ckpt;
     int kernel_id;
     unsigned long long *stamps = nullptr;  // BlpArgs::stamps (the measurement mode of tile_loop.hpp)
+    int *announce = nullptr;               // run<true> with a stop word: the counter in which the workgroup counts itself at its
+                                           // last look, less than LOOK_EVERY K-steps before the end of a tile that it finishes
 };
 
 // NWAVES: wavefronts per workgroup.  With eight (two per SIMD, 128 accumulator registers each) the
@@ -114,6 +116,7 @@ struct PipeKernel {
     static constexpr size_t CKPT_SLOT_BYTES = (size_t)WAVES * MI * NI * 16 * 64 * 4;  // one workgroup's accumulators
     static constexpr bool ckpt = CKPT;
     static constexpr bool early_stop = !CKPT;  // run() takes an early-stop word (see there)
+    static constexpr bool can_look = !CKPT;    // run<true>() looks at it again every few K-steps
     // The stop words are fetched with every stage (so that every wave issues the same number of
     // loads) but looked at every POLL_EVERY-th K-step: about every 2.5 us for either tile size.
     static constexpr int POLL_EVERY = BM >= 256 ? 2 : 4;
@@ -131,6 +134,7 @@ struct PipeKernel {
     // all claim at once while a few spare workgroups read the host flag (tile_loop.hpp): the flag
     // read takes 1-2 us, so without the second look a kernel launched just after the flag went up
     // would still run to its end.
+    template <bool LOOKS = false>
     static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0},
                                                int tile_index = 0, int kt0 = 0) {
         GP_PROBE(0);
@@ -138,6 +142,14 @@ struct PipeKernel {
         // (made wave-uniform by force: handed over in a vector register, the word would make the compiler treat every branch
         // that depends on it as divergent, and the barriers and hand-placed waits below assume uniform control flow)
         const bool early = !CKPT && __builtin_amdgcn_readfirstlane((int)(cc.stop_index != nullptr)) != 0;
+        // Long tiles look again every LOOK_EVERY K-steps (a K-step is 64 elements, a quarter to half a microsecond): the
+        // word is fetched by wavefront 0 at the top of the K-step in which the stage it travels with is fetched, in
+        // front of that stage's loads, and read by everybody at the end of that stage's K-step.  A tile that finds a
+        // stop recorded is given up (the caller withdraws the claim; the relaunch computes it from the start).
+        constexpr int LOOK_EVERY = 8;
+        static_assert(LOOK_EVERY >= STAGES, "a look is read before the next one is fetched");
+        // (an instantiation of its own, LOOKS: as a run-time switch the looks cost the short tiles 3 % of a ResNet-152 pass)
+        const bool looking = LOOKS && early;
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
         const int tid = threadIdx.x, lane = tid & 63;
@@ -242,7 +254,12 @@ struct PipeKernel {
                 const void *src = zero;
                 if (can_ckpt) {
                     if (wave == 0) src = cc.stop_index;
-                    else if (wave == 1 && blockIdx.x < 8 && cc.flag && ((sa.k0 / BK) & (8 * POLL_EVERY - 1)) == (int)blockIdx.x * POLL_EVERY) src = cc.flag;
+                    // Whose turn it is goes by the clock, not by the K position: workgroups that continue tiles left
+                    // at different depths are at different K positions, and turns taken by position then bunch up
+                    // (a stop took up to 44 us to be recorded).  A turn is 5.12 us (two looks of this workgroup at
+                    // least fall into it), eight turns a cycle.
+                    else if (wave == 1 && blockIdx.x < 8 && cc.flag && ((sa.k0 / BK) & (POLL_EVERY - 1)) == 0 &&
+                             (int)((wall_clock64() >> 9) & 7) == (int)blockIdx.x) src = cc.flag;
                 }
                 load_lds4(src, sa.sbase_poll + (unsigned)wave * 256);
             } else if (l < A_PW) {
@@ -405,6 +422,10 @@ struct PipeKernel {
             const int stage = kt % STAGES;
             StageAddr sa = {};
             if constexpr (ISSUE) sa = stage_addr(kt + STAGES - 1);
+            if constexpr (ISSUE && !CKPT) {
+                if (looking && wave == 0 && ((kt + STAGES - 1 - kt0) & (LOOK_EVERY - 1)) == 0)
+                    load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
+            }
             if constexpr (SPLITK) {
                 read_frags(0, stage, wave);  // the address arithmetic of the loads overlaps the LDS latency
                 if constexpr (ISSUE) static_for<0, NLOADS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
@@ -442,7 +463,8 @@ struct PipeKernel {
             }
             int stop_now = 0;
             if constexpr (!CKPT) {
-                if (early && kt == kt0) stop_now = __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1;
+                if ((early && kt == kt0) || (looking && kt > kt0 && ((kt - kt0) & (LOOK_EVERY - 1)) == 0))
+                    stop_now = __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1;
             }
             if constexpr (CKPT) {
                 const int sw = __builtin_amdgcn_readfirstlane(stop_word), fw = __builtin_amdgcn_readfirstlane(flag_word);
@@ -481,14 +503,22 @@ struct PipeKernel {
                 load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
         }
         int kt = kt0, stopped = 0;
+        // the K-step of the last look (the first K-step when the tile is too short for another)
+        const int kt_last_look = kt0 + (KT - 1 - kt0) / LOOK_EVERY * LOOK_EVERY;
+        auto announce = [&](int k) {
+            if constexpr (LOOKS)
+                if (looking && cc.announce && k == kt_last_look && tid == 0) __hip_atomic_fetch_add(cc.announce, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        };
         for (; kt + STAGES - 1 < KT; ++kt) {
             stopped = ktile(kt, false, IntC<1>{});
-            if (stopped) break;  // (CKPT: leave the tile here; otherwise only the early look at the first step can say so)
+            if (stopped) break;  // (CKPT: leave the tile here; otherwise only the looks can say so)
+            announce(kt);
         }
         if (!stopped)
             for (; kt < KT; ++kt) {
                 const int st = ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
                 if (!CKPT && st) { stopped = 1; break; }  // (a checkpointing body finishes a tile whose last stages are in flight)
+                announce(kt);
             }
         if (!CKPT && stopped) {
             wait_vmcnt<0>();  // operand loads still landing in LDS must not outlive the workgroup

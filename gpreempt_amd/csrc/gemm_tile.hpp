@@ -20,6 +20,7 @@ struct TileKernel {
     static constexpr int A_PER = (A_CHUNKS + NT - 1) / NT, B_PER = (B_CHUNKS + NT - 1) / NT;
     static constexpr size_t LDS_BYTES = (size_t)(BM + BN) * LDK * sizeof(T);
     static constexpr bool early_stop = false;
+    static constexpr bool can_look = false;
     static_assert(BK % KSTEP == 0 && WM % 32 == 0 && WN % 32 == 0, "tile shape");
     static_assert(A_CHUNKS % NT == 0 && B_CHUNKS % NT == 0, "loader shape");
 

@@ -158,6 +158,7 @@ struct WideKernel {
     static constexpr size_t CKPT_SLOT_BYTES = 0;
     static constexpr bool ckpt = false;
     static constexpr bool early_stop = true;  // as PipeKernel::run: a second look at the stop index when the first stage has landed
+    static constexpr bool can_look = true;
     static constexpr int PRE = GP_WIDE_PREFILL ? STAGES : STAGES - 1;  // stages asked for before the main loop
     static_assert(WAVES % 4 == 0 && WAVES >= 4 && WAVES <= 16, "4, 8, 12 or 16 wavefronts");
     static_assert(BM % 32 == 0 && BN % 32 == 0 && GROUPS % 4 == 0, "tile shape");
@@ -167,10 +168,18 @@ struct WideKernel {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 
     // Returns true when the early look found a stop recorded: the tile was not run.
+    template <bool LOOKS = false>
     static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0}) {
         GP_PROBE(0);
         __shared__ int early_slot[64];
         const bool early = __builtin_amdgcn_readfirstlane((int)(cc.stop_index != nullptr)) != 0;
+        // Long tiles look again every LOOK_EVERY stages (a stage is KB blocks of 64 K-elements: about a microsecond of a
+        // 32 x 32 x 25088 tile): the word is fetched by wavefront 0 in front of the loads of the stage it travels
+        // with, so that the wait for that stage covers it, and read by everybody behind that stage's barrier.  One
+        // landing slot is enough: the next fetch is issued LOOK_EVERY - (STAGES - 1) stages after this one was read.
+        constexpr int LOOK_EVERY = 4;
+        static_assert(LOOK_EVERY >= STAGES, "a look is read before the next one is fetched");
+        const bool looking = LOOKS && early;  // (an instantiation of its own, as in PipeKernel)
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
         const char *lds_c = (const char *)lds_t;
         const int tid = threadIdx.x, lane = tid & 63;
@@ -292,11 +301,19 @@ struct WideKernel {
             else wait_vmcnt<0>();
             __syncthreads();  // everyone's part of stage s is visible; the buffer of stage s-1 is free
             if (s == 0) GP_PROBE(2);
-            if (s == 0 && early && __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1) {
+            if (((s == 0 && early) || (looking && s > 0 && (s & (LOOK_EVERY - 1)) == 0)) && __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1) {
                 wait_vmcnt<0>();  // loads still landing in LDS must not outlive the workgroup
-                return true;
+                return true;      // the tile is given up: the caller withdraws the claim
             }
-            if (s >= PRE - (STAGES - 1) && s + STAGES - 1 < NS) issue(s + STAGES - 1);
+            if constexpr (LOOKS) {  // the last look: the workgroup counts itself (tile_fixed_early)
+                if (looking && cc.announce && s == (NS - 1) / LOOK_EVERY * LOOK_EVERY && tid == 0)
+                    __hip_atomic_fetch_add(cc.announce, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            if (s >= PRE - (STAGES - 1) && s + STAGES - 1 < NS) {
+                if (looking && wave == 0 && ((s + STAGES - 1) & (LOOK_EVERY - 1)) == 0)
+                    load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
+                issue(s + STAGES - 1);
+            }
             if (kb >= G) continue;  // (uniform) the other wavefronts only fetch
             const int stage = s % STAGES;
 #pragma unroll

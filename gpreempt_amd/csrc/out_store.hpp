@@ -20,17 +20,24 @@ constexpr bool kCoherentStores = false;
 
 typedef unsigned int out_u32x4 __attribute__((ext_vector_type(4)));
 
+// experiment switch: stand-alone kernels store their outputs with the nontemporal hint
+#ifdef GP_NT_STORES
+#define GP_PLAIN_STORE(T, p, v) __builtin_nontemporal_store((T)(v), (T *)(p))
+#else
+#define GP_PLAIN_STORE(T, p, v) (*(T *)(p) = (v))
+#endif
+
 __device__ __forceinline__ void st_out16(void *p, unsigned short v) {
     if (kCoherentStores) __hip_atomic_store((unsigned short *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *(unsigned short *)p = v;
+    else GP_PLAIN_STORE(unsigned short, p, v);
 }
 __device__ __forceinline__ void st_out32(void *p, unsigned int v) {
     if (kCoherentStores) __hip_atomic_store((unsigned int *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *(unsigned int *)p = v;
+    else GP_PLAIN_STORE(unsigned int, p, v);
 }
 __device__ __forceinline__ void st_out64(void *p, unsigned long long v) {
     if (kCoherentStores) __hip_atomic_store((unsigned long long *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *(unsigned long long *)p = v;
+    else GP_PLAIN_STORE(unsigned long long, p, v);
 }
 __device__ __forceinline__ void st_out128(void *p, out_u32x4 v) {
     if (kCoherentStores) {
@@ -38,12 +45,12 @@ __device__ __forceinline__ void st_out128(void *p, out_u32x4 v) {
         __hip_atomic_store((unsigned long long *)p, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         __hip_atomic_store((unsigned long long *)p + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     } else {
-        *(out_u32x4 *)p = v;
+        GP_PLAIN_STORE(out_u32x4, p, v);
     }
 }
 __device__ __forceinline__ void st_out8(void *p, unsigned char v) {
     if (kCoherentStores) __hip_atomic_store((unsigned char *)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    else *(unsigned char *)p = v;
+    else GP_PLAIN_STORE(unsigned char, p, v);
 }
 
 // typed element store

@@ -486,7 +486,7 @@ extern "C" int gp_program_launch(gp_program p, const gp_preempt_ctx *ctx, int re
         a.flag = nullptr; a.stop_index = p->own_stop(); a.inject_layer = -1; a.inject_claim = -1; a.poll_mask = 0;
     }
     if (grid < p->n_groups) grid = p->n_groups;  // every group needs at least one workgroup to serve its slices
-    if (info) { info->total_tiles = 0; for (auto &l : p->layers) info->total_tiles += l.total; info->shape[0] = n; info->shape[1] = a.launch_tag; info->shape[2] = 1; info->grid = (int)grid; info->block = 256; info->fixed_claims = 0; }
+    if (info) { info->total_tiles = 0; for (auto &l : p->layers) info->total_tiles += l.total; info->shape[0] = n; info->shape[1] = a.launch_tag; info->shape[2] = 1; info->grid = (int)grid; info->block = 256; info->fixed_claims = 0; info->front = 0; }
     switch (p->dtype) {
         case GP_F32: hipLaunchKernelGGL(program_kernel<float>, dim3((unsigned)grid), dim3(256), p->lds_bytes, native(s), a); break;
         case GP_F16: hipLaunchKernelGGL(program_kernel<_Float16>, dim3((unsigned)grid), dim3(256), p->lds_bytes, native(s), a); break;

@@ -57,7 +57,19 @@ struct BlpArgs {
     int spare;        // fixed claims only: the last `spare` workgroups of the grid have no claim and read the flag
     int poll_n[4];    // several counters, claims through them: the number of claims in the slices of counters 0..3
     unsigned long long *stamps;  // nullptr (the default) or device time stamps of the preemption (see "time stamps" below)
+    int front;        // the first `front` workgroups of the grid own no claim; the very first reads the flag until every
+                      // claim of the launch has been made (front_workgroup); the workers are numbered from `front` on
+    int *done;        // nullptr, or counters like `executed` (one per group, COUNTER_STRIDE apart) in which every worker of
+                      // every launch of this kernel counts itself when it leaves.  Set for launches of long tiles: the
+                      // front workgroup then reads the flag until the counters sum to done_target (most workers of
+                      // THIS launch have left: plan_launch), and the bodies look at the stop index
+                      // every few K-stages and give a tile up (the claim is withdrawn, the relaunch redoes it)
+    int done_target;
 };
+
+// a worker's number among the workers of the launch, and how many there are
+__device__ __forceinline__ int wg_id(const BlpArgs &b) { return (int)blockIdx.x - b.front; }
+__device__ __forceinline__ int wg_count(const BlpArgs &b) { return (int)gridDim.x - b.front; }
 
 // Device-scope atomics on ONE address complete at about one per 40 ns on MI355X: a kernel of a
 // few hundred tiles claimed from a single counter spends 10-20 us on claims alone.  A caller may
@@ -160,9 +172,11 @@ __device__ __forceinline__ int claim_tile(const BlpArgs &b, int grp, int slice_l
         const int c = atomicAdd(b.executed + grp * COUNTER_STRIDE, 1);
         if (c < slice_n) {
             claim = slice_lo + c;
+#ifndef GP_NO_INJECT  // (build switch for measuring what the test hook costs: nothing measurable)
             if (claim == b.inject_at && b.flag)
                 __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            if ((c & b.poll_mask) == 0 && b.flag && reads_flag(b, grp) &&
+#endif
+            if (b.front == 0 && (c & b.poll_mask) == 0 && b.flag && reads_flag(b, grp) &&
                 __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
                 record_stop(b.stop_index, b.kernel_id, b.stamps);
             // the polling workgroup still owes the tile it has just claimed
@@ -189,9 +203,9 @@ static_assert(kFixedClaimBits == (COUNTER_STRIDE - 1) * 32, "a bit per workgroup
 
 template <bool LOOK = true>
 __device__ __forceinline__ int claim_fixed(const BlpArgs &b, int grp) {
-    if ((int)blockIdx.x >= b.total) return -1;
+    if (wg_id(b) >= b.total) return -1;
     if (LOOK && __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1) return -1;
-    const int j = (int)blockIdx.x >> log2_pow2(b.groups);  // this workgroup's rank among those of its group
+    const int j = wg_id(b) >> log2_pow2(b.groups);  // this workgroup's rank among those of its group
     int *line = b.executed + grp * COUNTER_STRIDE;
     const int bit = 1 << (j & 31);
     if (b.fresh) {
@@ -200,11 +214,14 @@ __device__ __forceinline__ int claim_fixed(const BlpArgs &b, int grp) {
         return -1;  // made in an earlier launch
     }
     __hip_atomic_fetch_add(line, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const int claim = xcd_contiguous((int)blockIdx.x, b.total);
+    const int claim = xcd_contiguous(wg_id(b), b.total);
+#ifndef GP_NO_INJECT
     if (claim == b.inject_at && b.flag)
         __hip_atomic_store(b.flag, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+#endif
     // (with spare workgroups the flag is theirs to read: nobody's tile waits for host memory)
-    if (b.spare == 0 && (grp < 4 || b.poll_mask == 0) && (j & b.poll_mask) == 0 && b.flag &&
+    // (... and so it is with a workgroup in front that does nothing else)
+    if (b.spare == 0 && b.front == 0 && (grp < 4 || b.poll_mask == 0) && (j & b.poll_mask) == 0 && b.flag &&
         __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0)
         record_stop(b.stop_index, b.kernel_id, b.stamps);
     stamp_first_claim(b.stamps);
@@ -223,11 +240,83 @@ __device__ __forceinline__ bool spare_workgroup(const BlpArgs &b, bool fixed, bo
     return true;
 }
 
-// A workgroup of a preemptible launch leaves (every thread calls this; measurement mode only).
-__device__ __forceinline__ void leave_stamped(const BlpArgs &b) {
-    if (!b.stamps || !b.executed) return;
+// A launch of several rounds of workgroups with fixed claims (the hardware starts the later ones as earlier ones
+// retire) looks at the flag only when a workgroup starts, and those start in bursts, a tile's length apart: with
+// 40 us tiles (VGG-16's 512-channel 3 x 3 layers at batch 16) a stop took up to 43 us to be so much as recorded.
+// Such a launch gets `front` workgroups ahead of its workers (a multiple of 8, so that the workers keep their XCDs).
+// The first one stays: one lane reads the flag about every microsecond and records the stop, until a stop is
+// recorded, or every claim of the launch has been made (from then on no workgroup starts that a stop could hold
+// back), or its bounded number of looks is used up.  The others leave at once.  Returns true in a front workgroup.
+__device__ __forceinline__ bool front_workgroup(const BlpArgs &b, bool leader) {
+    if (b.front == 0 || (int)blockIdx.x >= b.front) return false;
+    const int tid = (int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z));
+    if (blockIdx.x != 0 || !b.flag) return true;
+    // Two wavefronts look.  The first reads the flag: a trip to host memory, 1-2 us, and a wavefront cannot end before
+    // its read has come back.  The second reads what lives in the device's memory, every lane one of the counters (at
+    // most 64 of them) and the stop index, a few times per microsecond, so that the end of the launch is noticed soon:
+    // the launch lasts until this workgroup has left, and with one wavefront that read the counters between two reads
+    // of the flag, it left 2-3 us after the point it waits for, which a kernel of 10 us with 3 us tiles feels
+    // (ResNet-152 b8: 3 % of a pass).  They tell each other through a word of LDS that it is time to go.
+    __shared__ int front_leave;
+    const int threads = (int)(blockDim.x * blockDim.y * blockDim.z);
+    const bool two = threads >= 128;  // (a smaller workgroup: one wavefront does both, one after the other)
+    if (tid == 0) front_leave = 0;
     __syncthreads();
-    if ((threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0)) stamp_exit_leader(b.stamps);
+    auto told = [&] { return __hip_atomic_load(&front_leave, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0; };
+    auto tell = [&] { __hip_atomic_store(&front_leave, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); };
+    // (with fixed claims word 0 of a line counts the claims made; handed out through the counters, a counter
+    // runs past its slice by one per workgroup that found it empty: either way the sum reaches the total
+    // no later than the last claim is made.  Long tiles: until most workers of this launch have left; they
+    // count themselves in leave_stamped)
+    const int *counters = b.done ? b.done : b.executed;
+    const int target = b.done ? b.done_target : b.total;
+    const int lanes = threads < 64 ? threads : 64;
+    auto device_look = [&](int lane) {  // true: a stop is recorded, or the launch is about to end
+        const int stop = __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int n = 0;  // (ds_bpermute reads 0 from a lane that is off)
+        for (int g = lane; g < b.groups; g += lanes) n += __hip_atomic_load(counters + g * COUNTER_STRIDE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int d = 32; d > 0; d >>= 1) n += __shfl_xor(n, d);
+        return __builtin_amdgcn_readfirstlane(stop) != -1 || __builtin_amdgcn_readfirstlane(n) >= target;
+    };
+    if (tid < 64) {
+        for (int look = 0; look < (1 << 17); ++look) {  // 1-2 us per look: at most about a quarter of a second
+            int flag = 0;
+            if (tid == 0) flag = __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            if (__builtin_amdgcn_readfirstlane(flag) != 0) {
+                if (tid == 0) record_stop(b.stop_index, b.kernel_id, b.stamps);
+                break;
+            }
+            if (two ? told() : device_look(tid)) break;
+            __builtin_amdgcn_s_sleep(4);
+        }
+        if (tid == 0) tell();
+    } else if (two && tid < 128) {
+        for (int look = 0; look < (1 << 19); ++look) {  // about half a microsecond per look
+            if (device_look(tid - 64) || told()) break;
+            __builtin_amdgcn_s_sleep(4);
+        }
+        if (tid == 64) tell();
+    }
+    return true;
+}
+
+// the counter of `done` in which this worker counts itself
+__device__ __forceinline__ int *done_counter(const BlpArgs &b) { return b.done + wg_group(wg_id(b), b.groups) * COUNTER_STRIDE; }
+
+// A worker of a preemptible launch leaves (every thread calls this).  Launches of long tiles count the leavers, for
+// the front workgroup; the measurement mode stamps the moment.
+__device__ __forceinline__ void leave_stamped(const BlpArgs &b, bool count = true) {
+    if (!b.executed || (!b.stamps && !b.done)) return;
+    if (wg_id(b) < 0 || (int)blockIdx.x >= (int)gridDim.x - b.spare) return;  // front and spare workgroups are no workers
+    const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    if (b.stamps) {
+        __syncthreads();
+        if (leader) stamp_exit_leader(b.stamps);
+    }
+    // (no value comes back: the atomic costs the leaver nothing; one line per group keeps them from queueing up on one address)
+    // (count == false: the body has counted the workgroup already, a few K-stages before the end of its tile)
+    if (b.done && count && leader) __hip_atomic_fetch_add(done_counter(b), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Runs body(TileIdx) for every tile this workgroup obtains.  All threads of the workgroup must
@@ -242,14 +331,15 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     // relaunch, and the claim that would only report "nothing left" (an atomic and a barrier at
     // the tail of every small kernel) is skipped.
     GP_DISP_PROBE(0);
-    const bool single = (int)gridDim.x >= b.total;
-    const bool fixed = fixed_claims(dynamic, b.groups, (int)gridDim.x, b.total);
+    if (front_workgroup(b, leader)) return;
+    const bool single = wg_count(b) >= b.total;
+    const bool fixed = fixed_claims(dynamic, b.groups, wg_count(b), b.total);
     // which counter this workgroup serves and the slice of the tile order that counter owns
-    const int grp = wg_group((int)blockIdx.x, b.groups);
+    const int grp = wg_group(wg_id(b), b.groups);
     int slice_lo = 0, slice_n = b.total;
     if (b.groups > 1 && !fixed) {
-        slice_lo = group_slice_begin(b.total, grp, b.groups, (int)gridDim.x);
-        slice_n = group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) - slice_lo;
+        slice_lo = group_slice_begin(b.total, grp, b.groups, wg_count(b));
+        slice_n = group_slice_begin(b.total, grp + 1, b.groups, wg_count(b)) - slice_lo;
     }
     if (spare_workgroup(b, fixed, leader)) return;
     // One loop and one call site for both modes, so that the body is inlined into the kernel and
@@ -257,7 +347,7 @@ __device__ __forceinline__ void tile_loop(const BlpArgs &b, Body &&body) {
     for (int it = 0;; ++it) {
         int idx;
         if (!dynamic) {
-            idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
+            idx = (it == 0 && wg_id(b) < b.total) ? xcd_contiguous(wg_id(b), b.total) : -1;
         } else {
             if (it == 0) GP_DISP_PROBE(1);
             if (leader) mailbox[it & 1] = fixed ? claim_fixed(b, grp) : claim_tile(b, grp, slice_lo, slice_n);
@@ -298,8 +388,9 @@ __device__ __forceinline__ void tile_plain(const BlpArgs &b, Body &&body) {
 __device__ __forceinline__ int fixed_claim_of_workgroup(const BlpArgs &b) {
     __shared__ int mailbox;
     const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
+    if (front_workgroup(b, leader)) return -1;
     if (spare_workgroup(b, true, leader)) return -1;
-    if (leader) mailbox = claim_fixed(b, wg_group((int)blockIdx.x, b.groups));
+    if (leader) mailbox = claim_fixed(b, wg_group(wg_id(b), b.groups));
     __syncthreads();
     return __builtin_amdgcn_readfirstlane(mailbox);
 }
@@ -309,8 +400,8 @@ __device__ __forceinline__ int fixed_claim_of_workgroup(const BlpArgs &b) {
 // (bit cleared, count lowered), so that the relaunch runs it.  The word is handed over only when
 // the launch has spare workgroups reading the flag: that read is what the second look waits for.
 __device__ __forceinline__ void unclaim_fixed(const BlpArgs &b) {
-    const int grp = wg_group((int)blockIdx.x, b.groups);
-    const int j = (int)blockIdx.x >> log2_pow2(b.groups);
+    const int grp = wg_group(wg_id(b), b.groups);
+    const int j = wg_id(b) >> log2_pow2(b.groups);
     int *line = b.executed + grp * COUNTER_STRIDE;
     __hip_atomic_fetch_and(line + 1 + (j >> 5), ~(1 << (j & 31)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __hip_atomic_fetch_add(line, -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -328,24 +419,28 @@ __device__ __forceinline__ void unclaim_fixed(const BlpArgs &b) {
 // a stop word that reaches the body in a vector register (a value merged from two branches does)
 // makes the compiler treat the body's control flow as divergent, and the body, whose barriers and
 // hand-placed waits assume uniform flow, then computes garbage for K of one step.
-template <class Body>
+// ANNOUNCES: a body that was handed a stop word counts its workgroup in b.done itself when it is a few K-stages from the
+// end of a tile that it finishes (so that the front workgroup is gone by the time the workers are: the launch lasts until
+// the last workgroup has left, and the front one needs a microsecond or two to notice and to get its read of the flag back).
+template <bool ANNOUNCES = false, class Body>
 __device__ __forceinline__ void tile_fixed_early(const BlpArgs &b, Body &&body) {
     const bool eager = b.fresh > 1;
     int idx;
     if (eager) {
         const bool leader = threadIdx.x == 0;
+        if (front_workgroup(b, leader)) return;
         if (spare_workgroup(b, true, leader)) return;
-        if ((int)blockIdx.x >= b.total) return;
-        if (leader) claim_fixed<false>(b, wg_group((int)blockIdx.x, b.groups));
-        idx = xcd_contiguous((int)blockIdx.x, b.total);
+        if (wg_id(b) >= b.total) { leave_stamped(b); return; }
+        if (leader) claim_fixed<false>(b, wg_group(wg_id(b), b.groups));
+        idx = xcd_contiguous(wg_id(b), b.total);
     } else {
         idx = fixed_claim_of_workgroup(b);
     }
     if (idx < 0) { leave_stamped(b); return; }
-    int *word = (eager || b.spare) ? b.stop_index : nullptr;
+    int *word = (eager || b.spare || b.front) ? b.stop_index : nullptr;
     const bool left = body(decode_tile(idx, b.sx, b.sy, b.order), word);
     if (left && threadIdx.x == 0) unclaim_fixed(b);
-    leave_stamped(b);
+    leave_stamped(b, !(ANNOUNCES && word != nullptr && !left));
 }
 
 template <class Body>
@@ -391,18 +486,19 @@ __device__ __forceinline__ void tile_loop_span(const BlpArgs &b, Body &&body) {
     __shared__ int mailbox[2];
     const bool dynamic = b.executed != nullptr;
     const bool leader = (threadIdx.x == 0) & (threadIdx.y == 0) & (threadIdx.z == 0);
-    const int grp = wg_group((int)blockIdx.x, b.groups);
-    const bool fixed = fixed_claims(dynamic, b.groups, (int)gridDim.x, b.total);
+    if (front_workgroup(b, leader)) return;
+    const int grp = wg_group(wg_id(b), b.groups);
+    const bool fixed = fixed_claims(dynamic, b.groups, wg_count(b), b.total);
     int slice_lo = 0, slice_n = b.total;
     if (b.groups > 1 && !fixed) {
-        slice_lo = group_slice_begin(b.total, grp, b.groups, (int)gridDim.x);
-        slice_n = group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) - slice_lo;
+        slice_lo = group_slice_begin(b.total, grp, b.groups, wg_count(b));
+        slice_n = group_slice_begin(b.total, grp + 1, b.groups, wg_count(b)) - slice_lo;
     }
     if (spare_workgroup(b, fixed, leader)) return;
     for (int it = 0;; ++it) {
         int idx;
         if (!dynamic) {
-            idx = (it == 0 && (int)blockIdx.x < b.total) ? xcd_contiguous((int)blockIdx.x, b.total) : -1;
+            idx = (it == 0 && wg_id(b) < b.total) ? xcd_contiguous(wg_id(b), b.total) : -1;
         } else {
             if (leader) mailbox[it & 1] = fixed ? claim_fixed(b, grp) : claim_tile(b, grp, slice_lo, slice_n);
             __syncthreads();
@@ -411,7 +507,7 @@ __device__ __forceinline__ void tile_loop_span(const BlpArgs &b, Body &&body) {
         if (idx < 0) { leave_stamped(b); return; }
         const int first = idx * b.batch;
         body(first, first + b.batch < b.tiles ? first + b.batch : b.tiles);
-        if ((int)gridDim.x >= b.total) { leave_stamped(b); return; }  // one claim per workgroup at most (see tile_loop)
+        if (wg_count(b) >= b.total) { leave_stamped(b); return; }  // one claim per workgroup at most (see tile_loop)
     }
 }
 
@@ -457,7 +553,15 @@ __device__ __forceinline__ void tile_loop_ckpt(const BlpArgs &b, Body &&body) {
                 if (it == 0 && hdr && hdr[0] == 1 && hdr[1] == b.kernel_id) {
                     // a tile this workgroup left half-way in an earlier launch comes first; it was
                     // counted when it was claimed
-                    if (__hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == -1) {
+                    // (the flag as well, by everybody: a launch that resumes stopped tiles may find the next request
+                    // already there, and reloading 256 KB of accumulators only to store them again is 30 us of a
+                    // preemption; the read costs a resumption one trip to host memory)
+                    bool stopped = __hip_atomic_load(b.stop_index, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != -1;
+                    if (!stopped && b.flag && __hip_atomic_load(b.flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0) {
+                        record_stop(b.stop_index, b.kernel_id, b.stamps);
+                        stopped = true;
+                    }
+                    if (!stopped) {
                         claim = hdr[2];
                         first = hdr[3];
                         hdr[0] = 0;

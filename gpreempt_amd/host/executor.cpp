@@ -203,10 +203,14 @@ Status BLPExecutor::init(std::string workload) {
     CUDA_RETURN_STATUS(gp_memcpy_h2d(dpStopIndex, &stopIndex, sizeof(int)));
     model->batchAddParam(&this->dpStop);
     model->batchAddParam(&this->dpStopIndex);
+    // (twice the claim counters: behind them, laid out alike, the counters of workers that have left a launch of
+    // long tiles; GPREEMPT_LONG_TILES=0 leaves them unused: such tiles are then finished, as the reference finishes them)
     const size_t counter_ints = model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride;
-    CUDA_RETURN_STATUS(gp_malloc(&executed, sizeof(int) * counter_ints));
-    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, counter_ints, nullptr));
+    CUDA_RETURN_STATUS(gp_malloc(&executed, sizeof(int) * counter_ints * 2));
+    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, counter_ints * 2, nullptr));
     CUDA_RETURN_STATUS(gp_stream_sync(nullptr));
+    const char *lt = std::getenv("GPREEMPT_LONG_TILES");
+    if (!(lt && *lt == '0')) model->set_done_counters(sizeof(int) * counter_ints);
     // GPREEMPT_SINGLE_COUNTER=1 selects the reference's one-counter-per-kernel layout (for A/B timing)
     const char *single = std::getenv("GPREEMPT_SINGLE_COUNTER");
     RETURN_STATUS(model->add_block_preemption_param(executed, (single && *single == '1') ? 1 : kCounterGroups));
@@ -259,6 +263,7 @@ Status BLPExecutor::execute(GPUstream stream) {
     RETURN_STATUS(reset_counters(stream));
     if (use_cuda_graph) {
         CUDA_RETURN_STATUS(gp_graph_launch(graph_exec, stream));
+        model->launched_once_more();  // (a resume relaunches kernel by kernel and has to know)
         return Status::Succ;
     }
     for (size_t i = 0; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
@@ -351,7 +356,7 @@ int64_t BLPExecutor::device_ticks_to_ns(unsigned long long ticks) const {
 
 Status BLPExecutor::reset_counters(GPUstream stream) {
     if (graph_compute) return Status::Succ;
-    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride, stream));
+    CUDA_RETURN_STATUS(gp_fill32_async(executed, 0, 2 * model->get_kernel_num() * (size_t)kCounterGroups * kCounterStride, stream));
     if (ckpt) CUDA_RETURN_STATUS(gp_ckpt_reset_async(ckpt, stream));  // a fresh run has no tile to continue
     // launches recorded into a graph are replayed with the arguments of the recording: never fresh
     model->counters_cleared(!use_cuda_graph);
@@ -377,7 +382,7 @@ Status BLPExecutor::read_counters(std::vector<int> &out) {
         long sum = 0;
         if (model->counter_groups() == 1) { out[i] = raw[i]; continue; }
         // slices follow the workgroup distribution of the last launch (device layer, tile_loop.hpp)
-        const long grid = std::max<long>(1, model->get_kernel_info(i).launch_params[0]);
+        const long grid = std::max<long>(1, (long)model->get_kernel_info(i).launch_params[0] - model->get_kernel_info(i).front_workgroups);  // the workers
         if (model->get_kernel_info(i).fixed_claims) {  // int 0 of every line is an exact count
             for (int g = 0; g < kCounterGroups; ++g) sum += raw[(i * kCounterGroups + g) * kCounterStride];
             out[i] = (int)sum;

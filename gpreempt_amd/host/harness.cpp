@@ -74,6 +74,12 @@ struct Load {
         next_trace = 0;
         std::sort(trace_ms.begin(), trace_ms.end());
     }
+    // When the request after the one being served arrives (0: not known, or never).
+    int64_t following() const {
+        if (type == "continuous") return 0;
+        if (type == "trace") return next_trace < trace_ms.size() ? begin + trace_ms[next_trace] * 1000000 : 0;
+        return frequency > 0 && next < end ? next : 0;
+    }
     // Returns false when the run is over.  A launch whose successor is already due is given up,
     // as in DISB ("always choose the newest frame", load.cpp:196-222).  *scheduled receives the
     // arrival time of the request that is served.
@@ -228,6 +234,8 @@ struct Shared {
     // finished, resubmission -> first tile claimed
     bool device_stamps = false;
     long corun_discard = 0;                 // the first requests of every priority-0 tenant are served but not counted
+    bool hold_backlog = true;               // see end_request
+    int64_t hold_us = 30;
     // busy_above[L]: time during which at least one request of a level above L (a smaller number)
     // was being served: what a continuous tenant of level L could not have used
     std::mutex busy_mu;
@@ -281,7 +289,7 @@ struct Tenant {
     void *gate_dev = nullptr;
     int *gate_timed_out = nullptr;          // device word set by a gate that gave up
     // the slowest drains of this tenant: how long, and which kernel the stop index named afterwards
-    struct Drain { double us; int stop_kernel; int queued; };
+    struct Drain { double us; int stop_kernel; int queued; unsigned long long stop_ticks = 0, exit_ticks = 0; int64_t raised = 0; double since_launch_us = 0; bool resumed = false; };
     std::vector<Drain> drains;
     bool have_ref_hash = false;
     uint64_t ref_hash = 0;
@@ -290,6 +298,8 @@ struct Tenant {
     std::vector<double> first_latencies;    // total latency of the first co-run requests, in arrival order
     long discarded = 0;
     int64_t resubmitted_ns = 0;             // device stamps: when the kernels of a stopped model were submitted again
+    bool holding = false;                   // the level stayed up after the last request (end_request)
+    long held = 0;                          // how often
     // one preemption (or resubmission) as the host and the GPU saw it: host clock nanoseconds and raw device ticks
     struct StampSample { int64_t raised = 0, drained = 0, resubmitted = 0; unsigned long long stop = 0, exit = 0, claim = 0; };
     std::vector<StampSample> stamp_samples;
@@ -396,6 +406,8 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
     Status st = ex->reset_counters(t.stream);
     size_t next = 0;
     int inflight = 0, head = 0, tail = 0;  // ring of 3 events, at most 2 in flight
+    int64_t first_launch_ns = 0;           // when the first kernel of this request, or of its latest resumption, was submitted
+    bool resumed = false;
     ex->running = true;
     sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
     while (st == Status::Succ && (next < n || inflight > 0)) {
@@ -413,6 +425,7 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             if (st != Status::Succ) { sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel); break; }
             const int stop = ex->last_stop_index();
             const int64_t raised = sh.domain->raised_ns(p);
+            unsigned long long stop_ticks = 0, exit_ticks = 0;
             if (ex->device_stamps_enabled()) {
                 // the GPU's own account of this preemption (and of the resume before it, if there was one)
                 BLPExecutor::DeviceStamps ds;
@@ -423,6 +436,7 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
                 if ((queued > 0 || stop >= 0) && raised > 0 && drained >= raised && ds.last_exit) {
                     smp.raised = raised; smp.drained = drained; smp.exit = ds.last_exit;
                     smp.stop = stop >= 0 ? ds.stop_recorded : 0;
+                    stop_ticks = smp.stop; exit_ticks = smp.exit;
                 }
                 if (t.resubmitted_ns && ds.first_claim) { smp.resubmitted = t.resubmitted_ns; smp.claim = ds.first_claim; }
                 if (smp.raised || smp.resubmitted) t.stamp_samples.push_back(smp);
@@ -438,15 +452,28 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
                     sh.preempt_latency.add(drain_us);
                 }
                 t.drains.push_back({drain_us, stop, queued});
+                t.drains.back().raised = raised; t.drains.back().stop_ticks = stop_ticks; t.drains.back().exit_ticks = exit_ticks;
+                t.drains.back().since_launch_us = (raised - first_launch_ns) / 1e3; t.drains.back().resumed = resumed;
             }
             while (sh.active_above(p) > 0) spin_pause();
             sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
-            if (stop >= 0) { next = (size_t)stop; ++t.preemptions; }  // kernels from the stopped one on are submitted again
+            if (stop >= 0) { next = (size_t)stop; ++t.preemptions; resumed = true; first_launch_ns = 0; }  // kernels from the stopped one on are submitted again
             if (stop >= 0 && ex->device_stamps_enabled()) t.resubmitted_ns = now_ns();
             continue;
         }
         if (next < n && inflight < 2) {
-            size_t end = std::min(n, next + (size_t)chunk_size());
+            // (a kernel of 3 GFLOP and more, 10 us and up, ends its chunk: behind such kernels the host keeps up with one
+            // chunk queued, and every queued kernel is one more to flush when a stop comes, 4-7 us apiece next to
+            // VGG-16 b16)
+            size_t end = next;
+            double flops = 0;
+            auto model = ex->get_model();
+            while (end < n && end - next < (size_t)chunk_size()) {
+                if (model) flops += model->get_kernel_info(end).flops;
+                ++end;
+                if (flops >= 3e9) break;
+            }
+            if (!first_launch_ns) first_launch_ns = now_ns();
             for (size_t i = next; i < end && st == Status::Succ; ++i) st = ex->launch_kernel(i, t.stream);
             if (st != Status::Succ) break;
             if (gp_event_record(t.chunk_events[tail], t.stream) != 0) { st = Status::Fail; break; }
@@ -586,12 +613,22 @@ static bool preempting_policy(const Shared &sh) { return is_wb(sh.policy); }
 // flag has to go up first.  This is where the reference posts its pre-preemption hint
 // (src/cuda-clients/gpreemptclient.cpp:203-219).  Raises the flag words of every lower level
 // (blpclient.cpp:185-188); end_request() lowers them when the level has no request left.
+// A tenant whose next request has arrived by the time this one ends (or will within hold_us) keeps its level up across
+// the two ("hold_backlog", on by default; loads with arrival times only).  Lowering the flag words for the instant
+// between two requests makes every lower level submit its stopped kernels again, and the raise that follows at once
+// finds them on their way onto the GPU: they have to start, pick their work up and leave again, the longest
+// preemptions there are (BERT-384 over the 8192^3 GEMM: 40-60 us of flag store to drained, one request in eight).
 void begin_request(Tenant &t, Shared &sh) {
     if (!preempting_policy(sh)) return;
+    if (t.holding) { t.holding = false; return; }  // the level is still up from the request before
     sh.domain->begin(t.priority);
 }
 void end_request(Tenant &t, Shared &sh) {
     if (!preempting_policy(sh)) return;
+    if (sh.hold_backlog && t.preprocess_us == 0 && !sh.stop.load(std::memory_order_acquire)) {
+        const int64_t f = t.load.following();
+        if (f != 0 && f <= now_ns() + sh.hold_us * 1000) { t.holding = true; ++t.held; return; }
+    }
     sh.domain->end(t.priority);
 }
 
@@ -677,6 +714,7 @@ void tenant_thread(Tenant *t, Shared *sh, std::atomic<int> *ready, int n_tasks, 
         }
     }
     if (sh->hp_requests > 0 && t->priority == 0 && !counted && sh->hp_unfinished.fetch_sub(1) == 1) sh->stop.store(true, std::memory_order_release);
+    if (t->holding) { t->holding = false; sh->domain->end(t->priority); }  // no request followed after all
 }
 
 }  // namespace
@@ -698,6 +736,8 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
     sh.hp_gate = cfg["hp_gate"].boolean(false);
     sh.device_stamps = cfg["device_stamps"].boolean(false);
     sh.corun_discard = (long)cfg["corun_discard"].number(0);
+    sh.hold_backlog = cfg["hold_backlog"].boolean(true);
+    sh.hold_us = (int64_t)cfg["hold_us"].number(30);
     const json::Value &tasks = cfg["tasks"];
     std::vector<std::unique_ptr<Tenant>> tenants;
     // Declared after `tenants`, so it runs first on every exit path: executors free device memory
@@ -803,6 +843,7 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
         o.set("queueing(us)") = t->queueing.to_json();
         o.set("standAlone(us)") = t->standalone.to_json();
         o.set("preemptions") = (long)t->preemptions;
+        o.set("levelHeldAcrossRequests") = t->held;
         double alone_thr = t->standalone.mean() > 0 ? 1e6 / t->standalone.mean() : 0;
         o.set("standAloneThroughput(req/s)") = alone_thr;
         if (t->priority == 0) {
@@ -830,6 +871,12 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
                 e.set("us") = t->drains[i].us;
                 e.set("stopKernel") = t->drains[i].stop_kernel;
                 e.set("chunksInFlight") = t->drains[i].queued;
+                e.set("sinceSubmission(us)") = t->drains[i].since_launch_us;
+                e.set("resumedBefore") = t->drains[i].resumed;
+                if (t->blp && t->blp->device_stamps_enabled() && t->drains[i].exit_ticks && t->blp->calibrate_device_clock(t->stream) == Status::Succ) {
+                    if (t->drains[i].stop_ticks) e.set("flagStore_to_stopRecorded(us)") = (t->blp->device_ticks_to_ns(t->drains[i].stop_ticks) - t->drains[i].raised) / 1e3;
+                    e.set("flagStore_to_lastWorkgroupExit(us)") = (t->blp->device_ticks_to_ns(t->drains[i].exit_ticks) - t->drains[i].raised) / 1e3;
+                }
                 if (model && t->drains[i].stop_kernel >= 0 && (size_t)t->drains[i].stop_kernel < model->get_kernel_num()) {
                     KernelInfo &k = model->get_kernel_info(t->drains[i].stop_kernel);
                     e.set("name") = k.name;

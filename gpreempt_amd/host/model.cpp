@@ -470,6 +470,10 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         ctx.ckpt = ckpt_;
         ctx.ckpt_bytes = ckpt_bytes_;
         ctx.stamps = (unsigned long long *)stamps_;
+        if (done_offset_) {
+            ctx.done = (int *)((char *)k.executed + done_offset_);
+            ctx.done_launches = idx < launches_.size() ? launches_[idx] : 0;
+        }
         pc = &ctx;
     }
     gp_launch_info info{};
@@ -488,10 +492,12 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
         case OpKind::Nop: break;
     }
     if (idx < fresh_.size()) fresh_[idx] = 0;  // launched (or refused): from here on only its counters know
+    if (idx < launches_.size() && rc == 0) ++launches_[idx];
     CUDA_RETURN_STATUS(rc);
     k.total_blocks = info.total_tiles;
     k.fixed_claims = info.fixed_claims != 0;
     k.launch_params[0] = (uint32_t)info.grid; k.launch_params[1] = 1; k.launch_params[2] = 1;
+    k.front_workgroups = info.front;
     k.launch_params[3] = (uint32_t)info.block; k.launch_params[4] = 1; k.launch_params[5] = 1;
     return Status::Succ;
 }

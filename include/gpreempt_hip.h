@@ -143,6 +143,16 @@ typedef struct gp_preempt_ctx {
                      /* with gp_ckpt_reset_async whenever the claim counters are cleared.  No       */
                      /* counterpart in the reference, whose tiles are never long enough to matter.  */
     unsigned long long ckpt_bytes;
+    int *done;       /* may be NULL.  Counters laid out like `executed` (counter_groups of them, 16 ints apart,  */
+                     /* cleared together with them) in which every worker workgroup of every launch of this     */
+                     /* kernel counts itself when it leaves.  With them a launch of long tiles (about 10^7      */
+                     /* multiply-adds and more per tile) keeps one workgroup in front of its workers reading    */
+                     /* the preempt flag until all of them have left, and its tiles look at the stop index every */
+                     /* few K-stages: a tile that finds a stop recorded is given up (its claim is withdrawn, the */
+                     /* relaunch computes it from the start: same bits).  The reference's wrapper can only stop  */
+                     /* between tiles (convert_to_blp.py:45-58); a 32 x 32 x 25088 tile of VGG-16's first dense  */
+                     /* layer runs 70 us.                                                                        */
+    int done_launches; /* launches of this kernel since `done` was cleared                                     */
     unsigned long long *stamps; /* may be NULL (the default).  A measurement mode: GP_STAMP_WORDS 64-bit words of   */
                      /* device memory that the kernels fill with the device's constant-rate clock             */
                      /* (gp_device_clock gives its rate and its offset to the host's monotonic clock):        */
@@ -168,6 +178,11 @@ typedef struct gp_launch_info {
     int block;          /* threads per workgroup                              */
     int fixed_claims;   /* 1: claims were fixed by workgroup index and recorded as bits (see  */
                         /* gp_preempt_ctx::fresh); 0: handed out through the counters          */
+    int front;          /* of `grid`, the workgroups in front of the workers that own no claim: a launch */
+                        /* with more claims than the device holds workgroups gets 8, the first of which  */
+                        /* reads the preempt flag about every microsecond while claims are still being   */
+                        /* made (the reference's wrapper reads it once per claim, convert_to_blp.py:45,   */
+                        /* which on this GPU leaves gaps as long as a tile)                               */
 } gp_launch_info;
 
 /* ---- operators ---------------------------------------------------------------------------

@@ -72,6 +72,7 @@ public:
     bool preemptible = false;
     int total_blocks = 0;
     bool fixed_claims = false;            // how the last launch recorded its claims (gp_launch_info)
+    int front_workgroups = 0;             // of launch_params[0], the workgroups that own no claim (gp_launch_info::front)
     GPUdeviceptr executed = nullptr;
     int kernel_id = 0;
     double flops = 0, bytes = 0;          // algorithmic work of one launch
@@ -148,7 +149,11 @@ public:
     // The claim counters have just been cleared (or are about to be, earlier on the same stream):
     // until its next launch every kernel is known to have made no claim (gp_preempt_ctx::fresh).
     // `on` = false withdraws that for all kernels (launches that are recorded and replayed).
-    void counters_cleared(bool on) { fresh_.assign(kernel_infos.size(), on ? 1 : 0); }
+    void counters_cleared(bool on) { fresh_.assign(kernel_infos.size(), on ? 1 : 0); launches_.assign(kernel_infos.size(), 0); }
+    // every kernel has been launched once more by something else than launch() (a replayed graph)
+    void launched_once_more() { for (int &n : launches_) ++n; }
+    // counters of the workers that have left, behind the claim counters (gp_preempt_ctx::done): byte distance from `executed`
+    void set_done_counters(size_t byte_offset) { done_offset_ = byte_offset; }
     // device-visible address of a host word that a program's last leaving workgroup sets to the
     // launch number returned by launch_program()
     void set_left_word(GPUdeviceptr p) { left_word_ = p; }
@@ -183,6 +188,8 @@ private:
     int counter_groups_ = 1;
     int poll_every_ = 0;
     std::vector<char> fresh_;
+    std::vector<int> launches_;           // per kernel: launches since the counters were cleared (gp_preempt_ctx::done_launches)
+    size_t done_offset_ = 0;              // 0: no done counters
     GPUdeviceptr left_word_ = nullptr;
     GPUdeviceptr ckpt_ = nullptr;
     size_t ckpt_bytes_ = 0;

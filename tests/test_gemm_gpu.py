@@ -198,11 +198,14 @@ def test_flag_set_before_launch(gp):
         gp.launch("gp_launch_gemm", p, st.ctx(poll_every=3))
 
 
-def test_flag_is_seen_after_the_first_four_counter_groups_ran_out(gp):
+@pytest.mark.parametrize("tile", [128, 64])
+def test_flag_is_seen_after_the_first_four_counter_groups_ran_out(gp, tile):
     """With 32 claim counters the first four groups read the flag for everybody.  A relaunch that finds their
     slices handed out (here: their counters set past the end by the test) while the flag is up must still
-    stop: the other groups take the reading over.  Lowering the flag and relaunching completes the work
-    with the bits of an uninterrupted run."""
+    stop: the other groups take the reading over (128 x 128 tiles: one workgroup per compute unit), or the
+    workgroup in front of the workers, which reads the flag for such a launch, has recorded the stop before
+    anybody claims (64 x 64 tiles).  Lowering the flag and relaunching completes the work with the bits of an
+    uninterrupted run."""
     rng = np.random.default_rng(21)
     M = N = 4096
     K = 256
@@ -211,7 +214,7 @@ def test_flag_is_seen_after_the_first_four_counter_groups_ran_out(gp):
     dA, dB = (gp.DevBuf.from_array(x, gp.F16) for x in (A, B))
     dC = gp.DevBuf(2 * M * N)
     p = gp.GemmParams(dtype=gp.F16, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, alpha=1.0, batch=1,
-                      tile_m=64, tile_n=64)
+                      tile_m=tile, tile_n=tile)
     gp.launch("gp_launch_gemm", p)
     gp.check(gp.lib().gp_stream_sync(None))
     base = dC.download().copy()
@@ -225,12 +228,16 @@ def test_flag_is_seen_after_the_first_four_counter_groups_ran_out(gp):
     dC.fill32(0)
     info = gp.launch("gp_launch_gemm", p, st.ctx(max_workgroups=512))
     gp.check(gp.lib().gp_stream_sync(None))
-    assert info.total_tiles == 4096 and info.grid < info.total_tiles and info.fixed_claims == 0
+    assert info.total_tiles == (4096 // tile) ** 2 and info.grid < info.total_tiles and info.fixed_claims == 0
     assert st.stop_index() == 0
     c = st.counters()[::S]
-    # the first claim of every group has a number that reads the flag: about one tile per workgroup (a second
-    # one where a tile ends before the read of host memory has come back), of the 3584 these groups own
-    assert 0 < int(c[4:].sum()) <= 2 * info.grid, c
+    if tile == 128:
+        # the first claim of every group has a number that reads the flag: about one tile per workgroup (a second
+        # one where a tile ends before the read of host memory has come back), of the tiles these groups own
+        assert info.front == 0 and 0 < int(c[4:].sum()) <= 2 * info.grid, c
+    else:
+        # the workgroup in front starts first and reads the flag first: hardly a claim is made before the stop is recorded
+        assert info.front == 8 and int(c[4:].sum()) <= 2 * info.grid, c
     assert not np.array_equal(dC.download(), base)
     # the four groups get their slices back; the flag comes down; the relaunch finishes everything
     now = st.counters()
@@ -908,3 +915,70 @@ def test_device_time_stamps_of_a_preemption(gp):
     assert info.fixed_claims == 1 and st.stop_index() == 0
     stop3, first3, last3, exits3 = st.read_stamps()
     assert stop3 and first3 and last3 >= stop3 and exits3 >= 1
+
+
+@pytest.mark.parametrize("family", ["wide", "pipe"])
+def test_long_tiles_are_given_up_on_a_stop_and_redone_bit_exact(gp, family):
+    """Tiles of 3 x 10^7 multiply-adds (about 100 us each; VGG-16's 25088-deep dense layer and ResNet-50's fp32
+    7 x 7 stage have such tiles) in a launch that has a workgroup per tile: with gp_preempt_ctx::done the launch keeps
+    a workgroup in front of its workers that reads the flag until they have all left, and the tiles look at the stop
+    index every few K-stages.  A flag raised by the host while the tiles run is recorded within microseconds, the
+    tiles are given up (their claims withdrawn), the launch is over long before a tile would have ended, and the
+    relaunch computes them from the start: the bits of an uninterrupted run."""
+    import time
+    dt, dtype = "f16", gp.F16
+    if family == "wide":
+        M, N, K, tm, tn, variant = 64, 2048, 32768, 32, 32, gp.MAT_WIDE
+    else:
+        M, N, K, tm, tn, variant = 1024, 1024, 8192, 64, 64, gp.MAT_PIPE
+    rng = np.random.default_rng(K)
+    A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), dt)
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32) * 0.02, dt)
+    dA, dB, dC = gp.DevBuf.from_array(A, dtype), gp.DevBuf.from_array(B, dtype), gp.DevBuf(M * N * 2)
+    p = gp.GemmParams(dtype=dtype, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, alpha=1.0, act=gp.ACT_RELU, batch=1,
+                      tile_m=tm, tile_n=tn, variant=variant)
+    stream = gp.Stream(1)
+    e0, e1 = gp.Event(), gp.Event()
+    e0.record(stream)
+    gp.launch("gp_launch_gemm", p, None, stream)
+    e1.record(stream); e1.sync()
+    whole_us = e0.elapsed_ms(e1) * 1e3
+    base = dC.download().copy()
+    assert rel_err(dC.download(dtype, (M, N))[:8], O.gemm_bias_act(A[:8], B, None, None, gp.ACT_RELU, b_is_nk=True)) < TOL[dt]
+    tick, off = C.c_double(0), C.c_double(0)
+    gp.check(gp.lib().gp_device_clock(None, 8, C.byref(tick), C.byref(off), None))
+    flag = gp.Flag()
+    st = gp.BlpState(1, flag, 32)
+    st.enable_done_counters()
+    st.enable_stamps()
+    given_up = 0
+    for attempt in range(6):
+        st.reset(); st.clear_stop(); flag.set(0)
+        st.stamps.upload(np.zeros(st.STAMP_WORDS, np.uint64))
+        dC.fill32(0x7E007E00)
+        info = gp.launch("gp_launch_gemm", p, st.ctx(fresh=1), stream)
+        t0 = time.perf_counter()
+        while time.perf_counter() - t0 < 15e-6 * (attempt + 1):  # the flag lands at another depth of the tiles every time
+            pass
+        flag.set(1)
+        stream.sync()
+        assert info.fixed_claims == 1 and info.front == 8 and info.total_tiles == (M // tm) * (N // tn)
+        made = int(st.counters().reshape(32, 16)[:, 0].sum())
+        left = int(st.done.download(np_dtype=np.int32).reshape(32, 16)[:, 0].sum())
+        assert left == info.grid - info.front  # every worker of the launch counted itself on its way out
+        stop, first, last_exit, exits = st.read_stamps()
+        if st.stop_index() == 0 and made < info.total_tiles:
+            given_up += 1
+            # the launch was over within microseconds of the recorded stop, not a tile's length later
+            assert (last_exit - stop) * tick.value < 25e3, ((last_exit - stop) * tick.value, whole_us)
+            part = dC.download(np_dtype=np.uint16).reshape(M // tm, tm, N // tn, tn)
+            untouched = int((part == 0x7E00).all(axis=(1, 3)).sum())
+            assert untouched == info.total_tiles - made  # a tile that was given up wrote nothing
+        # the host's resume: flag down, stop index re-armed, the same kernel again (its second launch since the reset)
+        flag.set(0)
+        st.clear_stop()
+        gp.launch("gp_launch_gemm", p, st.ctx(done_launches=1), stream)
+        stream.sync()
+        assert st.stop_index() == -1 and np.array_equal(dC.download(), base), attempt
+        assert int(st.counters().reshape(32, 16)[:, 0].sum()) == info.total_tiles
+    assert given_up >= 1, f"no attempt stopped the launch while its tiles ran (a plain launch takes {whole_us:.0f} us)"
