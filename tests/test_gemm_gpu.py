@@ -917,7 +917,7 @@ def test_device_time_stamps_of_a_preemption(gp):
     assert stop3 and first3 and last3 >= stop3 and exits3 >= 1
 
 
-@pytest.mark.parametrize("family", ["wide", "pipe"])
+@pytest.mark.parametrize("family", ["wide", "pipe", "pipe_two_rounds"])
 def test_long_tiles_are_given_up_on_a_stop_and_redone_bit_exact(gp, family):
     """Tiles of 3 x 10^7 multiply-adds (about 100 us each; VGG-16's 25088-deep dense layer and ResNet-50's fp32
     7 x 7 stage have such tiles) in a launch that has a workgroup per tile: with gp_preempt_ctx::done the launch keeps
@@ -929,8 +929,12 @@ def test_long_tiles_are_given_up_on_a_stop_and_redone_bit_exact(gp, family):
     dt, dtype = "f16", gp.F16
     if family == "wide":
         M, N, K, tm, tn, variant = 64, 2048, 32768, 32, 32, gp.MAT_WIDE
-    else:
+    elif family == "pipe":
         M, N, K, tm, tn, variant = 1024, 1024, 8192, 64, 64, gp.MAT_PIPE
+    else:
+        # 320 tiles of 128 x 128, one to a compute unit: two rounds of workgroups, a workgroup per claim all the same
+        # (a persistent grid would have to finish the tiles it is in), the front workgroup in one of the 256 places
+        M, N, K, tm, tn, variant = 2560, 2048, 4096, 128, 128, gp.MAT_PIPE
     rng = np.random.default_rng(K)
     A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), dt)
     B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32) * 0.02, dt)

@@ -224,3 +224,25 @@ def test_hp_gate_policy_option(gp):
     assert rep["tasks"]["hp"]["outputMismatches"] == 0 and rep["tasks"]["be"]["outputMismatches"] == 0
     # a gate that had given up would have cost its whole spin limit (seconds)
     assert rep["tasks"]["hp"]["totalLatency(us)"]["max"] < 50000
+
+
+def test_a_level_stays_up_across_back_to_back_requests(gp):
+    """Requests of the high-priority tenant that arrive while one is being served follow it at once.  With
+    "hold_backlog" (the default) the level's flag words stay up between the two, so the lower level is not sent
+    back onto the GPU for an instant only to be stopped again; without it the words go down and up per request, as
+    in the reference's client.  Either way every best-effort request returns the bits of an uninterrupted run."""
+    def run(hold):
+        cfg = {"time": 1.5, "policy": "wb-chunk-async", "warmups": 3, "standalone_runs": 10, "verify_outputs": True, "hold_backlog": hold, "tasks": [
+            {"id": "hp", "load": {"type": "poisson", "frequency": 4000, "seed": 11},
+             "client": {"name": "hp_rt", "model_name": "bert@layers=2,s=128", "priority": 0, "launch_mode": "launch"}},
+            {"id": "be", "load": {"type": "continuous"},
+             "client": {"name": "be_be", "model_name": "resnet50@b=2", "priority": 1, "launch_mode": "launch"}}]}
+        return _scenario(cfg)["tasks"]
+    held, plain = run(True), run(False)
+    assert held["hp"]["levelHeldAcrossRequests"] > 50, held["hp"]
+    assert plain["hp"]["levelHeldAcrossRequests"] == 0
+    for t in (held, plain):
+        assert t["hp"]["requests"] > 500 and t["be"]["requests"] > 20 and t["be"]["preemptions"] > 20
+        assert t["be"]["outputMismatches"] == 0 and t["hp"]["outputMismatches"] == 0
+    # a level that stays up stops the lower one less often for the same arrivals
+    assert held["be"]["preemptions"] < plain["be"]["preemptions"]
