@@ -387,7 +387,8 @@ def miniweather(steps=50):
     return {"workload": "miniweather 3200x1600 fp32, collision test case, 36 kernels per execute", "ms_per_execute": ms,
             "algorithmic_MB": nbytes / 1e6, "achieved_GBps": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / 8000.0,
             "mass_drift": abs(m1 - m0) / m0, "energy_drift": abs(e1 - e0) / e0, "executes": steps + 3,
-            "cpu_oracle_ms_per_execute_scaled": cpu_ms, "cpu_cores": 1}
+            "cpu_oracle_ms_per_execute_scaled": cpu_ms, "cpu_cores": 1,
+            "cpu_unit": "ms per execute on 1 core (numpy oracle on a 400 x 200 grid, scaled by cells)"}
 
 
 def graph_workloads(runs=5):
@@ -424,7 +425,8 @@ def graph_workloads(runs=5):
         cpu_s = (time.perf_counter() - t0) * info["edges"] / len(indices)
         out[kind] = {"ms_per_execute": dt * 1e3, "iterations": info["iterations"], "edges": info["edges"],
                      "edge_visits_per_s_upper_bound": info["edges"] * info["iterations"] / dt,
-                     "cpu_oracle_ms_scaled": cpu_s * 1e3, "cpu_cores": 1}
+                     "cpu_oracle_ms_scaled": cpu_s * 1e3, "cpu_cores": 1,
+                     "cpu_unit": "ms per run on 1 core (numpy oracle on a 2^16-vertex graph, scaled by edges)"}
         ex.destroy()
     return out
 
