@@ -30,7 +30,7 @@ CORUN_DISCARD = 5  # co-run requests of the high-priority tenant served before t
 # `bench.py --only roofline` (FETCH_SIZE, then WRITE_SIZE, each scaled by what the same counter reads
 # for the copy of `--only copycal`); the figures and commands are in the hbm_traffic summary
 # under profiles/.  Counters cannot be collected from inside this process.
-HBM_TRAFFIC_PER_LAUNCH = {("resnet152", "f16"): 10.57e6}
+HBM_TRAFFIC_PER_LAUNCH = {("resnet152", "f16"): 10.62e6}
 
 
 def scenario(steps, warmup, policy, hp_rate, be_model, hp_model, extra=None):
