@@ -602,7 +602,7 @@ def main():
     ap.add_argument("--be-model", default="resnet152")
     ap.add_argument("--only", default="", help="run one leg only: scenario | roofline | gemm | hbm | miniweather | graphs | cpu | copycal | vendor | hp")
     ap.add_argument("--cpu-requests", type=int, default=10, help="timed submissions per graph in the cpu_baseline leg")
-    ap.add_argument("--config-seconds", type=float, default=3.5, help="co-run time of the config 4 and config 5 scenario legs")
+    ap.add_argument("--config-seconds", type=float, default=5.0, help="co-run time of each of the config 2, 4 and 5 scenario legs")
     ap.add_argument("--gemm-operands", default="random", choices=("random", "const"), help="operands of the 8192^3 GEMM leg (--only gemm)")
     args = ap.parse_args()
     if args.gpus != 1:

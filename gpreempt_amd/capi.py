@@ -23,7 +23,8 @@ vp = C.c_void_p
 class PreemptCtx(C.Structure):
     _fields_ = [("flag", vp), ("stop_index", vp), ("executed", vp), ("kernel_id", C.c_int),
                 ("inject_at", C.c_int), ("max_workgroups", C.c_int), ("poll_every", C.c_int), ("counter_groups", C.c_int), ("fresh", C.c_int), ("left_host", vp),
-                ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong), ("done", vp), ("done_launches", C.c_int), ("stamps", vp)]
+                ("ckpt", vp), ("ckpt_bytes", C.c_ulonglong), ("done", vp), ("done_launches", C.c_int), ("stamps", vp),
+                ("started_host", vp), ("started_seq", C.c_int)]
 
 
 class LaunchInfo(C.Structure):
@@ -99,7 +100,7 @@ class EmbedParams(C.Structure):
 SYMBOLS = """gp_init gp_last_error gp_device_info gp_device_clock gp_stream_create gp_stream_destroy gp_stream_sync
 gp_stream_query gp_stream_priority gp_stream_set_priority gp_stream_native gp_event_create gp_event_destroy gp_event_record
 gp_event_sync gp_event_query gp_event_elapsed_ms gp_malloc gp_free gp_host_alloc gp_host_free gp_memcpy_h2d gp_memcpy_d2h
-gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_flag_relay_start
+gp_memcpy_h2d_async gp_memcpy_d2h_async gp_memcpy_d2d_async gp_fill32_async gp_flag_create gp_flag_destroy gp_store_word_async gp_flag_relay_start
 gp_launch_gemm gp_gemm_ln_supported gp_launch_gemm_noalloc gp_gemm_ckpt_bytes gp_conv_ckpt_bytes gp_ckpt_reset_async gp_launch_conv2d gp_launch_nchw_to_nhwc gp_launch_pool2d gp_launch_eltwise gp_launch_softmax
 gp_launch_layernorm gp_launch_attention gp_launch_miniweather gp_launch_graph gp_launch_embed gp_launch_gate gp_launch_noop gp_graph_begin gp_graph_end gp_graph_launch
 gp_graph_destroy gp_program_create gp_program_destroy gp_program_add_gemm gp_program_add_conv2d
@@ -301,12 +302,13 @@ class BlpState:
         if getattr(self, "done", None):
             self.done.upload(np.zeros(self.n * self.ints_per_kernel, np.int32))
 
-    def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0, fresh=0, done_launches=0):
+    def ctx(self, kernel_id=0, inject_at=-1, max_workgroups=0, poll_every=0, fresh=0, done_launches=0, started=None, started_seq=0):
         ck = getattr(self, "ckpt", None)
         return PreemptCtx(self.flag.dev, self.stop.ptr, self.executed.ptr + 4 * kernel_id * self.ints_per_kernel, kernel_id, inject_at, max_workgroups,
                           poll_every, self.groups if self.groups > 1 else 0, fresh, None, ck.ptr if ck else None, ck.nbytes if ck else 0,
                           (self.done.ptr + 4 * kernel_id * self.ints_per_kernel) if getattr(self, "done", None) else None, done_launches,
-                          self.stamps.ptr if getattr(self, "stamps", None) else None)
+                          self.stamps.ptr if getattr(self, "stamps", None) else None,
+                          started.dev if started is not None else None, started_seq)
 
     def enable_done_counters(self):
         """Counters of the workers that have left (gp_preempt_ctx::done), cleared by reset()."""

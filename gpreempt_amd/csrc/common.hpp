@@ -68,6 +68,7 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
         GP_REQUIRE(ctx->executed != nullptr && ctx->stop_index != nullptr, "preempt context needs executed and stop_index");
         blp->flag = ctx->flag; blp->stop_index = ctx->stop_index; blp->executed = ctx->executed;
         blp->kernel_id = ctx->kernel_id; blp->inject_at = ctx->inject_at; blp->stamps = ctx->stamps;
+        blp->started = ctx->started_host; blp->started_seq = ctx->started_seq;
         GP_REQUIRE(ctx->fresh >= 0 && ctx->fresh <= 2, "fresh is 0, 1 or 2");
         blp->fresh = ctx->fresh;
         int pe = ctx->poll_every > 0 ? ctx->poll_every : 8;
@@ -142,6 +143,7 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
     } else {
         blp->flag = nullptr; blp->stop_index = nullptr; blp->executed = nullptr;
         blp->kernel_id = 0; blp->inject_at = -1; blp->poll_mask = 0; blp->groups = 1; blp->fresh = 0; blp->spare = 0; blp->stamps = nullptr; blp->front = 0; blp->done = nullptr; blp->done_target = 0;
+        blp->started = nullptr; blp->started_seq = 0;
         for (int g = 0; g < 4; ++g) blp->poll_n[g] = 0;
         *grid = (int)total;
     }

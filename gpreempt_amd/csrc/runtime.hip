@@ -52,6 +52,11 @@ __global__ void clock_probe_kernel(unsigned long long *host_word) {
     if (threadIdx.x == 0) __hip_atomic_store(host_word, (unsigned long long)wall_clock64(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 }
 
+// stores a value where the host can see it: a marker that says "everything before me on this stream has left the GPU"
+__global__ void store_word_kernel(int *host_word, int value) {
+    if (threadIdx.x == 0) __hip_atomic_store(host_word, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 struct RelayArgs { const int *flags[8]; int *mirror; int n; const int *quit; unsigned long long spin_limit; };
 
 // Lane i mirrors flag word i into device memory; lane 0 also watches the quit word.
@@ -280,6 +285,13 @@ extern "C" int gp_device_clock(gp_stream s, int rounds, double *tick_ns, double 
     *tick_ns = tick;
     *offset_ns = best;
     if (ticks) *ticks = best_ticks;
+    return GP_SUCC;
+}
+
+extern "C" int gp_store_word_async(gp_stream s, int *word_dev, int value) {
+    GP_REQUIRE(word_dev != nullptr, "gp_store_word_async: null word");
+    hipLaunchKernelGGL(store_word_kernel, dim3(1), dim3(64), 0, native(s), word_dev, value);
+    GP_HIP(hipGetLastError());
     return GP_SUCC;
 }
 

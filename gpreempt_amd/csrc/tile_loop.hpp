@@ -65,7 +65,15 @@ struct BlpArgs {
                       // THIS launch have left: plan_launch), and the bodies look at the stop index
                       // every few K-stages and give a tile up (the claim is withdrawn, the relaunch redoes it)
     int done_target;
+    int *started;     // nullptr, or a word in host memory in which the first workgroup stores started_seq when it starts
+    int started_seq;  // (gp_preempt_ctx::started_host: the host's flow control when it submits kernel by kernel)
 };
+
+// The first workgroup tells the host that this launch has reached the GPU, i.e. that everything submitted before it on
+// the stream has left (a store to host memory: nobody waits for it).
+__device__ __forceinline__ void announce_start(const BlpArgs &b, bool leader) {
+    if (b.started && blockIdx.x == 0 && leader) __hip_atomic_store(b.started, b.started_seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
 
 // a worker's number among the workers of the launch, and how many there are
 __device__ __forceinline__ int wg_id(const BlpArgs &b) { return (int)blockIdx.x - b.front; }
@@ -248,6 +256,7 @@ __device__ __forceinline__ bool spare_workgroup(const BlpArgs &b, bool fixed, bo
 // recorded, or every claim of the launch has been made (from then on no workgroup starts that a stop could hold
 // back), or its bounded number of looks is used up.  The others leave at once.  Returns true in a front workgroup.
 __device__ __forceinline__ bool front_workgroup(const BlpArgs &b, bool leader) {
+    announce_start(b, leader);  // (here because every dispatcher loop comes through here first)
     if (b.front == 0 || (int)blockIdx.x >= b.front) return false;
     const int tid = (int)(threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z));
     if (blockIdx.x != 0 || !b.flag) return true;
@@ -542,6 +551,7 @@ __device__ __forceinline__ void tile_loop_ckpt(const BlpArgs &b, Body &&body) {
     const int grp = wg_group((int)blockIdx.x, b.groups);
     const int slice_lo = b.groups > 1 ? group_slice_begin(b.total, grp, b.groups, (int)gridDim.x) : 0;
     const int slice_n = (b.groups > 1 ? group_slice_begin(b.total, grp + 1, b.groups, (int)gridDim.x) : b.total) - slice_lo;
+    announce_start(b, leader);
     for (int it = 0;; ++it) {
         int idx, kt0 = 0;
         if (!dynamic) {

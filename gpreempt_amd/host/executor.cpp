@@ -168,6 +168,8 @@ BLPExecutor::~BLPExecutor() {
     if (stamps_host) gp_host_free(stamps_host);
     if (stop_host) gp_host_free(stop_host);
     if (left_host) gp_flag_destroy(left_host);
+    if (started_host) gp_flag_destroy(started_host);
+    if (mark_host) gp_flag_destroy(mark_host);
 }
 
 bool BLPExecutor::program_vacated() const {
@@ -299,6 +301,30 @@ Status BLPExecutor::resume(GPUstream stream) {
     if (use_program) return model->launch_program(stream, false, inject_kernel, inject_claim);
     for (size_t i = (size_t)stopIndex; i < get_kernel_num(); i++) RETURN_STATUS(launch_kernel(i, stream));
     return Status::Succ;
+}
+
+Status BLPExecutor::enable_launch_tracking() {
+    if (graph_compute || !model) return Status::Fail;
+    if (started_host) return Status::Succ;
+    CUDA_RETURN_STATUS(gp_flag_create(&started_host, &started_dev));
+    *started_host = 0;
+    model->set_started_word(started_dev);
+    return Status::Succ;
+}
+Status BLPExecutor::mark_stream(GPUstream stream) {
+    if (!mark_host) {
+        CUDA_RETURN_STATUS(gp_flag_create(&mark_host, &mark_dev));
+        *mark_host = 0;
+    }
+    mark_seq = mark_seq == 0x7fffffff ? 1 : mark_seq + 1;
+    CUDA_RETURN_STATUS(gp_store_word_async(stream, (int *)mark_dev, mark_seq));
+    return Status::Succ;
+}
+int BLPExecutor::launches_submitted() const { return model ? model->launch_number() : 0; }
+void BLPExecutor::restart_launch_tracking() {
+    if (!started_host || !model) return;
+    *started_host = 0;
+    model->restart_launch_numbers();
 }
 
 Status BLPExecutor::enable_device_stamps(GPUstream stream) {

@@ -356,6 +356,8 @@ Status init_tenant(Tenant &t, Shared &sh) {
         t.ex->capture_graph(t.stream);
     }
     if (chunked) for (int i = 0; i < 3; ++i) CUDA_RETURN_STATUS(gp_event_create(&t.chunk_events[i]));
+    static const bool use_events = [] { const char *e = getenv("GPREEMPT_CHUNK_EVENTS"); return e && *e == '1'; }();
+    if (chunked && !use_events && !t.ex->graph_workload()) RETURN_STATUS(t.blp->enable_launch_tracking());
     if (chunked && sh.device_stamps && !t.ex->graph_workload()) RETURN_STATUS(t.blp->enable_device_stamps(t.stream));
     return Status::Succ;
 }
@@ -388,6 +390,21 @@ Status drain(GPUstream s) {
     }
 }
 
+// The same for a tenant with launch tracking: a marker behind what is queued, then loads of host memory.  (The queue
+// is still asked now and then, so that an error on the stream ends the wait.)
+Status drain_marked(BLPExecutor *ex, GPUstream s) {
+    RETURN_STATUS(ex->mark_stream(s));
+    for (long i = 1;; ++i) {
+        if (ex->stream_left()) return Status::Succ;
+        if ((i & 0xffff) == 0) {
+            int idle = 0;
+            CUDA_RETURN_STATUS(gp_stream_query(s, &idle));
+            if (idle) return Status::Succ;
+        }
+        spin_pause();
+    }
+}
+
 // "wb-chunk" / "wb-chunk-async": the best-effort model is submitted launch by launch
 // (Executor::launch_kernel, the reference's own launch loop, src/executor.cpp:222-225) but never
 // more than two chunks of kernels ahead of the GPU.  A preempted model then has at most two chunks
@@ -400,24 +417,38 @@ static int chunk_size() {
     static const int v = [] { const char *e = getenv("GPREEMPT_CHUNK"); int c = e ? atoi(e) : 2; return c < 1 ? 1 : c; }();
     return v;
 }
+static int queue_depth() {
+    static const int v = [] { const char *e = getenv("GPREEMPT_QUEUE"); int c = e ? atoi(e) : 2; return c < 1 ? 1 : c; }();
+    return v;
+}
 Status infer_chunked(Tenant &t, Shared &sh, int p) {
     BLPExecutor *ex = t.blp;
     const size_t n = ex->get_kernel_num();
     Status st = ex->reset_counters(t.stream);
     size_t next = 0;
     int inflight = 0, head = 0, tail = 0;  // ring of 3 events, at most 2 in flight
+    // With launch tracking (BLPExecutor::enable_launch_tracking) no events are needed: every launch reports its start,
+    // and at most queue_depth() launches are kept submitted and not started (one, behind a kernel of 3 GFLOP or more).
+    const bool tracked = ex->launch_tracking_enabled();
+    if (tracked) ex->restart_launch_tracking();
+    double last_flops = 0;
+    bool tail_marked = false;              // the marker behind the model's last kernel has been submitted
     int64_t first_launch_ns = 0;           // when the first kernel of this request, or of its latest resumption, was submitted
     bool resumed = false;
     ex->running = true;
     sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
-    while (st == Status::Succ && (next < n || inflight > 0)) {
+    while (st == Status::Succ && (tracked || next < n || inflight > 0)) {
         if (sh.active_above(p) > 0) {
             // a higher level wants the GPU: stop feeding, let what is queued leave
-            st = drain(t.stream);
+            int queued = inflight;
+            // (tracked: the launches that have not started, and the one that has, if the tail marker has not run yet)
+            if (tracked) queued = ex->launches_submitted() - ex->launches_started() + (ex->launches_submitted() > 0 && !(tail_marked && ex->stream_left()) ? 1 : 0);
+            st = tracked ? drain_marked(ex, t.stream) : drain(t.stream);
+            tail_marked = false;
             if (st != Status::Succ) break;
             int64_t drained = now_ns();
-            const int queued = inflight;
             inflight = 0; head = tail;
+            if (tracked) ex->restart_launch_tracking();  // nothing of this tenant is in flight
             sh.on_gpu[p].fetch_sub(1, std::memory_order_acq_rel);
             // read the stop index back (and re-arm it) while the higher level has the GPU: nothing of
             // this tenant is in flight, and the blocking read-back (10-20 us) then costs nobody anything
@@ -459,6 +490,37 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
             sh.on_gpu[p].fetch_add(1, std::memory_order_acq_rel);
             if (stop >= 0) { next = (size_t)stop; ++t.preemptions; resumed = true; first_launch_ns = 0; }  // kernels from the stopped one on are submitted again
             if (stop >= 0 && ex->device_stamps_enabled()) t.resubmitted_ns = now_ns();
+            continue;
+        }
+        if (tracked) {
+            const int waiting = ex->launches_submitted() - ex->launches_started();
+            if (next < n && waiting < (last_flops >= 3e9 ? 1 : queue_depth())) {
+                if (!first_launch_ns) first_launch_ns = now_ns();
+                auto model = ex->get_model();
+                last_flops = model ? model->get_kernel_info(next).flops : 0;
+                st = ex->launch_kernel(next, t.stream);
+                ++next;
+                continue;
+            }
+            if (next >= n) {
+                if (!tail_marked) {
+                    st = ex->mark_stream(t.stream);
+                    tail_marked = true;
+                    continue;
+                }
+                if (ex->stream_left()) {
+                    tail_marked = false;
+                    // everything was submitted and has left the GPU; a late stop may still have cut it short
+                    st = ex->getStopPoint(t.stream);
+                    if (st == Status::Succ && ex->last_stop_index() >= 0) {
+                        next = (size_t)ex->last_stop_index(); ++t.preemptions;
+                        ex->restart_launch_tracking();
+                        continue;
+                    }
+                    break;
+                }
+            }
+            spin_pause();
             continue;
         }
         if (next < n && inflight < 2) {

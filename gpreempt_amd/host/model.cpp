@@ -474,6 +474,10 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
             ctx.done = (int *)((char *)k.executed + done_offset_);
             ctx.done_launches = idx < launches_.size() ? launches_[idx] : 0;
         }
+        if (started_) {
+            ctx.started_host = (int *)started_;
+            ctx.started_seq = launch_seq_ + 1;
+        }
         pc = &ctx;
     }
     gp_launch_info info{};
@@ -493,6 +497,7 @@ Status Model::launch(size_t idx, GPUstream stream, int inject_at) {
     }
     if (idx < fresh_.size()) fresh_[idx] = 0;  // launched (or refused): from here on only its counters know
     if (idx < launches_.size() && rc == 0) ++launches_[idx];
+    if (pc && started_ && rc == 0) ++launch_seq_;
     CUDA_RETURN_STATUS(rc);
     k.total_blocks = info.total_tiles;
     k.fixed_claims = info.fixed_claims != 0;

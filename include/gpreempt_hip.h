@@ -88,6 +88,11 @@ int gp_fill32_async(void *dev, uint32_t value, size_t count, gp_stream s);
  * with system-scope loads. */
 int gp_flag_create(volatile int **host_ptr, void **dev_ptr);
 int gp_flag_destroy(volatile int *host_ptr);
+/* A one-workgroup kernel on `s` that stores `value` in a gp_flag_create word (word_dev = its dev_ptr): when the host
+ * reads the value there, everything submitted to `s` before the call has left the GPU.  What a host that polls for
+ * "has my stream drained" (src/cuda-clients/blpclient.cpp:189-195 spins on a counter for the same purpose) uses
+ * instead of stream queries, which cost 3-5 us apiece once the stream's last command is a kernel. */
+int gp_store_word_async(gp_stream s, int *word_dev, int value);
 /* Flag relay: one small resident kernel copies n host flag words (device-visible addresses of
  * gp_flag_create flags, flags_dev[i]) into device memory (mirror[i]) whenever they change, so
  * that kernels can poll a device address on every claim instead of crossing PCIe; a host store
@@ -160,6 +165,12 @@ typedef struct gp_preempt_ctx {
                      /* words 8 + (workgroup mod 1024) whenever a workgroup of a preemptible launch leaves.    */
                      /* What                                                                                  */
                      /* src/cuda-clients/blpclient.cpp:185-195 measures from the host, measured on the GPU.    */
+    int *started_host; /* may be NULL: device-visible address of a gp_flag_create word.  The first workgroup of  */
+                     /* the launch stores started_seq there when it starts, i.e. when every launch before it  */
+                     /* on the stream has left the GPU.  A host that submits a model kernel by kernel          */
+                     /* (src/executor.cpp:222-225) reads the word to keep a bounded number of launches queued  */
+                     /* without events or queue queries, each of which costs the stream 3.7 us on MI355X.      */
+    int started_seq;
 } gp_preempt_ctx;
 enum { GP_STAMP_STOP = 0, GP_STAMP_FIRST_CLAIM = 1, GP_STAMP_EXIT0 = 8, GP_STAMP_EXIT_SLOTS = 1024, GP_STAMP_WORDS = 8 + 1024 };
 /* The device clock the stamps are taken from: *tick_ns = nominal nanoseconds per tick; *offset_ns = what to

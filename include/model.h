@@ -161,6 +161,11 @@ public:
     void set_checkpoint_workspace(GPUdeviceptr p, size_t bytes) { ckpt_ = p; ckpt_bytes_ = bytes; }
     // device time stamps of preemptions (gp_preempt_ctx::stamps); null = off
     void set_stamps(GPUdeviceptr p) { stamps_ = p; }
+    // A word of host memory (its device-visible address) in which every preemptible launch stores its number when its
+    // first workgroup starts (gp_preempt_ctx::started_host); launch numbers count from 1 after restart_launch_numbers().
+    void set_started_word(GPUdeviceptr p) { started_ = p; launch_seq_ = 0; }
+    void restart_launch_numbers() { launch_seq_ = 0; }
+    int launch_number() const { return launch_seq_; }
     // largest such workspace any kernel of the model can use (0: none can)
     size_t checkpoint_bytes_wanted() const;
     int last_launch_tag() const { return last_launch_tag_; }
@@ -194,6 +199,8 @@ private:
     GPUdeviceptr ckpt_ = nullptr;
     size_t ckpt_bytes_ = 0;
     GPUdeviceptr stamps_ = nullptr;
+    GPUdeviceptr started_ = nullptr;      // see set_started_word
+    int launch_seq_ = 0;
     int last_launch_tag_ = 0;
     std::string workload_, dtype_;
     std::shared_ptr<struct TvmExport> export_;

@@ -467,3 +467,38 @@ def test_deep_preemptible_convolution_takes_small_tiles_with_the_same_bits(gp):
     info = gp.launch("gp_launch_conv2d", p, st.ctx(fresh=1))
     sync(gp)
     assert info.total_tiles == (M // 128) * (Cc // 128) and np.array_equal(do.download(), base)
+
+
+def test_launches_report_their_start_and_a_marker_reports_the_end(gp):
+    """gp_preempt_ctx::started_host: the first workgroup of every preemptible launch stores the launch's number in
+    a word of host memory, in stream order, whichever dispatcher loop the kernel is built around; a
+    gp_store_word_async marker behind them says that all of them have left.  (What a host that submits kernel by
+    kernel polls instead of events and stream queries.)"""
+    import time
+    started, left = gp.Flag(), gp.Flag()
+    started.set(0); left.set(0)
+    flag = gp.Flag()
+    st = gp.BlpState(4, flag, 32)
+    stream = gp.Stream(1)
+    rng = np.random.default_rng(5)
+    M, N, K = 512, 512, 256
+    A = O.round_to(rng.uniform(-1, 1, (M, K)).astype(np.float32), "f16")
+    B = O.round_to(rng.uniform(-1, 1, (N, K)).astype(np.float32), "f16")
+    dA, dB, dC = gp.DevBuf.from_array(A, gp.F16), gp.DevBuf.from_array(B, gp.F16), gp.DevBuf(M * N * 2)
+    g = gp.GemmParams(dtype=gp.F16, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, alpha=1.0, act=gp.ACT_NONE, batch=1)
+    dX, dY = gp.DevBuf.from_array(A[:, :1].repeat(N, 1).copy(), gp.F16), gp.DevBuf(M * N * 2)
+    e = gp.EltwiseParams(dtype=gp.F16, rows=M, cols=N, a=dC.ptr, a_stride=N, b=dX.ptr, b_stride=N, scale=None, shift=None, out=dY.ptr, out_stride=N, act=gp.ACT_RELU)
+    seen = []
+    for seq, (fn, p, kid) in enumerate([("gp_launch_gemm", g, 0), ("gp_launch_eltwise", e, 1), ("gp_launch_gemm", g, 2), ("gp_launch_eltwise", e, 3)], start=1):
+        gp.launch(fn, p, st.ctx(kernel_id=kid, fresh=1, started=started, started_seq=seq), stream)
+    gp.check(gp.lib().gp_store_word_async(stream.h, gp.vp(left.dev), 77))
+    t0 = time.perf_counter()
+    while left.get() != 77 and time.perf_counter() - t0 < 5.0:
+        seen.append(started.get())
+    assert left.get() == 77, "the marker never ran"
+    # by the time the marker has run every launch before it has started (and left): the word holds the last number
+    assert started.get() == 4
+    assert seen == sorted(seen), "launch numbers went backwards"
+    stream.sync()
+    want = np.maximum(O.gemm_bias_act(A, B, None, None, gp.ACT_NONE, b_is_nk=True) + A[:, :1], 0)
+    assert rel_err(dY.download(gp.F16, (M, N)), want) < TOL["f16"]
