@@ -406,8 +406,10 @@ Status drain_marked(BLPExecutor *ex, GPUstream s) {
 }
 
 // "wb-chunk" / "wb-chunk-async": the best-effort model is submitted launch by launch
-// (Executor::launch_kernel, the reference's own launch loop, src/executor.cpp:222-225) but never
-// more than two chunks of kernels ahead of the GPU.  A preempted model then has at most two chunks
+// (Executor::launch_kernel, the reference's own launch loop, src/executor.cpp:222-225) but never far ahead of the
+// GPU: with launch tracking (the default) at most queue_depth() launches that have not started, as the launches
+// themselves report; without it (GPREEMPT_CHUNK_EVENTS=1) never
+// more than two chunks of kernels ahead of the GPU, by an event behind every chunk, which costs the stream 3.7 us.  A preempted model then has at most two chunks
 // of queued kernels to flush (each leaves at its first look at the stop index, about 4 us apiece
 // on MI355X) instead of the rest of the network, while every kernel keeps its own occupancy.
 // Measured with BERT over ResNet-152: chunks of 6 / 3 / 2 / 1 kernels drain in 44 / 32 / 28 / 23 us
