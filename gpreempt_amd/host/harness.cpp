@@ -435,6 +435,7 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
     if (tracked) ex->restart_launch_tracking();
     double last_flops = 0;
     bool tail_marked = false;              // the marker behind the model's last kernel has been submitted
+    unsigned long idle_spins = 0;
     int64_t first_launch_ns = 0;           // when the first kernel of this request, or of its latest resumption, was submitted
     bool resumed = false;
     ex->running = true;
@@ -521,6 +522,13 @@ Status infer_chunked(Tenant &t, Shared &sh, int p) {
                     }
                     break;
                 }
+            }
+            // (a launch that never reported its start would leave this loop waiting for it: the queue is asked now
+            // and then, and an idle queue means that everything submitted has run)
+            if ((++idle_spins & 0x3ffff) == 0) {
+                int idle = 0;
+                if (gp_stream_query(t.stream, &idle) != 0) { st = Status::Fail; break; }
+                if (idle && !tail_marked) ex->restart_launch_tracking();
             }
             spin_pause();
             continue;
