@@ -189,7 +189,7 @@ extern "C" int gpx_run_scenario(const char *config_json, char *report, size_t re
 extern "C" int gpx_preempt_probe(const char *workload, int trials, int use_graph, unsigned long long seed, char *report, size_t report_len) {
     return guarded("gpx_preempt_probe", [&] {
         std::string rep;
-        Status st = foo::preempt_probe(workload ? workload : "", trials, use_graph != 0, seed, rep);
+        Status st = foo::preempt_probe(workload ? workload : "", trials, use_graph, seed, rep);
         return copy_report(st, rep, report, report_len);
     });
 }

@@ -10,12 +10,12 @@
 
 int main(int argc, char **argv) {
     if (argc < 2) {
-        std::cout << "Usage: " << argv[0] << " config.json [policy] | --probe workload [trials]" << std::endl;
+        std::cout << "Usage: " << argv[0] << " config.json [policy] | --probe workload [trials] [0 = all kernels at once | 1 = as one program | 2 = kernel by kernel, bounded queue (default)]" << std::endl;
         return -1;
     }
     std::string report;
     if (std::strcmp(argv[1], "--probe") == 0 && argc >= 3) {
-        Status s = foo::preempt_probe(argv[2], argc > 3 ? std::atoi(argv[3]) : 200, true, 1, report);
+        Status s = foo::preempt_probe(argv[2], argc > 3 ? std::atoi(argv[3]) : 200, argc > 4 ? std::atoi(argv[4]) : 2, 1, report);
         std::cout << report << std::endl;
         return s == Status::Succ ? 0 : 1;
     }

@@ -1067,7 +1067,40 @@ Status run_scenario(const std::string &config_text, std::string &report_text) {
 // back; an injector raises the flag at random instants, waits for the stream to drain, notes
 // which kernel was stopped (the stop index) and how long the drain took, then clears the flag
 // and the model resumes.
-Status preempt_probe(const std::string &workload, int trials, bool use_graph, uint64_t seed, std::string &report_text) {
+// Kernels [from, n) of the executor's model submitted one by one, never more than queue_depth() launches ahead of the
+// GPU (one, behind a kernel of 3 GFLOP or more), as infer_chunked does for a tenant.  With raise_at != 0 the flag goes
+// up at that time (CLOCK_MONOTONIC nanoseconds) wherever the submission stands, and nothing more is submitted;
+// *raised then holds the time of the store.  Returns with the stream drained.
+static Status submit_tracked(BLPExecutor &ex, GPUstream stream, size_t from, volatile int *flag_host, int64_t raise_at, int64_t *raised) {
+    const size_t n = ex.get_kernel_num();
+    auto model = ex.get_model();
+    ex.restart_launch_tracking();
+    size_t next = from;
+    double last_flops = 0;
+    bool marked = false;
+    for (;;) {
+        if (raise_at && !*raised && now_ns() >= raise_at) {
+            *raised = now_ns();
+            *flag_host = 1;
+            break;
+        }
+        const int waiting = ex.launches_submitted() - ex.launches_started();
+        if (next < n && waiting < (last_flops >= 3e9 ? 1 : queue_depth())) {
+            last_flops = model ? model->get_kernel_info(next).flops : 0;
+            RETURN_STATUS(ex.launch_kernel(next, stream));
+            ++next;
+            continue;
+        }
+        if (next >= n) {
+            if (!marked) { RETURN_STATUS(ex.mark_stream(stream)); marked = true; }
+            else if (ex.stream_left() && !(raise_at && !*raised)) return Status::Succ;  // (a probe waits for its instant)
+        }
+        spin_pause();
+    }
+    return drain_marked(&ex, stream);
+}
+
+Status preempt_probe(const std::string &workload, int trials, int use_graph, uint64_t seed, std::string &report_text) {
     util::init_cuda();
     BLPExecutor ex;
     RETURN_STATUS(ex.init(workload));
@@ -1077,7 +1110,11 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
     ex.dpStop = flag_dev;
     GPUstream stream;
     CUDA_RETURN_STATUS(gp_stream_create(1, &stream));
-    if (use_graph) ex.capture_graph(stream);
+    // use_graph: 0 = every kernel launched at once (execute), 1 = the captured form (the whole-model program), 2 = kernel
+    // by kernel with a bounded queue, which is how the scenario runner feeds a best-effort tenant
+    const bool tracked = use_graph == 2;
+    if (use_graph == 1) ex.capture_graph(stream);
+    if (tracked) RETURN_STATUS(ex.enable_launch_tracking());
     // the GPU's own time stamps ride along (GPREEMPT_PROBE_STAMPS=0 switches them off)
     const char *ps = getenv("GPREEMPT_PROBE_STAMPS");
     const bool stamps = !(ps && *ps == '0') && ex.enable_device_stamps(stream) == Status::Succ;
@@ -1088,8 +1125,13 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
     Stats iso;
     for (int i = 0; i < 12; ++i) {
         int64_t t0 = now_ns();
-        RETURN_STATUS(ex.execute(stream));
-        RETURN_STATUS(drain(stream));
+        if (tracked) {
+            RETURN_STATUS(ex.reset_counters(stream));
+            RETURN_STATUS(submit_tracked(ex, stream, 0, flag_host, 0, nullptr));
+        } else {
+            RETURN_STATUS(ex.execute(stream));
+            RETURN_STATUS(drain(stream));
+        }
         if (i >= 2) iso.add((now_ns() - t0) / 1e3);
     }
     double span_us = iso.mean();
@@ -1099,13 +1141,19 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
     int hits = 0;
     for (int tr = 0; tr < trials; ++tr) {
         ex.running = true;
-        RETURN_STATUS(ex.execute(stream));
         int64_t wait = (int64_t)(rng.uniform01() * span_us * 0.95 * 1e3);
-        int64_t t0 = now_ns();
-        while (now_ns() - t0 < wait) spin_pause();
-        int64_t raised = now_ns();
-        *flag_host = 1;
-        RETURN_STATUS(drain(stream));
+        int64_t raised = 0;
+        if (tracked) {
+            RETURN_STATUS(ex.reset_counters(stream));
+            RETURN_STATUS(submit_tracked(ex, stream, 0, flag_host, now_ns() + wait, &raised));
+        } else {
+            RETURN_STATUS(ex.execute(stream));
+            int64_t t0 = now_ns();
+            while (now_ns() - t0 < wait) spin_pause();
+            raised = now_ns();
+            *flag_host = 1;
+            RETURN_STATUS(drain(stream));
+        }
         int64_t drained = now_ns();
         *flag_host = 0;
         BLPExecutor::DeviceStamps ds;
@@ -1115,10 +1163,20 @@ Status preempt_probe(const std::string &workload, int trials, bool use_graph, ui
             RETURN_STATUS(drain(stream));
         }
         int64_t r0 = now_ns();
-        RETURN_STATUS(ex.resume(stream));
-        int64_t r1 = now_ns();
-        int stop = ex.last_stop_index();
-        RETURN_STATUS(drain(stream));
+        int64_t r1 = r0;
+        int stop = -1;
+        if (tracked) {
+            // the tenant's resume: read the stop index back, submit from the stopped kernel on
+            RETURN_STATUS(ex.getStopPoint(stream));
+            stop = ex.last_stop_index();
+            r1 = now_ns();
+            if (stop >= 0) RETURN_STATUS(submit_tracked(ex, stream, (size_t)stop, flag_host, 0, nullptr));
+        } else {
+            RETURN_STATUS(ex.resume(stream));
+            r1 = now_ns();
+            stop = ex.last_stop_index();
+            RETURN_STATUS(drain(stream));
+        }
         if (stamps && stop >= 0) {
             BLPExecutor::DeviceStamps rs;
             RETURN_STATUS(ex.read_device_stamps(stream, rs));

@@ -11,6 +11,6 @@ namespace foo {
 Status run_scenario(const std::string &config_text, std::string &report_text);
 
 // Measures flag-store -> stream-drained latency of `workload` per stopped kernel.
-Status preempt_probe(const std::string &workload, int trials, bool use_graph, uint64_t seed, std::string &report_text);
+Status preempt_probe(const std::string &workload, int trials, int use_graph, uint64_t seed, std::string &report_text);
 
 }  // namespace foo

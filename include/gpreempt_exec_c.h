@@ -74,7 +74,10 @@ int gpx_miniweather_reductions(gpx_executor e, double *mass, double *te);
  * baseclient.cpp), "seq" (seqclient.cpp), "lco" (high-priority tasks only, rtonlyclient.cpp).
  * The JSON report is written to `report` (NUL-terminated, truncated to report_len). */
 int gpx_run_scenario(const char *config_json, char *report, size_t report_len);
-/* Per-kernel preemption / resume latency of one best-effort model (BASELINE config 2). */
+/* Per-kernel preemption / resume latency of one best-effort model (BASELINE config 2): `trials` inferences, each
+ * stopped at a random instant by the host and resumed (the protocol of src/tests/test-dnn-blp.cpp:36-42).
+ * use_graph: 0 = BLPExecutor::execute launches every kernel at once, 1 = the captured form (whole-model program),
+ * 2 = kernel by kernel with a bounded queue, as the scenario runner feeds a best-effort tenant. */
 int gpx_preempt_probe(const char *workload, int trials, int use_graph, unsigned long long seed, char *report, size_t report_len);
 /* Parses a TVM_MODEL_PARAMS file (ModelParamParser::parse_from_file, reference src/model.cpp:15-55):
  * returns the number of tensors (-1: missing or malformed); when `key` names a tensor, up to n of

@@ -150,3 +150,23 @@ def test_exported_model_as_best_effort_tenant(gp, tmp_path):
     assert hp["requests"] >= 40 and be["requests"] > 0 and be["preemptions"] > 0
     assert be["kernels"] == 1 + 1 + 1 + 4 * 4 + 1 + 1 + 1   # layout, stem, pool, four blocks of four convolutions, pool, classifier, softmax
     assert hp["outputMismatches"] == 0 and be["outputMismatches"] == 0
+
+
+@pytest.mark.parametrize("mode", [2, 1, 0])
+def test_preempt_probe_of_config2(gp, mode):
+    """BASELINE config 2 through gpx_preempt_probe: ResNet-50 fp32 b1 stopped at random instants by the host and
+    resumed (the protocol of src/tests/test-dnn-blp.cpp:36-42), fed kernel by kernel with a bounded queue (2), as
+    one persistent program (1) or with every kernel launched at once as BLPExecutor::execute does (0).  Every mode
+    reports its interruptions; the bounded queue, which is how a tenant is fed, drains in well under 50 us."""
+    from gpreempt_amd import executor as gx
+    buf = C.create_string_buffer(1 << 20)
+    rc = gx.lib().gpx_preempt_probe(b"resnet50", 80, mode, C.c_ulonglong(3), buf, C.c_size_t(len(buf)))
+    assert rc == 0, buf.value[:400]
+    r = json.loads(buf.value.decode())
+    assert r["kernels"] > 50 and r["trials"] == 80 and r["interrupted"] > 40
+    lat = r["preemptLatency(us)"]
+    assert lat["count"] == r["interrupted"] and 0 < lat["mean"] < 400
+    assert {"flagStore_to_stopRecorded", "stopRecorded_to_lastWorkgroupExit", "lastWorkgroupExit_to_hostNotices"} <= set(r["deviceStamps(us)"])
+    assert all(k["samples"] > 0 and k["preempt_max(us)"] >= k["preempt_mean(us)"] > 0 for k in r["perKernel"])
+    if mode == 2:
+        assert lat["p99"] < 50, lat
