@@ -170,3 +170,29 @@ def test_preempt_probe_of_config2(gp, mode):
     assert all(k["samples"] > 0 and k["preempt_max(us)"] >= k["preempt_mean(us)"] > 0 for k in r["perKernel"])
     if mode == 2:
         assert lat["p99"] < 50, lat
+
+
+def test_chunked_policy_with_an_event_per_chunk_still_works(gp, tmp_path):
+    """The chunked policies keep their queue short through the launches' own start reports by default; with
+    GPREEMPT_CHUNK_EVENTS=1 (read once per process, hence the child process) they fall back to an event behind
+    every chunk of GPREEMPT_CHUNK kernels.  Both ways the tenant is preempted and every request returns the bits of
+    an uninterrupted run."""
+    import os
+    import subprocess
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg = {"time": 1.5, "policy": "wb-chunk-async", "warmups": 3, "standalone_runs": 10, "verify_outputs": True, "tasks": [
+        {"id": "hp", "load": {"type": "poisson", "frequency": 300, "seed": 5},
+         "client": {"name": "hp", "model_name": "bert@layers=2,s=128", "priority": 0, "launch_mode": "launch"}},
+        {"id": "be", "load": {"type": "continuous"},
+         "client": {"name": "be", "model_name": "resnet50@b=2", "priority": 1, "launch_mode": "launch"}}]}
+    path = tmp_path / "cfg.json"
+    path.write_text(json.dumps(cfg))
+    for env_extra in ({"GPREEMPT_CHUNK_EVENTS": "1", "GPREEMPT_CHUNK": "3"}, {"GPREEMPT_QUEUE": "1"}):
+        out = subprocess.run([os.path.join(root, "gpreempt_amd", "gpreempt_bench"), str(path)], capture_output=True, text=True,
+                             env={**os.environ, **env_extra}, timeout=100)
+        assert out.returncode == 0, out.stderr[-400:]
+        rep = json.loads(out.stdout.strip().splitlines()[-1])
+        t = rep["tasks"]
+        assert t["hp"]["requests"] > 200 and t["be"]["requests"] > 50 and t["be"]["preemptions"] > 50, (env_extra, t["be"])
+        assert t["be"]["outputMismatches"] == 0 and t["hp"]["outputMismatches"] == 0
+        assert rep["preemptLatency(us)"]["count"] > 50 and rep["preemptLatency(us)"]["p99"] < 200
