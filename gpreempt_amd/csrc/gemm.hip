@@ -93,12 +93,16 @@ static int launch_mat(const MatPlan &pl, const gp_preempt_ctx *ctx, gp_stream s,
         });
         GP_HIP(once_rc);
     }
-    // Long tiles (2 * 10^7 multiply-adds of the 16-bit rate and more, 10-40 us depending on how many workgroups share a
+    // Long tiles (1.8 * 10^7 multiply-adds of the 16-bit rate and more, 10-40 us depending on how many workgroups share a
     // compute unit): what a stopped tenant would otherwise finish before it leaves.  The bodies that look at the stop
     // word every few K-stages can give such a tile up (tile_fixed_early).  Measured with the threshold at 0.8 / 2 / 4 * 10^7:
     // ResNet-50 fp32 b1 under a 500 req/s probe drains in 35 / 42 / 57 us (p99) and keeps 1046 / 1095 / 1094 req/s
-    // (a launch in this mode is about a microsecond longer).  GPREEMPT_LONG_TILE_MACS overrides it.
-    static const double long_macs = [] { const char *e = getenv("GPREEMPT_LONG_TILE_MACS"); return e && atof(e) > 0 ? atof(e) : 2e7; }();
+    // (a launch in this mode is about a microsecond longer).  The 64x64 tiles with K = 4608 and the 128x128 tiles with
+    // K = 1152 of VGG-16 have 1.89 * 10^7 each: with them in, BERT's drains of VGG-16 end within 48 us (p99) instead of
+    // 60, and a VGG-16 pass takes 4 % longer (those launches 13 %: the instantiation that looks runs its K-steps that
+    // much slower than the one that does not, although the two execute the same instructions per K-step to within a
+    // few scalar ones).  GPREEMPT_LONG_TILE_MACS overrides it.
+    static const double long_macs = [] { const char *e = getenv("GPREEMPT_LONG_TILE_MACS"); return e && atof(e) > 0 ? atof(e) : 1.8e7; }();
     const bool long_tiles = K::can_look && (double)K::bm * K::bn * pl.g.K * (pl.dtype == GP_F32 ? 8.0 : 1.0) >= long_macs;
     int rc = plan_launch(kern, K::NT, K::LDS_BYTES, pl.sx, pl.sy, pl.batch, ctx, &blp, &grid, info, 1, K::LDS_BYTES <= 64 * 1024 ? 4 : 1, long_tiles);
     if (rc) return rc;

@@ -88,7 +88,7 @@ struct LnWideKernel {
         }
         auto issue = [&](int s) {
             const int k0 = (s * KB + kb) * BK;
-            const unsigned sbase = lds0 + (unsigned)(s % STAGES) * STAGE_BYTES + (unsigned)kb * B_BLK_BYTES;
+            const unsigned sbase = lds0 + ((unsigned)s % STAGES) * STAGE_BYTES + (unsigned)kb * B_BLK_BYTES;
 #pragma unroll
             for (int j = 0; j < LPW; ++j) {
                 const bool ok = row_ok[j] & (k0 < g.K);   // whole blocks past the last one, when the stage is not full
@@ -187,7 +187,7 @@ struct LnWideKernel {
             else wait_vmcnt<0>();
             __syncthreads();  // stage s of B (and, the first time, the rows of A) visible; the buffer of stage s-1 is free
             if (s == 0) GP_PROBE(2);
-            if (s == 0 && early && __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1) {
+            if (s == 0 && early && __builtin_amdgcn_readfirstlane(read_lds_word(early_slot)) != -1) {
                 wait_vmcnt<0>();  // loads still landing in LDS must not outlive the workgroup
                 return true;
             }
@@ -211,7 +211,7 @@ struct LnWideKernel {
             }
             if (s >= PRE - (STAGES - 1) && s + STAGES - 1 < NS) issue(s + STAGES - 1);
             if (kb >= G) continue;  // (uniform) the other wavefronts only fetch
-            const int stage = s % STAGES;
+            const int stage = (int)((unsigned)s % STAGES);
 #pragma unroll
             for (int b = 0; b < KB; ++b) {
                 if (s * KB + b >= KT) break;

@@ -37,9 +37,16 @@ __device__ __forceinline__ void load_lds16(const void *gptr, unsigned lds_byte) 
                  : "memory", "m0");
 }
 
+// Reads a word that a load-to-LDS has written.  The pointer must carry the LDS address space: through a plain
+// `volatile int *` the read is a flat load, which counts as a vector-memory operation as well, and the wait that the
+// compiler puts behind it (vmcnt 0) also waits for every operand load the wavefront has in flight.
+__device__ __forceinline__ int read_lds_word(const int *p) {
+    return *(__attribute__((address_space(3))) volatile int *)(__attribute__((address_space(3))) void *)p;
+}
 // 4 bytes per lane: lane i's dword lands at lds_byte + 4*i.  Read past the caches (sc0 sc1): the
 // word is one that another workgroup or the host changes while this kernel runs.
 __device__ __forceinline__ void load_lds4(const void *gptr, unsigned lds_byte) {
+    lds_byte = __builtin_amdgcn_readfirstlane(lds_byte);  // (the same for every lane; the compiler may hold it in a vector register)
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off sc0 sc1"
                  :
                  : "v"(gptr), "s"(lds_byte)
@@ -87,8 +94,8 @@ struct CkptCtx {       // what a checkpointing body needs from the dispatcher, p
     void *ckpt;
     int kernel_id;
     unsigned long long *stamps = nullptr;  // BlpArgs::stamps (the measurement mode of tile_loop.hpp)
-    int *announce = nullptr;               // run<true> with a stop word: the counter in which the workgroup counts itself at its
-                                           // last look, less than LOOK_EVERY K-steps before the end of a tile that it finishes
+    int *announce = nullptr;               // run<true> with a stop word: the counter in which the workgroup counts itself at the
+                                           // top of the last K-step of a tile that it finishes
 };
 
 // NWAVES: wavefronts per workgroup.  With eight (two per SIMD, 128 accumulator registers each) the
@@ -138,7 +145,7 @@ struct PipeKernel {
     static __device__ __forceinline__ bool run(const MatArgs &g, TileIdx t, T *lds_t, CkptCtx cc = CkptCtx{nullptr, nullptr, nullptr, 0},
                                                int tile_index = 0, int kt0 = 0) {
         GP_PROBE(0);
-        __shared__ int early_slot[64];  // landing place of the early-stop word (lane 0's dword)
+        __shared__ int early_slot[LOOKS ? 192 : 64];  // landing places of the stop word (lane 0's dword of each 64): the early look's, then two that the later looks take in turn
         // (made wave-uniform by force: handed over in a vector register, the word would make the compiler treat every branch
         // that depends on it as divergent, and the barriers and hand-placed waits below assume uniform control flow)
         const bool early = !CKPT && __builtin_amdgcn_readfirstlane((int)(cc.stop_index != nullptr)) != 0;
@@ -146,7 +153,11 @@ struct PipeKernel {
         // word is fetched by wavefront 0 at the top of the K-step in which the stage it travels with is fetched, in
         // front of that stage's loads, and read by everybody at the end of that stage's K-step.  A tile that finds a
         // stop recorded is given up (the caller withdraws the claim; the relaunch computes it from the start).
+#ifdef GP_LOOK_EVERY
+        constexpr int LOOK_EVERY = GP_LOOK_EVERY;
+#else
         constexpr int LOOK_EVERY = 8;
+#endif
         static_assert(LOOK_EVERY >= STAGES, "a look is read before the next one is fetched");
         // (an instantiation of its own, LOOKS: as a run-time switch the looks cost the short tiles 3 % of a ResNet-152 pass)
         const bool looking = LOOKS && early;
@@ -231,8 +242,8 @@ struct PipeKernel {
         }
         auto stage_addr = [&](int kt) {
             StageAddr sa;
-            sa.sbase = lds0 + (unsigned)(kt % STAGES) * STAGE_BYTES;
-            sa.sbase_poll = lds0 + (unsigned)RING_BYTES + (unsigned)(kt % STAGES) * WAVES * 256;
+            sa.sbase = lds0 + ((unsigned)kt % STAGES) * STAGE_BYTES;
+            sa.sbase_poll = lds0 + (unsigned)RING_BYTES + ((unsigned)kt % STAGES) * WAVES * 256;
             sa.k0 = kt * BK;
             sa.r_u = nx_r; sa.s_u = nx_s;
             sa.tap_off = (nx_r * g.W + nx_s) * (int)g.lda + nx_ci;  // elements from the window origin
@@ -410,22 +421,31 @@ struct PipeKernel {
                 if constexpr (ISSUE) __builtin_amdgcn_sched_barrier(0);
             });
         };
+        const int KT = (g.K + BK - 1) / BK;
+        // A tile that is being finished counts its workgroup in cc.announce at the top of its last K-step, behind that step's
+        // wait for its operands: nothing the wavefront issues later is waited for before the epilogue.  (Counted at the last
+        // look instead, several K-steps from the end, the atomic stood in wavefront 0's queue in front of operand loads: the
+        // counts that the waits of the next K-steps rely on go down in the order of issue, so the whole workgroup waited for
+        // the atomic to be acknowledged, 6 us a tile with 512 workgroups resident.)
+        auto announce = [&]() {
+            if constexpr (LOOKS)
+                if (cc.announce && tid == 0) __hip_atomic_fetch_add(cc.announce, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        };
         // k-tile kt: wait for its stage, start fetching stage kt+STAGES-1 (ISSUE) and multiply.
-        auto ktile = [&](int kt, bool tail, auto issue_c) -> int {
+        auto ktile = [&](int kt, bool tail, auto issue_c, auto plain_c) -> int {
             constexpr bool ISSUE = decltype(issue_c)::value != 0;
+            constexpr bool PLAIN = decltype(plain_c)::value != 0;  // a K-step that cannot be the first of its tile and looks at nothing
             // stage kt has landed once at most the loads of the younger in-flight stages remain
             if (!tail) wait_vmcnt<(STAGES - 2) * NLOADS>();
             else wait_vmcnt<0>();
             int stop_word = -1, flag_word = 0;
             __syncthreads();  // everyone's part of stage kt is visible; stage kt-1's buffer is free
             if (kt == 0) GP_PROBE(2);
-            const int stage = kt % STAGES;
+            if constexpr (LOOKS && !ISSUE)
+                if (looking && kt == KT - 1 && kt > kt0) announce();
+            const int stage = (int)((unsigned)kt % STAGES);
             StageAddr sa = {};
             if constexpr (ISSUE) sa = stage_addr(kt + STAGES - 1);
-            if constexpr (ISSUE && !CKPT) {
-                if (looking && wave == 0 && ((kt + STAGES - 1 - kt0) & (LOOK_EVERY - 1)) == 0)
-                    load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
-            }
             if constexpr (SPLITK) {
                 read_frags(0, stage, wave);  // the address arithmetic of the loads overlaps the LDS latency
                 if constexpr (ISSUE) static_for<0, NLOADS>([&](auto lc) { issue_one(sa, decltype(lc)::value); });
@@ -434,7 +454,7 @@ struct PipeKernel {
                 constexpr int LAST = (KSTEPS - 1) & 1;
                 read_frags(0, stage, 0);
                 __builtin_amdgcn_sched_barrier(0);
-                if (kt > kt0) {
+                if (PLAIN || kt > kt0) {
                     phase(LAST, issue_c, sa, IntC<0>{});  // last k-step of stage kt-1 (in registers)
                 } else if constexpr (ISSUE) {
                     static_for<0, NM>([&](auto qc) {  // first k-tile: phase 0 has loads but no MFMAs
@@ -451,8 +471,8 @@ struct PipeKernel {
                         // last phase, whose MFMAs cover the LDS latency (read at the top of the k-tile they cost
                         // 12 % of a VGG-16 layer: the wait for them came in front of the first fragment reads)
                         if (can_ckpt && (kt & (POLL_EVERY - 1)) == 0) {
-                            stop_word = pollw[((kt % STAGES) * WAVES + 0) * 64];
-                            flag_word = pollw[((kt % STAGES) * WAVES + 1) * 64];
+                            stop_word = pollw[(((unsigned)kt % STAGES) * WAVES + 0) * 64];
+                            flag_word = pollw[(((unsigned)kt % STAGES) * WAVES + 1) * 64];
                         }
                     }
                     read_frags((ks + 1) & 1, stage, ks + 1);
@@ -462,9 +482,8 @@ struct PipeKernel {
                 __builtin_amdgcn_sched_barrier(0);
             }
             int stop_now = 0;
-            if constexpr (!CKPT) {
-                if ((early && kt == kt0) || (looking && kt > kt0 && ((kt - kt0) & (LOOK_EVERY - 1)) == 0))
-                    stop_now = __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1;
+            if constexpr (!CKPT && !PLAIN) {
+                if (early && kt == kt0) stop_now = __builtin_amdgcn_readfirstlane(read_lds_word(early_slot)) != -1;
             }
             if constexpr (CKPT) {
                 const int sw = __builtin_amdgcn_readfirstlane(stop_word), fw = __builtin_amdgcn_readfirstlane(flag_word);
@@ -491,7 +510,6 @@ struct PipeKernel {
         if (bias && vec_ok && epi_n < g.N) bias_raw = *(const Vec4<T> *)(bias + epi_n);
 
         // ---- main loop ------------------------------------------------------------------------
-        const int KT = (g.K + BK - 1) / BK;
         GP_PROBE(1);
         __syncthreads();  // the previous tile of this workgroup may still be reading LDS
 #pragma unroll
@@ -503,22 +521,35 @@ struct PipeKernel {
                 load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)early_slot);
         }
         int kt = kt0, stopped = 0;
-        // the K-step of the last look (the first K-step when the tile is too short for another)
-        const int kt_last_look = kt0 + (KT - 1 - kt0) / LOOK_EVERY * LOOK_EVERY;
-        auto announce = [&](int k) {
-            if constexpr (LOOKS)
-                if (looking && cc.announce && k == kt_last_look && tid == 0) __hip_atomic_fetch_add(cc.announce, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        };
+        // Later looks: after the first K-step the tile goes on in runs of LOOK_EVERY K-steps, as many as fit in front
+        // of the last STAGES-1 K-steps.  Wavefront 0 fetches the word in front of a run, everybody reads it behind
+        // the run (the waits and barriers of the K-steps between have made it land and be seen), and the runs take two
+        // landing places in turn, so that the fetch for the next run cannot overwrite a word that a slower wavefront
+        // has still to read.  A run has no way out in the middle: a K-step that may leave the loop, or that tests
+        // whether it is time to look, made the whole loop a quarter slower on 64x64 tiles with K = 4608.
+        const int runs = looking ? max(KT - (kt0 + 1) - (STAGES - 1), 0) / LOOK_EVERY : 0;
         for (; kt + STAGES - 1 < KT; ++kt) {
-            stopped = ktile(kt, false, IntC<1>{});
+            stopped = ktile(kt, false, IntC<1>{}, IntC<0>{});
             if (stopped) break;  // (CKPT: leave the tile here; otherwise only the looks can say so)
-            announce(kt);
+            if constexpr (LOOKS) {
+                if (looking && kt == kt0) {
+                    for (int r = 0; r < runs; ++r) {
+                        int *slot = early_slot + 64 + 64 * (r & 1);
+                        if (wave == 0) load_lds4(cc.stop_index, (unsigned)(size_t)(__attribute__((address_space(3))) void *)slot);
+#pragma nounroll
+                        for (int i = 0; i < LOOK_EVERY; ++i) ktile(++kt, false, IntC<1>{}, IntC<1>{});
+                        if (__builtin_amdgcn_readfirstlane(read_lds_word(slot)) != -1) { stopped = 1; break; }
+                    }
+                    if (stopped) break;
+                }
+            }
         }
         if (!stopped)
             for (; kt < KT; ++kt) {
-                const int st = ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{});
+                const int st = ktile(kt, KT - kt - 1 < STAGES - 2, IntC<0>{}, IntC<0>{});
                 if (!CKPT && st) { stopped = 1; break; }  // (a checkpointing body finishes a tile whose last stages are in flight)
-                announce(kt);
+                if constexpr (LOOKS)
+                    if (looking && kt == kt0 && kt == KT - 1) announce();  // (a tile of one K-step: its early look has just said go on)
             }
         if (!CKPT && stopped) {
             wait_vmcnt<0>();  // operand loads still landing in LDS must not outlive the workgroup

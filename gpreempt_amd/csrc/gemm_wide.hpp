@@ -249,7 +249,7 @@ struct WideKernel {
         }
         auto issue = [&](int s) {
             const int k0 = (s * KB + kb) * BK;          // first K element of this wavefront group's block
-            const unsigned sbase = lds0 + (unsigned)(s % STAGES) * STAGE_BYTES + (unsigned)kb * BLK_BYTES;
+            const unsigned sbase = lds0 + ((unsigned)s % STAGES) * STAGE_BYTES + (unsigned)kb * BLK_BYTES;
             const unsigned tap_bit = (k0 < g.K && nx_tap < 32) ? 1u << nx_tap : 0u;  // blocks past K have no tap
             const int tap_off = (nx_r * g.W + nx_s) * (int)g.lda + nx_ci;  // elements from the window's origin
 #pragma unroll
@@ -301,12 +301,15 @@ struct WideKernel {
             else wait_vmcnt<0>();
             __syncthreads();  // everyone's part of stage s is visible; the buffer of stage s-1 is free
             if (s == 0) GP_PROBE(2);
-            if (((s == 0 && early) || (looking && s > 0 && (s & (LOOK_EVERY - 1)) == 0)) && __builtin_amdgcn_readfirstlane(*(volatile int *)early_slot) != -1) {
+            if (((s == 0 && early) || (looking && s > 0 && (s & (LOOK_EVERY - 1)) == 0)) && __builtin_amdgcn_readfirstlane(read_lds_word(early_slot)) != -1) {
                 wait_vmcnt<0>();  // loads still landing in LDS must not outlive the workgroup
                 return true;      // the tile is given up: the caller withdraws the claim
             }
-            if constexpr (LOOKS) {  // the last look: the workgroup counts itself (tile_fixed_early)
-                if (looking && cc.announce && s == (NS - 1) / LOOK_EVERY * LOOK_EVERY && tid == 0)
+            if constexpr (LOOKS) {
+                // the last stage: the workgroup counts itself (tile_fixed_early).  Not earlier: an atomic in front of operand
+                // loads is waited for with them (the waits count in the order of issue), and its acknowledgement takes
+                // microseconds when every resident workgroup sends one.
+                if (looking && cc.announce && s == NS - 1 && tid == 0)
                     __hip_atomic_fetch_add(cc.announce, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
             if (s >= PRE - (STAGES - 1) && s + STAGES - 1 < NS) {
@@ -315,7 +318,7 @@ struct WideKernel {
                 issue(s + STAGES - 1);
             }
             if (kb >= G) continue;  // (uniform) the other wavefronts only fetch
-            const int stage = s % STAGES;
+            const int stage = (int)((unsigned)s % STAGES);
 #pragma unroll
             for (int b = 0; b < KB; ++b) {
                 // a block past the last one holds zeros; it is skipped, not multiplied, so that the sum

@@ -324,7 +324,7 @@ __device__ __forceinline__ void leave_stamped(const BlpArgs &b, bool count = tru
         if (leader) stamp_exit_leader(b.stamps);
     }
     // (no value comes back: the atomic costs the leaver nothing; one line per group keeps them from queueing up on one address)
-    // (count == false: the body has counted the workgroup already, a few K-stages before the end of its tile)
+    // (count == false: the body has counted the workgroup already, at the top of the last K-step of its tile)
     if (b.done && count && leader) __hip_atomic_fetch_add(done_counter(b), 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
@@ -428,9 +428,10 @@ __device__ __forceinline__ void unclaim_fixed(const BlpArgs &b) {
 // a stop word that reaches the body in a vector register (a value merged from two branches does)
 // makes the compiler treat the body's control flow as divergent, and the body, whose barriers and
 // hand-placed waits assume uniform flow, then computes garbage for K of one step.
-// ANNOUNCES: a body that was handed a stop word counts its workgroup in b.done itself when it is a few K-stages from the
-// end of a tile that it finishes (so that the front workgroup is gone by the time the workers are: the launch lasts until
-// the last workgroup has left, and the front one needs a microsecond or two to notice and to get its read of the flag back).
+// ANNOUNCES: a body that was handed a stop word counts its workgroup in b.done itself at the top of the last K-step of a
+// tile that it finishes, a microsecond or two before it leaves (so that the front workgroup is gone by the time the
+// workers are: the launch lasts until the last workgroup has left, and the front one needs a microsecond or two to notice
+// and to get its read of the flag back).
 template <bool ANNOUNCES = false, class Body>
 __device__ __forceinline__ void tile_fixed_early(const BlpArgs &b, Body &&body) {
     const bool eager = b.fresh > 1;
