@@ -153,11 +153,7 @@ struct PipeKernel {
         // word is fetched by wavefront 0 at the top of the K-step in which the stage it travels with is fetched, in
         // front of that stage's loads, and read by everybody at the end of that stage's K-step.  A tile that finds a
         // stop recorded is given up (the caller withdraws the claim; the relaunch computes it from the start).
-#ifdef GP_LOOK_EVERY
-        constexpr int LOOK_EVERY = GP_LOOK_EVERY;
-#else
         constexpr int LOOK_EVERY = 8;
-#endif
         static_assert(LOOK_EVERY >= STAGES, "a look is read before the next one is fetched");
         // (an instantiation of its own, LOOKS: as a run-time switch the looks cost the short tiles 3 % of a ResNet-152 pass)
         const bool looking = LOOKS && early;
@@ -525,8 +521,8 @@ struct PipeKernel {
         // of the last STAGES-1 K-steps.  Wavefront 0 fetches the word in front of a run, everybody reads it behind
         // the run (the waits and barriers of the K-steps between have made it land and be seen), and the runs take two
         // landing places in turn, so that the fetch for the next run cannot overwrite a word that a slower wavefront
-        // has still to read.  A run has no way out in the middle: a K-step that may leave the loop, or that tests
-        // whether it is time to look, made the whole loop a quarter slower on 64x64 tiles with K = 4608.
+        // has still to read.  A run has no way out in the middle and tests nothing: its K-steps are the plain ones of the
+        // steady state.
         const int runs = looking ? max(KT - (kt0 + 1) - (STAGES - 1), 0) / LOOK_EVERY : 0;
         for (; kt + STAGES - 1 < KT; ++kt) {
             stopped = ktile(kt, false, IntC<1>{}, IntC<0>{});
