@@ -150,9 +150,10 @@ typedef struct gp_preempt_ctx {
     unsigned long long ckpt_bytes;
     int *done;       /* may be NULL.  Counters laid out like `executed` (counter_groups of them, 16 ints apart,  */
                      /* cleared together with them) in which every worker workgroup of every launch of this     */
-                     /* kernel counts itself when it leaves.  With them a launch of long tiles (about 10^7      */
-                     /* multiply-adds and more per tile) keeps one workgroup in front of its workers reading    */
-                     /* the preempt flag until all of them have left, and its tiles look at the stop index every */
+                     /* kernel counts itself when it leaves (a K-step earlier when it finishes its tile).  With  */
+                     /* them a launch of long tiles (1.8 * 10^7 multiply-adds and more per tile) keeps one       */
+                     /* workgroup in front of its workers reading the preempt flag until half of the last round  */
+                     /* of them has counted itself, and its tiles look at the stop index every                    */
                      /* few K-stages: a tile that finds a stop recorded is given up (its claim is withdrawn, the */
                      /* relaunch computes it from the start: same bits).  The reference's wrapper can only stop  */
                      /* between tiles (convert_to_blp.py:45-58); a 32 x 32 x 25088 tile of VGG-16's first dense  */
