@@ -986,3 +986,68 @@ def test_long_tiles_are_given_up_on_a_stop_and_redone_bit_exact(gp, family):
         assert st.stop_index() == -1 and np.array_equal(dC.download(), base), attempt
         assert int(st.counters().reshape(32, 16)[:, 0].sum()) == info.total_tiles
     assert given_up >= 1, f"no attempt stopped the launch while its tiles ran (a plain launch takes {whole_us:.0f} us)"
+
+
+_LOOKS_SWEEP = r'''
+import sys, numpy as np
+sys.path.insert(0, sys.argv[1])
+from gpreempt_amd import capi as gp
+gp.init(0)
+rng = np.random.default_rng(11)
+flag = gp.Flag()
+cases = 0
+for variant, tm, tn, M, N, ks in ((gp.MAT_PIPE, 64, 64, 256, 256, (64, 128, 192, 256, 320, 704, 768, 832, 1280)),
+                                  (gp.MAT_PIPE, 128, 128, 256, 256, (64, 192, 256, 704, 1216)),
+                                  (gp.MAT_WIDE, 32, 32, 64, 128, (1024, 2048, 3072, 5120, 9216))):
+    for K in ks:
+        A = rng.uniform(-1, 1, (M, K)).astype(np.float16)
+        B = (rng.uniform(-1, 1, (N, K)) * 0.05).astype(np.float16)
+        dA, dB, dC = gp.DevBuf.from_array(A, gp.F16), gp.DevBuf.from_array(B, gp.F16), gp.DevBuf(M * N * 2)
+        p = gp.GemmParams(dtype=gp.F16, M=M, N=N, K=K, A=dA.ptr, lda=K, B=dB.ptr, ldb=K, b_is_nk=1, C=dC.ptr, ldc=N, alpha=1.0, act=gp.ACT_NONE,
+                          batch=1, tile_m=tm, tile_n=tn, variant=variant)
+        gp.launch("gp_launch_gemm", p, None)
+        gp.check(gp.lib().gp_stream_sync(None))
+        base = dC.download().copy()
+        tiles = (M // tm) * (N // tn)
+        st = gp.BlpState(1, flag, 32)
+        st.enable_done_counters()
+        # (1) no stop: the bits of the plain launch, and every worker counted itself exactly once
+        flag.set(0); st.reset(); st.clear_stop(); dC.fill32(0x7E007E00)
+        info = gp.launch("gp_launch_gemm", p, st.ctx(fresh=1))
+        gp.check(gp.lib().gp_stream_sync(None))
+        assert info.fixed_claims == 1 and info.front == 8 and info.total_tiles == tiles, (variant, tm, K, info.fixed_claims, info.front)
+        assert np.array_equal(dC.download(), base), ("bits", variant, tm, K)
+        done = int(st.done.download(np_dtype=np.int32).reshape(32, 16)[:, 0].sum())
+        assert done == info.grid - info.front, ("done", variant, tm, K, done, info.grid)
+        # (2) the flag up before the launch: tiles are given up wherever they are; the relaunch finishes the rest
+        flag.set(1); st.reset(); st.clear_stop(); dC.fill32(0x7E007E00)
+        info = gp.launch("gp_launch_gemm", p, st.ctx(fresh=1))
+        gp.check(gp.lib().gp_stream_sync(None))
+        made = int(st.counters().reshape(32, 16)[:, 0].sum())
+        done = int(st.done.download(np_dtype=np.int32).reshape(32, 16)[:, 0].sum())
+        assert done == info.grid - info.front, ("done after stop", variant, tm, K, done)
+        part = dC.download(np_dtype=np.uint16).reshape(M // tm, tm, N // tn, tn)
+        assert int((part == 0x7E00).all(axis=(1, 3)).sum()) == tiles - made, ("untouched", variant, tm, K, made)
+        flag.set(0); st.clear_stop()
+        gp.launch("gp_launch_gemm", p, st.ctx(done_launches=1))
+        gp.check(gp.lib().gp_stream_sync(None))
+        assert np.array_equal(dC.download(), base), ("bits after resume", variant, tm, K)
+        assert int(st.counters().reshape(32, 16)[:, 0].sum()) == tiles
+        cases += 1
+print("OK", cases)
+'''
+
+
+def test_looks_at_every_count_of_k_steps(gp):
+    """The instantiation that looks again during a tile, on tiles of 1 to 20 K-steps (no run of 8, exactly one, one and
+    a rest, two; fewer K-steps than stages) and on split-K tiles of 4 to 36 stages: the bits of the plain launch, every
+    worker counted once in gp_preempt_ctx::done whether it finished its tile or gave it up, and a launch that finds
+    the flag up leaves its tiles unwritten for the relaunch.  The threshold that selects the instantiation is read
+    once per process, hence the child process with GPREEMPT_LONG_TILE_MACS=1."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", _LOOKS_SWEEP, root], capture_output=True, text=True, timeout=110,
+                         env={**os.environ, "GPREEMPT_LONG_TILE_MACS": "1"})
+    assert out.returncode == 0 and out.stdout.strip().startswith("OK 19"), (out.stdout[-300:], out.stderr[-1500:])
