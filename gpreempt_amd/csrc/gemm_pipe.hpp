@@ -150,11 +150,11 @@ struct PipeKernel {
         // that depends on it as divergent, and the barriers and hand-placed waits below assume uniform control flow)
         const bool early = !CKPT && __builtin_amdgcn_readfirstlane((int)(cc.stop_index != nullptr)) != 0;
         // Long tiles look again every LOOK_EVERY K-steps (a K-step is 64 elements, a quarter to half a microsecond): the
-        // word is fetched by wavefront 0 at the top of the K-step in which the stage it travels with is fetched, in
-        // front of that stage's loads, and read by everybody at the end of that stage's K-step.  A tile that finds a
-        // stop recorded is given up (the caller withdraws the claim; the relaunch computes it from the start).
+        // word is fetched by wavefront 0 in front of a run of LOOK_EVERY K-steps and read by everybody behind the run
+        // (the main loop below).  A tile that finds a stop recorded is given up (the caller withdraws the claim; the
+        // relaunch computes it from the start).
         constexpr int LOOK_EVERY = 8;
-        static_assert(LOOK_EVERY >= STAGES, "a look is read before the next one is fetched");
+        static_assert(LOOK_EVERY >= STAGES, "the waits of a run's K-steps cover the fetch in front of it");
         // (an instantiation of its own, LOOKS: as a run-time switch the looks cost the short tiles 3 % of a ResNet-152 pass)
         const bool looking = LOOKS && early;
         const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) void *)lds_t;
