@@ -131,8 +131,8 @@ int plan_launch(Kernel kernel, int block, size_t lds_bytes, int sx, int sy, int 
             *grid = workers;
             blp->spare = 0; blp->front = 8;
             blp->done = ctx->done;
-            // (the front workgroup leaves when half of the last round of workers has counted itself, which a worker does a
-            // few K-stages before the end of its tile: the microsecond or two in which the front workgroup notices and
+            // (the front workgroup leaves when half of the last round of workers has counted itself, which a worker does at
+            // the top of the last K-step of its tile: the microsecond or two in which the front workgroup notices and
             // gets its last read of the flag back would otherwise come on top of every launch, 2.5 us on each of
             // ResNet-50's fp32 kernels)
             const int last_round = (int)(workers < resident ? workers : resident);
